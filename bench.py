@@ -1,0 +1,180 @@
+#!/usr/bin/env python3
+"""Benchmark of the paged decode-attention hot path on one MI355X.
+
+One step = one ``pa_decode`` call (split-K pass + reduction pass) over one
+batch of the synthetic workload, inputs resident in HBM.  The headline
+workload is BASELINE configuration 4 (Llama-3-8B shape, B=256, bf16 pool,
+lognormal context lengths, seed 1004).  Prints one JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1]
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
+
+# HBM traffic of one decode_split_kernel launch on workload c4, from
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/); None until measured.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c4", "c5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
+    return ap.parse_args()
+
+
+def cpu_baseline(w, budget_s: float):
+    """Time the vectorised CPU restatement (index gather + SDPA per sequence) on a bounded sample."""
+    from oracle import paged_oracle as po
+
+    threads = torch.get_num_threads()
+    order = np.argsort(w.seq_lens)  # shortest first so the sample can be cut to the budget
+    tables = [w.block_tables[i].tolist() for i in order]
+    lens = w.seq_lens[order]
+    q = w.q[torch.from_numpy(order)][:, None]
+    k_pool, v_pool = w.k_pool, w.v_pool
+    if w.kv_format == "fp8_e4m3":  # the CPU path of the fp8 workload is dequantise-then-attend
+        kb, ks = po.quantize_kv_e4m3(k_pool, w.block_size)
+        vb, vs = po.quantize_kv_e4m3(v_pool, w.block_size)
+        k_pool = po.dequantize_kv_e4m3(kb, ks, w.block_size).to(w.dtype)
+        v_pool = po.dequantize_kv_e4m3(vb, vs, w.block_size).to(w.dtype)
+    done_tokens, done_seqs, t0 = 0, 0, time.perf_counter()
+    while done_seqs < len(lens) and time.perf_counter() - t0 < budget_s:
+        n = min(4, len(lens) - done_seqs)
+        sl = slice(done_seqs, done_seqs + n)
+        po.decode_per_sequence(q[sl], k_pool, v_pool, tables[sl], lens[sl], w.block_size, w.scale)
+        done_seqs += n
+        done_tokens += int(lens[sl].sum())
+    dt = time.perf_counter() - t0
+    kv_size = w.q.element_size()
+    sample_bytes = done_tokens * w.num_kv_heads * w.head_dim * 2 * kv_size
+    return {
+        "value": sample_bytes / dt / 1e9,
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "tokens_per_s": done_seqs / dt,
+        "sample": f"{done_seqs} shortest of {len(lens)} sequences of {w.name} ({done_tokens} keys), "
+                  f"per-sequence index gather + torch SDPA on {threads} threads, {dt:.1f} s",
+    }
+
+
+def main() -> int:
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1", file=sys.stderr)
+        return 2
+    from research_amd import _lib, ops
+    from research_amd.workloads import make_decode
+
+    _lib.load()  # no fallback: raises if the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    t_gen = time.perf_counter()
+    w = make_decode(args.workload)
+    t_gen = time.perf_counter() - t_gen
+
+    q = w.q.to(dev)
+    if w.kv_format == "fp8_e4m3":
+        k_pool, k_scale = ops.quantize_kv_e4m3(w.k_pool.to(dev), w.block_size)
+        v_pool, v_scale = ops.quantize_kv_e4m3(w.v_pool.to(dev), w.block_size)
+    else:
+        k_pool, v_pool, k_scale, v_scale = w.k_pool.to(dev), w.v_pool.to(dev), None, None
+    tables = torch.from_numpy(w.padded_tables()).to(dev)
+    lens = torch.from_numpy(w.seq_lens.astype(np.int32)).to(dev)
+    chunk = ops.decode_plan(w.total_tokens, w.batch, w.num_kv_heads, w.block_size)
+    total_chunks = int((-(-w.seq_lens // chunk)).sum())
+    ws = torch.empty(ops.decode_workspace_bytes(total_chunks, w.batch, w.num_q_heads, w.head_dim),
+                     dtype=torch.uint8, device=dev)
+    out = torch.empty_like(q)
+
+    def step(entry="pa_decode"):
+        ops.decode(q, k_pool, v_pool, tables, lens, w.block_size, w.scale, chunk, total_chunks, ws,
+                   k_scale=k_scale, v_scale=v_scale, out=out, entry=entry)
+
+    def timed(entry, steps):
+        """Average milliseconds per launch: HIP events on the launch stream around `steps` calls."""
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        start.record()
+        for _ in range(steps):
+            step(entry)
+        stop.record()
+        torch.cuda.synchronize()
+        return start.elapsed_time(stop) / steps
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    wall = time.perf_counter()
+    ms_step = timed("pa_decode", args.steps)
+    wall = time.perf_counter() - wall
+    ms_split = timed("pa_decode_split", args.steps)  # the dominant kernel alone
+    ms_reduce = timed("pa_decode_reduce", args.steps)
+
+    alg_bytes = w.algorithmic_bytes()
+    achieved = alg_bytes / (ms_split * 1e-3) / 1e9
+    traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
+    result = {
+        "metric": "decode-attn HBM GB/s",
+        "value": alg_bytes / (ms_step * 1e-3) / 1e9,
+        "unit": "GB/s",
+        "pct_of_hbm_peak": 100.0 * alg_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+        "tokens_per_s": w.batch / (ms_step * 1e-3),
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "wall_ms_per_step": wall * 1e3 / args.steps,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16" if w.dtype == torch.bfloat16 else str(w.dtype).replace("torch.", ""),
+        "data": "synthetic",
+        "config": {
+            "workload": {"c1": "c1 fp32 decode B=4", "c2": "c2 Qwen3-0.6B-shaped decode B=64 bf16",
+                         "c4": "c4 Llama-3-8B-shaped decode B=256 bf16 paged KV",
+                         "c5": "c5 long-context fp8-e4m3 KV decode B=8"}[args.workload],
+            "batch": w.batch, "num_q_heads": w.num_q_heads, "num_kv_heads": w.num_kv_heads,
+            "head_dim": w.head_dim, "block_size": w.block_size, "total_keys": w.total_tokens,
+            "max_len": int(w.seq_lens.max()), "kv_format": w.kv_format or str(w.dtype).replace("torch.", ""),
+            "chunk_tokens": chunk, "total_chunks": total_chunks, "algorithmic_bytes": alg_bytes,
+            "seed": 1000 + int(args.workload[1]), "generate_s": round(t_gen, 1),
+        },
+        "roofline": {
+            "bound": "hbm", "kernel": "decode_split_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
+            "kernel_ms": ms_split, "reduce_kernel_ms": ms_reduce,
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,192 @@
+/*
+ * paged_attn.h - C ABI of libpaged_attn.so: paged-KV attention for one MI355X
+ * (gfx950) behind the attention / KV-cache call surface of the `rollouts`
+ * inference engine.
+ *
+ * Conventions for every entry point
+ *   - plain pointers and sizes; device pointers unless the name says host;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *     work is enqueued asynchronously on it, nothing synchronises;
+ *   - the return value is a status: PA_OK, or a negative PA_ERR_* after which
+ *     pa_last_error() (thread-local text) says what was wrong.  Arguments are
+ *     checked on the host before any HIP call, so a rejected call has touched
+ *     neither the GPU nor its buffers;
+ *   - the library allocates nothing: the caller owns inputs, outputs and the
+ *     decode workspace;
+ *   - indices read from device memory (slots, block ids) are range-checked by
+ *     the kernels against `total_slots` / `num_blocks`: an out-of-range index
+ *     is skipped (append) or reads as zeros (gather, attention), never a fault.
+ *
+ * Pool layout (fixed by the reference, attention/config.py:43-45, one layer's
+ * slice): element [slot][kv_head][d] at ((slot*num_kv_heads)+kv_head)*head_dim+d,
+ * slot = block_id*block_size + offset_in_block.
+ *
+ * Reference citations are relative to rollouts/rollouts/inference/.
+ */
+#ifndef PAGED_ATTN_H
+#define PAGED_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PA_OK 0
+#define PA_ERR_INVALID_ARG (-1) /* NULL pointer, negative size, inconsistent dims */
+#define PA_ERR_UNSUPPORTED (-2) /* dtype / head_dim / group size has no kernel */
+#define PA_ERR_WORKSPACE (-3)   /* decode workspace missing or too small */
+#define PA_ERR_HIP (-4)         /* a HIP launch reported an error */
+
+/* element types of q / out / the KV pool */
+#define PA_F32 0
+#define PA_BF16 1
+#define PA_F16 2
+#define PA_FP8_E4M3 3 /* OCP e4m3fn, KV pool only; q/out stay 16- or 32-bit */
+
+/* Library ABI version (bumped when a signature changes). */
+int pa_version(void);
+
+/* Text of the calling thread's most recent error; "" if none. */
+const char *pa_last_error(void);
+
+/* Bytes per element of a PA_* dtype, or 0 for an unknown code. */
+int pa_dtype_bytes(int dtype);
+
+/*
+ * KV append / scatter.  Replaces FlexAttentionBackend._store_kv
+ * (attention/flex_backend.py:116-142):
+ *     for i in range(n_tokens): s = slots[i]
+ *         if s >= 0: k_cache[s] = k_src[i]; v_cache[s] = v_src[i]
+ * A pure byte copy of rows of num_kv_heads*head_dim elements; rows whose slot
+ * is negative (the reference's filter, :139-142) or >= total_slots are
+ * dropped.  Duplicate slots in one call: which source row wins is unspecified
+ * (as for the reference's index_put on a GPU).
+ *   k_cache,v_cache : one layer's pool slice, [total_slots][row]
+ *   k_src,v_src     : [n_tokens][row], contiguous
+ *   slots           : int64[n_tokens]
+ *   elem_bytes      : 1, 2 or 4; row bytes must be a multiple of 4
+ */
+int pa_kv_scatter(void *k_cache, void *v_cache, const void *k_src, const void *v_src,
+                  const int64_t *slots, int64_t n_tokens, int64_t total_slots,
+                  int num_kv_heads, int head_dim, int elem_bytes, void *stream);
+
+/*
+ * Block-table gather.  Replaces FlexAttentionBackend._gather_kv_from_cache
+ * (attention/flex_backend.py:233-279):
+ *     out[b][pos] = cache[bt[b][pos / bs] * bs + pos % bs]   for pos < seq_lens[b]
+ * and zeros for pos >= seq_lens[b], for positions whose block-table entry is
+ * missing (the reference's short-table case, :274; here: entry < 0, entry >=
+ * num_blocks, or pos / bs >= bt_stride), up to max_len.  Bit-exact copy.
+ *   block_tables : int32[batch][bt_stride], row-padded with -1
+ *   seq_lens     : int32[batch]
+ *   k_out,v_out  : [batch][max_len][row], every byte is written
+ */
+int pa_kv_gather(const void *k_cache, const void *v_cache, void *k_out, void *v_out,
+                 const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
+                 int batch, int64_t max_len, int64_t num_blocks, int block_size,
+                 int num_kv_heads, int head_dim, int elem_bytes, void *stream);
+
+/*
+ * Split-K planning for pa_decode (host arithmetic only, no GPU call).
+ * pa_decode cuts every sequence into chunks of `chunk_tokens` keys (a multiple
+ * of block_size); one workgroup pass handles one chunk of one sequence and the
+ * partial results are merged by a reduction pass.
+ *   pa_decode_chunk_tokens   : suggested chunk size for a batch holding
+ *                              total_tokens keys (sum of seq_lens); <= 0 on error
+ *   pa_decode_workspace_bytes: workspace needed when the batch has at most
+ *                              total_chunks = sum_b ceil(seq_lens[b]/chunk_tokens)
+ *                              chunks (batch*ceil(max_seq_len/chunk_tokens) is
+ *                              always enough); 0 on error
+ */
+int pa_decode_chunk_tokens(int64_t total_tokens, int batch, int num_kv_heads, int block_size);
+size_t pa_decode_workspace_bytes(int64_t total_chunks, int batch, int num_q_heads, int head_dim);
+
+/*
+ * Paged decode attention.  Replaces FlexAttentionBackend._decode_attention
+ * (attention/flex_backend.py:187-231) together with the gather and the GQA
+ * repeat_interleave it performs: for sequence b and query head h
+ *     kvh = h / (num_q_heads / num_kv_heads)
+ *     out[b][h] = softmax_j( scale * q[b][h] . K[b][j][kvh] ) . V[b][j][kvh],  j < seq_lens[b]
+ * with K/V rows addressed through the block table as in pa_kv_gather; a
+ * position whose block-table entry is missing acts as an all-zero key and
+ * value (logit 0), as it does in the reference.  Accumulation is fp32.
+ *   q, out        : [batch][num_q_heads][head_dim], dtype q_dtype
+ *   kv_dtype      : q_dtype, or PA_FP8_E4M3 with k_scale/v_scale =
+ *                   float[num_blocks][num_kv_heads] (value = fp8 * scale)
+ *   extra_zero_keys: NULL, or int32[batch]: that many additional all-zero
+ *                   keys take part in sequence b's softmax.  The reference
+ *                   zero-pads ragged batches to the longest sequence without a
+ *                   mask (:253-264, :227-229); passing max_len - seq_lens[b]
+ *                   reproduces it.
+ *   chunk_tokens, total_chunks, workspace(_bytes): see the planning calls.
+ *   A sequence of length 0 with no extra keys yields zeros.
+ */
+int pa_decode(const void *q, const void *k_cache, const void *v_cache, void *out,
+              const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
+              const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale,
+              int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+              int64_t num_blocks, float scale, int q_dtype, int kv_dtype, int chunk_tokens,
+              int64_t total_chunks, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The two passes of pa_decode as separate calls, same arguments: pa_decode ==
+ * pa_decode_split followed by pa_decode_reduce on the same stream and
+ * workspace.  For callers that time or schedule the passes separately, or
+ * merge several split passes' workspaces themselves.  (The reference has one
+ * fused call site, attention/flex_backend.py:227-229; these have no separate
+ * counterpart there.)
+ */
+int pa_decode_split(const void *q, const void *k_cache, const void *v_cache, void *out,
+                    const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
+                    const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale,
+                    int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+                    int64_t num_blocks, float scale, int q_dtype, int kv_dtype, int chunk_tokens,
+                    int64_t total_chunks, void *workspace, size_t workspace_bytes, void *stream);
+int pa_decode_reduce(const void *q, const void *k_cache, const void *v_cache, void *out,
+                     const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
+                     const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale,
+                     int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+                     int64_t num_blocks, float scale, int q_dtype, int kv_dtype, int chunk_tokens,
+                     int64_t total_chunks, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Causal prefill attention over a paged context.  Covers both
+ * FlexAttentionBackend._prefill_attention (attention/flex_backend.py:144-185,
+ * the is_causal SDPA over the step's own K/V) and chunked prefill over cached
+ * prefix blocks (a composition the reference does not have): for sequence b
+ * the q_lens[b] query rows are the LAST q_lens[b] positions of a context of
+ * ctx_lens[b] keys, and row i attends keys j <= ctx_lens[b] - q_lens[b] + i.
+ * The keys are read through the block table, so the step's new K/V must have
+ * been appended (pa_kv_scatter) first.  Sequences that list the same block
+ * ids share those blocks.
+ *   q, out   : [total_q][num_q_heads][head_dim] packed rows, sequence b's rows
+ *              start at q_starts[b]; dtype PA_BF16 or PA_F16 (MFMA path) or
+ *              PA_F32 (vector path)
+ *   ctx_lens, q_lens, q_starts : int32[batch]
+ *   max_q_len: upper bound of q_lens (grid sizing)
+ */
+int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, void *out,
+                     const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
+                     const int32_t *q_lens, const int32_t *q_starts, int batch, int max_q_len,
+                     int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+                     int64_t num_blocks, float scale, int dtype, void *stream);
+
+/*
+ * fp8-e4m3 pool construction (no counterpart in the reference; its oracle is
+ * "dequantise, then attend in fp32").  For every (block, kv head):
+ *     s = max|x| / 448  (s = 1 when the block is all zero)
+ *     dst = e4m3fn_rne(x / s),  scale[block][kv_head] = s
+ *   src   : [num_blocks*block_size][num_kv_heads][head_dim], src_dtype F32/BF16/F16
+ *   dst   : same shape, one byte per element
+ *   scale : float[num_blocks][num_kv_heads]
+ */
+int pa_quantize_kv_e4m3(const void *src, void *dst, float *scale, int64_t num_blocks,
+                        int block_size, int num_kv_heads, int head_dim, int src_dtype,
+                        void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PAGED_ATTN_H */

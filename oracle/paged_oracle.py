@@ -1,0 +1,315 @@
+"""CPU restatement of the reference's paged attention path.  TEST INFRASTRUCTURE.
+
+Nothing in the product imports this file: it exists so that tests, the smoke
+check and the CPU-baseline leg of the benchmark can compare the HIP path with
+an independent statement of what the reference computes.  It never imports
+the reference; each function cites the reference lines it restates
+(paths relative to rollouts/rollouts/inference/).
+
+Two families:
+
+* ``*_literal`` functions follow the reference statement by statement with the
+  same PyTorch calls (Python gather loop, ``repeat_interleave``,
+  ``scaled_dot_product_attention``).  They are the timed CPU baseline and the
+  arbiter for the reference's ragged-batch zero-padding behaviour.
+* the numpy functions compute the same mathematics directly in float64
+  (explicit softmax) at exact sequence lengths; they are what the HIP results
+  are compared with.
+
+How each function is pinned (see tests/test_oracle.py):
+  kv_scatter            the reference's own assertion (slots 0..3 -> rows 0..3,
+                        examples/inference/test_kv_cache.py:106-111), closed form
+  kv_gather_padded      closed form slot = bt[pos//bs]*bs + pos%bs, brute force
+                        loop on small pools, gather(scatter(x)) = x
+  paged_decode          pure-Python softmax on tiny inputs; torch SDPA on the
+                        gathered tensors; invariance under pool permutation;
+                        GQA vs explicitly expanded heads; constant V
+  paged_decode(pad_zero_keys=True)
+                        equals ``decode_literal`` (SDPA over the zero-padded
+                        batch) and the closed form with (Lmax-L) extra e^(-m)
+                        terms in the denominator
+  dense_prefill         torch SDPA is_causal=True with the recipe and tolerance
+                        of the reference's test (test_kv_cache.py:321-342)
+  paged_prefill_chunk   rows [P:P+C] of dense_prefill over the whole sequence;
+                        P=0 equals dense_prefill
+  quantize_kv_e4m3      torch.float8_e4m3fn conversion (library definition of
+                        OCP e4m3fn, round to nearest even), known values
+                        464 -> 448, 2**-10 -> 0, max 448
+Parity unpinned by any test of the reference itself: decode values, the
+gather and ragged batches (the reference only asserts shapes there).
+"""
+
+from __future__ import annotations
+
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+# --------------------------------------------------------------------------- helpers
+
+
+def to_f64(x) -> np.ndarray:
+    if isinstance(x, torch.Tensor):
+        return x.detach().to(torch.float64).cpu().numpy()
+    return np.asarray(x, dtype=np.float64)
+
+
+def slot_of(blocks: Sequence[int], pos: int, block_size: int) -> int:
+    """Slot of token position ``pos``; -1 if the table is too short (context.py:35-42, :78-85)."""
+    idx = pos // block_size
+    if idx >= len(blocks):
+        return -1
+    return int(blocks[idx]) * block_size + pos % block_size
+
+
+# --------------------------------------------------------------------------- scatter / gather
+
+
+def kv_scatter(k_cache, v_cache, k_src, v_src, slots: Sequence[int]) -> None:
+    """In place: ``cache[s] = src[i]`` for every ``s = slots[i] >= 0`` (flex_backend.py:116-142).
+
+    ``*_cache``: one layer ``[total_slots, Hkv, D]``; ``*_src``: ``[N, Hkv, D]``
+    (numpy arrays or torch tensors; rows are copied, never converted).
+    """
+    slots = np.asarray(slots, dtype=np.int64)
+    assert slots.shape[0] == k_src.shape[0] == v_src.shape[0]
+    keep = np.nonzero(slots >= 0)[0]
+    for i in keep:  # in order, so that on duplicate slots the last writer wins as on CPU
+        k_cache[int(slots[i])] = k_src[int(i)]
+        v_cache[int(slots[i])] = v_src[int(i)]
+
+
+def kv_gather_padded(k_cache, v_cache, block_tables, seq_lens, block_size: int):
+    """Zero-padded ``[B, max(seq_lens), Hkv, D]`` gather (flex_backend.py:233-279).
+
+    Positions past a sequence's length, and positions whose block index is past
+    the end of that sequence's table (:274), stay zero.  Works on numpy arrays
+    or torch tensors and returns the same kind.
+    """
+    num_seqs, max_len = len(block_tables), int(max(seq_lens))
+    shape = (num_seqs, max_len) + tuple(k_cache.shape[1:])
+    if isinstance(k_cache, torch.Tensor):
+        k_out = torch.zeros(shape, dtype=k_cache.dtype)
+        v_out = torch.zeros(shape, dtype=v_cache.dtype)
+    else:
+        k_out = np.zeros(shape, dtype=k_cache.dtype)
+        v_out = np.zeros(shape, dtype=v_cache.dtype)
+    for b, (blocks, n) in enumerate(zip(block_tables, seq_lens)):
+        blocks = np.asarray(blocks, dtype=np.int64)
+        n_ok = min(int(n), len(blocks) * block_size)
+        if n_ok <= 0:
+            continue
+        pos = np.arange(n_ok)
+        slots = blocks[pos // block_size] * block_size + pos % block_size
+        if isinstance(k_cache, torch.Tensor):
+            idx = torch.from_numpy(slots)
+            k_out[b, :n_ok] = k_cache[idx]
+            v_out[b, :n_ok] = v_cache[idx]
+        else:
+            k_out[b, :n_ok] = k_cache[slots]
+            v_out[b, :n_ok] = v_cache[slots]
+    return k_out, v_out
+
+
+def kv_gather_loop(k_cache, v_cache, block_tables, seq_lens, block_size: int):
+    """The reference's two-level loop, token by token (flex_backend.py:266-277).  Small inputs only."""
+    num_seqs, max_len = len(block_tables), int(max(seq_lens))
+    shape = (num_seqs, max_len) + tuple(k_cache.shape[1:])
+    k_out = torch.zeros(shape, dtype=k_cache.dtype)
+    v_out = torch.zeros(shape, dtype=v_cache.dtype)
+    for b, (blocks, n) in enumerate(zip(block_tables, seq_lens)):
+        for pos in range(int(n)):
+            slot = slot_of(blocks, pos, block_size)
+            if slot >= 0:
+                k_out[b, pos] = k_cache[slot]
+                v_out[b, pos] = v_cache[slot]
+    return k_out, v_out
+
+
+# --------------------------------------------------------------------------- attention (float64, explicit)
+
+
+def _attend_rows(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, n_zero: int = 0,
+                 causal_offset: Optional[int] = None) -> np.ndarray:
+    """softmax(scale * q k^T) v for one kv head group.
+
+    q ``[R, n_rep, D]``, k/v ``[L, D]`` -> ``[R, n_rep, D]``.  ``n_zero`` extra
+    all-zero keys (logit 0, value 0) join the softmax.  ``causal_offset``: row
+    r may only see keys ``j <= causal_offset + r``.
+    """
+    logits = scale * np.einsum("rhd,ld->rhl", q, k)  # [R, n_rep, L]
+    if causal_offset is not None:
+        rows = np.arange(q.shape[0])[:, None, None]
+        cols = np.arange(k.shape[0])[None, None, :]
+        logits = np.where(cols <= causal_offset + rows, logits, -np.inf)
+    m = logits.max(axis=-1, keepdims=True) if logits.shape[-1] else np.full(logits.shape[:-1] + (1,), -np.inf)
+    if n_zero > 0:
+        m = np.maximum(m, 0.0)
+    m = np.where(np.isfinite(m), m, 0.0)
+    p = np.exp(logits - m)
+    den = p.sum(axis=-1, keepdims=True) + n_zero * np.exp(-m)
+    out = np.einsum("rhl,ld->rhd", p, v)
+    with np.errstate(invalid="ignore", divide="ignore"):
+        return np.where(den > 0, out / den, 0.0)
+
+
+def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, block_size: int, scale: float,
+                 pad_zero_keys: bool = False) -> np.ndarray:
+    """Decode attention at exact lengths (flex_backend.py:187-231 with a length mask).
+
+    q ``[B, Hq, D]``; caches ``[total_slots, Hkv, D]``; returns float64 ``[B, Hq, D]``.
+    Query head h reads kv head ``h // (Hq/Hkv)`` - the mapping ``repeat_interleave``
+    on dim 1 produces (:215-217).  Positions whose block is missing from the
+    table are all-zero keys, as in the reference's gather (:274).  With
+    ``pad_zero_keys`` every sequence additionally sees ``max(seq_lens) - len``
+    zero keys: the reference's unmasked attention over the zero-padded batch.
+    A sequence with no keys at all yields zeros.
+    """
+    q, kc, vc = to_f64(q), to_f64(k_cache), to_f64(v_cache)
+    batch, hq, d = q.shape
+    hkv = kc.shape[1]
+    n_rep = hq // hkv
+    max_len = int(max(seq_lens)) if len(seq_lens) else 0
+    out = np.zeros((batch, hq, d))
+    for b in range(batch):
+        n = int(seq_lens[b])
+        blocks = np.asarray(block_tables[b], dtype=np.int64)
+        n_ok = max(0, min(n, len(blocks) * block_size))
+        pos = np.arange(n_ok)
+        slots = blocks[pos // block_size] * block_size + pos % block_size
+        n_zero = (n - n_ok) + (max_len - n if pad_zero_keys else 0)
+        for g in range(hkv):
+            qg = q[b, g * n_rep : (g + 1) * n_rep][None]  # [1, n_rep, D]
+            out[b, g * n_rep : (g + 1) * n_rep] = _attend_rows(qg, kc[slots, g], vc[slots, g], scale, n_zero)[0]
+    return out
+
+
+def dense_prefill(q, k, v, scale: float) -> np.ndarray:
+    """Causal attention over the step's own K/V (flex_backend.py:144-185, SDPA is_causal=True).
+
+    q ``[B, T, Hq, D]``, k/v ``[B, T, Hkv, D]`` -> float64 ``[B, T, Hq, D]``.
+    """
+    q, k, v = to_f64(q), to_f64(k), to_f64(v)
+    batch, t, hq, d = q.shape
+    hkv = k.shape[2]
+    n_rep = hq // hkv
+    out = np.zeros_like(q)
+    for b in range(batch):
+        for g in range(hkv):
+            sl = slice(g * n_rep, (g + 1) * n_rep)
+            out[b, :, sl] = _attend_rows(q[b, :, sl], k[b, :, g], v[b, :, g], scale, causal_offset=0)
+    return out
+
+
+def paged_prefill_chunk(q, k_cache, v_cache, block_tables, prefix_lens, chunk_lens, block_size: int,
+                        scale: float) -> np.ndarray:
+    """Chunked prefill over a cached prefix (composition; not a reference function).
+
+    Defined as: gather keys ``0 .. P+C-1`` through the block table
+    (flex_backend.py:233-279) and attend with a bottom-right aligned causal
+    mask, i.e. chunk row i (absolute position P+i) sees keys ``j <= P+i``.
+    The chunk's own K/V must already be in the cache.  q ``[B, Cmax, Hq, D]``;
+    rows past ``chunk_lens[b]`` give zeros.
+    """
+    q, kc, vc = to_f64(q), to_f64(k_cache), to_f64(v_cache)
+    batch, cmax, hq, d = q.shape
+    hkv = kc.shape[1]
+    n_rep = hq // hkv
+    out = np.zeros_like(q)
+    for b in range(batch):
+        p, c = int(prefix_lens[b]), int(chunk_lens[b])
+        blocks = np.asarray(block_tables[b], dtype=np.int64)
+        pos = np.arange(p + c)
+        slots = blocks[pos // block_size] * block_size + pos % block_size
+        for g in range(hkv):
+            sl = slice(g * n_rep, (g + 1) * n_rep)
+            out[b, :c, sl] = _attend_rows(q[b, :c, sl], kc[slots, g], vc[slots, g], scale, causal_offset=p)
+    return out
+
+
+# --------------------------------------------------------------------------- literal restatement (torch)
+
+
+def decode_literal(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables, seq_lens,
+                   block_size: int, scale: float, vectorised_gather: bool = False) -> torch.Tensor:
+    """The reference's decode, statement by statement (flex_backend.py:187-231, :233-279).
+
+    q ``[B, 1, Hq, D]`` -> ``[B, 1, Hq, D]``.  Gathers a zero-padded batch with
+    the token loop (or its vectorised equivalent), expands kv heads with
+    ``repeat_interleave`` and calls SDPA without any mask.
+    """
+    gather = kv_gather_padded if vectorised_gather else kv_gather_loop
+    k_g, v_g = gather(k_cache, v_cache, block_tables, seq_lens, block_size)
+    n_rep = q.shape[2] // k_cache.shape[1]
+    qt = q.transpose(1, 2)
+    kt, vt = k_g.transpose(1, 2), v_g.transpose(1, 2)
+    if n_rep > 1:
+        kt = kt.repeat_interleave(n_rep, dim=1)
+        vt = vt.repeat_interleave(n_rep, dim=1)
+    out = torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, is_causal=False, scale=scale)
+    return out.transpose(1, 2)
+
+
+def decode_per_sequence(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables, seq_lens,
+                        block_size: int, scale: float) -> torch.Tensor:
+    """Vectorised CPU restatement at exact lengths: per sequence index-gather + SDPA.
+
+    The same library calls as the reference, minus the padding; this is the
+    CPU baseline that stays runnable at the large configurations.
+    """
+    batch, _, hq, d = q.shape
+    n_rep = hq // k_cache.shape[1]
+    out = torch.empty_like(q)
+    for b in range(batch):
+        n = int(seq_lens[b])
+        blocks = np.asarray(block_tables[b], dtype=np.int64)
+        pos = np.arange(n)
+        idx = torch.from_numpy(blocks[pos // block_size] * block_size + pos % block_size)
+        kt = k_cache[idx].transpose(0, 1).unsqueeze(0)  # [1, Hkv, L, D]
+        vt = v_cache[idx].transpose(0, 1).unsqueeze(0)
+        if n_rep > 1:
+            kt = kt.repeat_interleave(n_rep, dim=1)
+            vt = vt.repeat_interleave(n_rep, dim=1)
+        qt = q[b : b + 1].transpose(1, 2)
+        out[b : b + 1] = torch.nn.functional.scaled_dot_product_attention(
+            qt, kt, vt, is_causal=False, scale=scale).transpose(1, 2)
+    return out
+
+
+def prefill_literal(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float) -> torch.Tensor:
+    """The reference's prefill, statement by statement (flex_backend.py:144-185)."""
+    n_rep = q.shape[2] // k.shape[2]
+    qt, kt, vt = q.transpose(1, 2), k.transpose(1, 2), v.transpose(1, 2)
+    if n_rep > 1:
+        kt = kt.repeat_interleave(n_rep, dim=1)
+        vt = vt.repeat_interleave(n_rep, dim=1)
+    return torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, is_causal=True, scale=scale).transpose(1, 2)
+
+
+# --------------------------------------------------------------------------- fp8 e4m3 pool
+
+
+def quantize_kv_e4m3(pool: torch.Tensor, block_size: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per-(block, kv head) absmax quantisation to OCP e4m3fn.
+
+    pool ``[num_blocks*block_size, Hkv, D]`` (any float type) ->
+    (``uint8`` bytes of the same shape, ``float32 [num_blocks, Hkv]`` scales)
+    with scale = absmax/448 (1 for an all-zero tile) and byte = e4m3fn(x/scale),
+    both divisions in fp32, conversion round-to-nearest-even (torch's).
+    """
+    slots, hkv, d = pool.shape
+    nb = slots // block_size
+    x = pool.to(torch.float32).reshape(nb, block_size, hkv, d)
+    amax = x.abs().amax(dim=(1, 3))  # [nb, hkv]
+    scale = torch.where(amax > 0, amax / torch.tensor(448.0, dtype=torch.float32), torch.ones_like(amax))
+    y = (x / scale[:, None, :, None]).to(torch.float8_e4m3fn)
+    return y.reshape(slots, hkv, d).view(torch.uint8), scale
+
+
+def dequantize_kv_e4m3(bits: torch.Tensor, scale: torch.Tensor, block_size: int) -> torch.Tensor:
+    """float32 pool from e4m3fn bytes and per-(block, head) scales."""
+    slots, hkv, d = bits.shape
+    nb = slots // block_size
+    x = bits.view(torch.float8_e4m3fn).to(torch.float32).reshape(nb, block_size, hkv, d)
+    return (x * scale[:, None, :, None]).reshape(slots, hkv, d)

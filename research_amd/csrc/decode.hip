@@ -1,0 +1,185 @@
+// Host entry points of paged decode attention: argument checks, split-K
+// planning arithmetic, workspace layout and the two launches.  The kernels are
+// in decode_impl.h and are instantiated per pool element type in
+// decode_inst_*.hip.
+#include "decode_impl.h"
+
+namespace pa_decode_detail {
+
+KernelSet pa_pick_kernels(int q_dtype, int kv_dtype, int d, int nrep_t) {
+    if (kv_dtype == PA_FP8_E4M3) return pa_kernels_fp8(q_dtype, d, nrep_t);
+    if (q_dtype != kv_dtype) return KernelSet{};
+    if (q_dtype == PA_BF16) return pa_kernels_bf16(d, nrep_t);
+    if (q_dtype == PA_F16) return pa_kernels_f16(d, nrep_t);
+    if (q_dtype == PA_F32) return pa_kernels_f32(d, nrep_t);
+    return KernelSet{};
+}
+
+int pa_fill_head_mapping(PoolArgs &p, int num_q_heads, int num_kv_heads, int head_dim, int kv_dtype) {
+    const int kv_bytes = pa_dtype_bytes(kv_dtype);
+    if (kv_bytes == 0 || (head_dim != 32 && head_dim != 64 && head_dim != 128 && head_dim != 256)) return 0;
+    const int lpr = head_dim * kv_bytes / 16;  // lanes per K/V row
+    const int rpw = 64 / lpr;                  // rows per wave load
+    int hpw = 1;                               // kv heads per wave load: power of two dividing num_kv_heads
+    while (hpw * 2 <= rpw && num_kv_heads % (hpw * 2) == 0) hpw *= 2;
+    const int n_rep = num_q_heads / num_kv_heads;
+    int nrep_t = 1;
+    while (nrep_t < n_rep && nrep_t < 8) nrep_t *= 2;
+    p.hq = num_q_heads;
+    p.hkv = num_kv_heads;
+    p.n_rep = n_rep;
+    p.hpw = hpw;
+    p.tpw = rpw / hpw;
+    p.n_hgroups = num_kv_heads / hpw;
+    p.n_rgroups = (n_rep + nrep_t - 1) / nrep_t;
+    return nrep_t;
+}
+
+}  // namespace pa_decode_detail
+
+using namespace pa_decode_detail;
+
+namespace {
+
+size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+
+// workspace = [chunk_prefix int32[batch+1]] [part_ml float[cap][hq][2]] [part_acc float[cap][hq][D]]
+struct WsLayout {
+    size_t prefix_off, ml_off, acc_off, total;
+};
+WsLayout ws_layout(int64_t cap, int batch, int hq, int d) {
+    WsLayout w;
+    w.prefix_off = 0;
+    w.ml_off = align_up((size_t)(batch + 1) * 4, 256);
+    w.acc_off = w.ml_off + align_up((size_t)cap * hq * 2 * 4, 256);
+    w.total = w.acc_off + align_up((size_t)cap * hq * d * 4, 256);
+    return w;
+}
+
+int num_cus() {
+    static int cached = 0;
+    if (cached == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess ||
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        cached = n;
+    }
+    return cached;
+}
+
+}  // namespace
+
+extern "C" int pa_decode_chunk_tokens(int64_t total_tokens, int batch, int num_kv_heads, int block_size) {
+    pa_clear_error();
+    if (total_tokens < 0 || batch < 0 || num_kv_heads <= 0 || block_size <= 0)
+        return pa_fail(PA_ERR_INVALID_ARG, "pa_decode_chunk_tokens: negative size or non-positive head count / block size");
+    // Aim for a few thousand chunks across the batch, between 256 and 1024 keys
+    // each: enough work items to keep 256 CUs busy through the tail, few enough
+    // that the partials stay a small fraction of the KV bytes.
+    int64_t target = 256;
+    const int64_t want_chunks = 4096;
+    while (target < 1024 && total_tokens / target > want_chunks) target *= 2;
+    int64_t blocks = (target + block_size - 1) / block_size;
+    if (blocks < 1) blocks = 1;
+    return (int)(blocks * block_size);
+}
+
+extern "C" size_t pa_decode_workspace_bytes(int64_t total_chunks, int batch, int num_q_heads, int head_dim) {
+    pa_clear_error();
+    if (total_chunks < 0 || batch < 0 || num_q_heads <= 0 || head_dim <= 0) {
+        pa_fail(PA_ERR_INVALID_ARG, "pa_decode_workspace_bytes: negative size or non-positive head count / head_dim");
+        return 0;
+    }
+    return ws_layout(total_chunks, batch, num_q_heads, head_dim).total;
+}
+
+namespace {
+
+enum { kPhaseSplit = 1, kPhaseReduce = 2 };
+
+int decode_launch(int phases, const void *q, const void *k_cache, const void *v_cache, void *out,
+                  const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
+                  const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale, int batch,
+                  int num_q_heads, int num_kv_heads, int head_dim, int block_size, int64_t num_blocks, float scale,
+                  int q_dtype, int kv_dtype, int chunk_tokens, int64_t total_chunks, void *workspace,
+                  size_t workspace_bytes, void *stream) {
+    pa_clear_error();
+    PA_REQUIRE(batch >= 0, "batch=%d is negative", batch);
+    PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, "head counts / head_dim must be positive");
+    PA_REQUIRE(num_q_heads % num_kv_heads == 0, "num_q_heads=%d is not a multiple of num_kv_heads=%d",
+               num_q_heads, num_kv_heads);
+    PA_REQUIRE(block_size > 0, "block_size=%d must be positive", block_size);
+    PA_REQUIRE(num_blocks >= 0 && bt_stride >= 0, "num_blocks / bt_stride must be non-negative");
+    PA_REQUIRE(num_blocks * (int64_t)block_size < (1ll << 40), "pool of %lld blocks is too large", (long long)num_blocks);
+    PA_REQUIRE(chunk_tokens > 0 && chunk_tokens % block_size == 0,
+               "chunk_tokens=%d is not a positive multiple of block_size=%d", chunk_tokens, block_size);
+    PA_REQUIRE(total_chunks >= 0 && total_chunks < (1ll << 30), "total_chunks=%lld out of range",
+               (long long)total_chunks);
+    DecodeArgs a;
+    const int nrep_t = pa_fill_head_mapping(a.p, num_q_heads, num_kv_heads, head_dim, kv_dtype);
+    const KernelSet ks = nrep_t ? pa_pick_kernels(q_dtype, kv_dtype, head_dim, nrep_t) : KernelSet{};
+    if (!ks.split)
+        return pa_fail(PA_ERR_UNSUPPORTED, "pa_decode: no kernel for q_dtype=%d kv_dtype=%d head_dim=%d", q_dtype,
+                       kv_dtype, head_dim);
+    PA_REQUIRE(batch <= kMaxBatch, "batch=%d above the %d sequences one call handles", batch, kMaxBatch);
+    if (batch == 0) return PA_OK;
+    PA_REQUIRE(q && out && seq_lens, "NULL q / out / seq_lens");
+    PA_REQUIRE(k_cache && v_cache, "NULL cache pointer");
+    PA_REQUIRE(block_tables || bt_stride == 0, "NULL block_tables with bt_stride=%lld", (long long)bt_stride);
+    PA_REQUIRE(kv_dtype != PA_FP8_E4M3 || (k_scale && v_scale), "fp8 KV needs k_scale and v_scale");
+    PA_REQUIRE(pa_aligned16(k_cache) && pa_aligned16(v_cache), "cache pointers must be 16-byte aligned");
+    const WsLayout w = ws_layout(total_chunks, batch, num_q_heads, head_dim);
+    if (!workspace || workspace_bytes < w.total)
+        return pa_fail(PA_ERR_WORKSPACE, "pa_decode: workspace of %zu bytes, need %zu", workspace_bytes, w.total);
+    PA_REQUIRE(((uintptr_t)workspace & 255u) == 0, "workspace must be 256-byte aligned");
+
+    a.p.k = k_cache; a.p.v = v_cache; a.p.bt = block_tables; a.p.bt_stride = bt_stride;
+    a.p.k_scale = k_scale; a.p.v_scale = v_scale;
+    a.p.bs = block_size; a.p.num_blocks = num_blocks;
+    a.p.scale_log2 = scale * 1.4426950408889634f;
+    a.q = q; a.out = out; a.seq_lens = seq_lens; a.extra_zero = extra_zero_keys;
+    a.batch = batch;
+    a.chunk_blocks = chunk_tokens / block_size;
+    a.chunk_cap = total_chunks;
+    char *ws = (char *)workspace;
+    a.chunk_prefix = (int32_t *)(ws + w.prefix_off);
+    a.part_ml = (float *)(ws + w.ml_off);
+    a.part_acc = (float *)(ws + w.acc_off);
+
+    hipStream_t s = (hipStream_t)stream;
+    const int64_t max_items = total_chunks * a.p.n_hgroups * a.p.n_rgroups;
+    const int64_t persistent = (int64_t)num_cus() * 4;
+    // At least one workgroup always runs: it publishes the chunk prefix the
+    // reduction pass reads, even when there is no chunk to process.
+    const int64_t want = max_items < persistent ? max_items : persistent;
+    const unsigned grid = (unsigned)(want < 1 ? 1 : want);
+    if (phases & kPhaseSplit) {
+        ks.split<<<dim3(grid), dim3(kThreads), (size_t)(batch + 1) * sizeof(int), s>>>(a);
+        PA_CHECK_LAUNCH("pa_decode split pass");
+    }
+    if (phases & kPhaseReduce) {
+        int red_threads = head_dim < 64 ? 64 : head_dim;
+        if (red_threads > 256) red_threads = 256;
+        ks.reduce<<<dim3((unsigned)(batch * num_q_heads)), dim3(red_threads), 0, s>>>(a);
+        PA_CHECK_LAUNCH("pa_decode reduction pass");
+    }
+    return PA_OK;
+}
+
+}  // namespace
+
+#define PA_DECODE_PARAMS                                                                                       \
+    const void *q, const void *k_cache, const void *v_cache, void *out, const int32_t *block_tables,          \
+        int64_t bt_stride, const int32_t *seq_lens, const int32_t *extra_zero_keys, const float *k_scale,      \
+        const float *v_scale, int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,      \
+        int64_t num_blocks, float scale, int q_dtype, int kv_dtype, int chunk_tokens, int64_t total_chunks,    \
+        void *workspace, size_t workspace_bytes, void *stream
+#define PA_DECODE_ARGS                                                                                         \
+    q, k_cache, v_cache, out, block_tables, bt_stride, seq_lens, extra_zero_keys, k_scale, v_scale, batch,     \
+        num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, q_dtype, kv_dtype, chunk_tokens,   \
+        total_chunks, workspace, workspace_bytes, stream
+
+extern "C" int pa_decode(PA_DECODE_PARAMS) { return decode_launch(kPhaseSplit | kPhaseReduce, PA_DECODE_ARGS); }
+extern "C" int pa_decode_split(PA_DECODE_PARAMS) { return decode_launch(kPhaseSplit, PA_DECODE_ARGS); }
+extern "C" int pa_decode_reduce(PA_DECODE_PARAMS) { return decode_launch(kPhaseReduce, PA_DECODE_ARGS); }

@@ -1,0 +1,457 @@
+// Paged attention of single query rows for gfx950: the split-K decode kernel,
+// its reduction pass, and a row-per-workgroup kernel that evaluates causal
+// prefill one query row at a time (the vector path for element types that
+// have no matrix-core kernel).
+//
+// Work decomposition (decode)
+//   Every sequence is cut into chunks of `chunk_blocks` pool blocks.  One work
+//   item = (chunk, group of kv heads, group of <= NREP query heads per kv
+//   head).  A persistent grid of 256-thread workgroups walks the items with a
+//   grid stride; each workgroup first builds the per-sequence chunk prefix sum
+//   in LDS (seq_lens live on the device, the host never reads them) and finds
+//   an item's sequence by binary search in it.
+//
+// Lane layout (wave64)
+//   A K or V row of one (token, kv head) is D elements = LPR lanes x 16 bytes,
+//   so one 128-bit load instruction of a wave fetches RPW = 64/LPR rows.  The
+//   pool is token-major ([slot][kv_head][d]); the RPW rows are mapped to HPW
+//   neighbouring kv heads of TPW consecutive tokens (HPW*TPW = RPW) so that a
+//   wave's load covers HPW*D contiguous elements per token.  The NREP query
+//   heads that share a kv head are all evaluated from the same registers: each
+//   K/V byte is loaded once.
+//
+// Softmax
+//   base-2 online softmax in fp32 per row group, rescaled once per batch of U
+//   token steps; the partial (m, l, acc) of the 4 waves x TPW token rows are
+//   merged through LDS.  Decode writes one partial per (chunk, query head) to
+//   the workspace and a second kernel merges the chunks of a sequence.
+#pragma once
+#include "pa_common.h"
+
+namespace pa_decode_detail {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / PA_WAVE;
+constexpr int kMaxBatch = 8192;      // sequences per call (their chunk prefix sum lives in LDS)
+constexpr float kNegBig = -1.0e30f;  // finite stand-in for -inf in running maxima
+
+// What every kernel of this file needs to know about the pool and the heads.
+struct PoolArgs {
+    const void *k, *v;
+    const int32_t *bt;
+    int64_t bt_stride;
+    const float *k_scale, *v_scale;
+    int hq, hkv, n_rep, bs;
+    int64_t num_blocks;
+    float scale_log2;  // softmax scale * log2(e)
+    int hpw, tpw, n_hgroups, n_rgroups;
+};
+
+struct DecodeArgs {
+    PoolArgs p;
+    const void *q;
+    void *out;
+    const int32_t *seq_lens;
+    const int32_t *extra_zero;
+    int batch;
+    int chunk_blocks;
+    int64_t chunk_cap;      // partial slots the workspace holds
+    float *part_acc;        // [chunk_cap][hq][D]
+    float *part_ml;         // [chunk_cap][hq][2]
+    int32_t *chunk_prefix;  // [batch+1], written by the split pass for the reduction pass
+};
+
+struct RowwiseArgs {
+    PoolArgs p;
+    const void *q;
+    void *out;
+    const int32_t *ctx_lens, *q_lens, *q_starts;
+    int batch;
+    int max_q_len;
+};
+
+__device__ __forceinline__ uint4 ld16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }
+
+template <typename KV, int D> struct RowShape {
+    static constexpr int EPL = pa_vec16<KV>::N;  // elements per lane per 16-byte load
+    static constexpr int LPR = D / EPL;          // lanes per row
+    static constexpr int RPW = PA_WAVE / LPR;    // rows per wave load
+    static_assert(D % EPL == 0 && LPR >= 1 && LPR <= 64 && (LPR & (LPR - 1)) == 0, "row shape");
+};
+
+// Fixed role of a lane within its wave.
+struct LaneRole {
+    int row, lir, head_local, tok_local, d0;
+};
+template <typename KV, int D> __device__ __forceinline__ LaneRole lane_role(int lane, const PoolArgs &p) {
+    using S = RowShape<KV, D>;
+    LaneRole r;
+    r.row = lane / S::LPR;
+    r.lir = lane - r.row * S::LPR;
+    r.head_local = r.row % p.hpw;
+    r.tok_local = r.row / p.hpw;
+    r.d0 = r.lir * S::EPL;
+    return r;
+}
+
+// Running softmax state of one row group for NREP query heads.
+template <int NREP, int EPL> struct RowState {
+    float m[NREP], l[NREP], acc[NREP][EPL];
+    int zero_keys;  // keys of missing blocks (logit 0, value 0) seen by this row group
+    __device__ __forceinline__ void init() {
+#pragma unroll
+        for (int r = 0; r < NREP; ++r) {
+            m[r] = kNegBig;
+            l[r] = 0.f;
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) acc[r][e] = 0.f;
+        }
+        zero_keys = 0;
+    }
+    __device__ __forceinline__ void fold_zero_keys() {
+        if (zero_keys <= 0) return;
+#pragma unroll
+        for (int r = 0; r < NREP; ++r) {
+            const float mn = fmaxf(m[r], 0.f);
+            const float alpha = __builtin_amdgcn_exp2f(m[r] - mn);
+            l[r] = l[r] * alpha + (float)zero_keys * __builtin_amdgcn_exp2f(-mn);
+#pragma unroll
+            for (int e = 0; e < EPL; ++e) acc[r][e] *= alpha;
+            m[r] = mn;
+        }
+        zero_keys = 0;
+    }
+};
+
+// This lane's slice of the NREP query heads of kv head `kvh`, pre-multiplied by
+// scale*log2(e).  `qrow` points at [num_q_heads][D] of the query row.
+template <typename QT, int D, int NREP, int EPL>
+__device__ __forceinline__ void load_q(float (&qf)[NREP][EPL], const QT *qrow, const PoolArgs &p, int kvh,
+                                       int rep0, int d0) {
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) {
+        const bool live = rep0 + r < p.n_rep;
+        const QT *qp = qrow + ((int64_t)kvh * p.n_rep + rep0 + (live ? r : 0)) * D + d0;
+#pragma unroll
+        for (int e = 0; e < EPL; ++e) qf[r][e] = live ? pa_scalar<QT>::load(qp + e) * p.scale_log2 : 0.f;
+    }
+}
+
+// Attend keys [0, L) restricted to blocks blk_begin, blk_begin+blk_step, ... < blk_end
+// of the block-table row `bt_row`, for kv head `kvh`.
+template <typename KV, int D, int NREP, int U>
+__device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EPL> &st,
+                                              const float (&qf)[NREP][RowShape<KV, D>::EPL], const PoolArgs &p,
+                                              const int32_t *bt_row, int L, int blk_begin, int blk_end,
+                                              int blk_step, const LaneRole &role, int kvh) {
+    using S = RowShape<KV, D>;
+    constexpr int EPL = S::EPL;
+    constexpr bool kFp8 = sizeof(KV) == 1;
+    const int64_t tok_stride = (int64_t)p.hkv * D * sizeof(KV);  // bytes between tokens
+
+    for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
+        const int ntok = min(p.bs, L - blk * p.bs);
+        const int64_t bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
+        if (bid < 0 || bid >= p.num_blocks) {
+            if (role.tok_local == 0) st.zero_keys += ntok;
+            continue;
+        }
+        const int64_t base = ((bid * p.bs) * p.hkv + kvh) * (int64_t)(D * sizeof(KV)) + (int64_t)role.lir * 16;
+        const char *kp = reinterpret_cast<const char *>(p.k) + base;
+        const char *vp = reinterpret_cast<const char *>(p.v) + base;
+        float ks = 1.f, vs = 1.f;
+        if (kFp8) {
+            ks = p.k_scale[bid * p.hkv + kvh];
+            vs = p.v_scale[bid * p.hkv + kvh];
+        }
+        for (int t0 = 0; t0 < ntok; t0 += p.tpw * U) {
+            uint4 kraw[U], vraw[U];
+            bool ok[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int t = t0 + u * p.tpw + role.tok_local;
+                ok[u] = t < ntok;
+                kraw[u] = ok[u] ? ld16(kp + t * tok_stride) : uint4{0, 0, 0, 0};
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int t = t0 + u * p.tpw + role.tok_local;
+                vraw[u] = ok[u] ? ld16(vp + t * tok_stride) : uint4{0, 0, 0, 0};
+            }
+            float s[U][NREP];
+            float mx[NREP];
+#pragma unroll
+            for (int r = 0; r < NREP; ++r) mx[r] = st.m[r];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float kf[EPL];
+                pa_vec16<KV>::unpack(kraw[u], kf);
+#pragma unroll
+                for (int r = 0; r < NREP; ++r) {
+                    float d = 0.f;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) d = fmaf(qf[r][e], kf[e], d);
+                    d = pa_group_sum<S::LPR>(d);
+                    if (kFp8) d *= ks;
+                    s[u][r] = ok[u] ? d : -INFINITY;
+                    mx[r] = fmaxf(mx[r], s[u][r]);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < NREP; ++r) {
+                const float alpha = __builtin_amdgcn_exp2f(st.m[r] - mx[r]);
+                st.m[r] = mx[r];
+                st.l[r] *= alpha;
+#pragma unroll
+                for (int e = 0; e < EPL; ++e) st.acc[r][e] *= alpha;
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float vf[EPL];
+                pa_vec16<KV>::unpack(vraw[u], vf);
+#pragma unroll
+                for (int r = 0; r < NREP; ++r) {
+                    float pr = __builtin_amdgcn_exp2f(s[u][r] - st.m[r]);  // 0 for masked steps
+                    st.l[r] += pr;
+                    if (kFp8) pr *= vs;
+#pragma unroll
+                    for (int e = 0; e < EPL; ++e) st.acc[r][e] = fmaf(pr, vf[e], st.acc[r][e]);
+                }
+            }
+        }
+    }
+}
+
+// Merge the kWaves*TPW row-group partials of every (kv head of the group,
+// query head r) through LDS and hand (qh, d, num, M, den) of the merged
+// partial to `emit`; out = num/den, M is the base-2 running maximum.
+template <typename KV, int D, int NREP, typename Emit>
+__device__ __forceinline__ void merge_rows(RowState<NREP, RowShape<KV, D>::EPL> &st,
+                                           float (*s_part)[D + 2], const PoolArgs &p, const LaneRole &role,
+                                           int wave, int tid, int hg, int rep0, Emit emit) {
+    using S = RowShape<KV, D>;
+    st.fold_zero_keys();
+    const int prow = wave * S::RPW + role.row;  // = wave*RPW + tok_local*hpw + head_local
+#pragma unroll
+    for (int r = 0; r < NREP; ++r) {
+        if (rep0 + r >= p.n_rep) break;  // uniform over the workgroup
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < S::EPL; ++e) s_part[prow][role.d0 + e] = st.acc[r][e];
+        if (role.lir == 0) {
+            s_part[prow][D] = st.m[r];
+            s_part[prow][D + 1] = st.l[r];
+        }
+        __syncthreads();
+        for (int o = tid; o < p.hpw * D; o += kThreads) {
+            const int hl = o / D, d = o - hl * D;
+            float M = kNegBig;
+            for (int w = 0; w < kWaves; ++w)
+                for (int t = 0; t < p.tpw; ++t) M = fmaxf(M, s_part[w * S::RPW + t * p.hpw + hl][D]);
+            float num = 0.f, den = 0.f;
+            for (int w = 0; w < kWaves; ++w)
+                for (int t = 0; t < p.tpw; ++t) {
+                    const float *pr = s_part[w * S::RPW + t * p.hpw + hl];
+                    const float wgt = __builtin_amdgcn_exp2f(pr[D] - M);
+                    num = fmaf(wgt, pr[d], num);
+                    den = fmaf(wgt, pr[D + 1], den);
+                }
+            emit((hg * p.hpw + hl) * p.n_rep + rep0 + r, d, num, M, den);
+        }
+    }
+    __syncthreads();
+}
+
+template <typename KV, typename QT, int D, int NREP, int U>
+__global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs a) {
+    using S = RowShape<KV, D>;
+    extern __shared__ int s_prefix[];  // batch + 1 entries, sized at launch
+    __shared__ int s_scan[kThreads];
+    __shared__ float s_part[kWaves * S::RPW][D + 2];
+
+    const PoolArgs &p = a.p;
+    const int tid = threadIdx.x;
+    const int lane = tid & (PA_WAVE - 1);
+    const int wave = tid / PA_WAVE;
+    const int B = a.batch;
+
+    // ---- chunk prefix sum over the batch -------------------------------
+    {
+        const int per = (B + kThreads - 1) / kThreads;
+        const int lo = min(B, tid * per), hi = min(B, lo + per);
+        auto chunks_of = [&](int b) {
+            const int L = max(0, a.seq_lens[b]);
+            const int nblk = (L + p.bs - 1) / p.bs;
+            return (nblk + a.chunk_blocks - 1) / a.chunk_blocks;
+        };
+        int sum = 0;
+        for (int b = lo; b < hi; ++b) sum += chunks_of(b);
+        s_scan[tid] = sum;
+        __syncthreads();
+        for (int off = 1; off < kThreads; off <<= 1) {
+            const int add = tid >= off ? s_scan[tid - off] : 0;
+            __syncthreads();
+            s_scan[tid] += add;
+            __syncthreads();
+        }
+        int run = s_scan[tid] - sum;  // exclusive
+        for (int b = lo; b < hi; ++b) {
+            s_prefix[b] = run;
+            run += chunks_of(b);
+        }
+        if (tid == kThreads - 1) s_prefix[B] = s_scan[tid];
+        __syncthreads();
+        if (blockIdx.x == 0)
+            for (int b = tid; b <= B; b += kThreads) a.chunk_prefix[b] = s_prefix[b];
+    }
+    const int total_chunks = s_prefix[B];
+    const int64_t n_items = (int64_t)total_chunks * p.n_hgroups * p.n_rgroups;
+    const LaneRole role = lane_role<KV, D>(lane, p);
+
+    for (int64_t item = blockIdx.x; item < n_items; item += gridDim.x) {
+        // item -> (chunk, rep group, head group); head group fastest
+        const int hg = (int)(item % p.n_hgroups);
+        const int64_t rest = item / p.n_hgroups;
+        const int rg = (int)(rest % p.n_rgroups);
+        const int gchunk = (int)(rest / p.n_rgroups);
+        if (gchunk >= a.chunk_cap) continue;  // workspace smaller than promised: never write outside it
+        int lo = 0, hi = B;  // last b with prefix[b] <= gchunk
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (s_prefix[mid] <= gchunk) lo = mid; else hi = mid;
+        }
+        const int b = lo;
+        const int c = gchunk - s_prefix[lo];
+        const int L = a.seq_lens[b];
+        const int nblk = (L + p.bs - 1) / p.bs;
+        const int blk0 = c * a.chunk_blocks;
+        const int blk1 = min(nblk, blk0 + a.chunk_blocks);
+        const int kvh = hg * p.hpw + role.head_local;
+        const int rep0 = rg * NREP;
+
+        float qf[NREP][S::EPL];
+        load_q<QT, D, NREP, S::EPL>(qf, reinterpret_cast<const QT *>(a.q) + (int64_t)b * p.hq * D, p, kvh, rep0,
+                                    role.d0);
+        RowState<NREP, S::EPL> st;
+        st.init();
+        attend_blocks<KV, D, NREP, U>(st, qf, p, p.bt + (int64_t)b * p.bt_stride, L, blk0 + wave, blk1, kWaves,
+                                      role, kvh);
+        merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
+                                [&](int qh, int d, float num, float M, float den) {
+                                    const int64_t slot = (int64_t)gchunk * p.hq + qh;
+                                    a.part_acc[slot * D + d] = num;
+                                    if (d == 0) {
+                                        a.part_ml[slot * 2] = M;
+                                        a.part_ml[slot * 2 + 1] = den;
+                                    }
+                                });
+    }
+}
+
+// Merge the chunk partials of one (sequence, query head); thread d owns out[d].
+template <typename QT, int D>
+__global__ void decode_reduce_kernel(const DecodeArgs a) {
+    const int hq = a.p.hq;
+    const int b = blockIdx.x / hq;
+    const int qh = blockIdx.x - b * hq;
+    const int c0 = a.chunk_prefix[b], c1 = (int)min((int64_t)a.chunk_prefix[b + 1], a.chunk_cap);
+    float M = kNegBig;
+    for (int c = c0; c < c1; ++c) M = fmaxf(M, a.part_ml[((int64_t)c * hq + qh) * 2]);
+    const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
+    if (ez > 0) M = fmaxf(M, 0.f);
+    for (int d = threadIdx.x; d < D; d += blockDim.x) {
+        float num = 0.f, den = 0.f;
+        for (int c = c0; c < c1; ++c) {
+            const int64_t slot = (int64_t)c * hq + qh;
+            const float w = __builtin_amdgcn_exp2f(a.part_ml[slot * 2] - M);
+            num = fmaf(w, a.part_acc[slot * D + d], num);
+            den = fmaf(w, a.part_ml[slot * 2 + 1], den);
+        }
+        if (ez > 0) den += (float)ez * __builtin_amdgcn_exp2f(-M);
+        const float o = den > 0.f ? num / den : 0.f;
+        pa_scalar<QT>::store(reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * D + d, o);
+    }
+}
+
+// Causal prefill, one workgroup per (sequence, query row, head group, rep
+// group): query row i of sequence b attends keys [0, ctx_len - q_len + i].
+template <typename KV, typename QT, int D, int NREP, int U>
+__global__ __launch_bounds__(kThreads) void prefill_rowwise_kernel(const RowwiseArgs a) {
+    using S = RowShape<KV, D>;
+    __shared__ float s_part[kWaves * S::RPW][D + 2];
+    const PoolArgs &p = a.p;
+    const int tid = threadIdx.x;
+    const int lane = tid & (PA_WAVE - 1);
+    const int wave = tid / PA_WAVE;
+    const int b = blockIdx.z;
+    const int i = blockIdx.y;
+    const int q_len = a.q_lens[b];
+    if (i >= q_len) return;  // uniform over the workgroup
+    const int hg = blockIdx.x % p.n_hgroups;
+    const int rg = blockIdx.x / p.n_hgroups;
+    const int L = min(a.ctx_lens[b], a.ctx_lens[b] - q_len + i + 1);
+    const LaneRole role = lane_role<KV, D>(lane, p);
+    const int kvh = hg * p.hpw + role.head_local;
+    const int rep0 = rg * NREP;
+    const int64_t qrow = (int64_t)a.q_starts[b] + i;
+
+    float qf[NREP][S::EPL];
+    load_q<QT, D, NREP, S::EPL>(qf, reinterpret_cast<const QT *>(a.q) + qrow * p.hq * D, p, kvh, rep0, role.d0);
+    RowState<NREP, S::EPL> st;
+    st.init();
+    const int nblk = L > 0 ? (L + p.bs - 1) / p.bs : 0;
+    attend_blocks<KV, D, NREP, U>(st, qf, p, p.bt + (int64_t)b * p.bt_stride, L, wave, nblk, kWaves, role, kvh);
+    QT *orow = reinterpret_cast<QT *>(a.out) + qrow * p.hq * D;
+    merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
+                            [&](int qh, int d, float num, float M, float den) {
+                                pa_scalar<QT>::store(orow + (int64_t)qh * D + d, den > 0.f ? num / den : 0.f);
+                            });
+}
+
+typedef void (*split_fn)(const DecodeArgs);
+typedef void (*reduce_fn)(const DecodeArgs);
+typedef void (*rowwise_fn)(const RowwiseArgs);
+
+struct KernelSet {
+    split_fn split = nullptr;
+    reduce_fn reduce = nullptr;
+    rowwise_fn rowwise = nullptr;
+};
+
+template <typename KV, typename QT, int D> KernelSet kernels_for_d(int nrep_t) {
+    constexpr int U = sizeof(KV) == 1 ? 4 : 8;
+    KernelSet k;
+    k.reduce = decode_reduce_kernel<QT, D>;
+    switch (nrep_t) {
+    case 1: k.split = decode_split_kernel<KV, QT, D, 1, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 1, U>; break;
+    case 2: k.split = decode_split_kernel<KV, QT, D, 2, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 2, U>; break;
+    case 4: k.split = decode_split_kernel<KV, QT, D, 4, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 4, U>; break;
+    case 8: k.split = decode_split_kernel<KV, QT, D, 8, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 8, U>; break;
+    }
+    return k;
+}
+
+template <typename KV, typename QT> KernelSet kernels_for(int d, int nrep_t) {
+    switch (d) {
+    case 32: return kernels_for_d<KV, QT, 32>(nrep_t);
+    case 64: return kernels_for_d<KV, QT, 64>(nrep_t);
+    case 128: return kernels_for_d<KV, QT, 128>(nrep_t);
+    case 256: return kernels_for_d<KV, QT, 256>(nrep_t);
+    }
+    return KernelSet{};
+}
+
+// one definition each, in decode_inst_<type>.hip
+KernelSet pa_kernels_bf16(int d, int nrep_t);
+KernelSet pa_kernels_f16(int d, int nrep_t);
+KernelSet pa_kernels_f32(int d, int nrep_t);
+KernelSet pa_kernels_fp8(int q_dtype, int d, int nrep_t);
+
+// Kernel set for (q dtype, KV dtype, head_dim, padded group size), empty if none.
+KernelSet pa_pick_kernels(int q_dtype, int kv_dtype, int d, int nrep_t);
+
+// Head-mapping fields of PoolArgs derived from the shapes; returns the padded
+// group size (template NREP) or 0 when head_dim / dtype has no kernel.
+int pa_fill_head_mapping(PoolArgs &p, int num_q_heads, int num_kv_heads, int head_dim, int kv_dtype);
+
+}  // namespace pa_decode_detail

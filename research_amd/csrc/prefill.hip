@@ -1,0 +1,43 @@
+// Host entry point of causal prefill attention over a paged context.
+#include "decode_impl.h"
+
+using namespace pa_decode_detail;
+
+extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, void *out,
+                                const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
+                                const int32_t *q_lens, const int32_t *q_starts, int batch, int max_q_len,
+                                int num_q_heads, int num_kv_heads, int head_dim, int block_size,
+                                int64_t num_blocks, float scale, int dtype, void *stream) {
+    pa_clear_error();
+    PA_REQUIRE(batch >= 0 && max_q_len >= 0, "batch=%d max_q_len=%d must be non-negative", batch, max_q_len);
+    PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, "head counts / head_dim must be positive");
+    PA_REQUIRE(num_q_heads % num_kv_heads == 0, "num_q_heads=%d is not a multiple of num_kv_heads=%d",
+               num_q_heads, num_kv_heads);
+    PA_REQUIRE(block_size > 0, "block_size=%d must be positive", block_size);
+    PA_REQUIRE(num_blocks >= 0 && bt_stride >= 0, "num_blocks / bt_stride must be non-negative");
+    PA_REQUIRE(num_blocks * (int64_t)block_size < (1ll << 40), "pool of %lld blocks is too large", (long long)num_blocks);
+    PA_REQUIRE(dtype == PA_F32 || dtype == PA_BF16 || dtype == PA_F16, "dtype=%d is not F32, BF16 or F16", dtype);
+    RowwiseArgs a;
+    const int nrep_t = pa_fill_head_mapping(a.p, num_q_heads, num_kv_heads, head_dim, dtype);
+    const KernelSet ks = nrep_t ? pa_pick_kernels(dtype, dtype, head_dim, nrep_t) : KernelSet{};
+    if (!ks.rowwise)
+        return pa_fail(PA_ERR_UNSUPPORTED, "pa_prefill_paged: no kernel for dtype=%d head_dim=%d", dtype, head_dim);
+    PA_REQUIRE(batch <= 65535 && max_q_len <= 65535, "batch=%d / max_q_len=%d above 65535", batch, max_q_len);
+    if (batch == 0 || max_q_len == 0) return PA_OK;
+    PA_REQUIRE(q && out && ctx_lens && q_lens && q_starts, "NULL q / out / ctx_lens / q_lens / q_starts");
+    PA_REQUIRE(k_cache && v_cache, "NULL cache pointer");
+    PA_REQUIRE(block_tables || bt_stride == 0, "NULL block_tables with bt_stride=%lld", (long long)bt_stride);
+    PA_REQUIRE(pa_aligned16(k_cache) && pa_aligned16(v_cache), "cache pointers must be 16-byte aligned");
+
+    a.p.k = k_cache; a.p.v = v_cache; a.p.bt = block_tables; a.p.bt_stride = bt_stride;
+    a.p.k_scale = nullptr; a.p.v_scale = nullptr;
+    a.p.bs = block_size; a.p.num_blocks = num_blocks;
+    a.p.scale_log2 = scale * 1.4426950408889634f;
+    a.q = q; a.out = out; a.ctx_lens = ctx_lens; a.q_lens = q_lens; a.q_starts = q_starts;
+    a.batch = batch; a.max_q_len = max_q_len;
+    hipStream_t s = (hipStream_t)stream;
+    ks.rowwise<<<dim3((unsigned)(a.p.n_hgroups * a.p.n_rgroups), (unsigned)max_q_len, (unsigned)batch),
+                 dim3(kThreads), 0, s>>>(a);
+    PA_CHECK_LAUNCH("pa_prefill_paged");
+    return PA_OK;
+}

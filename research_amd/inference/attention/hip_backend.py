@@ -1,0 +1,321 @@
+"""Paged-KV attention backend for MI355X behind the reference's call surface.
+
+``HipPagedAttentionBackend`` has the constructor, attributes and methods of
+the reference's ``FlexAttentionBackend``
+(rollouts/rollouts/inference/attention/flex_backend.py:11-285) and can stand in
+for it inside an ``Attention`` layer.  Where the reference issues PyTorch
+indexing / ``scaled_dot_product_attention`` calls, this class passes raw device
+pointers of the same tensors to the C ABI of ``libpaged_attn.so``; torch is used
+for device memory and the current stream only.  There is no eager fallback: a
+missing library, or tensors that are not on a HIP device, raise.
+
+Differences from the reference, all deliberate:
+
+* Decode attends exactly ``seq_lens[b]`` keys per sequence.  The reference
+  zero-pads a ragged batch to its longest sequence and attends without a mask
+  (flex_backend.py:253-264, :227-229), which lets the padding keys (logit 0)
+  take softmax mass; the two agree whenever all lengths are equal (always for
+  batch 1).  ``pad_zero_keys=True`` reproduces the reference's ragged result.
+* ``ctx.prefix_lens`` (an added, optional context field) selects chunked
+  prefill: the chunk's queries attend the cached prefix and the chunk itself,
+  both read from the pool through the block table.
+* ``ctx.block_mask`` objects and ``config.sliding_window`` are not supported
+  and raise ``NotImplementedError`` instead of being ignored.
+"""
+
+from __future__ import annotations
+
+from collections import OrderedDict
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+from torch import Tensor
+
+from ... import _lib, ops
+from ..types import InferenceContext
+from .config import CacheConfig
+
+_COMPUTE_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
+
+
+class _StepTensors:
+    """Device copies of one context's integer fields, built once per step."""
+
+    __slots__ = ("ctx", "slots", "tables", "bt_stride", "seq_lens", "extra_zero", "total_chunks", "chunk_tokens",
+                 "ctx_lens", "q_lens", "q_starts", "max_q_len")
+
+    def __init__(self, ctx: InferenceContext) -> None:
+        self.ctx = ctx  # keeps id(ctx) alive while the entry is cached
+        self.slots = self.tables = self.seq_lens = self.extra_zero = None
+        self.ctx_lens = self.q_lens = self.q_starts = None
+        self.bt_stride = self.total_chunks = self.chunk_tokens = self.max_q_len = 0
+
+
+def _padded_tables(block_tables: Sequence[Sequence[int]]) -> np.ndarray:
+    width = max((len(row) for row in block_tables), default=0)
+    out = np.full((len(block_tables), max(width, 1)), -1, dtype=np.int32)
+    for i, row in enumerate(block_tables):
+        if len(row):
+            out[i, : len(row)] = np.asarray(row, dtype=np.int64)
+    return out
+
+
+class HipPagedAttentionBackend:
+    def __init__(self, config: CacheConfig, pad_zero_keys: bool = False) -> None:
+        self._lib = _lib.load()  # raises if the HIP library has not been built
+        self.config = config
+        self.num_heads_per_kv = 1  # until set_num_heads(), as in the reference (flex_backend.py:31,43-45)
+        self.scale = config.head_dim**-0.5
+        self.pad_zero_keys = pad_zero_keys
+        self._mask_cache: dict = {}
+        self._step_cache: "OrderedDict[int, _StepTensors]" = OrderedDict()
+        self._workspace: Optional[Tensor] = None
+
+        if config.kv_format not in (None, "fp8_e4m3"):
+            raise ValueError(f"unknown kv_format {config.kv_format!r}")
+        if config.dtype not in _COMPUTE_DTYPES:
+            raise ValueError(f"unsupported cache dtype {config.dtype}")
+        self._fp8 = config.kv_format == "fp8_e4m3"
+        pool_dtype = torch.float8_e4m3fn if self._fp8 else config.dtype
+        # one allocation per tensor for all layers, zero-initialised (flex_backend.py:38-41)
+        self.k_cache = torch.zeros(config.cache_shape, dtype=pool_dtype, device=config.device)
+        self.v_cache = torch.zeros(config.cache_shape, dtype=pool_dtype, device=config.device)
+        self.k_scale = self.v_scale = None
+        if self._fp8:
+            shape = (config.num_layers, config.num_blocks, config.num_kv_heads)
+            self.k_scale = torch.ones(shape, dtype=torch.float32, device=config.device)
+            self.v_scale = torch.ones(shape, dtype=torch.float32, device=config.device)
+
+    # ------------------------------------------------------------------ small surface
+    def set_num_heads(self, num_heads: int) -> None:
+        self.num_heads_per_kv = num_heads // self.config.num_kv_heads
+
+    def get_block_mask(self, batch_size: int, seq_len: int) -> object:
+        if self.config.sliding_window is None:
+            return None  # plain causal needs no mask object (flex_backend.py:62-63)
+        raise NotImplementedError("sliding_window masks are not supported by the HIP backend")
+
+    def clear_mask_cache(self) -> None:
+        self._mask_cache.clear()
+
+    def clear_cache(self) -> None:
+        self.k_cache.zero_()
+        self.v_cache.zero_()
+        if self._fp8:
+            self.k_scale.fill_(1.0)
+            self.v_scale.fill_(1.0)
+        self._mask_cache.clear()
+        self._step_cache.clear()
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, q: Tensor, k: Tensor, v: Tensor, layer_idx: int, ctx: InferenceContext) -> Tensor:
+        """Append this step's K/V, then attend (flex_backend.py:89-114).
+
+        The append runs first, so a decode step sees its own token.
+        """
+        if ctx.slot_mapping is not None:
+            self._store_kv(k, v, layer_idx, ctx.slot_mapping, _step=self._step(ctx))
+        if ctx.is_prefill:
+            if ctx.prefix_lens is not None:
+                return self._prefill_paged(q, layer_idx, ctx)
+            return self._prefill_attention(q, k, v, ctx)
+        return self._decode_attention(q, layer_idx, ctx)
+
+    __call__ = forward
+
+    # ------------------------------------------------------------------ helpers
+    def _require_device(self, *tensors: Tensor) -> torch.device:
+        for t in tensors:
+            if t.device.type != "cuda":
+                raise RuntimeError(
+                    "HipPagedAttentionBackend computes only on a HIP device; "
+                    f"got a tensor on {t.device} (there is no CPU implementation)"
+                )
+        return tensors[0].device
+
+    def _step(self, ctx: InferenceContext) -> _StepTensors:
+        key = id(ctx)
+        hit = self._step_cache.get(key)
+        if hit is not None and hit.ctx is ctx:
+            self._step_cache.move_to_end(key)
+            return hit
+        entry = _StepTensors(ctx)
+        self._step_cache[key] = entry
+        while len(self._step_cache) > 4:
+            self._step_cache.popitem(last=False)
+        return entry
+
+    def _to_device(self, array: np.ndarray) -> Tensor:
+        return torch.from_numpy(array).to(self.k_cache.device)
+
+    def _tables(self, step: _StepTensors, block_tables) -> None:
+        if step.tables is None:
+            padded = _padded_tables(block_tables)
+            step.tables, step.bt_stride = self._to_device(padded), padded.shape[1]
+
+    def _workspace_for(self, nbytes: int) -> Tensor:
+        if self._workspace is None or self._workspace.numel() < nbytes:
+            self._workspace = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=self.k_cache.device)
+        return self._workspace
+
+    def _layer(self, layer_idx: int) -> Tuple[Tensor, Tensor]:
+        return self.k_cache[layer_idx], self.v_cache[layer_idx]
+
+    # ------------------------------------------------------------------ KV append
+    def _store_kv(self, k: Tensor, v: Tensor, layer_idx: int, slot_mapping: Tuple[int, ...],
+                  _step: Optional[_StepTensors] = None) -> None:
+        """``cache[layer, slot] = row`` for every non-negative slot (flex_backend.py:116-142)."""
+        cfg = self.config
+        if self._fp8:
+            raise NotImplementedError("appending to an fp8 pool: quantise a filled pool with quantize_from()")
+        k_flat = k.reshape(-1, cfg.num_kv_heads, cfg.head_dim)
+        v_flat = v.reshape(-1, cfg.num_kv_heads, cfg.head_dim)
+        n = len(slot_mapping)
+        if n != k_flat.shape[0]:
+            # the reference fails in its boolean-mask indexing with this error type
+            raise IndexError(
+                f"The shape of the mask [{n}] at index 0 does not match the shape of the indexed tensor "
+                f"{list(k_flat.shape)} at index 0"
+            )
+        if k_flat.dtype != self.k_cache.dtype or v_flat.dtype != self.v_cache.dtype:
+            raise RuntimeError("Index put requires the source and destination dtypes match")
+        if n == 0:
+            return
+        if _step is not None and _step.slots is not None:
+            slots = _step.slots
+        else:
+            host = np.asarray(slot_mapping, dtype=np.int64)
+            if host.max() >= cfg.total_slots:
+                raise IndexError(
+                    f"index {int(host.max())} is out of bounds for dimension 0 with size {cfg.total_slots}")
+            self._require_device(k_flat, v_flat, self.k_cache)
+            slots = self._to_device(host)
+            if _step is not None:
+                _step.slots = slots
+        k_flat, v_flat = k_flat.contiguous(), v_flat.contiguous()
+        kc, vc = self._layer(layer_idx)
+        ops.kv_scatter(kc, vc, k_flat, v_flat, slots)
+
+    # ------------------------------------------------------------------ gather
+    def _gather_kv_from_cache(self, layer_idx: int, block_tables, seq_lens) -> Tuple[Tensor, Tensor]:
+        """Zero-padded ``[num_seqs, max(seq_lens), Hkv, D]`` copies (flex_backend.py:233-279)."""
+        cfg = self.config
+        num_seqs, max_len = len(block_tables), max(seq_lens)
+        self._require_device(self.k_cache)
+        tables = self._to_device(_padded_tables(block_tables))
+        lens = self._to_device(np.asarray(seq_lens, dtype=np.int32)[:num_seqs])
+        kc, vc = self._layer(layer_idx)
+        return ops.kv_gather(kc, vc, tables, lens, max_len, cfg.block_size)
+
+    # ------------------------------------------------------------------ decode
+    def _decode_attention(self, q: Tensor, layer_idx: int, ctx: InferenceContext) -> Tensor:
+        """One query token per sequence over its cached keys (flex_backend.py:187-231)."""
+        batch, seq_len, num_heads, head_dim = q.shape
+        assert seq_len == 1, "Decode should have seq_len=1"
+        if ctx.block_tables is None or ctx.seq_lens is None:
+            raise ValueError("Decode requires block_tables and seq_lens in context")
+        if ctx.block_mask is not None:
+            raise NotImplementedError("block_mask objects are not supported by the HIP backend")
+        cfg = self.config
+        self._require_device(q, self.k_cache)
+        step = self._step(ctx)
+        if step.seq_lens is None:
+            lens = np.asarray(ctx.seq_lens, dtype=np.int64)[:batch]
+            self._tables(step, ctx.block_tables[:batch])
+            step.seq_lens = self._to_device(lens.astype(np.int32))
+            step.chunk_tokens = ops.decode_plan(int(lens.sum()), batch, cfg.num_kv_heads, cfg.block_size)
+            step.total_chunks = int((-(-np.maximum(lens, 0) // step.chunk_tokens)).sum())
+            if self.pad_zero_keys and batch > 0:
+                step.extra_zero = self._to_device((lens.max() - lens).astype(np.int32))
+        q3 = q.contiguous().view(batch, num_heads, head_dim)
+        ws = self._workspace_for(ops.decode_workspace_bytes(step.total_chunks, batch, num_heads, head_dim))
+        kc, vc = self._layer(layer_idx)
+        ksc = self.k_scale[layer_idx] if self._fp8 else None
+        vsc = self.v_scale[layer_idx] if self._fp8 else None
+        out = ops.decode(q3, kc, vc, step.tables, step.seq_lens, cfg.block_size, self.scale, step.chunk_tokens,
+                         step.total_chunks, ws, step.extra_zero, ksc, vsc)
+        return out.view(batch, 1, num_heads, head_dim)
+
+    # ------------------------------------------------------------------ prefill
+    def _prefill_attention(self, q: Tensor, k: Tensor, v: Tensor, ctx: InferenceContext) -> Tensor:
+        """Causal attention over the step's own K/V, cache not read (flex_backend.py:144-185).
+
+        The dense ``[B, T, Hkv, D]`` inputs are handed to the paged kernel as a
+        pool of ``B`` blocks of ``T`` tokens with the identity block table.
+        """
+        if ctx.block_mask is not None or self.config.sliding_window is not None:
+            raise NotImplementedError("block_mask / sliding_window are not supported by the HIP backend")
+        batch, seq_len, num_heads, head_dim = q.shape
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        if out.numel() == 0:
+            return out
+        dev = self._require_device(q, k, v)
+        num_kv = k.shape[2]
+        if num_heads != num_kv * self.num_heads_per_kv:
+            raise RuntimeError(
+                f"q has {num_heads} heads but k/v have {num_kv} x num_heads_per_kv={self.num_heads_per_kv}")
+        ar = torch.arange(batch, dtype=torch.int32, device=dev)
+        lens = torch.full((batch,), seq_len, dtype=torch.int32, device=dev)
+        ops.prefill_paged(
+            q.contiguous().view(batch * seq_len, num_heads, head_dim),
+            k.contiguous().view(batch * seq_len, num_kv, head_dim),
+            v.contiguous().view(batch * seq_len, num_kv, head_dim),
+            ar.reshape(batch, 1).contiguous(), lens, lens, ar * seq_len, seq_len, seq_len, self.scale,
+            out=out.view(batch * seq_len, num_heads, head_dim))
+        return out
+
+    def _prefill_paged(self, q: Tensor, layer_idx: int, ctx: InferenceContext) -> Tensor:
+        """Chunked prefill: ``q[b]`` holds the last ``T`` positions of a context of ``seq_lens[b]`` keys."""
+        if ctx.block_mask is not None or self.config.sliding_window is not None:
+            raise NotImplementedError("block_mask / sliding_window are not supported by the HIP backend")
+        if ctx.block_tables is None or ctx.seq_lens is None:
+            raise ValueError("Chunked prefill requires block_tables and seq_lens in context")
+        if self._fp8:
+            raise NotImplementedError("chunked prefill over an fp8 pool")
+        cfg = self.config
+        batch, seq_len, num_heads, head_dim = q.shape
+        out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+        if out.numel() == 0:
+            return out
+        self._require_device(q, self.k_cache)
+        step = self._step(ctx)
+        if step.ctx_lens is None:
+            totals = np.asarray(ctx.seq_lens, dtype=np.int64)[:batch]
+            chunk = totals - np.asarray(ctx.prefix_lens, dtype=np.int64)[:batch]
+            if (chunk < 0).any() or (chunk > seq_len).any():
+                raise ValueError("prefix_lens / seq_lens do not describe chunks of at most q.shape[1] tokens")
+            self._tables(step, ctx.block_tables[:batch])
+            step.ctx_lens = self._to_device(totals.astype(np.int32))
+            step.q_lens = self._to_device(chunk.astype(np.int32))
+            step.q_starts = self._to_device((np.arange(batch, dtype=np.int64) * seq_len).astype(np.int32))
+            step.max_q_len = int(chunk.max()) if batch else 0
+        out.zero_()  # rows past a sequence's chunk length are padding and stay zero
+        kc, vc = self._layer(layer_idx)
+        ops.prefill_paged(q.contiguous().view(batch * seq_len, num_heads, head_dim), kc, vc, step.tables,
+                          step.ctx_lens, step.q_lens, step.q_starts, step.max_q_len, cfg.block_size, self.scale,
+                          out=out.view(batch * seq_len, num_heads, head_dim))
+        return out
+
+    # ------------------------------------------------------------------ fp8 pool
+    def quantize_from(self, k_pool: Tensor, v_pool: Tensor, layer_idx: int) -> None:
+        """Fill one layer of an fp8 pool from full-precision pools of the same shape.
+
+        ``k_pool`` / ``v_pool``: ``[total_slots, Hkv, D]`` in fp32, bf16 or fp16.
+        Each (block, kv head) tile gets scale = absmax/448 and is stored as
+        e4m3fn(x / scale).
+        """
+        if not self._fp8:
+            raise RuntimeError("quantize_from() needs CacheConfig(kv_format='fp8_e4m3')")
+        cfg = self.config
+        self._require_device(k_pool, v_pool, self.k_cache)
+        for src, dst, scale in ((k_pool, self.k_cache, self.k_scale), (v_pool, self.v_cache, self.v_scale)):
+            if tuple(src.shape) != cfg.cache_shape[1:]:
+                raise ValueError(f"pool of shape {tuple(src.shape)}, expected {cfg.cache_shape[1:]}")
+            bits, sc = ops.quantize_kv_e4m3(src.contiguous(), cfg.block_size)
+            dst[layer_idx].copy_(bits)
+            scale[layer_idx].copy_(sc)
+
+
+# name under which code written for the reference finds its backend
+FlexAttentionBackend = HipPagedAttentionBackend

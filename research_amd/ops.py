@@ -1,0 +1,109 @@
+"""Tensor-level wrappers of the C ABI (one function per ``pa_*`` entry point).
+
+Each wrapper takes torch tensors that already live on the HIP device, passes
+their raw pointers, sizes and the current stream to ``libpaged_attn.so`` and
+raises ``PagedAttnError`` on a negative status.  No computation happens in
+Python and nothing is routed to torch kernels.
+"""
+
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+from torch import Tensor
+
+from . import _lib
+
+PA_DTYPE = {torch.float32: _lib.PA_F32, torch.bfloat16: _lib.PA_BF16, torch.float16: _lib.PA_F16,
+            torch.float8_e4m3fn: _lib.PA_FP8_E4M3, torch.uint8: _lib.PA_FP8_E4M3}
+
+
+def _ptr(t: Optional[Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _stream(t: Tensor) -> Optional[int]:
+    if t.device.type != "cuda":
+        raise RuntimeError(f"libpaged_attn computes only on a HIP device; got a tensor on {t.device}")
+    return torch.cuda.current_stream(t.device).cuda_stream or None
+
+
+def _run(name: str, *args) -> None:
+    _lib.check(name, getattr(_lib.load(), name)(*args))
+
+
+def kv_scatter(k_cache: Tensor, v_cache: Tensor, k_src: Tensor, v_src: Tensor, slots: Tensor) -> None:
+    """``cache[slots[i]] = src[i]``; caches ``[total_slots, Hkv, D]``, src ``[N, Hkv, D]``, slots int64 ``[N]``."""
+    total_slots, hkv, d = k_cache.shape
+    _run("pa_kv_scatter", _ptr(k_cache), _ptr(v_cache), _ptr(k_src), _ptr(v_src), _ptr(slots), slots.numel(),
+         total_slots, hkv, d, k_cache.element_size(), _stream(k_cache))
+
+
+def kv_gather(k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, seq_lens: Tensor, max_len: int,
+              block_size: int) -> Tuple[Tensor, Tensor]:
+    """Zero-padded ``[B, max_len, Hkv, D]`` copies; block_tables int32 ``[B, W]`` (-1 padded), seq_lens int32."""
+    total_slots, hkv, d = k_cache.shape
+    batch = block_tables.shape[0]
+    k_out = torch.empty((batch, max_len, hkv, d), dtype=k_cache.dtype, device=k_cache.device)
+    v_out = torch.empty_like(k_out)
+    _run("pa_kv_gather", _ptr(k_cache), _ptr(v_cache), _ptr(k_out), _ptr(v_out), _ptr(block_tables),
+         block_tables.shape[1], _ptr(seq_lens), batch, max_len, total_slots // block_size, block_size, hkv, d,
+         k_cache.element_size(), _stream(k_cache))
+    return k_out, v_out
+
+
+def decode_plan(total_tokens: int, batch: int, num_kv_heads: int, block_size: int) -> int:
+    """Chunk size (keys) the library suggests for this batch."""
+    chunk = _lib.load().pa_decode_chunk_tokens(total_tokens, batch, num_kv_heads, block_size)
+    if chunk <= 0:
+        raise _lib.PagedAttnError("pa_decode_chunk_tokens", chunk, _lib.last_error())
+    return chunk
+
+
+def decode_workspace_bytes(total_chunks: int, batch: int, num_q_heads: int, head_dim: int) -> int:
+    return int(_lib.load().pa_decode_workspace_bytes(total_chunks, batch, num_q_heads, head_dim))
+
+
+def decode(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, seq_lens: Tensor, block_size: int,
+           scale: float, chunk_tokens: int, total_chunks: int, workspace: Tensor,
+           extra_zero_keys: Optional[Tensor] = None, k_scale: Optional[Tensor] = None,
+           v_scale: Optional[Tensor] = None, out: Optional[Tensor] = None, entry: str = "pa_decode") -> Tensor:
+    """Paged decode attention; q ``[B, Hq, D]`` -> out ``[B, Hq, D]`` (same dtype).
+
+    ``entry`` may name ``pa_decode_split`` or ``pa_decode_reduce`` to run one pass only.
+    """
+    batch, hq, d = q.shape
+    total_slots, hkv, _ = k_cache.shape
+    if out is None:
+        out = torch.empty_like(q)
+    _run(entry, _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_tables), block_tables.shape[1],
+         _ptr(seq_lens), _ptr(extra_zero_keys), _ptr(k_scale), _ptr(v_scale), batch, hq, hkv, d, block_size,
+         total_slots // block_size, float(scale), PA_DTYPE[q.dtype], PA_DTYPE[k_cache.dtype], chunk_tokens,
+         total_chunks, _ptr(workspace), workspace.numel() * workspace.element_size(), _stream(q))
+    return out
+
+
+def prefill_paged(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, ctx_lens: Tensor,
+                  q_lens: Tensor, q_starts: Tensor, max_q_len: int, block_size: int, scale: float,
+                  out: Optional[Tensor] = None) -> Tensor:
+    """Causal prefill over a paged context; q ``[total_q, Hq, D]`` packed rows."""
+    _, hq, d = q.shape
+    total_slots, hkv, _ = k_cache.shape
+    if out is None:
+        out = torch.empty_like(q)
+    _run("pa_prefill_paged", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_tables),
+         block_tables.shape[1], _ptr(ctx_lens), _ptr(q_lens), _ptr(q_starts), block_tables.shape[0], max_q_len, hq,
+         hkv, d, block_size, total_slots // block_size, float(scale), PA_DTYPE[q.dtype], _stream(q))
+    return out
+
+
+def quantize_kv_e4m3(pool: Tensor, block_size: int) -> Tuple[Tensor, Tensor]:
+    """e4m3fn bytes (as ``torch.float8_e4m3fn``) and ``float32 [num_blocks, Hkv]`` scales of a pool."""
+    total_slots, hkv, d = pool.shape
+    num_blocks = total_slots // block_size
+    dst = torch.empty(pool.shape, dtype=torch.float8_e4m3fn, device=pool.device)
+    scale = torch.empty((num_blocks, hkv), dtype=torch.float32, device=pool.device)
+    _run("pa_quantize_kv_e4m3", _ptr(pool), _ptr(dst), _ptr(scale), num_blocks, block_size, hkv, d,
+         PA_DTYPE[pool.dtype], _stream(pool))
+    return dst, scale

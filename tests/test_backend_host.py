@@ -1,0 +1,124 @@
+"""Host-side behaviour of the backend class that needs no GPU: construction,
+attribute surface and the error conventions of the reference
+(rollouts/rollouts/inference/attention/flex_backend.py)."""
+
+import pytest
+import torch
+
+from research_amd.inference import Attention, CacheConfig, FlexAttentionBackend, HipPagedAttentionBackend
+from research_amd.inference import InferenceContext
+
+
+def _cfg(**kw):
+    base = dict(num_layers=2, num_kv_heads=4, head_dim=32, num_blocks=16, block_size=4, device="cpu")
+    base.update(kw)
+    return CacheConfig(**base)
+
+
+def test_cache_config_surface():
+    cfg = CacheConfig(num_layers=3, num_kv_heads=8, head_dim=128)
+    assert (cfg.num_blocks, cfg.block_size, cfg.sliding_window, cfg.dtype, cfg.device) == (
+        1024, 16, None, torch.bfloat16, "cuda")
+    assert cfg.total_slots == 16384 and cfg.cache_shape == (3, 16384, 8, 128)
+    # config.py:47-58 of the reference hashes exactly this tuple
+    assert hash(cfg) == hash((3, 8, 128, 1024, 16, None, "torch.bfloat16", "cuda"))
+    assert cfg == CacheConfig(num_layers=3, num_kv_heads=8, head_dim=128)
+    with pytest.raises(Exception):
+        cfg.num_layers = 4
+
+
+def test_backend_attributes_match_reference_surface():
+    be = HipPagedAttentionBackend(_cfg())
+    assert FlexAttentionBackend is HipPagedAttentionBackend
+    assert be.num_heads_per_kv == 1 and be.scale == 32**-0.5
+    assert be.k_cache.shape == (2, 64, 4, 32) and be.k_cache.dtype == torch.bfloat16
+    assert not be.k_cache.any() and not be.v_cache.any()
+    be.set_num_heads(9)
+    assert be.num_heads_per_kv == 2  # integer division, as the reference
+    assert be.get_block_mask(2, 8) is None
+    be.clear_mask_cache()
+    be.k_cache[0, 0] = 1
+    be.clear_cache()
+    assert not be.k_cache.any()
+    for name in ("forward", "_store_kv", "_prefill_attention", "_decode_attention", "_gather_kv_from_cache"):
+        assert callable(getattr(be, name))
+
+
+def test_decode_error_conventions():
+    be = HipPagedAttentionBackend(_cfg())
+    be.set_num_heads(8)
+    q2 = torch.zeros(1, 2, 8, 32, dtype=torch.bfloat16)
+    ctx = InferenceContext(is_prefill=False, block_tables=((0,),), seq_lens=(1,))
+    with pytest.raises(AssertionError):  # flex_backend.py:199
+        be._decode_attention(q2, 0, ctx)
+    q1 = q2[:, :1]
+    with pytest.raises(ValueError, match="Decode requires block_tables and seq_lens"):  # :201-202
+        be._decode_attention(q1, 0, InferenceContext(is_prefill=False))
+    with pytest.raises(NotImplementedError):
+        be._decode_attention(q1, 0, InferenceContext(is_prefill=False, block_tables=((0,),), seq_lens=(1,),
+                                                     block_mask=object()))
+
+
+def test_store_kv_error_conventions():
+    be = HipPagedAttentionBackend(_cfg())
+    k = torch.zeros(1, 4, 4, 32, dtype=torch.bfloat16)
+    with pytest.raises(IndexError, match="shape of the mask"):
+        be._store_kv(k, k, 0, (0, 1, 2))
+    with pytest.raises(RuntimeError, match="dtypes match"):
+        be._store_kv(k.float(), k.float(), 0, (0, 1, 2, 3))
+    be._store_kv(k[:, :0], k[:, :0], 0, ())  # nothing to store, no device needed
+
+
+def test_no_cpu_execution_path():
+    """Tensors on the CPU must raise; there is nothing to fall back to."""
+    be = HipPagedAttentionBackend(_cfg())
+    be.set_num_heads(8)
+    k = torch.zeros(1, 4, 4, 32, dtype=torch.bfloat16)
+    q = torch.zeros(1, 4, 8, 32, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="HIP device"):
+        be._store_kv(k, k, 0, (0, 1, 2, 3))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        be.forward(q, k, k, 0, InferenceContext(is_prefill=True))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        be.forward(q[:, :1], k[:, :1], k[:, :1], 0,
+                   InferenceContext(is_prefill=False, block_tables=((0,),), seq_lens=(1,)))
+    with pytest.raises(RuntimeError, match="HIP device"):
+        be._gather_kv_from_cache(0, ((0,),), (3,))
+
+
+def test_out_of_range_slot_is_an_index_error():
+    be = HipPagedAttentionBackend(_cfg())
+    k = torch.zeros(1, 2, 4, 32, dtype=torch.bfloat16)
+    with pytest.raises(IndexError, match="out of bounds"):
+        be._store_kv(k, k, 0, (0, 64))
+
+
+def test_unsupported_features_raise():
+    be = HipPagedAttentionBackend(_cfg(sliding_window=4))
+    with pytest.raises(NotImplementedError):
+        be.get_block_mask(1, 8)
+    with pytest.raises(ValueError):
+        HipPagedAttentionBackend(_cfg(kv_format="int4"))
+    with pytest.raises(ValueError):
+        HipPagedAttentionBackend(_cfg(dtype=torch.float64))
+
+
+def test_fp8_pool_layout():
+    be = HipPagedAttentionBackend(_cfg(kv_format="fp8_e4m3"))
+    assert be.k_cache.dtype == torch.float8_e4m3fn and be.k_cache.shape == (2, 64, 4, 32)
+    assert be.k_scale.shape == (2, 16, 4) and be.k_scale.dtype == torch.float32 and (be.v_scale == 1).all()
+
+
+def test_attention_layer_delegates():
+    calls = []
+
+    class Probe:
+        def forward(self, q, k, v, layer_idx, ctx):
+            calls.append((layer_idx, ctx))
+            return q
+
+    layer = Attention(layer_idx=3, backend=Probe())
+    ctx = InferenceContext(is_prefill=True)
+    x = torch.zeros(1)
+    assert layer(x, x, x, ctx) is x and calls == [(3, ctx)]
+    assert list(layer.parameters()) == []

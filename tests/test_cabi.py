@@ -1,0 +1,138 @@
+"""The C ABI without a GPU: the library loads, exports every symbol the header
+declares, and rejects bad arguments with a status code and a message before it
+touches any device (so none of these calls computes anything)."""
+
+import ctypes
+import os
+import re
+
+import pytest
+
+from research_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "paged_attn.h")
+
+
+def _declared_functions():
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    return sorted(set(re.findall(r"\b(pa_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    names = _declared_functions()
+    assert len(names) >= 10
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in paged_attn.h but not exported"
+
+
+def test_binding_table_matches_header():
+    assert sorted(_lib.SIGNATURES) == _declared_functions()
+
+
+def test_version_and_dtype_sizes():
+    lib = _lib.load()
+    assert lib.pa_version() == 1
+    assert [lib.pa_dtype_bytes(c) for c in (0, 1, 2, 3, 4, -1)] == [4, 2, 2, 1, 0, 0]
+
+
+def test_missing_library_fails_loudly(tmp_path):
+    with pytest.raises(FileNotFoundError, match="no other implementation"):
+        _lib.load(str(tmp_path / "libpaged_attn.so"))
+
+
+FAKE = ctypes.c_void_p(0x1000)  # never dereferenced: every call below is rejected first
+
+
+def _status(name, *args):
+    lib = _lib.load()
+    rc = getattr(lib, name)(*args)
+    return rc, _lib.last_error()
+
+
+def test_scatter_argument_errors():
+    rc, msg = _status("pa_kv_scatter", FAKE, FAKE, FAKE, FAKE, FAKE, 4, 64, 8, 128, 3, None)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "elem_bytes" in msg
+    rc, msg = _status("pa_kv_scatter", FAKE, FAKE, FAKE, FAKE, FAKE, -1, 64, 8, 128, 2, None)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "n_tokens" in msg
+    rc, msg = _status("pa_kv_scatter", None, FAKE, FAKE, FAKE, FAKE, 4, 64, 8, 128, 2, None)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
+    rc, msg = _status("pa_kv_scatter", FAKE, FAKE, FAKE, FAKE, FAKE, 4, 64, 1, 3, 1, None)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "multiple of 4" in msg
+    # nothing to do is fine and needs no pointers
+    assert _status("pa_kv_scatter", None, None, None, None, None, 0, 64, 8, 128, 2, None)[0] == _lib.PA_OK
+
+
+def test_gather_argument_errors():
+    rc, msg = _status("pa_kv_gather", FAKE, FAKE, FAKE, FAKE, FAKE, 4, FAKE, 2, 16, 8, 0, 8, 128, 2, None)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "block_size" in msg
+    rc, msg = _status("pa_kv_gather", FAKE, FAKE, None, FAKE, FAKE, 4, FAKE, 2, 16, 8, 16, 8, 128, 2, None)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
+    assert _status("pa_kv_gather", None, None, None, None, None, 0, None, 0, 0, 8, 16, 8, 128, 2, None)[0] == 0
+
+
+def _decode_args(**kw):
+    a = dict(q=FAKE, k=FAKE, v=FAKE, out=FAKE, bt=FAKE, bt_stride=4, lens=FAKE, ez=None, ks=None, vs=None,
+             batch=2, hq=32, hkv=8, d=128, bs=16, nb=64, scale=0.088, qd=_lib.PA_BF16, kvd=_lib.PA_BF16,
+             chunk=256, chunks=2, ws=FAKE, ws_bytes=1 << 30, stream=None)
+    a.update(kw)
+    return [a[k] for k in ("q", "k", "v", "out", "bt", "bt_stride", "lens", "ez", "ks", "vs", "batch", "hq", "hkv",
+                           "d", "bs", "nb", "scale", "qd", "kvd", "chunk", "chunks", "ws", "ws_bytes", "stream")]
+
+
+def test_decode_argument_errors():
+    rc, msg = _status("pa_decode", *_decode_args(hq=30))
+    assert rc == _lib.PA_ERR_INVALID_ARG and "multiple of num_kv_heads" in msg
+    rc, msg = _status("pa_decode", *_decode_args(chunk=250))
+    assert rc == _lib.PA_ERR_INVALID_ARG and "chunk_tokens" in msg
+    rc, msg = _status("pa_decode", *_decode_args(d=96))
+    assert rc == _lib.PA_ERR_UNSUPPORTED and "head_dim=96" in msg
+    rc, msg = _status("pa_decode", *_decode_args(qd=_lib.PA_F32))
+    assert rc == _lib.PA_ERR_UNSUPPORTED  # q and pool types must match unless the pool is fp8
+    rc, msg = _status("pa_decode", *_decode_args(kvd=_lib.PA_FP8_E4M3))
+    assert rc == _lib.PA_ERR_INVALID_ARG and "k_scale" in msg
+    rc, msg = _status("pa_decode", *_decode_args(ws_bytes=1024))
+    assert rc == _lib.PA_ERR_WORKSPACE and "need" in msg
+    rc, msg = _status("pa_decode", *_decode_args(ws=None))
+    assert rc == _lib.PA_ERR_WORKSPACE
+    rc, msg = _status("pa_decode", *_decode_args(batch=10000))
+    assert rc == _lib.PA_ERR_INVALID_ARG and "sequences one call handles" in msg
+    rc, msg = _status("pa_decode", *_decode_args(q=None))
+    assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
+    assert _status("pa_decode", *_decode_args(batch=0, q=None, ws=None, ws_bytes=0))[0] == _lib.PA_OK
+
+
+def test_decode_planning_arithmetic():
+    lib = _lib.load()
+    assert lib.pa_decode_chunk_tokens(604, 4, 2, 16) == 256
+    assert lib.pa_decode_chunk_tokens(840539, 256, 8, 16) == 256
+    assert lib.pa_decode_chunk_tokens(10_000_000, 64, 8, 16) == 1024
+    assert lib.pa_decode_chunk_tokens(1000, 4, 2, 48) == 288  # rounded up to whole blocks
+    assert lib.pa_decode_chunk_tokens(-1, 4, 2, 16) == _lib.PA_ERR_INVALID_ARG
+    small = lib.pa_decode_workspace_bytes(1, 1, 1, 32)
+    big = lib.pa_decode_workspace_bytes(1000, 256, 32, 128)
+    assert 0 < small < big and big >= 1000 * 32 * 130 * 4
+    assert lib.pa_decode_workspace_bytes(-1, 1, 1, 32) == 0 and "pa_decode_workspace_bytes" in _lib.last_error()
+
+
+def test_prefill_and_quantize_argument_errors():
+    args = [FAKE, FAKE, FAKE, FAKE, FAKE, 4, FAKE, FAKE, FAKE, 2, 16, 32, 8, 128, 16, 64, 0.088, _lib.PA_FP8_E4M3,
+            None]
+    rc, msg = _status("pa_prefill_paged", *args)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "dtype" in msg
+    args[-2] = _lib.PA_BF16
+    args[13] = 80
+    rc, msg = _status("pa_prefill_paged", *args)
+    assert rc == _lib.PA_ERR_UNSUPPORTED
+    rc, msg = _status("pa_quantize_kv_e4m3", FAKE, FAKE, FAKE, 4, 16, 8, 128, _lib.PA_FP8_E4M3, None)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "src_dtype" in msg
+    rc, msg = _status("pa_quantize_kv_e4m3", None, FAKE, FAKE, 4, 16, 8, 128, _lib.PA_F32, None)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
+
+
+def test_error_text_is_cleared_by_a_good_call():
+    _status("pa_kv_scatter", FAKE, FAKE, FAKE, FAKE, FAKE, -1, 64, 8, 128, 2, None)
+    assert _lib.last_error() != ""
+    assert _status("pa_kv_scatter", None, None, None, None, None, 0, 64, 8, 128, 2, None)[0] == 0
+    assert _lib.last_error() == ""

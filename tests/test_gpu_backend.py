@@ -1,0 +1,191 @@
+"""The backend class on the GPU: the flows of the reference's own script
+(rollouts/examples/inference/test_kv_cache.py:81-178, :276-345) run against
+this backend, with values checked where the reference only checks shapes."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_oracle as po
+from research_amd.inference import (
+    Attention,
+    CacheConfig,
+    FlexAttentionBackend,
+    InferenceContext,
+    PagedKVCache,
+    allocate_and_build_context,
+    build_chunked_prefill_context,
+    build_decode_context,
+    extend_and_build_context,
+)
+from research_amd.workloads import make_decode, make_prefill_c3
+from tests.gpu_helpers import announce, assert_close
+
+pytestmark = pytest.mark.gpu
+
+
+def test_store_kv_like_the_reference_script():
+    announce("backend store_kv")
+    config = CacheConfig(num_layers=2, num_kv_heads=4, head_dim=32, num_blocks=16, block_size=4, device="cuda")
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(8)
+    k = torch.randn(1, 4, 4, 32, device="cuda", dtype=torch.bfloat16)
+    v = torch.randn(1, 4, 4, 32, device="cuda", dtype=torch.bfloat16)
+    backend._store_kv(k, v, layer_idx=0, slot_mapping=tuple(range(4)))
+    assert torch.allclose(backend.k_cache[0, 0], k[0, 0])
+    assert torch.allclose(backend.v_cache[0, 3], v[0, 3])
+    assert not backend.k_cache[1].any() and not backend.k_cache[0, 4:].any()
+
+
+def test_attention_correctness_like_the_reference_script():
+    announce("backend prefill correctness")
+    config = CacheConfig(num_layers=1, num_kv_heads=2, head_dim=32, num_blocks=16, block_size=16, device="cuda")
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(4)
+    torch.manual_seed(42)
+    q = torch.randn(2, 8, 4, 32, device="cuda", dtype=torch.bfloat16)
+    k = torch.randn(2, 8, 2, 32, device="cuda", dtype=torch.bfloat16)
+    v = torch.randn(2, 8, 2, 32, device="cuda", dtype=torch.bfloat16)
+    ctx = InferenceContext(is_prefill=True, slot_mapping=None, seq_lens=(8, 8), max_seq_len=8)
+    ours = backend.forward(q, k, v, layer_idx=0, ctx=ctx)
+    ref = po.prefill_literal(q.cpu().float(), k.cpu().float(), v.cpu().float(), 32**-0.5)
+    diff = (ours.cpu().float() - ref).abs()
+    assert diff.max().item() < 0.01 and diff.mean().item() < 0.001
+    assert not backend.k_cache.any()  # slot_mapping=None: cache untouched
+
+
+def test_end_to_end_like_the_reference_script_with_values():
+    announce("backend end to end")
+    cache = PagedKVCache(num_blocks=16, block_size=4)
+    config = CacheConfig(num_layers=2, num_kv_heads=4, head_dim=32, num_blocks=16, block_size=4, device="cuda")
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(8)
+    layer = Attention(layer_idx=1, backend=backend)
+    torch.manual_seed(1)
+    ctx, cached = allocate_and_build_context(cache, seq_id=0, token_ids=[1, 2, 3, 4, 5])
+    q = torch.randn(1, 5, 8, 32, device="cuda", dtype=torch.bfloat16)
+    k = torch.randn(1, 5, 4, 32, device="cuda", dtype=torch.bfloat16)
+    v = torch.randn(1, 5, 4, 32, device="cuda", dtype=torch.bfloat16)
+    out = layer(q, k, v, ctx)
+    assert out.shape == (1, 5, 8, 32) and out.is_contiguous()
+    assert_close(out, po.dense_prefill(q.cpu(), k.cpu(), v.cpu(), backend.scale), 2e-2, "prefill")
+
+    # the sequence's last block is partial, so append_token does not grow it and position 5 still fits block 1
+    ctx = extend_and_build_context(cache, seq_id=0, new_token=6, current_len=5)
+    q1 = torch.randn(1, 1, 8, 32, device="cuda", dtype=torch.bfloat16)
+    k1 = torch.randn(1, 1, 4, 32, device="cuda", dtype=torch.bfloat16)
+    v1 = torch.randn(1, 1, 4, 32, device="cuda", dtype=torch.bfloat16)
+    out = layer(q1, k1, v1, ctx)
+    assert out.shape == (1, 1, 8, 32)
+    k_all, v_all = torch.cat([k, k1], 1).cpu(), torch.cat([v, v1], 1).cpu()
+    want = po.dense_prefill(torch.cat([torch.zeros_like(q), q1], 1).cpu(), k_all, v_all, backend.scale)[:, 5:]
+    assert_close(out, want, 2e-2, "decode sees prompt + its own token")
+    kg, vg = backend._gather_kv_from_cache(1, ctx.block_tables, ctx.seq_lens)
+    assert torch.equal(kg.cpu(), k_all) and torch.equal(vg.cpu(), v_all)
+    assert not backend.k_cache[0].any()  # only layer 1 was written
+
+    cache.deallocate(seq_id=0)
+    assert cache.num_free_blocks() == 16
+    backend.clear_cache()
+    assert not backend.k_cache.any() and not backend.v_cache.any()
+
+
+def test_dropped_token_when_the_table_cannot_grow():
+    """allocate() of exactly one partial block, then decode until the block is full:
+    the reference's allocator never adds a block (no hash on a partial block), the
+    context builder emits slot -1, the append drops the row and the gather reads zeros."""
+    announce("backend dropped token")
+    cache = PagedKVCache(num_blocks=4, block_size=2)
+    config = CacheConfig(num_layers=1, num_kv_heads=1, head_dim=32, num_blocks=4, block_size=2, device="cuda",
+                         dtype=torch.float32)
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(2)
+    ctx, _ = allocate_and_build_context(cache, 0, [7])
+    torch.manual_seed(2)
+    k0, v0 = torch.randn(1, 1, 1, 32, device="cuda"), torch.randn(1, 1, 1, 32, device="cuda")
+    backend.forward(torch.randn(1, 1, 2, 32, device="cuda"), k0, v0, 0, ctx)
+    ks, vs = [k0], [v0]
+    for cur in (1, 2):
+        ctx = extend_and_build_context(cache, 0, new_token=9, current_len=cur)
+        k1, v1 = torch.randn(1, 1, 1, 32, device="cuda"), torch.randn(1, 1, 1, 32, device="cuda")
+        q1 = torch.randn(1, 1, 2, 32, device="cuda")
+        out = backend.forward(q1, k1, v1, 0, ctx)
+        ks.append(k1)
+        vs.append(v1)
+    assert ctx.slot_mapping == (-1,) and ctx.seq_lens == (3,) and len(ctx.block_tables[0]) == 1
+    lit = po.decode_literal(q1.cpu(), backend.k_cache[0].cpu(), backend.v_cache[0].cpu(), ctx.block_tables,
+                            ctx.seq_lens, 2, backend.scale)
+    assert_close(out, lit, 1e-5, "third token was dropped, attends as a zero key")
+    assert torch.equal(backend.k_cache[0, : 2].cpu(), torch.cat(ks[:2], 1)[0])
+
+
+def test_ragged_decode_both_semantics_on_c1():
+    announce("backend c1 decode masked / pad_zero_keys")
+    w = make_decode("c1")
+    tables = tuple(tuple(int(b) for b in t) for t in w.block_tables)
+    lens = tuple(int(n) for n in w.seq_lens)
+    ctx = InferenceContext(is_prefill=False, block_tables=tables, seq_lens=lens, max_seq_len=max(lens))
+    for pad in (False, True):
+        config = CacheConfig(num_layers=1, num_kv_heads=2, head_dim=64, num_blocks=128, block_size=16,
+                             dtype=torch.float32, device="cuda")
+        backend = FlexAttentionBackend(config, pad_zero_keys=pad)
+        backend.set_num_heads(8)
+        backend.k_cache[0].copy_(w.k_pool)
+        backend.v_cache[0].copy_(w.v_pool)
+        out = backend.forward(w.q[:, None].cuda(), None, None, 0, ctx)
+        want = po.paged_decode(w.q, w.k_pool, w.v_pool, tables, lens, 16, w.scale, pad_zero_keys=pad)
+        assert_close(out[:, 0], want, 1e-5, f"pad_zero_keys={pad}")
+        if pad:
+            lit = po.decode_literal(w.q[:, None], w.k_pool, w.v_pool, tables, lens, 16, w.scale,
+                                    vectorised_gather=True)
+            assert_close(out, lit, 1e-5, "literal reference restatement")
+
+
+def test_chunked_prefill_through_the_backend_with_allocator_shared_prefix():
+    """Two prompts with a common 32-token prefix: the allocator hands out the same
+    leading block ids, the second prompt is prefilled as a chunk over the cached prefix."""
+    announce("backend chunked prefill")
+    bs = 16
+    cache = PagedKVCache(num_blocks=32, block_size=bs)
+    config = CacheConfig(num_layers=1, num_kv_heads=2, head_dim=64, num_blocks=32, block_size=bs, device="cuda")
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(4)
+    rng = np.random.default_rng(3)
+    prefix = rng.integers(0, 100, 32).tolist()
+    a, b = prefix + [1, 2, 3], prefix + [4, 5, 6, 7, 8]
+    torch.manual_seed(4)
+    ctx_a, _ = allocate_and_build_context(cache, 0, a)
+    qa = torch.randn(1, len(a), 4, 64, device="cuda", dtype=torch.bfloat16)
+    ka = torch.randn(1, len(a), 2, 64, device="cuda", dtype=torch.bfloat16)
+    va = torch.randn(1, len(a), 2, 64, device="cuda", dtype=torch.bfloat16)
+    backend.forward(qa, ka, va, 0, ctx_a)
+    blocks_b = cache.allocate(1, b)
+    assert cache.get_cached_tokens(1) == 32 and blocks_b[:2] == ctx_a.block_tables[0][:2]
+    ctx_b = build_chunked_prefill_context(cache, [1], [32], [len(b) - 32], [blocks_b])
+    qb = torch.randn(1, 5, 4, 64, device="cuda", dtype=torch.bfloat16)
+    kb = torch.randn(1, 5, 2, 64, device="cuda", dtype=torch.bfloat16)
+    vb = torch.randn(1, 5, 2, 64, device="cuda", dtype=torch.bfloat16)
+    out = backend.forward(qb, kb, vb, 0, ctx_b)
+    k_full = torch.cat([ka[:, :32], kb], 1).cpu()
+    v_full = torch.cat([va[:, :32], vb], 1).cpu()
+    q_full = torch.cat([torch.zeros(1, 32, 4, 64, dtype=torch.bfloat16), qb.cpu()], 1)
+    want = po.dense_prefill(q_full, k_full, v_full, backend.scale)[:, 32:]
+    assert_close(out, want, 2e-2, "chunk over allocator-shared prefix")
+
+
+def test_fp8_backend_decode():
+    announce("backend fp8 decode")
+    w = make_decode("c5", batch=2, len_range=(500, 2000))
+    config = CacheConfig(num_layers=1, num_kv_heads=8, head_dim=128, num_blocks=w.num_blocks, block_size=16,
+                         device="cuda", kv_format="fp8_e4m3")
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(32)
+    backend.quantize_from(w.k_pool.cuda(), w.v_pool.cuda(), 0)
+    tables = tuple(tuple(int(b) for b in t) for t in w.block_tables)
+    lens = tuple(int(n) for n in w.seq_lens)
+    ctx = build_decode_context(PagedKVCache(1, 16), [0, 1], list(lens), list(tables))
+    ctx = InferenceContext(is_prefill=False, block_tables=ctx.block_tables, seq_lens=ctx.seq_lens)
+    out = backend.forward(w.q[:, None].cuda(), None, None, 0, ctx)
+    kd = po.dequantize_kv_e4m3(backend.k_cache[0].cpu().view(torch.uint8), backend.k_scale[0].cpu(), 16)
+    vd = po.dequantize_kv_e4m3(backend.v_cache[0].cpu().view(torch.uint8), backend.v_scale[0].cpu(), 16)
+    assert_close(out[:, 0], po.paged_decode(w.q, kd, vd, tables, lens, 16, w.scale), 6e-2, "fp8 backend")

@@ -1,0 +1,171 @@
+"""Paged decode attention on the GPU against the CPU checker, through the C ABI.
+
+Tolerances (absolute on |want|<=1, relative above): 1e-5 for the fp32 pool,
+2e-2 for bf16/fp16 pools with fp32 accumulation, 6e-2 for the fp8-e4m3 pool
+against dequantise-then-attend.
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_oracle as po
+from research_amd import ops
+from research_amd.workloads import make_decode
+from tests.gpu_helpers import DEV, announce, assert_close, run_decode
+
+pytestmark = pytest.mark.gpu
+
+
+def _lists(w):
+    return [t.tolist() for t in w.block_tables]
+
+
+def _gpu_decode(w, **kw):
+    return run_decode(w.q.to(DEV), w.k_pool.to(DEV), w.v_pool.to(DEV), _lists(w), w.seq_lens, w.block_size, w.scale,
+                      **kw)
+
+
+def test_c1_fp32_masked_and_pad_zero_keys():
+    """BASELINE config 1 in both semantics; the padded one against the literal restatement too."""
+    announce("decode c1 fp32")
+    w = make_decode("c1")
+    want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, w.block_size, w.scale)
+    assert_close(_gpu_decode(w), want, 1e-5, "c1 masked")
+    pad = (w.seq_lens.max() - w.seq_lens).tolist()
+    got = _gpu_decode(w, extra_zero=pad)
+    want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, w.block_size, w.scale, pad_zero_keys=True)
+    assert_close(got, want, 1e-5, "c1 pad_zero_keys")
+    lit = po.decode_literal(w.q[:, None], w.k_pool, w.v_pool, _lists(w), w.seq_lens, w.block_size, w.scale,
+                            vectorised_gather=True)[:, 0]
+    assert_close(got, lit, 1e-5, "c1 vs literal reference restatement")
+
+
+def test_c2_bf16_full_size():
+    """BASELINE config 2 at full size (B=64, 141 622 keys)."""
+    announce("decode c2 bf16 full")
+    w = make_decode("c2")
+    assert w.total_tokens == 141622
+    want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, w.block_size, w.scale)
+    assert_close(_gpu_decode(w), want, 2e-2, "c2")
+
+
+def test_c4_shape_reduced_batch():
+    """BASELINE config 4's shape (Hq=32, Hkv=8, D=128, lognormal lengths) on 24 sequences."""
+    announce("decode c4 reduced")
+    w = make_decode("c4", batch=24, len_range=(64, 6000))
+    want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, w.block_size, w.scale)
+    assert_close(_gpu_decode(w), want, 2e-2, "c4 reduced")
+
+
+def test_split_count_does_not_change_the_result():
+    announce("decode split invariance")
+    w = make_decode("c4", batch=12, len_range=(64, 5000), seed=77)
+    ref = _gpu_decode(w, chunk_tokens=16 * 1024).float()  # one chunk per sequence
+    for chunk in (16, 64, 256, 1024):
+        assert_close(_gpu_decode(w, chunk_tokens=chunk).float(), ref, 1e-2, f"chunk={chunk}")
+
+
+def test_pool_permutation_and_constant_values():
+    announce("decode permutation / constant V")
+    w = make_decode("c2", batch=5, len_range=(30, 400), seed=5)
+    base = _gpu_decode(w).float()
+    rng = np.random.default_rng(0)
+    perm = rng.permutation(w.num_blocks)  # new id of block i is perm[i]
+    src = torch.from_numpy(np.argsort(perm))  # block living at new position j
+    bs = w.block_size
+    k2 = w.k_pool.reshape(w.num_blocks, bs, *w.k_pool.shape[1:])[src].reshape(w.k_pool.shape)
+    v2 = w.v_pool.reshape(w.num_blocks, bs, *w.v_pool.shape[1:])[src].reshape(w.v_pool.shape)
+    tables2 = [perm[t].tolist() for t in w.block_tables]
+    moved = run_decode(w.q.to(DEV), k2.to(DEV), v2.to(DEV), tables2, w.seq_lens, bs, w.scale).float()
+    assert torch.equal(moved, base)  # same arithmetic in the same order: bit-identical
+    row = torch.linspace(-2, 2, w.head_dim).to(w.dtype)
+    vconst = row.expand_as(w.v_pool).contiguous()
+    out = run_decode(w.q.to(DEV), w.k_pool.to(DEV), vconst.to(DEV), _lists(w), w.seq_lens, bs, w.scale)
+    assert_close(out, row.float().expand(w.batch, w.num_q_heads, w.head_dim), 1e-2, "constant V")
+
+
+@pytest.mark.parametrize("hq,hkv,d,dtype", [
+    (14, 2, 64, torch.bfloat16),   # group of 7 (Qwen2.5-0.5B), padded to 8 in the kernel
+    (8, 4, 32, torch.bfloat16),    # the reference script's shape (test_kv_cache.py:131-136)
+    (6, 6, 128, torch.float16),    # MHA, 6 kv heads: two per wave load
+    (3, 1, 256, torch.bfloat16),   # MQA, group of 3, D=256
+    (32, 2, 128, torch.float32),   # group of 16: two passes of 8
+    (5, 5, 64, torch.float32),     # odd head count: one kv head per wave load
+])
+def test_head_layouts(hq, hkv, d, dtype):
+    announce(f"decode heads hq={hq} hkv={hkv} d={d} {dtype}")
+    rng = np.random.default_rng(hq * 1000 + d)
+    bs, nb = 4, 64
+    lens = [37, 1, 100, 64, 5]
+    perm = rng.permutation(nb)
+    tables, at = [], 0
+    for n in lens:
+        c = -(-n // bs)
+        tables.append(perm[at : at + c].tolist())
+        at += c
+    q = torch.from_numpy(rng.standard_normal((len(lens), hq, d)).astype(np.float32)).to(dtype)
+    kp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
+    vp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
+    want = po.paged_decode(q, kp, vp, tables, lens, bs, d**-0.5)
+    got = run_decode(q.to(DEV), kp.to(DEV), vp.to(DEV), tables, lens, bs, d**-0.5, chunk_tokens=32)
+    assert_close(got, want, 1e-5 if dtype == torch.float32 else 2e-2, "head layout")
+
+
+def test_edge_cases_empty_short_table_and_garbage_tail():
+    announce("decode edge cases")
+    rng = np.random.default_rng(21)
+    bs, nb, hq, hkv, d = 16, 12, 8, 2, 64
+    q = torch.from_numpy(rng.standard_normal((4, hq, d)).astype(np.float32))
+    kp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32))
+    vp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32))
+    tables = [[3, 7], [], [5], [9, 1, 0]]
+    lens = [20, 0, 40, 33]  # seq 1 empty; seq 2's table covers 16 of its 40 keys
+    # poison everything past each sequence's length inside its last block: must never be read as a key
+    kp[7 * bs + 4 : 8 * bs] = float("nan")
+    vp[7 * bs + 4 : 8 * bs] = float("inf")
+    kp[0 * bs + 1 : 1 * bs] = float("nan")
+    vp[0 * bs + 1 : 1 * bs] = float("nan")
+    want = po.paged_decode(q, kp, vp, tables, lens, bs, 0.125)
+    got = run_decode(q.to(DEV), kp.to(DEV), vp.to(DEV), tables, lens, bs, 0.125)
+    assert_close(got, want, 1e-5, "edge")
+    assert not got[1].any()  # empty sequence -> zeros
+    lit = po.decode_literal(q[2:3, None], kp, vp, tables[2:3], lens[2:3], bs, 0.125)[:, 0]
+    assert_close(got[2:3], lit, 1e-5, "short table vs literal restatement")
+
+
+def test_block_ids_outside_the_pool_do_not_fault():
+    announce("decode bad block ids")
+    rng = np.random.default_rng(22)
+    bs, nb = 16, 4
+    q = torch.from_numpy(rng.standard_normal((1, 4, 64)).astype(np.float32))
+    kp = torch.from_numpy(rng.standard_normal((nb * bs, 2, 64)).astype(np.float32))
+    vp = torch.from_numpy(rng.standard_normal((nb * bs, 2, 64)).astype(np.float32))
+    got = run_decode(q.to(DEV), kp.to(DEV), vp.to(DEV), [[2, 1000, -3]], [48], bs, 0.125)
+    want = po.paged_decode(q, kp, vp, [[2]], [48], bs, 0.125)  # the two bad blocks act as missing ones
+    assert_close(got, want, 1e-5, "bad ids")
+
+
+def test_quantize_matches_torch_e4m3_bit_for_bit():
+    announce("quantize e4m3")
+    w = make_decode("c5", batch=3, len_range=(50, 300))
+    w.k_pool[5 * 16 : 6 * 16, 3] = 0  # an all-zero tile
+    for src in (w.k_pool, w.v_pool.float(), w.v_pool.to(torch.float16)):
+        bits, scale = ops.quantize_kv_e4m3(src.to(DEV), w.block_size)
+        eb, es = po.quantize_kv_e4m3(src, w.block_size)
+        assert torch.equal(scale.cpu(), es)
+        assert torch.equal(bits.cpu().view(torch.uint8), eb)
+
+
+def test_c5_fp8_reduced():
+    """BASELINE config 5's shape with shorter contexts: e4m3 pool, per-(block, head) scales, bf16 q."""
+    announce("decode c5 fp8 reduced")
+    w = make_decode("c5", batch=4, len_range=(3000, 9000))
+    kb, ks = ops.quantize_kv_e4m3(w.k_pool.to(DEV), w.block_size)
+    vb, vs = ops.quantize_kv_e4m3(w.v_pool.to(DEV), w.block_size)
+    kd = po.dequantize_kv_e4m3(kb.cpu().view(torch.uint8), ks.cpu(), w.block_size)
+    vd = po.dequantize_kv_e4m3(vb.cpu().view(torch.uint8), vs.cpu(), w.block_size)
+    want = po.paged_decode(w.q, kd, vd, _lists(w), w.seq_lens, w.block_size, w.scale)
+    got = run_decode(w.q.to(DEV), kb, vb, _lists(w), w.seq_lens, w.block_size, w.scale, k_scale=ks, v_scale=vs)
+    assert_close(got, want, 6e-2, "c5 fp8")
+    assert_close(got, want, 2e-2, "c5 fp8 (the arithmetic itself is as tight as bf16)")

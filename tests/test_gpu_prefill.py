@@ -1,0 +1,99 @@
+"""Causal prefill on the GPU against the CPU checker: the dense case the
+reference has (its own recipe and tolerance) and chunked prefill over shared
+prefix blocks."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_oracle as po
+from research_amd import ops
+from research_amd.workloads import make_prefill_c3
+from tests.gpu_helpers import DEV, announce, assert_close, tables_to_device
+
+pytestmark = pytest.mark.gpu
+
+
+def _i32(x):
+    return torch.tensor(list(x), dtype=torch.int32, device=DEV)
+
+
+def _run_chunked(w, q=None):
+    """Append prefix and chunks, then prefill every chunk over its prefix, all on the device."""
+    shape = (w.num_blocks * w.block_size, w.num_kv_heads, w.head_dim)
+    kc = torch.zeros(shape, dtype=w.dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    ops.kv_scatter(kc, vc, w.k_prefix.to(DEV), w.v_prefix.to(DEV), torch.from_numpy(w.prefix_slots()).to(DEV))
+    ops.kv_scatter(kc, vc, w.k_chunk.reshape(-1, *shape[1:]).to(DEV), w.v_chunk.reshape(-1, *shape[1:]).to(DEV),
+                   torch.from_numpy(w.chunk_slots()).to(DEV))
+    S, C = w.num_seqs, w.chunk_len
+    q = w.q if q is None else q
+    out = ops.prefill_paged(q.reshape(S * C, w.num_q_heads, w.head_dim).to(DEV), kc, vc,
+                            tables_to_device(w.block_tables), _i32([w.prefix_len + C] * S), _i32([C] * S),
+                            _i32(np.arange(S) * C), C, w.block_size, w.scale)
+    return out.reshape(S, C, w.num_q_heads, w.head_dim), kc, vc
+
+
+def test_dense_prefill_reference_recipe():
+    """B=2,T=8,Hq=4,Hkv=2,D=32 bf16, seed 42; bars max<0.01, mean<0.001 (test_kv_cache.py:276-345)."""
+    announce("prefill reference recipe")
+    torch.manual_seed(42)
+    q = torch.randn(2, 8, 4, 32).to(torch.bfloat16)
+    k = torch.randn(2, 8, 2, 32).to(torch.bfloat16)
+    v = torch.randn(2, 8, 2, 32).to(torch.bfloat16)
+    out = ops.prefill_paged(q.reshape(16, 4, 32).to(DEV), k.reshape(16, 2, 32).to(DEV), v.reshape(16, 2, 32).to(DEV),
+                            _i32([0, 1]).reshape(2, 1), _i32([8, 8]), _i32([8, 8]), _i32([0, 8]), 8, 8, 32**-0.5)
+    ref = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(1, 2), k.transpose(1, 2).repeat_interleave(2, 1), v.transpose(1, 2).repeat_interleave(2, 1),
+        is_causal=True).transpose(1, 2)
+    diff = (out.reshape(2, 8, 4, 32).cpu().float() - ref.float()).abs()
+    assert diff.max() < 0.01 and diff.mean() < 0.001
+    assert_close(out.reshape(2, 8, 4, 32), po.dense_prefill(q, k, v, 32**-0.5), 2e-2, "dense prefill")
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2), (torch.float16, 2e-2)])
+def test_chunked_prefill_small(dtype, tol):
+    announce(f"chunked prefill small {dtype}")
+    w = make_prefill_c3(num_seqs=3, prefix_len=48, chunk_len=21, num_q_heads=8, num_kv_heads=2, head_dim=64,
+                        dtype=dtype)
+    got, kc, vc = _run_chunked(w)
+    want = po.paged_prefill_chunk(w.q, kc.cpu(), vc.cpu(), w.block_tables, [48] * 3, [21] * 3, w.block_size, w.scale)
+    assert_close(got, want, tol, "chunked small")
+
+
+def test_chunked_prefill_ragged_chunks_and_prefixes():
+    announce("chunked prefill ragged")
+    rng = np.random.default_rng(31)
+    bs, nb, hq, hkv, d = 16, 40, 4, 2, 64
+    prefix, chunk = [0, 32, 19], [17, 5, 30]
+    cmax = 30
+    perm = rng.permutation(nb)
+    tables, at = [], 0
+    for p, c in zip(prefix, chunk):
+        n = -(-(p + c) // bs)
+        tables.append(perm[at : at + n].tolist())
+        at += n
+    kc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32))
+    vc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32))
+    q = torch.from_numpy(rng.standard_normal((3, cmax, hq, d)).astype(np.float32))
+    want = po.paged_prefill_chunk(q, kc, vc, tables, prefix, chunk, bs, 0.125)
+    out = torch.zeros(3 * cmax, hq, d, device=DEV)
+    ops.prefill_paged(q.reshape(3 * cmax, hq, d).to(DEV), kc.to(DEV), vc.to(DEV), tables_to_device(tables),
+                      _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk), _i32(np.arange(3) * cmax), cmax, bs,
+                      0.125, out=out)
+    assert_close(out.reshape(3, cmax, hq, d), want, 1e-5, "ragged chunks")
+
+
+def test_c3_reduced_shared_prefix():
+    """BASELINE config 3's head shape with 4 sequences sharing a 512-token prefix, 64-token chunks."""
+    announce("chunked prefill c3 reduced")
+    w = make_prefill_c3(num_seqs=4, prefix_len=512, chunk_len=64)
+    got, kc, vc = _run_chunked(w)
+    want = po.paged_prefill_chunk(w.q, kc.cpu(), vc.cpu(), w.block_tables, [512] * 4, [64] * 4, w.block_size, w.scale)
+    assert_close(got, want, 2e-2, "c3 reduced")
+    # equals rows [P:P+C] of full causal attention over prefix+chunk for one sequence
+    s = 2
+    full = po.dense_prefill(torch.cat([torch.zeros(512, 32, 128, dtype=w.dtype), w.q[s]])[None],
+                            torch.cat([w.k_prefix, w.k_chunk[s]])[None], torch.cat([w.v_prefix, w.v_chunk[s]])[None],
+                            w.scale)
+    assert_close(got[s], full[0, 512:], 2e-2, "rows of the full-sequence prefill")
