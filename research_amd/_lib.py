@@ -82,6 +82,13 @@ def load(path: Optional[str] = None) -> ctypes.CDLL:
             f"{target} is missing: build it with `python -m research_amd.build` "
             "(hipcc --offload-arch=gfx950); this backend has no other implementation"
         )
+    # The library needs libamdhip64.so.7.  PyTorch-ROCm ships its own copy under
+    # that soname; importing torch first makes the loader bind this library to
+    # the runtime torch already uses.  Loaded the other way round the process
+    # ends up with two HIP runtimes and launches fail with "no ROCm-capable
+    # device" on pointers that belong to the other one.
+    import torch  # noqa: F401
+
     lib = ctypes.CDLL(target)
     for name, (restype, argtypes) in SIGNATURES.items():
         fn = getattr(lib, name)  # AttributeError names the missing symbol
