@@ -111,15 +111,12 @@ def main() -> int:
         k_pool, v_pool, k_scale, v_scale = w.k_pool.to(dev), w.v_pool.to(dev), None, None
     tables = torch.from_numpy(w.padded_tables()).to(dev)
     lens = torch.from_numpy(w.seq_lens.astype(np.int32)).to(dev)
-    chunk = ops.decode_plan(w.total_tokens, w.batch, w.num_kv_heads, w.block_size)
-    total_chunks = int((-(-w.seq_lens // chunk)).sum())
-    ws = torch.empty(ops.decode_workspace_bytes(total_chunks, w.batch, w.num_q_heads, w.head_dim),
-                     dtype=torch.uint8, device=dev)
+    ws = ops.decode_workspace(q, k_pool)
     out = torch.empty_like(q)
 
     def step(entry="pa_decode"):
-        ops.decode(q, k_pool, v_pool, tables, lens, w.block_size, w.scale, chunk, total_chunks, ws,
-                   k_scale=k_scale, v_scale=v_scale, out=out, entry=entry)
+        ops.decode(q, k_pool, v_pool, tables, lens, w.block_size, w.scale, ws, k_scale=k_scale, v_scale=v_scale,
+                   out=out, entry=entry)
 
     def timed(entry, steps):
         """Average milliseconds per launch: HIP events on the launch stream around `steps` calls."""
@@ -173,7 +170,7 @@ def main() -> int:
             "batch": w.batch, "num_q_heads": w.num_q_heads, "num_kv_heads": w.num_kv_heads,
             "head_dim": w.head_dim, "block_size": w.block_size, "total_keys": w.total_tokens,
             "max_len": int(w.seq_lens.max()), "kv_format": w.kv_format or str(w.dtype).replace("torch.", ""),
-            "chunk_tokens": chunk, "total_chunks": total_chunks, "algorithmic_bytes": alg_bytes,
+            "algorithmic_bytes": alg_bytes,
             "seed": 1000 + int(args.workload[1]), "generate_s": round(t_gen, 1),
         },
         "roofline": {

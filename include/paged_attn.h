@@ -89,19 +89,16 @@ int pa_kv_gather(const void *k_cache, const void *v_cache, void *k_out, void *v_
                  int num_kv_heads, int head_dim, int elem_bytes, void *stream);
 
 /*
- * Split-K planning for pa_decode (host arithmetic only, no GPU call).
- * pa_decode cuts every sequence into chunks of `chunk_tokens` keys (a multiple
- * of block_size); one workgroup pass handles one chunk of one sequence and the
- * partial results are merged by a reduction pass.
- *   pa_decode_chunk_tokens   : suggested chunk size for a batch holding
- *                              total_tokens keys (sum of seq_lens); <= 0 on error
- *   pa_decode_workspace_bytes: workspace needed when the batch has at most
- *                              total_chunks = sum_b ceil(seq_lens[b]/chunk_tokens)
- *                              chunks (batch*ceil(max_seq_len/chunk_tokens) is
- *                              always enough); 0 on error
+ * Workspace of pa_decode in bytes (host arithmetic only, no GPU call); 0 on
+ * error.  pa_decode splits the batch's pool blocks evenly over a machine-sized
+ * grid of workgroups; a sequence whose blocks fall into several workgroups
+ * leaves one partial result per piece in the workspace.  The size depends on
+ * the shapes only, never on the sequence lengths, so one allocation serves
+ * every step of a model.  Alignment: 256 bytes.  Contents need not be
+ * initialised and are not kept between calls.
  */
-int pa_decode_chunk_tokens(int64_t total_tokens, int batch, int num_kv_heads, int block_size);
-size_t pa_decode_workspace_bytes(int64_t total_chunks, int batch, int num_q_heads, int head_dim);
+size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                                 int kv_dtype);
 
 /*
  * Paged decode attention.  Replaces FlexAttentionBackend._decode_attention
@@ -111,8 +108,9 @@ size_t pa_decode_workspace_bytes(int64_t total_chunks, int batch, int num_q_head
  *     out[b][h] = softmax_j( scale * q[b][h] . K[b][j][kvh] ) . V[b][j][kvh],  j < seq_lens[b]
  * with K/V rows addressed through the block table as in pa_kv_gather; a
  * position whose block-table entry is missing acts as an all-zero key and
- * value (logit 0), as it does in the reference.  Accumulation is fp32.
- *   q, out        : [batch][num_q_heads][head_dim], dtype q_dtype
+ * value (logit 0), as it does in the reference.  Accumulation is fp32.  All
+ * integer inputs stay on the device: the host never reads seq_lens.
+ *   q, out        : [batch][num_q_heads][head_dim], dtype q_dtype, 16-byte aligned
  *   kv_dtype      : q_dtype, or PA_FP8_E4M3 with k_scale/v_scale =
  *                   float[num_blocks][num_kv_heads] (value = fp8 * scale)
  *   extra_zero_keys: NULL, or int32[batch]: that many additional all-zero
@@ -120,36 +118,36 @@ size_t pa_decode_workspace_bytes(int64_t total_chunks, int batch, int num_q_head
  *                   zero-pads ragged batches to the longest sequence without a
  *                   mask (:253-264, :227-229); passing max_len - seq_lens[b]
  *                   reproduces it.
- *   chunk_tokens, total_chunks, workspace(_bytes): see the planning calls.
- *   A sequence of length 0 with no extra keys yields zeros.
+ *   batch         : at most 8192 sequences per call
+ *   workspace     : pa_decode_workspace_bytes(...) bytes
+ *   A sequence of length 0 yields zeros.
  */
 int pa_decode(const void *q, const void *k_cache, const void *v_cache, void *out,
               const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
               const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale,
               int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-              int64_t num_blocks, float scale, int q_dtype, int kv_dtype, int chunk_tokens,
-              int64_t total_chunks, void *workspace, size_t workspace_bytes, void *stream);
+              int64_t num_blocks, float scale, int q_dtype, int kv_dtype, void *workspace,
+              size_t workspace_bytes, void *stream);
 
 /*
  * The two passes of pa_decode as separate calls, same arguments: pa_decode ==
  * pa_decode_split followed by pa_decode_reduce on the same stream and
- * workspace.  For callers that time or schedule the passes separately, or
- * merge several split passes' workspaces themselves.  (The reference has one
- * fused call site, attention/flex_backend.py:227-229; these have no separate
- * counterpart there.)
+ * workspace.  For callers that time or schedule the passes separately.  (The
+ * reference has one fused call site, attention/flex_backend.py:227-229; these
+ * have no separate counterpart there.)
  */
 int pa_decode_split(const void *q, const void *k_cache, const void *v_cache, void *out,
                     const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
                     const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale,
                     int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-                    int64_t num_blocks, float scale, int q_dtype, int kv_dtype, int chunk_tokens,
-                    int64_t total_chunks, void *workspace, size_t workspace_bytes, void *stream);
+                    int64_t num_blocks, float scale, int q_dtype, int kv_dtype, void *workspace,
+                    size_t workspace_bytes, void *stream);
 int pa_decode_reduce(const void *q, const void *k_cache, const void *v_cache, void *out,
                      const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
                      const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale,
                      int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-                     int64_t num_blocks, float scale, int q_dtype, int kv_dtype, int chunk_tokens,
-                     int64_t total_chunks, void *workspace, size_t workspace_bytes, void *stream);
+                     int64_t num_blocks, float scale, int q_dtype, int kv_dtype, void *workspace,
+                     size_t workspace_bytes, void *stream);
 
 /*
  * Causal prefill attention over a paged context.  Covers both

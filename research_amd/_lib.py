@@ -37,13 +37,11 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int64, c_int,
          c_int, c_int, c_int, c_void_p],
     ),
-    "pa_decode_chunk_tokens": (c_int, [c_int64, c_int, c_int, c_int]),
-    "pa_decode_workspace_bytes": (c_size_t, [c_int64, c_int, c_int, c_int]),
+    "pa_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "pa_decode": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
-         c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_int, c_int64, c_void_p, c_size_t,
-         c_void_p],
+         c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "pa_decode_split": None,   # same signature as pa_decode, filled in below
     "pa_decode_reduce": None,

@@ -2,6 +2,8 @@
 // planning arithmetic, workspace layout and the two launches.  The kernels are
 // in decode_impl.h and are instantiated per pool element type in
 // decode_inst_*.hip.
+#include <stdlib.h>
+
 #include "decode_impl.h"
 
 namespace pa_decode_detail {
@@ -43,16 +45,22 @@ namespace {
 
 size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
 
-// workspace = [chunk_prefix int32[batch+1]] [part_ml float[cap][hq][2]] [part_acc float[cap][hq][D]]
+constexpr int kMaxSplitGrid = 4096;  // upper bound of the split pass's grid, fixes the workspace size
+
+// workspace = [block_prefix int32[batch+1]] [part_ml float[slots][heads][2]] [part_acc float[slots][heads][D]]
+// with heads = hpw * NREP query heads of one plane and slots = kMaxSplitGrid + planes * batch.
 struct WsLayout {
     size_t prefix_off, ml_off, acc_off, total;
+    int64_t slots;
 };
-WsLayout ws_layout(int64_t cap, int batch, int hq, int d) {
+WsLayout ws_layout(int batch, const PoolArgs &p, int nrep_t, int d) {
     WsLayout w;
+    const size_t heads = (size_t)p.hpw * nrep_t;
+    w.slots = (int64_t)kMaxSplitGrid + (int64_t)p.n_hgroups * p.n_rgroups * batch;
     w.prefix_off = 0;
     w.ml_off = align_up((size_t)(batch + 1) * 4, 256);
-    w.acc_off = w.ml_off + align_up((size_t)cap * hq * 2 * 4, 256);
-    w.total = w.acc_off + align_up((size_t)cap * hq * d * 4, 256);
+    w.acc_off = w.ml_off + align_up((size_t)w.slots * heads * 2 * 4, 256);
+    w.total = w.acc_off + align_up((size_t)w.slots * heads * d * 4, 256);
     return w;
 }
 
@@ -68,33 +76,17 @@ int num_cus() {
     return cached;
 }
 
-}  // namespace
-
-extern "C" int pa_decode_chunk_tokens(int64_t total_tokens, int batch, int num_kv_heads, int block_size) {
-    pa_clear_error();
-    if (total_tokens < 0 || batch < 0 || num_kv_heads <= 0 || block_size <= 0)
-        return pa_fail(PA_ERR_INVALID_ARG, "pa_decode_chunk_tokens: negative size or non-positive head count / block size");
-    // Aim for a few thousand chunks across the batch, between 256 and 1024 keys
-    // each: enough work items to keep 256 CUs busy through the tail, few enough
-    // that the partials stay a small fraction of the KV bytes.
-    int64_t target = 256;
-    const int64_t want_chunks = 4096;
-    while (target < 1024 && total_tokens / target > want_chunks) target *= 2;
-    int64_t blocks = (target + block_size - 1) / block_size;
-    if (blocks < 1) blocks = 1;
-    return (int)(blocks * block_size);
-}
-
-extern "C" size_t pa_decode_workspace_bytes(int64_t total_chunks, int batch, int num_q_heads, int head_dim) {
-    pa_clear_error();
-    if (total_chunks < 0 || batch < 0 || num_q_heads <= 0 || head_dim <= 0) {
-        pa_fail(PA_ERR_INVALID_ARG, "pa_decode_workspace_bytes: negative size or non-positive head count / head_dim");
-        return 0;
+// Workgroups of the split pass per CU.  PA_DECODE_WGS_PER_CU overrides the
+// default (a tuning aid; read once).
+int wgs_per_cu() {
+    static int cached = 0;
+    if (cached == 0) {
+        const char *e = getenv("PA_DECODE_WGS_PER_CU");
+        const int v = e ? atoi(e) : 0;
+        cached = v >= 1 && v <= 16 ? v : 2;
     }
-    return ws_layout(total_chunks, batch, num_q_heads, head_dim).total;
+    return cached;
 }
-
-namespace {
 
 enum { kPhaseSplit = 1, kPhaseReduce = 2 };
 
@@ -102,8 +94,7 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
                   const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
                   const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale, int batch,
                   int num_q_heads, int num_kv_heads, int head_dim, int block_size, int64_t num_blocks, float scale,
-                  int q_dtype, int kv_dtype, int chunk_tokens, int64_t total_chunks, void *workspace,
-                  size_t workspace_bytes, void *stream) {
+                  int q_dtype, int kv_dtype, void *workspace, size_t workspace_bytes, void *stream) {
     pa_clear_error();
     PA_REQUIRE(batch >= 0, "batch=%d is negative", batch);
     PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, "head counts / head_dim must be positive");
@@ -112,10 +103,8 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     PA_REQUIRE(block_size > 0, "block_size=%d must be positive", block_size);
     PA_REQUIRE(num_blocks >= 0 && bt_stride >= 0, "num_blocks / bt_stride must be non-negative");
     PA_REQUIRE(num_blocks * (int64_t)block_size < (1ll << 40), "pool of %lld blocks is too large", (long long)num_blocks);
-    PA_REQUIRE(chunk_tokens > 0 && chunk_tokens % block_size == 0,
-               "chunk_tokens=%d is not a positive multiple of block_size=%d", chunk_tokens, block_size);
-    PA_REQUIRE(total_chunks >= 0 && total_chunks < (1ll << 30), "total_chunks=%lld out of range",
-               (long long)total_chunks);
+    PA_REQUIRE((int64_t)block_size * num_kv_heads * head_dim * 4 < (1ll << 31),
+               "one block of %d tokens x %d heads x %d is too large", block_size, num_kv_heads, head_dim);
     DecodeArgs a;
     const int nrep_t = pa_fill_head_mapping(a.p, num_q_heads, num_kv_heads, head_dim, kv_dtype);
     const KernelSet ks = nrep_t ? pa_pick_kernels(q_dtype, kv_dtype, head_dim, nrep_t) : KernelSet{};
@@ -128,8 +117,9 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     PA_REQUIRE(k_cache && v_cache, "NULL cache pointer");
     PA_REQUIRE(block_tables || bt_stride == 0, "NULL block_tables with bt_stride=%lld", (long long)bt_stride);
     PA_REQUIRE(kv_dtype != PA_FP8_E4M3 || (k_scale && v_scale), "fp8 KV needs k_scale and v_scale");
-    PA_REQUIRE(pa_aligned16(k_cache) && pa_aligned16(v_cache), "cache pointers must be 16-byte aligned");
-    const WsLayout w = ws_layout(total_chunks, batch, num_q_heads, head_dim);
+    PA_REQUIRE(pa_aligned16(k_cache) && pa_aligned16(v_cache) && pa_aligned16(q),
+               "q and cache pointers must be 16-byte aligned");
+    const WsLayout w = ws_layout(batch, a.p, nrep_t, head_dim);
     if (!workspace || workspace_bytes < w.total)
         return pa_fail(PA_ERR_WORKSPACE, "pa_decode: workspace of %zu bytes, need %zu", workspace_bytes, w.total);
     PA_REQUIRE(((uintptr_t)workspace & 255u) == 0, "workspace must be 256-byte aligned");
@@ -140,22 +130,18 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     a.p.scale_log2 = scale * 1.4426950408889634f;
     a.q = q; a.out = out; a.seq_lens = seq_lens; a.extra_zero = extra_zero_keys;
     a.batch = batch;
-    a.chunk_blocks = chunk_tokens / block_size;
-    a.chunk_cap = total_chunks;
+    a.slot_cap = w.slots;
     char *ws = (char *)workspace;
-    a.chunk_prefix = (int32_t *)(ws + w.prefix_off);
+    a.block_prefix = (int32_t *)(ws + w.prefix_off);
     a.part_ml = (float *)(ws + w.ml_off);
     a.part_acc = (float *)(ws + w.acc_off);
 
     hipStream_t s = (hipStream_t)stream;
-    const int64_t max_items = total_chunks * a.p.n_hgroups * a.p.n_rgroups;
-    const int64_t persistent = (int64_t)num_cus() * 4;
-    // At least one workgroup always runs: it publishes the chunk prefix the
-    // reduction pass reads, even when there is no chunk to process.
-    const int64_t want = max_items < persistent ? max_items : persistent;
-    const unsigned grid = (unsigned)(want < 1 ? 1 : want);
+    int grid = num_cus() * wgs_per_cu();
+    if (grid > kMaxSplitGrid) grid = kMaxSplitGrid;
+    a.split_grid = grid;
     if (phases & kPhaseSplit) {
-        ks.split<<<dim3(grid), dim3(kThreads), (size_t)(batch + 1) * sizeof(int), s>>>(a);
+        ks.split<<<dim3((unsigned)grid), dim3(kThreads), (size_t)(batch + 1) * sizeof(int), s>>>(a);
         PA_CHECK_LAUNCH("pa_decode split pass");
     }
     if (phases & kPhaseReduce) {
@@ -169,16 +155,33 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
 
 }  // namespace
 
+extern "C" size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads, int head_dim,
+                                            int kv_dtype) {
+    pa_clear_error();
+    PoolArgs p;
+    if (batch < 0 || num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) {
+        pa_fail(PA_ERR_INVALID_ARG, "pa_decode_workspace_bytes: negative batch or inconsistent head counts");
+        return 0;
+    }
+    const int nrep_t = pa_fill_head_mapping(p, num_q_heads, num_kv_heads, head_dim, kv_dtype);
+    if (!nrep_t) {
+        pa_fail(PA_ERR_UNSUPPORTED, "pa_decode_workspace_bytes: no kernel for kv_dtype=%d head_dim=%d", kv_dtype,
+                head_dim);
+        return 0;
+    }
+    return ws_layout(batch, p, nrep_t, head_dim).total;
+}
+
 #define PA_DECODE_PARAMS                                                                                       \
     const void *q, const void *k_cache, const void *v_cache, void *out, const int32_t *block_tables,          \
         int64_t bt_stride, const int32_t *seq_lens, const int32_t *extra_zero_keys, const float *k_scale,      \
         const float *v_scale, int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,      \
-        int64_t num_blocks, float scale, int q_dtype, int kv_dtype, int chunk_tokens, int64_t total_chunks,    \
-        void *workspace, size_t workspace_bytes, void *stream
+        int64_t num_blocks, float scale, int q_dtype, int kv_dtype, void *workspace, size_t workspace_bytes,   \
+        void *stream
 #define PA_DECODE_ARGS                                                                                         \
     q, k_cache, v_cache, out, block_tables, bt_stride, seq_lens, extra_zero_keys, k_scale, v_scale, batch,     \
-        num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, q_dtype, kv_dtype, chunk_tokens,   \
-        total_chunks, workspace, workspace_bytes, stream
+        num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, q_dtype, kv_dtype, workspace,      \
+        workspace_bytes, stream
 
 extern "C" int pa_decode(PA_DECODE_PARAMS) { return decode_launch(kPhaseSplit | kPhaseReduce, PA_DECODE_ARGS); }
 extern "C" int pa_decode_split(PA_DECODE_PARAMS) { return decode_launch(kPhaseSplit, PA_DECODE_ARGS); }

@@ -4,12 +4,13 @@
 // have no matrix-core kernel).
 //
 // Work decomposition (decode)
-//   Every sequence is cut into chunks of `chunk_blocks` pool blocks.  One work
-//   item = (chunk, group of kv heads, group of <= NREP query heads per kv
-//   head).  A persistent grid of 256-thread workgroups walks the items with a
-//   grid stride; each workgroup first builds the per-sequence chunk prefix sum
-//   in LDS (seq_lens live on the device, the host never reads them) and finds
-//   an item's sequence by binary search in it.
+//   plane = (group of <= NREP query heads per kv head, group of HPW kv heads).
+//   The (plane, sequence, pool block) space is flattened and cut into equal
+//   ranges, one per 256-thread workgroup of a grid sized to the machine, so
+//   that every workgroup streams the same number of blocks however ragged the
+//   batch is.  Each workgroup first builds the per-sequence block prefix sum in
+//   LDS (seq_lens live on the device, the host never reads them) and finds the
+//   sequences of its range by binary search in it.
 //
 // Lane layout (wave64)
 //   A K or V row of one (token, kv head) is D elements = LPR lanes x 16 bytes,
@@ -23,9 +24,13 @@
 // Softmax
 //   base-2 online softmax in fp32 per row group, rescaled once per batch of U
 //   token steps; the partial (m, l, acc) of the 4 waves x TPW token rows are
-//   merged through LDS.  Decode writes one partial per (chunk, query head) to
-//   the workspace and a second kernel merges the chunks of a sequence.
+//   merged through LDS.  A sequence that one workgroup covers alone is written
+//   out directly; where a sequence straddles workgroup ranges each piece leaves
+//   a partial in the workspace and a second kernel merges them.
 #pragma once
+#include <type_traits>
+#include <utility>
+
 #include "pa_common.h"
 
 namespace pa_decode_detail {
@@ -54,11 +59,11 @@ struct DecodeArgs {
     const int32_t *seq_lens;
     const int32_t *extra_zero;
     int batch;
-    int chunk_blocks;
-    int64_t chunk_cap;      // partial slots the workspace holds
-    float *part_acc;        // [chunk_cap][hq][D]
-    float *part_ml;         // [chunk_cap][hq][2]
-    int32_t *chunk_prefix;  // [batch+1], written by the split pass for the reduction pass
+    int split_grid;         // workgroups of the split pass (the reduction pass needs the same number)
+    int64_t slot_cap;       // partial slots the workspace holds
+    float *part_acc;        // [slot_cap][hpw*NREP][D]
+    float *part_ml;         // [slot_cap][hpw*NREP][2]
+    int32_t *block_prefix;  // [batch+1], written by the split pass for the reduction pass
 };
 
 struct RowwiseArgs {
@@ -71,6 +76,13 @@ struct RowwiseArgs {
 };
 
 __device__ __forceinline__ uint4 ld16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }
+
+// 16-byte load of pool data: used once, so it carries the non-temporal hint.
+__device__ __forceinline__ uint4 ld16_stream(const void *p) {
+    typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+    const u4 v = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p));
+    return uint4{v[0], v[1], v[2], v[3]};
+}
 
 template <typename KV, int D> struct RowShape {
     static constexpr int EPL = pa_vec16<KV>::N;  // elements per lane per 16-byte load
@@ -171,12 +183,12 @@ __device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EP
             for (int u = 0; u < U; ++u) {
                 const int t = t0 + u * p.tpw + role.tok_local;
                 ok[u] = t < ntok;
-                kraw[u] = ok[u] ? ld16(kp + t * tok_stride) : uint4{0, 0, 0, 0};
+                kraw[u] = ok[u] ? ld16_stream(kp + t * tok_stride) : uint4{0, 0, 0, 0};
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int t = t0 + u * p.tpw + role.tok_local;
-                vraw[u] = ok[u] ? ld16(vp + t * tok_stride) : uint4{0, 0, 0, 0};
+                vraw[u] = ok[u] ? ld16_stream(vp + t * tok_stride) : uint4{0, 0, 0, 0};
             }
             float s[U][NREP];
             float mx[NREP];
@@ -222,6 +234,56 @@ __device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EP
     }
 }
 
+}  // namespace pa_decode_detail
+
+#include "decode_pk16.h"
+
+namespace pa_decode_detail {
+
+// One wave's pass over its blocks of one query row: picks the packed 16-bit
+// loop where it applies (bf16/fp16 pool, head_dim 64 or 128), else the generic
+// fp32 loop.  Returns the row-group state in the generic form merge_rows takes.
+template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
+    using S = RowShape<KV, D>;
+    static constexpr bool kPacked = sizeof(KV) == 2 && std::is_same<KV, QT>::value && (D == 64 || D == 128);
+
+    static __device__ __forceinline__ RowState<NREP, S::EPL> run(const PoolArgs &p, const QT *qrow,
+                                                                  const int32_t *bt_row, int L, int blk_begin,
+                                                                  int blk_end, int blk_step, const LaneRole &role,
+                                                                  int lane, int kvh, int rep0) {
+        RowState<NREP, S::EPL> out;
+        if constexpr (kPacked) {
+            using HS = HeadScatter<NREP, D / 8>;
+            uint32_t qpk[NREP][4];
+#pragma unroll
+            for (int r = 0; r < NREP; ++r) {
+                const bool live = rep0 + r < p.n_rep;
+                const uint4 raw = live ? ld16(qrow + ((int64_t)kvh * p.n_rep + rep0 + r) * D + role.d0)
+                                       : uint4{0, 0, 0, 0};
+                qpk[r][0] = raw.x; qpk[r][1] = raw.y; qpk[r][2] = raw.z; qpk[r][3] = raw.w;
+            }
+            PkState<NREP, HS::VPL> st;
+            st.init();
+            const int lane_voff = role.tok_local * (p.hkv * D * 2) + kvh * (D * 2) + role.lir * 16;
+            attend_blocks_pk<KV, D, NREP, U>(st, qpk, p, bt_row, L, blk_begin, blk_end, blk_step, lane, lane_voff,
+                                             role.tok_local == 0);
+            StaticFor<NREP>::run([&](auto h) {
+                out.m[h.value] = HS::template bcast<h.value>(st.m);
+                out.l[h.value] = HS::template bcast<h.value>(st.l);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) out.acc[h.value][e] = st.acc[h.value][e];
+            });
+            out.zero_keys = st.zero_keys;
+        } else {
+            float qf[NREP][S::EPL];
+            load_q<QT, D, NREP, S::EPL>(qf, qrow, p, kvh, rep0, role.d0);
+            out.init();
+            attend_blocks<KV, D, NREP, U>(out, qf, p, bt_row, L, blk_begin, blk_end, blk_step, role, kvh);
+        }
+        return out;
+    }
+};
+
 // Merge the kWaves*TPW row-group partials of every (kv head of the group,
 // query head r) through LDS and hand (qh, d, num, M, den) of the merged
 // partial to `emit`; out = num/den, M is the base-2 running maximum.
@@ -262,30 +324,53 @@ __device__ __forceinline__ void merge_rows(RowState<NREP, RowShape<KV, D>::EPL> 
     __syncthreads();
 }
 
+// Which workgroup of a grid of G owns flattened block unit u of total T:
+// workgroup w owns [floor(w*T/G), floor((w+1)*T/G)).
+__device__ __forceinline__ int64_t unit_begin(int64_t w, int64_t total, int64_t grid) { return w * total / grid; }
+__device__ __forceinline__ int owner_of(int64_t u, int64_t total, int64_t grid) {
+    return (int)(((u + 1) * grid - 1) / total);
+}
+
+// Finish one (sequence, query head): fold `ez` extra all-zero keys into the
+// merged (num, M, den) and normalise.
+__device__ __forceinline__ float finish_row(float num, float M, float den, int ez) {
+    if (ez > 0) {
+        const float mn = fmaxf(M, 0.f);
+        const float alpha = __builtin_amdgcn_exp2f(M - mn);
+        num *= alpha;
+        den = den * alpha + (float)ez * __builtin_amdgcn_exp2f(-mn);
+    }
+    return den > 0.f ? num / den : 0.f;
+}
+
+// Split pass.  The (plane, sequence, block) space - plane = (rep group, head
+// group) - is flattened in that order and cut into gridDim.x equal ranges, one
+// per workgroup, so every workgroup streams the same number of pool blocks
+// whatever the length distribution.  A range may cover the tail of one
+// sequence, several whole sequences and the head of another.  A sequence that
+// lies inside one range is finished in place; otherwise the workgroup leaves a
+// partial in slot (workgroup index + plane*batch + sequence), unique because
+// both terms only grow along the flattened order.
 template <typename KV, typename QT, int D, int NREP, int U>
 __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs a) {
     using S = RowShape<KV, D>;
-    extern __shared__ int s_prefix[];  // batch + 1 entries, sized at launch
+    extern __shared__ int s_prefix[];  // batch + 1 entries: blocks before each sequence
     __shared__ int s_scan[kThreads];
     __shared__ float s_part[kWaves * S::RPW][D + 2];
 
     const PoolArgs &p = a.p;
     const int tid = threadIdx.x;
     const int lane = tid & (PA_WAVE - 1);
-    const int wave = tid / PA_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / PA_WAVE);
     const int B = a.batch;
 
-    // ---- chunk prefix sum over the batch -------------------------------
+    // ---- block prefix sum over the batch --------------------------------
     {
         const int per = (B + kThreads - 1) / kThreads;
         const int lo = min(B, tid * per), hi = min(B, lo + per);
-        auto chunks_of = [&](int b) {
-            const int L = max(0, a.seq_lens[b]);
-            const int nblk = (L + p.bs - 1) / p.bs;
-            return (nblk + a.chunk_blocks - 1) / a.chunk_blocks;
-        };
+        auto blocks_of = [&](int b) { return (max(0, a.seq_lens[b]) + p.bs - 1) / p.bs; };
         int sum = 0;
-        for (int b = lo; b < hi; ++b) sum += chunks_of(b);
+        for (int b = lo; b < hi; ++b) sum += blocks_of(b);
         s_scan[tid] = sum;
         __syncthreads();
         for (int off = 1; off < kThreads; off <<= 1) {
@@ -297,79 +382,116 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
         int run = s_scan[tid] - sum;  // exclusive
         for (int b = lo; b < hi; ++b) {
             s_prefix[b] = run;
-            run += chunks_of(b);
+            run += blocks_of(b);
         }
         if (tid == kThreads - 1) s_prefix[B] = s_scan[tid];
         __syncthreads();
         if (blockIdx.x == 0)
-            for (int b = tid; b <= B; b += kThreads) a.chunk_prefix[b] = s_prefix[b];
+            for (int b = tid; b <= B; b += kThreads) a.block_prefix[b] = s_prefix[b];
     }
-    const int total_chunks = s_prefix[B];
-    const int64_t n_items = (int64_t)total_chunks * p.n_hgroups * p.n_rgroups;
+    const int64_t per_plane = s_prefix[B];
+    const int planes = p.n_hgroups * p.n_rgroups;
+    const int64_t total = per_plane * planes;
     const LaneRole role = lane_role<KV, D>(lane, p);
+    if (total == 0) return;
 
-    for (int64_t item = blockIdx.x; item < n_items; item += gridDim.x) {
-        // item -> (chunk, rep group, head group); head group fastest
-        const int hg = (int)(item % p.n_hgroups);
-        const int64_t rest = item / p.n_hgroups;
-        const int rg = (int)(rest % p.n_rgroups);
-        const int gchunk = (int)(rest / p.n_rgroups);
-        if (gchunk >= a.chunk_cap) continue;  // workspace smaller than promised: never write outside it
-        int lo = 0, hi = B;  // last b with prefix[b] <= gchunk
+    int64_t cur = unit_begin(blockIdx.x, total, gridDim.x);
+    const int64_t end = unit_begin((int64_t)blockIdx.x + 1, total, gridDim.x);
+    while (cur < end) {
+        const int plane = (int)(cur / per_plane);
+        const int off = (int)(cur - plane * per_plane);
+        int lo = 0, hi = B;  // last b with prefix[b] <= off
         while (hi - lo > 1) {
             const int mid = (lo + hi) >> 1;
-            if (s_prefix[mid] <= gchunk) lo = mid; else hi = mid;
+            if (s_prefix[mid] <= off) lo = mid; else hi = mid;
         }
         const int b = lo;
-        const int c = gchunk - s_prefix[lo];
-        const int L = a.seq_lens[b];
-        const int nblk = (L + p.bs - 1) / p.bs;
-        const int blk0 = c * a.chunk_blocks;
-        const int blk1 = min(nblk, blk0 + a.chunk_blocks);
+        const int nblk = s_prefix[b + 1] - s_prefix[b];
+        const int blk0 = off - s_prefix[b];
+        const int blk1 = (int)min((int64_t)nblk, blk0 + (end - cur));
+        const int hg = plane % p.n_hgroups;
+        const int rg = plane / p.n_hgroups;
         const int kvh = hg * p.hpw + role.head_local;
         const int rep0 = rg * NREP;
+        const int L = a.seq_lens[b];
 
-        float qf[NREP][S::EPL];
-        load_q<QT, D, NREP, S::EPL>(qf, reinterpret_cast<const QT *>(a.q) + (int64_t)b * p.hq * D, p, kvh, rep0,
-                                    role.d0);
-        RowState<NREP, S::EPL> st;
-        st.init();
-        attend_blocks<KV, D, NREP, U>(st, qf, p, p.bt + (int64_t)b * p.bt_stride, L, blk0 + wave, blk1, kWaves,
-                                      role, kvh);
-        merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
-                                [&](int qh, int d, float num, float M, float den) {
-                                    const int64_t slot = (int64_t)gchunk * p.hq + qh;
-                                    a.part_acc[slot * D + d] = num;
-                                    if (d == 0) {
-                                        a.part_ml[slot * 2] = M;
-                                        a.part_ml[slot * 2 + 1] = den;
-                                    }
-                                });
+        RowState<NREP, S::EPL> st = Attender<KV, QT, D, NREP, U>::run(
+            p, reinterpret_cast<const QT *>(a.q) + (int64_t)b * p.hq * D, p.bt + (int64_t)b * p.bt_stride, L,
+            blk0 + wave, blk1, kWaves, role, lane, kvh, rep0);
+        if (blk0 == 0 && blk1 == nblk) {
+            // the whole sequence is ours: write the output row
+            const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
+            QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * D;
+            merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
+                                    [&](int qh, int d, float num, float M, float den) {
+                                        pa_scalar<QT>::store(orow + (int64_t)qh * D + d, finish_row(num, M, den, ez));
+                                    });
+        } else {
+            const int64_t slot = (int64_t)blockIdx.x + (int64_t)plane * B + b;
+            if (slot < a.slot_cap) {  // never write outside the workspace
+                float *acc = a.part_acc + slot * (p.hpw * NREP * D);
+                float *ml = a.part_ml + slot * (p.hpw * NREP * 2);
+                merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
+                                        [&](int qh, int d, float num, float M, float den) {
+                                            const int kv = qh / p.n_rep;
+                                            const int idx = (kv - hg * p.hpw) * NREP + (qh - kv * p.n_rep - rep0);
+                                            acc[idx * D + d] = num;
+                                            if (d == 0) {
+                                                ml[idx * 2] = M;
+                                                ml[idx * 2 + 1] = den;
+                                            }
+                                        });
+            }
+        }
+        cur += blk1 - blk0;
     }
 }
 
-// Merge the chunk partials of one (sequence, query head); thread d owns out[d].
-template <typename QT, int D>
+// Reduction pass: one workgroup per (sequence, query head), thread d owns
+// out[d].  Rows the split pass finished in place are skipped; empty sequences
+// get their zeros (or the all-zero-keys result) here.
+template <typename QT, int D, int NREP>
 __global__ void decode_reduce_kernel(const DecodeArgs a) {
-    const int hq = a.p.hq;
+    const PoolArgs &p = a.p;
+    const int hq = p.hq;
     const int b = blockIdx.x / hq;
     const int qh = blockIdx.x - b * hq;
-    const int c0 = a.chunk_prefix[b], c1 = (int)min((int64_t)a.chunk_prefix[b + 1], a.chunk_cap);
-    float M = kNegBig;
-    for (int c = c0; c < c1; ++c) M = fmaxf(M, a.part_ml[((int64_t)c * hq + qh) * 2]);
+    const int kv = qh / p.n_rep, rep = qh - kv * p.n_rep;
+    const int hg = kv / p.hpw, rg = rep / NREP;
+    const int plane = rg * p.n_hgroups + hg;
+    const int idx = (kv - hg * p.hpw) * NREP + (rep - rg * NREP);
+    const int64_t per_plane = a.block_prefix[a.batch];
+    const int64_t total = per_plane * p.n_hgroups * p.n_rgroups;
+    const int nblk = a.block_prefix[b + 1] - a.block_prefix[b];
     const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
-    if (ez > 0) M = fmaxf(M, 0.f);
+    QT *orow = reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * D;
+    if (nblk == 0) {
+        for (int d = threadIdx.x; d < D; d += blockDim.x) pa_scalar<QT>::store(orow + d, 0.f);
+        return;
+    }
+    const int64_t u0 = plane * per_plane + a.block_prefix[b];
+    const int w0 = owner_of(u0, total, a.split_grid), w1 = owner_of(u0 + nblk - 1, total, a.split_grid);
+    if (w0 == w1) return;  // finished by the split pass
+    const int64_t key = (int64_t)plane * a.batch + b;
+    const int stride_acc = p.hpw * NREP * D, stride_ml = p.hpw * NREP * 2;
+    // a workgroup whose range is empty (more workgroups than blocks) left no partial
+    auto has_piece = [&](int w) {
+        return unit_begin(w, total, a.split_grid) < unit_begin((int64_t)w + 1, total, a.split_grid) &&
+               w + key < a.slot_cap;
+    };
+    float M = kNegBig;
+    for (int w = w0; w <= w1; ++w)
+        if (has_piece(w)) M = fmaxf(M, a.part_ml[(w + key) * stride_ml + idx * 2]);
     for (int d = threadIdx.x; d < D; d += blockDim.x) {
         float num = 0.f, den = 0.f;
-        for (int c = c0; c < c1; ++c) {
-            const int64_t slot = (int64_t)c * hq + qh;
-            const float w = __builtin_amdgcn_exp2f(a.part_ml[slot * 2] - M);
-            num = fmaf(w, a.part_acc[slot * D + d], num);
-            den = fmaf(w, a.part_ml[slot * 2 + 1], den);
+        for (int w = w0; w <= w1; ++w) {
+            if (!has_piece(w)) continue;
+            const int64_t slot = w + key;
+            const float wgt = __builtin_amdgcn_exp2f(a.part_ml[slot * stride_ml + idx * 2] - M);
+            num = fmaf(wgt, a.part_acc[slot * stride_acc + idx * D + d], num);
+            den = fmaf(wgt, a.part_ml[slot * stride_ml + idx * 2 + 1], den);
         }
-        if (ez > 0) den += (float)ez * __builtin_amdgcn_exp2f(-M);
-        const float o = den > 0.f ? num / den : 0.f;
-        pa_scalar<QT>::store(reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * D + d, o);
+        pa_scalar<QT>::store(orow + d, finish_row(num, M, den, ez));
     }
 }
 
@@ -382,7 +504,7 @@ __global__ __launch_bounds__(kThreads) void prefill_rowwise_kernel(const Rowwise
     const PoolArgs &p = a.p;
     const int tid = threadIdx.x;
     const int lane = tid & (PA_WAVE - 1);
-    const int wave = tid / PA_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(tid / PA_WAVE);
     const int b = blockIdx.z;
     const int i = blockIdx.y;
     const int q_len = a.q_lens[b];
@@ -395,12 +517,10 @@ __global__ __launch_bounds__(kThreads) void prefill_rowwise_kernel(const Rowwise
     const int rep0 = rg * NREP;
     const int64_t qrow = (int64_t)a.q_starts[b] + i;
 
-    float qf[NREP][S::EPL];
-    load_q<QT, D, NREP, S::EPL>(qf, reinterpret_cast<const QT *>(a.q) + qrow * p.hq * D, p, kvh, rep0, role.d0);
-    RowState<NREP, S::EPL> st;
-    st.init();
     const int nblk = L > 0 ? (L + p.bs - 1) / p.bs : 0;
-    attend_blocks<KV, D, NREP, U>(st, qf, p, p.bt + (int64_t)b * p.bt_stride, L, wave, nblk, kWaves, role, kvh);
+    RowState<NREP, S::EPL> st = Attender<KV, QT, D, NREP, U>::run(
+        p, reinterpret_cast<const QT *>(a.q) + qrow * p.hq * D, p.bt + (int64_t)b * p.bt_stride, L, wave, nblk,
+        kWaves, role, lane, kvh, rep0);
     QT *orow = reinterpret_cast<QT *>(a.out) + qrow * p.hq * D;
     merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
                             [&](int qh, int d, float num, float M, float den) {
@@ -421,12 +541,11 @@ struct KernelSet {
 template <typename KV, typename QT, int D> KernelSet kernels_for_d(int nrep_t) {
     constexpr int U = sizeof(KV) == 1 ? 4 : 8;
     KernelSet k;
-    k.reduce = decode_reduce_kernel<QT, D>;
     switch (nrep_t) {
-    case 1: k.split = decode_split_kernel<KV, QT, D, 1, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 1, U>; break;
-    case 2: k.split = decode_split_kernel<KV, QT, D, 2, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 2, U>; break;
-    case 4: k.split = decode_split_kernel<KV, QT, D, 4, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 4, U>; break;
-    case 8: k.split = decode_split_kernel<KV, QT, D, 8, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 8, U>; break;
+    case 1: k.reduce = decode_reduce_kernel<QT, D, 1>; k.split = decode_split_kernel<KV, QT, D, 1, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 1, U>; break;
+    case 2: k.reduce = decode_reduce_kernel<QT, D, 2>; k.split = decode_split_kernel<KV, QT, D, 2, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 2, U>; break;
+    case 4: k.reduce = decode_reduce_kernel<QT, D, 4>; k.split = decode_split_kernel<KV, QT, D, 4, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 4, U>; break;
+    case 8: k.reduce = decode_reduce_kernel<QT, D, 8>; k.split = decode_split_kernel<KV, QT, D, 8, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 8, U>; break;
     }
     return k;
 }

@@ -1,0 +1,266 @@
+// Packed 16-bit inner loop of single-query-row paged attention (bf16 / fp16
+// pools, head_dim 64 or 128) for gfx950.
+//
+// The generic loop converts every K/V element to fp32 and spends most of its
+// issue slots on conversions, per-head cross-lane sums and redundant softmax
+// arithmetic.  This loop keeps the pool data packed:
+//   * q.k: v_dot2 on the raw 16-bit pairs (fp32 accumulate), no conversion;
+//   * the NREP per-head partial dots of a lane are combined over the LPR lanes
+//     of a row with a reduce-scatter in DPP moves, so each lane ends up owning
+//     the logit of ONE (token, head) (two for NREP = 8) and the exp2 / running
+//     max / running sum are evaluated once, not once per lane;
+//   * p.v: two tokens at a time, v_perm interleaves their V pairs and v_dot2
+//     accumulates p(t0)*v(t0)+p(t1)*v(t1) with p rounded to the pool type; the
+//     p pair of head h is broadcast inside the quad by a DPP move;
+//   * loads are buffer loads against a per-block descriptor whose size is the
+//     number of valid bytes in the block: rows past the sequence end read as
+//     zero without a branch, and no index can leave the block.
+#pragma once
+#include "pa_common.h"
+
+namespace pa_decode_detail {
+
+typedef unsigned int pa_u4 __attribute__((ext_vector_type(4)));
+
+// Cache policy of the K/V stream: every byte is used once, so the loads carry
+// the non-temporal hint (bit 1 of the buffer-load policy operand = "nt").
+// Measured on MI355X with a pure read of 3.4 GB in 32 KiB pages: 6.2 TB/s with
+// default loads, 7.0 TB/s with nt loads.
+constexpr int kStreamPolicy = 2;
+
+template <typename KV> struct Pk16;
+template <> struct Pk16<pa_bf16> {
+    typedef __bf16 v2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
+    }
+    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+        v2 r = {(__bf16)lo, (__bf16)hi};
+        return __builtin_bit_cast(uint32_t, r);
+    }
+};
+template <> struct Pk16<pa_f16> {
+    typedef _Float16 v2 __attribute__((ext_vector_type(2)));
+    static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
+    }
+    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+        v2 r = {(_Float16)lo, (_Float16)hi};
+        return __builtin_bit_cast(uint32_t, r);
+    }
+};
+
+template <int CTRL, int BANKS = 0xf> __device__ __forceinline__ float dpp_mov(float old, float x) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old),
+                                                                 __builtin_bit_cast(int, x), CTRL, 0xf, BANKS, false));
+}
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_mov_u(uint32_t x) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, CTRL, 0xf, 0xf, true);
+}
+
+// How NREP per-head values of a lane are combined over the LPR lanes of a row.
+// After reduce(): a lane at quad position c = lane & 3 owns VPL totals, those
+// of heads head_base(c) .. head_base(c)+VPL-1.
+template <int NREP, int LPR> struct HeadScatter {
+    static_assert(LPR == 8 || LPR == 16, "rows of 8 or 16 lanes");
+    static constexpr int SC = NREP >= 4 ? 2 : (NREP == 2 ? 1 : 0);  // scatter steps (xor 1, xor 2)
+    static constexpr int VPL = NREP >> SC;                            // values a lane keeps
+
+    static __device__ __forceinline__ void reduce(const float (&s)[NREP], float (&out)[VPL], int lane) {
+        constexpr int H1 = SC >= 1 ? NREP / 2 : NREP;
+        float t[H1];
+        if (SC >= 1) {
+            const bool odd = lane & 1;
+#pragma unroll
+            for (int i = 0; i < H1; ++i) {
+                const float keep = odd ? s[i + H1] : s[i];
+                const float send = odd ? s[i] : s[i + H1];
+                t[i] = keep + dpp_mov<0xB1>(0.f, send);  // quad_perm [1,0,3,2]
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < H1; ++i) t[i] = s[i] + dpp_mov<0xB1>(0.f, s[i]);
+        }
+        if (SC == 2) {
+            const bool up = lane & 2;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                const float keep = up ? t[i + VPL] : t[i];
+                const float send = up ? t[i] : t[i + VPL];
+                out[i] = keep + dpp_mov<0x4E>(0.f, send);  // quad_perm [2,3,0,1]
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) out[i] = t[i] + dpp_mov<0x4E>(0.f, t[i]);
+        }
+        // remaining levels keep the quad position: every quad of the row gets the row total
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            if (LPR == 16) {
+                out[i] += dpp_mov<0x124>(0.f, out[i]);  // row_ror:4
+                out[i] += dpp_mov<0x128>(0.f, out[i]);  // row_ror:8
+            } else {
+                // partner quad inside the row of 8: from 4 lanes below for banks 1,3, from 4 lanes above for banks 0,2
+                float other = dpp_mov<0x114, 0xa>(0.f, out[i]);   // row_shr:4
+                other = dpp_mov<0x104, 0x5>(other, out[i]);       // row_shl:4
+                out[i] += other;
+            }
+        }
+    }
+
+    // quad position and slot that hold head h
+    static constexpr int pos_of(int h) {
+        return SC == 2 ? ((h / (NREP / 2)) | (((h / VPL) & 1) << 1)) : (SC == 1 ? h : 0);
+    }
+    static constexpr int slot_of(int h) { return SC == 2 ? h % VPL : 0; }
+
+    template <int H> static __device__ __forceinline__ float bcast(const float (&x)[VPL]) {
+        if (SC == 0) return x[0];
+        return dpp_mov<pos_of(H) * 0x55>(0.f, x[slot_of(H)]);
+    }
+    template <int H> static __device__ __forceinline__ uint32_t bcast_u(const uint32_t (&x)[VPL]) {
+        if (SC == 0) return x[0];
+        return dpp_mov_u<pos_of(H) * 0x55>(x[slot_of(H)]);
+    }
+};
+
+template <int NREP, int VPL> struct PkState {
+    float m[VPL], l[VPL];
+    float acc[NREP][8];
+    int zero_keys;
+    __device__ __forceinline__ void init() {
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) { m[j] = -1.0e30f; l[j] = 0.f; }
+#pragma unroll
+        for (int r = 0; r < NREP; ++r)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[r][e] = 0.f;
+        zero_keys = 0;
+    }
+};
+
+template <int N> struct StaticFor {
+    template <typename F> static __device__ __forceinline__ void run(F &&f) {
+        StaticFor<N - 1>::run(f);
+        f(std::integral_constant<int, N - 1>{});
+    }
+};
+template <> struct StaticFor<0> {
+    template <typename F> static __device__ __forceinline__ void run(F &&) {}
+};
+
+// Attend keys [0, L) of blocks blk_begin, blk_begin+blk_step, ... < blk_end.
+// qpk[r][i]: raw 16-bit pairs of this lane's 8 query elements of head r.
+template <typename KV, int D, int NREP, int U>
+__device__ __forceinline__ void attend_blocks_pk(PkState<NREP, HeadScatter<NREP, D / 8>::VPL> &st,
+                                                 const uint32_t (&qpk)[NREP][4], const PoolArgs &p,
+                                                 const int32_t *bt_row, int L, int blk_begin, int blk_end,
+                                                 int blk_step, int lane, int lane_voff, bool count_zero_keys) {
+    static_assert(U % 2 == 0, "tokens are consumed in pairs");
+    constexpr int LPR = D / 8;
+    using HS = HeadScatter<NREP, LPR>;
+    using PK = Pk16<KV>;
+    constexpr int VPL = HS::VPL;
+    const int tok_stride = p.hkv * D * 2;  // bytes between tokens
+    const int tok_local = (lane / LPR) / p.hpw;
+
+    for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
+        const int ntok = min(p.bs, L - blk * p.bs);
+        const int64_t bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
+        if (bid < 0 || bid >= p.num_blocks) {
+            if (count_zero_keys) st.zero_keys += ntok;
+            continue;
+        }
+        // descriptor of the valid part of this block: reads past it return 0
+        const int64_t block_off = bid * p.bs * (int64_t)tok_stride;
+        const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(reinterpret_cast<const char *>(p.k) + block_off), 0, ntok * tok_stride, 0x00020000);
+        const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(reinterpret_cast<const char *>(p.v) + block_off), 0, ntok * tok_stride, 0x00020000);
+
+        for (int t0 = 0; t0 < ntok; t0 += p.tpw * U) {
+            pa_u4 kraw[U], vraw[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                kraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rk, lane_voff + (t0 + u * p.tpw) * tok_stride, 0, kStreamPolicy);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                vraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rv, lane_voff + (t0 + u * p.tpw) * tok_stride, 0, kStreamPolicy);
+
+            // ---- logits: one (token, head) per lane -----------------------
+            float sv[U][VPL];
+            const bool partial = ntok - t0 < p.tpw * U;  // uniform
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float s[NREP];
+#pragma unroll
+                for (int r = 0; r < NREP; ++r) {
+                    float d = PK::dot2(kraw[u][0], qpk[r][0], 0.f);
+                    d = PK::dot2(kraw[u][1], qpk[r][1], d);
+                    d = PK::dot2(kraw[u][2], qpk[r][2], d);
+                    s[r] = PK::dot2(kraw[u][3], qpk[r][3], d);
+                }
+                HS::reduce(s, sv[u], lane);
+#pragma unroll
+                for (int j = 0; j < VPL; ++j) sv[u][j] *= p.scale_log2;
+                if (partial) {
+                    const bool ok = t0 + u * p.tpw + tok_local < ntok;
+#pragma unroll
+                    for (int j = 0; j < VPL; ++j) sv[u][j] = ok ? sv[u][j] : -INFINITY;
+                }
+            }
+            // ---- running maximum; rescale only when some lane's maximum grew ----
+            float mx[VPL];
+            bool grew = false;
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) {
+                mx[j] = st.m[j];
+#pragma unroll
+                for (int u = 0; u < U; ++u) mx[j] = fmaxf(mx[j], sv[u][j]);
+                grew |= mx[j] > st.m[j];
+            }
+            if (__builtin_amdgcn_ballot_w64(grew) != 0) {
+                float alpha[VPL];
+#pragma unroll
+                for (int j = 0; j < VPL; ++j) {
+                    alpha[j] = __builtin_amdgcn_exp2f(st.m[j] - mx[j]);
+                    st.m[j] = mx[j];
+                    st.l[j] *= alpha[j];
+                }
+                StaticFor<NREP>::run([&](auto h) {
+                    const float a = HS::template bcast<h.value>(alpha);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) st.acc[h.value][e] *= a;
+                });
+            }
+            // ---- p.v, two tokens per step ----------------------------------
+#pragma unroll
+            for (int u = 0; u < U; u += 2) {
+                uint32_t ppk[VPL];
+#pragma unroll
+                for (int j = 0; j < VPL; ++j) {
+                    const float p0 = __builtin_amdgcn_exp2f(sv[u][j] - st.m[j]);  // 0 for masked tokens
+                    const float p1 = __builtin_amdgcn_exp2f(sv[u + 1][j] - st.m[j]);
+                    st.l[j] += p0 + p1;
+                    ppk[j] = PK::pack(p0, p1);
+                }
+                uint32_t lo[4], hi[4];  // (v_t0[2i], v_t1[2i]) and (v_t0[2i+1], v_t1[2i+1])
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    lo[i] = __builtin_amdgcn_perm(vraw[u + 1][i], vraw[u][i], 0x05040100u);
+                    hi[i] = __builtin_amdgcn_perm(vraw[u + 1][i], vraw[u][i], 0x07060302u);
+                }
+                StaticFor<NREP>::run([&](auto h) {
+                    const uint32_t pb = HS::template bcast_u<h.value>(ppk);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        st.acc[h.value][2 * i] = PK::dot2(lo[i], pb, st.acc[h.value][2 * i]);
+                        st.acc[h.value][2 * i + 1] = PK::dot2(hi[i], pb, st.acc[h.value][2 * i + 1]);
+                    }
+                });
+            }
+        }
+    }
+}
+
+}  // namespace pa_decode_detail

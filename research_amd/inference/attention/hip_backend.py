@@ -42,14 +42,14 @@ _COMPUTE_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
 class _StepTensors:
     """Device copies of one context's integer fields, built once per step."""
 
-    __slots__ = ("ctx", "slots", "tables", "bt_stride", "seq_lens", "extra_zero", "total_chunks", "chunk_tokens",
-                 "ctx_lens", "q_lens", "q_starts", "max_q_len")
+    __slots__ = ("ctx", "slots", "tables", "bt_stride", "seq_lens", "extra_zero", "ctx_lens", "q_lens", "q_starts",
+                 "max_q_len")
 
     def __init__(self, ctx: InferenceContext) -> None:
         self.ctx = ctx  # keeps id(ctx) alive while the entry is cached
         self.slots = self.tables = self.seq_lens = self.extra_zero = None
         self.ctx_lens = self.q_lens = self.q_starts = None
-        self.bt_stride = self.total_chunks = self.chunk_tokens = self.max_q_len = 0
+        self.bt_stride = self.max_q_len = 0
 
 
 def _padded_tables(block_tables: Sequence[Sequence[int]]) -> np.ndarray:
@@ -224,17 +224,16 @@ class HipPagedAttentionBackend:
             lens = np.asarray(ctx.seq_lens, dtype=np.int64)[:batch]
             self._tables(step, ctx.block_tables[:batch])
             step.seq_lens = self._to_device(lens.astype(np.int32))
-            step.chunk_tokens = ops.decode_plan(int(lens.sum()), batch, cfg.num_kv_heads, cfg.block_size)
-            step.total_chunks = int((-(-np.maximum(lens, 0) // step.chunk_tokens)).sum())
             if self.pad_zero_keys and batch > 0:
                 step.extra_zero = self._to_device((lens.max() - lens).astype(np.int32))
         q3 = q.contiguous().view(batch, num_heads, head_dim)
-        ws = self._workspace_for(ops.decode_workspace_bytes(step.total_chunks, batch, num_heads, head_dim))
+        ws = self._workspace_for(
+            ops.decode_workspace_bytes(batch, num_heads, cfg.num_kv_heads, head_dim, self.k_cache.dtype))
         kc, vc = self._layer(layer_idx)
         ksc = self.k_scale[layer_idx] if self._fp8 else None
         vsc = self.v_scale[layer_idx] if self._fp8 else None
-        out = ops.decode(q3, kc, vc, step.tables, step.seq_lens, cfg.block_size, self.scale, step.chunk_tokens,
-                         step.total_chunks, ws, step.extra_zero, ksc, vsc)
+        out = ops.decode(q3, kc, vc, step.tables, step.seq_lens, cfg.block_size, self.scale, ws, step.extra_zero,
+                         ksc, vsc)
         return out.view(batch, 1, num_heads, head_dim)
 
     # ------------------------------------------------------------------ prefill

@@ -53,22 +53,26 @@ def kv_gather(k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, seq_lens: 
     return k_out, v_out
 
 
-def decode_plan(total_tokens: int, batch: int, num_kv_heads: int, block_size: int) -> int:
-    """Chunk size (keys) the library suggests for this batch."""
-    chunk = _lib.load().pa_decode_chunk_tokens(total_tokens, batch, num_kv_heads, block_size)
-    if chunk <= 0:
-        raise _lib.PagedAttnError("pa_decode_chunk_tokens", chunk, _lib.last_error())
-    return chunk
+def decode_workspace_bytes(batch: int, num_q_heads: int, num_kv_heads: int, head_dim: int,
+                           kv_dtype: torch.dtype) -> int:
+    """Bytes of workspace ``decode`` needs for these shapes (independent of the sequence lengths)."""
+    n = int(_lib.load().pa_decode_workspace_bytes(batch, num_q_heads, num_kv_heads, head_dim, PA_DTYPE[kv_dtype]))
+    if n == 0:
+        raise _lib.PagedAttnError("pa_decode_workspace_bytes", 0, _lib.last_error())
+    return n
 
 
-def decode_workspace_bytes(total_chunks: int, batch: int, num_q_heads: int, head_dim: int) -> int:
-    return int(_lib.load().pa_decode_workspace_bytes(total_chunks, batch, num_q_heads, head_dim))
+def decode_workspace(q: Tensor, k_cache: Tensor) -> Tensor:
+    """A fresh workspace tensor sized for ``decode(q, k_cache, ...)``."""
+    batch, hq, d = q.shape
+    n = decode_workspace_bytes(batch, hq, k_cache.shape[1], d, k_cache.dtype)
+    return torch.empty(n, dtype=torch.uint8, device=q.device)
 
 
 def decode(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, seq_lens: Tensor, block_size: int,
-           scale: float, chunk_tokens: int, total_chunks: int, workspace: Tensor,
-           extra_zero_keys: Optional[Tensor] = None, k_scale: Optional[Tensor] = None,
-           v_scale: Optional[Tensor] = None, out: Optional[Tensor] = None, entry: str = "pa_decode") -> Tensor:
+           scale: float, workspace: Tensor, extra_zero_keys: Optional[Tensor] = None,
+           k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None, out: Optional[Tensor] = None,
+           entry: str = "pa_decode") -> Tensor:
     """Paged decode attention; q ``[B, Hq, D]`` -> out ``[B, Hq, D]`` (same dtype).
 
     ``entry`` may name ``pa_decode_split`` or ``pa_decode_reduce`` to run one pass only.
@@ -79,8 +83,8 @@ def decode(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, se
         out = torch.empty_like(q)
     _run(entry, _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_tables), block_tables.shape[1],
          _ptr(seq_lens), _ptr(extra_zero_keys), _ptr(k_scale), _ptr(v_scale), batch, hq, hkv, d, block_size,
-         total_slots // block_size, float(scale), PA_DTYPE[q.dtype], PA_DTYPE[k_cache.dtype], chunk_tokens,
-         total_chunks, _ptr(workspace), workspace.numel() * workspace.element_size(), _stream(q))
+         total_slots // block_size, float(scale), PA_DTYPE[q.dtype], PA_DTYPE[k_cache.dtype], _ptr(workspace),
+         workspace.numel() * workspace.element_size(), _stream(q))
     return out
 
 

@@ -22,19 +22,14 @@ def tables_to_device(tables, width=None):
     return torch.from_numpy(out).to(DEV)
 
 
-def run_decode(q, k_pool, v_pool, tables, seq_lens, block_size, scale, chunk_tokens=None, extra_zero=None,
-               k_scale=None, v_scale=None):
+def run_decode(q, k_pool, v_pool, tables, seq_lens, block_size, scale, extra_zero=None, k_scale=None, v_scale=None,
+               wgs_per_call=None):
     """q [B,Hq,D] and pools already on the device; tables/seq_lens host lists.  Returns a device tensor."""
-    lens = np.asarray(seq_lens, dtype=np.int64)
-    batch, hq, d = q.shape
-    hkv = k_pool.shape[1]
-    if chunk_tokens is None:
-        chunk_tokens = ops.decode_plan(int(lens.sum()), batch, hkv, block_size)
-    total_chunks = int((-(-np.maximum(lens, 0) // chunk_tokens)).sum())
-    ws = torch.empty(max(ops.decode_workspace_bytes(total_chunks, batch, hq, d), 256), dtype=torch.uint8, device=DEV)
+    lens = np.asarray(seq_lens, dtype=np.int32)
+    ws = ops.decode_workspace(q, k_pool)
     ez = None if extra_zero is None else torch.from_numpy(np.asarray(extra_zero, dtype=np.int32)).to(DEV)
-    return ops.decode(q, k_pool, v_pool, tables_to_device(tables), torch.from_numpy(lens.astype(np.int32)).to(DEV),
-                      block_size, scale, chunk_tokens, total_chunks, ws, ez, k_scale, v_scale)
+    return ops.decode(q, k_pool, v_pool, tables_to_device(tables), torch.from_numpy(lens).to(DEV), block_size, scale,
+                      ws, ez, k_scale, v_scale)
 
 
 def assert_close(got, want, tol, what=""):

@@ -75,17 +75,20 @@ def test_gather_argument_errors():
 def _decode_args(**kw):
     a = dict(q=FAKE, k=FAKE, v=FAKE, out=FAKE, bt=FAKE, bt_stride=4, lens=FAKE, ez=None, ks=None, vs=None,
              batch=2, hq=32, hkv=8, d=128, bs=16, nb=64, scale=0.088, qd=_lib.PA_BF16, kvd=_lib.PA_BF16,
-             chunk=256, chunks=2, ws=FAKE, ws_bytes=1 << 30, stream=None)
+             ws=FAKE, ws_bytes=1 << 30, stream=None)
     a.update(kw)
     return [a[k] for k in ("q", "k", "v", "out", "bt", "bt_stride", "lens", "ez", "ks", "vs", "batch", "hq", "hkv",
-                           "d", "bs", "nb", "scale", "qd", "kvd", "chunk", "chunks", "ws", "ws_bytes", "stream")]
+                           "d", "bs", "nb", "scale", "qd", "kvd", "ws", "ws_bytes", "stream")]
 
 
 def test_decode_argument_errors():
     rc, msg = _status("pa_decode", *_decode_args(hq=30))
     assert rc == _lib.PA_ERR_INVALID_ARG and "multiple of num_kv_heads" in msg
-    rc, msg = _status("pa_decode", *_decode_args(chunk=250))
-    assert rc == _lib.PA_ERR_INVALID_ARG and "chunk_tokens" in msg
+    rc, msg = _status("pa_decode", *_decode_args(bs=0))
+    assert rc == _lib.PA_ERR_INVALID_ARG and "block_size" in msg
+    for entry in ("pa_decode_split", "pa_decode_reduce"):
+        rc, msg = _status(entry, *_decode_args(hq=30))
+        assert rc == _lib.PA_ERR_INVALID_ARG
     rc, msg = _status("pa_decode", *_decode_args(d=96))
     assert rc == _lib.PA_ERR_UNSUPPORTED and "head_dim=96" in msg
     rc, msg = _status("pa_decode", *_decode_args(qd=_lib.PA_F32))
@@ -103,17 +106,18 @@ def test_decode_argument_errors():
     assert _status("pa_decode", *_decode_args(batch=0, q=None, ws=None, ws_bytes=0))[0] == _lib.PA_OK
 
 
-def test_decode_planning_arithmetic():
+def test_decode_workspace_arithmetic():
     lib = _lib.load()
-    assert lib.pa_decode_chunk_tokens(604, 4, 2, 16) == 256
-    assert lib.pa_decode_chunk_tokens(840539, 256, 8, 16) == 256
-    assert lib.pa_decode_chunk_tokens(10_000_000, 64, 8, 16) == 1024
-    assert lib.pa_decode_chunk_tokens(1000, 4, 2, 48) == 288  # rounded up to whole blocks
-    assert lib.pa_decode_chunk_tokens(-1, 4, 2, 16) == _lib.PA_ERR_INVALID_ARG
-    small = lib.pa_decode_workspace_bytes(1, 1, 1, 32)
-    big = lib.pa_decode_workspace_bytes(1000, 256, 32, 128)
-    assert 0 < small < big and big >= 1000 * 32 * 130 * 4
-    assert lib.pa_decode_workspace_bytes(-1, 1, 1, 32) == 0 and "pa_decode_workspace_bytes" in _lib.last_error()
+    small = lib.pa_decode_workspace_bytes(1, 1, 1, 32, _lib.PA_F32)
+    c4 = lib.pa_decode_workspace_bytes(256, 32, 8, 128, _lib.PA_BF16)
+    # (4096 + planes*batch) slots of hpw*NREP heads x (D+2) floats: shapes only, no lengths
+    assert 0 < small < c4 and c4 >= (4096 + 2 * 256) * 16 * 130 * 4
+    assert c4 % 256 == 0
+    assert lib.pa_decode_workspace_bytes(256, 32, 8, 128, _lib.PA_FP8_E4M3) > 0
+    assert lib.pa_decode_workspace_bytes(-1, 32, 8, 128, _lib.PA_BF16) == 0
+    assert "pa_decode_workspace_bytes" in _lib.last_error()
+    assert lib.pa_decode_workspace_bytes(4, 32, 8, 96, _lib.PA_BF16) == 0
+    assert lib.pa_decode_workspace_bytes(4, 30, 8, 128, _lib.PA_BF16) == 0
 
 
 def test_prefill_and_quantize_argument_errors():

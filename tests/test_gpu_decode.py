@@ -58,12 +58,30 @@ def test_c4_shape_reduced_batch():
     assert_close(_gpu_decode(w), want, 2e-2, "c4 reduced")
 
 
-def test_split_count_does_not_change_the_result():
-    announce("decode split invariance")
+def test_result_does_not_depend_on_the_partition():
+    """Where the workgroup ranges cut the sequences depends on the batch around them:
+    alone, every sequence is split over the whole grid; in the batch most are whole."""
+    announce("decode partition invariance")
     w = make_decode("c4", batch=12, len_range=(64, 5000), seed=77)
-    ref = _gpu_decode(w, chunk_tokens=16 * 1024).float()  # one chunk per sequence
-    for chunk in (16, 64, 256, 1024):
-        assert_close(_gpu_decode(w, chunk_tokens=chunk).float(), ref, 1e-2, f"chunk={chunk}")
+    tables = _lists(w)
+    q, kp, vp = w.q.to(DEV), w.k_pool.to(DEV), w.v_pool.to(DEV)
+    together = run_decode(q, kp, vp, tables, w.seq_lens, w.block_size, w.scale).float()
+    want = po.paged_decode(w.q, w.k_pool, w.v_pool, tables, w.seq_lens, w.block_size, w.scale)
+    assert_close(together, want, 2e-2, "batch")
+    for b in range(w.batch):
+        alone = run_decode(q[b : b + 1], kp, vp, tables[b : b + 1], w.seq_lens[b : b + 1], w.block_size, w.scale)
+        assert_close(alone.float(), together[b : b + 1], 1e-2, f"sequence {b} alone")
+    order = list(range(w.batch))[::-1]
+    rev = run_decode(q[order], kp, vp, [tables[i] for i in order], w.seq_lens[order], w.block_size, w.scale).float()
+    assert_close(rev, together[order], 1e-2, "reversed batch")
+
+
+def test_long_single_sequence_is_split_over_the_grid():
+    """One 40 000-key sequence: thousands of blocks, every workgroup gets a piece, one merged row."""
+    announce("decode single long sequence")
+    w = make_decode("c2", batch=1, len_range=(40000, 40000), seed=9)
+    want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, w.block_size, w.scale)
+    assert_close(_gpu_decode(w), want, 2e-2, "single long sequence")
 
 
 def test_pool_permutation_and_constant_values():
@@ -108,7 +126,7 @@ def test_head_layouts(hq, hkv, d, dtype):
     kp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
     vp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
     want = po.paged_decode(q, kp, vp, tables, lens, bs, d**-0.5)
-    got = run_decode(q.to(DEV), kp.to(DEV), vp.to(DEV), tables, lens, bs, d**-0.5, chunk_tokens=32)
+    got = run_decode(q.to(DEV), kp.to(DEV), vp.to(DEV), tables, lens, bs, d**-0.5)
     assert_close(got, want, 1e-5 if dtype == torch.float32 else 2e-2, "head layout")
 
 
