@@ -28,7 +28,7 @@ HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
 
 # HBM traffic of one decode_split_kernel launch on workload c4, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {"c4": 3455256371}  # profiles/decode_c4_bf16.md: fetch 3 447 663 616 + write 7 592 755
 
 
 def parse_args():

@@ -117,7 +117,7 @@ class HipPagedAttentionBackend:
         if ctx.slot_mapping is not None:
             self._store_kv(k, v, layer_idx, ctx.slot_mapping, _step=self._step(ctx))
         if ctx.is_prefill:
-            if ctx.prefix_lens is not None:
+            if getattr(ctx, "prefix_lens", None) is not None:  # absent on the reference's own context type
                 return self._prefill_paged(q, layer_idx, ctx)
             return self._prefill_attention(q, k, v, ctx)
         return self._decode_attention(q, layer_idx, ctx)
