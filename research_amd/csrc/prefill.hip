@@ -1,5 +1,7 @@
 // Host entry point of causal prefill attention over a paged context.
-#include "decode_impl.h"
+#include <stdlib.h>
+
+#include "prefill_mfma.h"
 
 using namespace pa_decode_detail;
 
@@ -36,6 +38,19 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     a.q = q; a.out = out; a.ctx_lens = ctx_lens; a.q_lens = q_lens; a.q_starts = q_starts;
     a.batch = batch; a.max_q_len = max_q_len;
     hipStream_t s = (hipStream_t)stream;
+    // bf16 / fp16 with head_dim 32, 64, 128 run on the matrix cores; PA_PREFILL_ROWWISE=1 forces the
+    // vector kernel (used to cross-check the two paths).
+    static const bool force_rowwise = [] { const char *e = getenv("PA_PREFILL_ROWWISE"); return e && e[0] == '1'; }();
+    const prefill_mfma_fn mfma = force_rowwise ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim);
+    if (mfma) {
+        PA_REQUIRE(pa_aligned16(q) && pa_aligned16(out), "q and out must be 16-byte aligned");
+        const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
+        const int groups = (row_blocks * a.p.n_rep + kPfWaves - 1) / kPfWaves;
+        PA_REQUIRE(groups <= 65535, "max_q_len=%d is too long for one launch", max_q_len);
+        mfma<<<dim3((unsigned)num_kv_heads, (unsigned)groups, (unsigned)batch), dim3(256), 0, s>>>(a);
+        PA_CHECK_LAUNCH("pa_prefill_paged (matrix-core kernel)");
+        return PA_OK;
+    }
     ks.rowwise<<<dim3((unsigned)(a.p.n_hgroups * a.p.n_rgroups), (unsigned)max_q_len, (unsigned)batch),
                  dim3(kThreads), 0, s>>>(a);
     PA_CHECK_LAUNCH("pa_prefill_paged");
