@@ -25,6 +25,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, vendor figure
 
 # HBM traffic of one decode_split_kernel launch on workload c4, from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/); None until measured.
@@ -36,7 +37,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c4", "c5"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -84,6 +85,105 @@ def cpu_baseline(w, budget_s: float):
     }
 
 
+def timed_ms(fn, steps):
+    """Average milliseconds per call: HIP events on the launch stream around `steps` calls."""
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def bench_prefill_c3(args, dev) -> int:
+    """Workload c3: append 32 x 256 new K/V rows, then chunked causal prefill over 2048 shared prefix keys.
+
+    One step = pa_kv_scatter + pa_prefill_paged.  The value is the step's attention FLOP rate; the roofline
+    entry is the matrix-core prefill kernel alone; the append is reported beside it in GB/s.
+    """
+    from oracle import paged_oracle as po
+    from research_amd import ops
+    from research_amd.workloads import make_prefill_c3
+
+    w = make_prefill_c3()
+    S, C, P = w.num_seqs, w.chunk_len, w.prefix_len
+    shape = (w.num_blocks * w.block_size, w.num_kv_heads, w.head_dim)
+    kc = torch.zeros(shape, dtype=w.dtype, device=dev)
+    vc = torch.zeros_like(kc)
+    ops.kv_scatter(kc, vc, w.k_prefix.to(dev), w.v_prefix.to(dev), torch.from_numpy(w.prefix_slots()).to(dev))
+    k_new = w.k_chunk.reshape(S * C, *shape[1:]).to(dev)
+    v_new = w.v_chunk.reshape(S * C, *shape[1:]).to(dev)
+    slots = torch.from_numpy(w.chunk_slots()).to(dev)
+    q = w.q.reshape(S * C, w.num_q_heads, w.head_dim).to(dev)
+    tables = torch.from_numpy(np.stack(w.block_tables).astype(np.int32)).to(dev)
+    ctx = torch.full((S,), P + C, dtype=torch.int32, device=dev)
+    ql = torch.full((S,), C, dtype=torch.int32, device=dev)
+    qs = torch.arange(S, dtype=torch.int32, device=dev) * C
+    out = torch.empty_like(q)
+
+    def append():
+        ops.kv_scatter(kc, vc, k_new, v_new, slots)
+
+    def prefill():
+        ops.prefill_paged(q, kc, vc, tables, ctx, ql, qs, C, w.block_size, w.scale, out=out)
+
+    def step():
+        append()
+        prefill()
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    for _ in range(args.warmup):
+        step()
+    ms_step = timed_ms(step, args.steps)
+    ms_prefill = timed_ms(prefill, args.steps)
+    ms_append = timed_ms(append, args.steps)
+    flops = w.attention_flops()
+    achieved = flops / (ms_prefill * 1e-3) / 1e12
+    result = {
+        "metric": "prefill-attn TFLOP/s", "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "tokens_per_s": S * C / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "c3 shared-prefix chunked prefill + KV append, 32 x (2048 + 256), bf16",
+                   "num_seqs": S, "prefix_len": P, "chunk_len": C, "num_q_heads": w.num_q_heads,
+                   "num_kv_heads": w.num_kv_heads, "head_dim": w.head_dim, "block_size": w.block_size,
+                   "attention_flops": flops, "append_bytes": w.append_bytes(), "seed": 1003},
+        "roofline": {"bound": "mfma", "kernel": "prefill_mfma_kernel", "achieved": achieved,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": None, "kernel_ms": ms_prefill},
+        "append": {"kernel": "kv_scatter_kernel", "kernel_ms": ms_append,
+                   "achieved_gbps": w.append_bytes() / (ms_append * 1e-3) / 1e9, "peak_gbps": HBM_PEAK_GBPS},
+    }
+    if not args.no_cpu_baseline:
+        threads = torch.get_num_threads()
+        n = 4  # sequences of the sample
+        kcc, vcc = kc.cpu(), vc.cpu()
+        t0 = time.perf_counter()
+        for s in range(n):
+            blocks = np.asarray(w.block_tables[s])
+            pos = np.arange(P + C)
+            idx = torch.from_numpy(blocks[pos // w.block_size] * w.block_size + pos % w.block_size)
+            k_full, v_full = kcc[idx][None], vcc[idx][None]
+            q_full = torch.cat([torch.zeros(P, w.num_q_heads, w.head_dim, dtype=w.dtype), w.q[s]])[None]
+            po.prefill_literal(q_full, k_full, v_full, w.scale)
+        dt = time.perf_counter() - t0
+        result["cpu_baseline"] = {
+            "value": flops / S * n / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{n} of {S} sequences: index gather of prefix+chunk, then the reference's full-sequence causal "
+                      f"SDPA over {P + C} tokens (rows {P}..{P + C - 1} are the chunk), {threads} threads, {dt:.1f} s; "
+                      "FLOPs counted for the chunk rows only",
+        }
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -98,6 +198,8 @@ def main() -> int:
         return 2
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    if args.workload == "c3":
+        return bench_prefill_c3(args, dev)
 
     t_gen = time.perf_counter()
     w = make_decode(args.workload)

@@ -41,7 +41,9 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     // bf16 / fp16 with head_dim 32, 64, 128 run on the matrix cores; PA_PREFILL_ROWWISE=1 forces the
     // vector kernel (used to cross-check the two paths).
     static const bool force_rowwise = [] { const char *e = getenv("PA_PREFILL_ROWWISE"); return e && e[0] == '1'; }();
-    const prefill_mfma_fn mfma = force_rowwise ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim);
+    // (its softmax takes the running maximum of the unscaled logits, which needs scale > 0)
+    const prefill_mfma_fn mfma =
+        force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
     if (mfma) {
         PA_REQUIRE(pa_aligned16(q) && pa_aligned16(out), "q and out must be 16-byte aligned");
         const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;

@@ -20,9 +20,14 @@
 //   (GQA packing: K/V are fetched once per kv head, not per query head).
 //   grid.x = kv head (fastest): with 8 XCDs a kv head's K/V stays in one XCD's
 //   L2 while all sequences and row blocks that share prefix blocks re-read it.
-//   K/V tiles of 64 keys go global -> registers -> LDS (next tile's loads are
-//   in flight while the current tile is multiplied); rows are padded in LDS
-//   so the 128-bit operand reads and the transpose reads are conflict free.
+//   K/V tiles of 64 keys go global -> LDS directly (global_load_lds, 16 bytes per
+//   lane, no staging registers) into one of two buffers, so the next tile's
+//   loads are in flight while the current tile is multiplied and there is one
+//   barrier per tile.  A direct load puts lane i's 16 bytes at base + 16*i, so
+//   rows cannot be padded; instead each lane fetches the chunk that belongs at
+//   its position under an XOR swizzle of the chunk index by the row, chosen so
+//   that the 128-bit operand reads (16 rows, same chunk) and the transpose
+//   reads (4 rows x 64 bytes) each touch all 64 banks once.
 #pragma once
 #include "decode_impl.h"
 
@@ -65,33 +70,36 @@ constexpr int kPfKeys = 64;   // keys per K/V tile
 constexpr int kPfRows = 64;   // query rows per wave
 constexpr int kPfWaves = 4;
 
-template <int D> struct PfLds {
-    static constexpr int kRowBytesK = D * 2 + 16;               // +16 B: 16 keys x 16 B hit 64 distinct banks
-    static constexpr int kRowBytesV = D * 2 + (D >= 64 ? 64 : 0);  // 4 keys x 64 B hit 64 distinct banks
-    static constexpr int kBytesK = kPfKeys * kRowBytesK;
-    static constexpr int kBytesV = kPfKeys * kRowBytesV;
+// LDS tile geometry and swizzles for head_dim D (rows of D*2 bytes = CPR chunks of 16 bytes).
+template <int D> struct PfTile {
+    static constexpr int RB = D * 2;            // row bytes
+    static constexpr int CPR = D / 8;           // 16-byte chunks per row
+    static constexpr int RPL = 64 / CPR;        // rows one wave-wide direct load covers
+    static constexpr int NL = CPR / 4;          // direct loads per wave, tile and tensor (16 rows per wave)
+    static constexpr int BYTES = kPfKeys * RB;  // one tensor's tile
+    static constexpr int RDIV = 16 / CPR;       // rows that share a 256-byte bank line
+    // K: 16 consecutive rows read the same chunk -> 16 distinct 16-byte bank groups
+    static __device__ __forceinline__ int swz_k(int row) { return (row / RDIV) % CPR; }
+    // V: 4 consecutive rows each read 4 consecutive chunks -> 4 distinct 64-byte bank groups
+    static __device__ __forceinline__ int swz_v(int row) { return CPR >= 8 ? ((row / RDIV) % (CPR / 4)) * 4 : 0; }
 };
 
-template <typename T, int D>
+template <typename T, int D, bool BS16>
 __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
     using X4 = typename M::x4;
-    using L = PfLds<D>;
-    constexpr int KS = D / 16;            // k-steps of the first product
-    constexpr int DT = D / 32;            // 32-wide d tiles of the second product
-    constexpr int CPR = D / 8;            // 16-byte chunks per K/V row
-    constexpr int LD = (kPfKeys * CPR) / 256;  // chunks a thread loads per tile and tensor
-    static_assert(LD >= 1, "tile smaller than the workgroup");
-    __shared__ __attribute__((aligned(16))) char s_k[L::kBytesK];
-    __shared__ __attribute__((aligned(16))) char s_v[L::kBytesV];
+    using G = PfTile<D>;
+    constexpr int KS = D / 16;  // k-steps of the first product
+    constexpr int DT = D / 32;  // 32-wide d tiles of the second product
+    __shared__ __attribute__((aligned(1024))) char s_buf[2][2][G::BYTES];  // [buffer][K, V][tile]
 
     const PoolArgs &p = a.p;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int half = lane >> 5;   // which 16 of the 32 keys / d values of a result tile
-    const int col = lane & 31;    // query row inside a 32-row tile
+    const int half = lane >> 5;  // which 16 of the 32 keys / d values of a result tile
+    const int col = lane & 31;   // query row inside a 32-row tile
 
     const int kvh = blockIdx.x;
     const int b = blockIdx.z;
@@ -136,134 +144,173 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) 
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) o[nt][dt][i] = 0.f;
-    float m_run[2] = {kNegBig, kNegBig}, l_run[2] = {0.f, 0.f};
+    // running maximum of the raw (unscaled) logits, the same times scale*log2e, and the running sum
+    float m_raw[2] = {kNegBig, kNegBig}, m_sc[2] = {kNegBig * p.scale_log2, kNegBig * p.scale_log2};
+    float l_run[2] = {0.f, 0.f};
 
-    // ---- cooperative tile loader: thread -> (key, 16-byte chunk) ------------
+    // ---- tile loader: wave w brings rows 16w..16w+15 of the tile, NL direct loads per tensor ----
     const int32_t *bt_row = p.bt + (int64_t)b * p.bt_stride;
     const int64_t tok_stride = (int64_t)p.hkv * D * 2;
-    uint4 kst[LD], vst[LD];
-    auto fetch = [&](int tile) {
+    const char *pool_k = reinterpret_cast<const char *>(p.k) + (int64_t)kvh * D * 2;
+    const char *pool_v = reinterpret_cast<const char *>(p.v) + (int64_t)kvh * D * 2;
+    const int ld_row = lane / G::CPR, ld_slot = lane % G::CPR;
+    auto issue = [&](int tile, int buf) {
 #pragma unroll
-        for (int i = 0; i < LD; ++i) {
-            const int idx = tid + 256 * i;
-            const int kk = idx / CPR, c = idx - kk * CPR;
-            const int key = tile * kPfKeys + kk;
-            kst[i] = vst[i] = uint4{0, 0, 0, 0};
-            if (key < ctx_len) {
+        for (int j = 0; j < G::NL; ++j) {
+            const int row = 16 * wave + j * G::RPL + ld_row;  // row of the tile this lane fills
+            const int key = tile * kPfKeys + row;
+            int64_t bid = -1;
+            int tok = 0;
+            if (BS16) {
+                const int blk = tile * 4 + wave;  // uniform: the wave's 16 rows are one pool block
+                bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
+                tok = j * G::RPL + ld_row;
+            } else if (key < ctx_len) {
                 const int blk = key / p.bs;
-                const int64_t bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
-                if (bid >= 0 && bid < p.num_blocks) {
-                    const int64_t off = (bid * p.bs + (key - blk * p.bs)) * tok_stride + (int64_t)kvh * D * 2 + c * 16;
-                    kst[i] = ld16(reinterpret_cast<const char *>(p.k) + off);
-                    vst[i] = ld16(reinterpret_cast<const char *>(p.v) + off);
-                }
+                bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
+                tok = key - blk * p.bs;
+            }
+            const bool ok = key < ctx_len && bid >= 0 && bid < p.num_blocks;
+            char *dst_k = &s_buf[buf][0][(16 * wave + j * G::RPL) * G::RB];  // uniform; lane i lands at +16*i
+            char *dst_v = &s_buf[buf][1][(16 * wave + j * G::RPL) * G::RB];
+            if (ok) {
+                const int64_t off = (bid * p.bs + tok) * tok_stride;
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void *)(pool_k + off + ((ld_slot ^ G::swz_k(row)) * 16)),
+                    (__attribute__((address_space(3))) void *)dst_k, 16, 0, 0);
+                __builtin_amdgcn_global_load_lds(
+                    (const __attribute__((address_space(1))) void *)(pool_v + off + ((ld_slot ^ G::swz_v(row)) * 16)),
+                    (__attribute__((address_space(3))) void *)dst_v, 16, 0, 0);
+            } else {
+                // past the context end or a missing block: all-zero key and value rows
+                *reinterpret_cast<uint4 *>(dst_k + lane * 16) = uint4{0, 0, 0, 0};
+                *reinterpret_cast<uint4 *>(dst_v + lane * 16) = uint4{0, 0, 0, 0};
             }
         }
     };
-    auto stash = [&]() {
+
+    // ---- per-lane byte offsets of the operand reads inside a tile ----
+    int k_ofs[KS];  // K operand: key row `col` (+32 per subtile), chunk 2*ks + half
 #pragma unroll
-        for (int i = 0; i < LD; ++i) {
-            const int idx = tid + 256 * i;
-            const int kk = idx / CPR, c = idx - kk * CPR;
-            *reinterpret_cast<uint4 *>(s_k + kk * L::kRowBytesK + c * 16) = kst[i];
-            *reinterpret_cast<uint4 *>(s_v + kk * L::kRowBytesV + c * 16) = vst[i];
+    for (int ks = 0; ks < KS; ++ks) k_ofs[ks] = col * G::RB + (((2 * ks + half) ^ G::swz_k(col)) * 16);
+    // V^T transpose read: 16-lane group g covers d = 16*(g%2).., keys 4*(g/2)..; source lane s of the group
+    // supplies the 8 bytes at key +s/4, d +4*(s%4)
+    const int g16 = lane >> 4, s16 = lane & 15;
+    const int v_key = 4 * (g16 >> 1) + (s16 >> 2);
+    int v_ofs[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+        v_ofs[dt] = v_key * G::RB + ((((4 * dt) ^ G::swz_v(v_key)) + 2 * (g16 & 1) + ((s16 & 3) >> 1)) * 16) + 8 * (s16 & 1);
+
+    const float c = p.scale_log2;
+
+    // one 32-key subtile of the current tile for this wave's 64 rows
+    auto subtile = [&](const char *tk, const char *tv, int key_base, auto mask_tag) {
+        constexpr bool kMask = decltype(mask_tag)::value;
+        // ---- S^T = K . Q^T: operand reads run two k-steps ahead of the products ----
+        f32x16 s[2];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[nt][i] = 0.f;
+        X8 ka[KS];
+#pragma unroll
+        for (int ks = 0; ks < KS && ks < 2; ++ks)
+            ka[ks] = __builtin_bit_cast(X8, *reinterpret_cast<const uint4 *>(tk + k_ofs[ks]));
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            if (ks + 2 < KS) ka[ks + 2] = __builtin_bit_cast(X8, *reinterpret_cast<const uint4 *>(tk + k_ofs[ks + 2]));
+            s[0] = M::mma(ka[ks], qreg[0][ks], s[0]);
+            s[1] = M::mma(ka[ks], qreg[1][ks], s[1]);
+        }
+        // first V^T operands are requested before the softmax arithmetic
+        X4 vlo[DT], vhi[DT];
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            vlo[dt] = M::tr_read(tv + v_ofs[dt]);
+            vhi[dt] = M::tr_read(tv + v_ofs[dt] + 8 * G::RB);
+        }
+        // ---- online softmax per row (= per lane); P^T is packed in place ----
+        uint32_t pp[2][8];
+#pragma unroll
+        for (int nt = 0; nt < 2; ++nt) {
+            if (kMask) {
+                const int limit = min(ctx_len - 1, prefix + row0 + 32 * nt + col) - key_base - 4 * half;
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[nt][i] = 8 * (i >> 2) + (i & 3) <= limit ? s[nt][i] : -INFINITY;
+            }
+            float mx = fmaxf(s[nt][0], s[nt][1]);
+#pragma unroll
+            for (int i = 2; i < 16; ++i) mx = fmaxf(mx, s[nt][i]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m_raw[nt]) != 0, 0)) {
+                const float m_new = fmaxf(m_raw[nt], mx);
+                const float alpha = __builtin_amdgcn_exp2f((m_raw[nt] - m_new) * c);
+                l_run[nt] *= alpha;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) o[nt][dt][i] *= alpha;
+                m_raw[nt] = m_new;
+                m_sc[nt] = m_new * c;
+            }
+            float sum = 0.f;
+#pragma unroll
+            for (int i = 0; i < 16; i += 2) {
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(s[nt][i], c, -m_sc[nt]));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(s[nt][i + 1], c, -m_sc[nt]));
+                sum += p0 + p1;
+                pp[nt][i >> 1] = M::pack(p0, p1);
+            }
+            l_run[nt] += sum;
+        }
+        // ---- O^T += V^T . P^T.  k-step ks2 uses result rows 8*ks2..8*ks2+7 of the lane, i.e. keys
+        //      key_base + 16*ks2 + 8*(e/4) + 4*half + e%4 for operand element e ----
+#pragma unroll
+        for (int ks2 = 0; ks2 < 2; ++ks2) {
+            X8 pb[2];
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt) {
+                const uint4 raw = uint4{pp[nt][4 * ks2], pp[nt][4 * ks2 + 1], pp[nt][4 * ks2 + 2], pp[nt][4 * ks2 + 3]};
+                pb[nt] = __builtin_bit_cast(X8, raw);
+            }
+            X8 va[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { va[dt][e] = vlo[dt][e]; va[dt][4 + e] = vhi[dt][e]; }
+            if (ks2 == 0) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {  // operands of the second k-step, in flight during the first
+                    vlo[dt] = M::tr_read(tv + 16 * G::RB + v_ofs[dt]);
+                    vhi[dt] = M::tr_read(tv + 24 * G::RB + v_ofs[dt]);
+                }
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                o[0][dt] = M::mma(va[dt], pb[0], o[0][dt]);
+                o[1][dt] = M::mma(va[dt], pb[1], o[1][dt]);
+            }
         }
     };
 
-    // per-lane byte offsets of the operand reads inside a tile
-    const int k_rd = col * L::kRowBytesK + half * 16;  // + 32-key subtile, + 32*ks
-    // V^T transpose read: 16-lane group g = lane/16 covers d = 16*(g%2).., keys 4*(g/2)..; source lane s of the
-    // group reads the 8 bytes at key +s/4, d +4*(s%4)
-    const int g16 = lane >> 4, s16 = lane & 15;
-    const int v_rd = (4 * (g16 >> 1) + (s16 >> 2)) * L::kRowBytesV + (16 * (g16 & 1) + 4 * (s16 & 3)) * 2;
-
-    fetch(0);
+    issue(0, 0);
     for (int tile = 0; tile < n_tiles; ++tile) {
-        __syncthreads();  // everyone is done reading the previous tile
-        stash();
-        __syncthreads();
-        if (tile + 1 < n_tiles) fetch(tile + 1);  // in flight during the products below
+        const int buf = tile & 1;
+        __builtin_amdgcn_s_waitcnt(0);  // this wave's direct loads and zero fills of `tile` have landed
+        __syncthreads();                // ... and everyone's; everyone is also done reading the other buffer
+        if (tile + 1 < n_tiles) issue(tile + 1, buf ^ 1);
         const int key0 = tile * kPfKeys;
         if (key0 >= my_keys) continue;  // this wave's rows end before this tile (uniform per wave)
         // masking is needed only where the tile reaches past the first row's causal limit or the context end
         const bool need_mask = key0 + kPfKeys > prefix + row0 + 1 || key0 + kPfKeys > ctx_len;
-
-#pragma unroll
-        for (int kt = 0; kt < 2; ++kt) {
-            // ---- S^T = K . Q^T for 32 keys x 64 rows ---------------------
-            f32x16 s[2];
-#pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) s[nt][i] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                const uint4 raw = *reinterpret_cast<const uint4 *>(s_k + kt * 32 * L::kRowBytesK + k_rd + ks * 32);
-                const X8 ka = __builtin_bit_cast(X8, raw);
-                s[0] = M::mma(ka, qreg[0][ks], s[0]);
-                s[1] = M::mma(ka, qreg[1][ks], s[1]);
-            }
-            // ---- online softmax per row (= per lane), P^T packed in place ----
-            uint32_t pp[2][8];
-#pragma unroll
-            for (int nt = 0; nt < 2; ++nt) {
-                float v[16];
-#pragma unroll
-                for (int i = 0; i < 16; ++i) v[i] = s[nt][i] * p.scale_log2;
-                if (need_mask) {
-                    const int limit = min(ctx_len - 1, prefix + row0 + 32 * nt + col);  // last visible key
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int key = key0 + 32 * kt + 4 * half + 8 * (i >> 2) + (i & 3);
-                        v[i] = key <= limit ? v[i] : -INFINITY;
-                    }
-                }
-                float mx = v[0];
-#pragma unroll
-                for (int i = 1; i < 16; ++i) mx = fmaxf(mx, v[i]);
-                mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-                const float m_new = fmaxf(m_run[nt], mx);
-                if (__builtin_amdgcn_ballot_w64(m_new > m_run[nt]) != 0) {
-                    const float alpha = __builtin_amdgcn_exp2f(m_run[nt] - m_new);
-                    l_run[nt] *= alpha;
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) o[nt][dt][i] *= alpha;
-                    m_run[nt] = m_new;
-                }
-                float sum = 0.f;
-#pragma unroll
-                for (int i = 0; i < 16; i += 2) {
-                    const float p0 = __builtin_amdgcn_exp2f(v[i] - m_run[nt]);
-                    const float p1 = __builtin_amdgcn_exp2f(v[i + 1] - m_run[nt]);
-                    sum += p0 + p1;
-                    pp[nt][i >> 1] = M::pack(p0, p1);
-                }
-                l_run[nt] += sum;
-            }
-            // ---- O^T += V^T . P^T: k-step ks2 uses result rows 8*ks2..8*ks2+7 of the lane, i.e. keys
-            //      32*kt + 8*(2*ks2 + e/4) + 4*half + e%4 for operand element e ----
-#pragma unroll
-            for (int ks2 = 0; ks2 < 2; ++ks2) {
-                X8 pb[2];
-#pragma unroll
-                for (int nt = 0; nt < 2; ++nt) {
-                    const uint4 raw = uint4{pp[nt][4 * ks2], pp[nt][4 * ks2 + 1], pp[nt][4 * ks2 + 2], pp[nt][4 * ks2 + 3]};
-                    pb[nt] = __builtin_bit_cast(X8, raw);
-                }
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    const char *vp = s_v + (32 * kt + 16 * ks2) * L::kRowBytesV + v_rd + dt * 64;
-                    const X4 lo = M::tr_read(vp);                        // keys +0..3 (+4 for the upper half-wave)
-                    const X4 hi = M::tr_read(vp + 8 * L::kRowBytesV);   // keys +8..11
-                    X8 va;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) { va[e] = lo[e]; va[4 + e] = hi[e]; }
-                    o[0][dt] = M::mma(va, pb[0], o[0][dt]);
-                    o[1][dt] = M::mma(va, pb[1], o[1][dt]);
-                }
-            }
+        const char *tk = &s_buf[buf][0][0], *tv = &s_buf[buf][1][0];
+        if (need_mask) {
+            subtile(tk, tv, key0, std::true_type{});
+            subtile(tk + 32 * G::RB, tv + 32 * G::RB, key0 + 32, std::true_type{});
+        } else {
+            subtile(tk, tv, key0, std::false_type{});
+            subtile(tk + 32 * G::RB, tv + 32 * G::RB, key0 + 32, std::false_type{});
         }
     }
 
@@ -290,6 +337,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) 
 }
 
 typedef void (*prefill_mfma_fn)(const RowwiseArgs);
-prefill_mfma_fn pa_prefill_mfma_kernel(int dtype, int d);  // nullptr if the shape has no matrix-core kernel
+// nullptr if the shape has no matrix-core kernel; `bs16` selects the variant for pools of 16-token blocks
+prefill_mfma_fn pa_prefill_mfma_kernel(int dtype, int d, bool bs16);
 
 }  // namespace pa_decode_detail

@@ -3,16 +3,16 @@
 
 namespace pa_decode_detail {
 
-prefill_mfma_fn pa_prefill_mfma_kernel(int dtype, int d) {
-    if (dtype == PA_BF16) {
-        if (d == 32) return prefill_mfma_kernel<pa_bf16, 32>;
-        if (d == 64) return prefill_mfma_kernel<pa_bf16, 64>;
-        if (d == 128) return prefill_mfma_kernel<pa_bf16, 128>;
-    } else if (dtype == PA_F16) {
-        if (d == 32) return prefill_mfma_kernel<pa_f16, 32>;
-        if (d == 64) return prefill_mfma_kernel<pa_f16, 64>;
-        if (d == 128) return prefill_mfma_kernel<pa_f16, 128>;
-    }
+template <typename T> static prefill_mfma_fn by_shape(int d, bool bs16) {
+    if (d == 32) return bs16 ? prefill_mfma_kernel<T, 32, true> : prefill_mfma_kernel<T, 32, false>;
+    if (d == 64) return bs16 ? prefill_mfma_kernel<T, 64, true> : prefill_mfma_kernel<T, 64, false>;
+    if (d == 128) return bs16 ? prefill_mfma_kernel<T, 128, true> : prefill_mfma_kernel<T, 128, false>;
+    return nullptr;
+}
+
+prefill_mfma_fn pa_prefill_mfma_kernel(int dtype, int d, bool bs16) {
+    if (dtype == PA_BF16) return by_shape<pa_bf16>(d, bs16);
+    if (dtype == PA_F16) return by_shape<pa_f16>(d, bs16);
     return nullptr;
 }
 
