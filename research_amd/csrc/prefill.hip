@@ -49,7 +49,7 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
         const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
         const int groups = (row_blocks * a.p.n_rep + kPfWaves - 1) / kPfWaves;
         PA_REQUIRE(groups <= 65535, "max_q_len=%d is too long for one launch", max_q_len);
-        mfma<<<dim3((unsigned)num_kv_heads, (unsigned)groups, (unsigned)batch), dim3(256), 0, s>>>(a);
+        mfma<<<dim3((unsigned)num_kv_heads, (unsigned)groups, (unsigned)batch), dim3(kPfThreads), 0, s>>>(a);
         PA_CHECK_LAUNCH("pa_prefill_paged (matrix-core kernel)");
         return PA_OK;
     }

@@ -14,8 +14,10 @@
 // order, so P never moves between lanes.
 //
 // Work split
-//   workgroup = 4 waves; a wave owns 64 query rows (two 32-row MFMA column
-//   tiles) of ONE query head; the 4 waves of a workgroup take 4 consecutive
+//   workgroup = 8 waves (two per SIMD, so one wave's softmax arithmetic runs
+//   under the other's matrix instructions); a wave owns 32 query rows (one MFMA
+//   column tile) of ONE query head and keeps everything in ordinary VGPRs
+//   (64 accumulators + 32 for Q + 16 for S); the 8 waves take 8 consecutive
 //   (row block, query head of the kv head) tasks, so they share every K/V tile
 //   (GQA packing: K/V are fetched once per kv head, not per query head).
 //   grid.x = kv head (fastest): with 8 XCDs a kv head's K/V stays in one XCD's
@@ -67,15 +69,16 @@ template <> struct Mfma16<pa_f16> {
 };
 
 constexpr int kPfKeys = 64;   // keys per K/V tile
-constexpr int kPfRows = 64;   // query rows per wave
-constexpr int kPfWaves = 4;
+constexpr int kPfRows = 32;   // query rows per wave
+constexpr int kPfWaves = 8;
+constexpr int kPfThreads = kPfWaves * 64;
 
 // LDS tile geometry and swizzles for head_dim D (rows of D*2 bytes = CPR chunks of 16 bytes).
 template <int D> struct PfTile {
     static constexpr int RB = D * 2;            // row bytes
     static constexpr int CPR = D / 8;           // 16-byte chunks per row
     static constexpr int RPL = 64 / CPR;        // rows one wave-wide direct load covers
-    static constexpr int NL = CPR / 4;          // direct loads per wave, tile and tensor (16 rows per wave)
+    static constexpr int LOADS = CPR;           // wave-wide direct loads per tile and tensor
     static constexpr int BYTES = kPfKeys * RB;  // one tensor's tile
     static constexpr int RDIV = 16 / CPR;       // rows that share a 256-byte bank line
     // K: 16 consecutive rows read the same chunk -> 16 distinct 16-byte bank groups
@@ -85,7 +88,7 @@ template <int D> struct PfTile {
 };
 
 template <typename T, int D, bool BS16>
-__global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) {
+__global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
     using X4 = typename M::x4;
@@ -99,7 +102,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) 
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5;  // which 16 of the 32 keys / d values of a result tile
-    const int col = lane & 31;   // query row inside a 32-row tile
+    const int col = lane & 31;   // query row inside the wave's 32-row tile
 
     const int kvh = blockIdx.x;
     const int b = blockIdx.z;
@@ -123,32 +126,29 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) 
     const int wg_keys = min(ctx_len, prefix + min(q_len, (last_task / p.n_rep) * kPfRows + kPfRows));
     const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys;
 
-    // ---- Q^T operand: row = row0 + 32*nt + col, d = 16*ks + 8*half .. +8 ----
+    // ---- Q^T operand: row = row0 + col, d = 16*ks + 8*half .. +8 ----
     const T *qbase = reinterpret_cast<const T *>(a.q) + ((int64_t)a.q_starts[b] * p.hq + qh) * D;
-    X8 qreg[2][KS];
-#pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-        const int row = row0 + 32 * nt + col;
+    X8 qreg[KS];
+    {
+        const int row = row0 + col;
         const bool ok = live && row < q_len;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             uint4 raw = ok ? ld16(qbase + (int64_t)row * p.hq * D + 16 * ks + 8 * half) : uint4{0, 0, 0, 0};
-            qreg[nt][ks] = __builtin_bit_cast(X8, raw);
+            qreg[ks] = __builtin_bit_cast(X8, raw);
         }
     }
 
-    f32x16 o[2][DT];
+    f32x16 o[DT];
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) o[nt][dt][i] = 0.f;
+        for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
     // running maximum of the raw (unscaled) logits, the same times scale*log2e, and the running sum
-    float m_raw[2] = {kNegBig, kNegBig}, m_sc[2] = {kNegBig * p.scale_log2, kNegBig * p.scale_log2};
-    float l_run[2] = {0.f, 0.f};
+    const float c = p.scale_log2;
+    float m_raw = kNegBig, m_sc = kNegBig * c, l_run = 0.f;
 
-    // ---- tile loader: wave w brings rows 16w..16w+15 of the tile, NL direct loads per tensor ----
+    // ---- tile loader: wave-wide direct load l covers rows l*RPL .. of the tile; wave w issues l = w, w+8, ... ----
     const int32_t *bt_row = p.bt + (int64_t)b * p.bt_stride;
     const int64_t tok_stride = (int64_t)p.hkv * D * 2;
     const char *pool_k = reinterpret_cast<const char *>(p.k) + (int64_t)kvh * D * 2;
@@ -156,23 +156,25 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) 
     const int ld_row = lane / G::CPR, ld_slot = lane % G::CPR;
     auto issue = [&](int tile, int buf) {
 #pragma unroll
-        for (int j = 0; j < G::NL; ++j) {
-            const int row = 16 * wave + j * G::RPL + ld_row;  // row of the tile this lane fills
+        for (int l0 = 0; l0 < G::LOADS; l0 += kPfWaves) {
+            const int l = l0 + wave;  // uniform
+            if (l >= G::LOADS) break;
+            const int row = l * G::RPL + ld_row;  // row of the tile this lane fills
             const int key = tile * kPfKeys + row;
             int64_t bid = -1;
             int tok = 0;
             if (BS16) {
-                const int blk = tile * 4 + wave;  // uniform: the wave's 16 rows are one pool block
+                const int blk = tile * 4 + (l * G::RPL) / 16;  // uniform: the load's rows lie in one pool block
                 bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
-                tok = j * G::RPL + ld_row;
+                tok = (l * G::RPL) % 16 + ld_row;
             } else if (key < ctx_len) {
                 const int blk = key / p.bs;
                 bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
                 tok = key - blk * p.bs;
             }
             const bool ok = key < ctx_len && bid >= 0 && bid < p.num_blocks;
-            char *dst_k = &s_buf[buf][0][(16 * wave + j * G::RPL) * G::RB];  // uniform; lane i lands at +16*i
-            char *dst_v = &s_buf[buf][1][(16 * wave + j * G::RPL) * G::RB];
+            char *dst_k = &s_buf[buf][0][l * G::RPL * G::RB];  // uniform; lane i lands at +16*i
+            char *dst_v = &s_buf[buf][1][l * G::RPL * G::RB];
             if (ok) {
                 const int64_t off = (bid * p.bs + tok) * tok_stride;
                 __builtin_amdgcn_global_load_lds(
@@ -202,28 +204,23 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) 
     for (int dt = 0; dt < DT; ++dt)
         v_ofs[dt] = v_key * G::RB + ((((4 * dt) ^ G::swz_v(v_key)) + 2 * (g16 & 1) + ((s16 & 3) >> 1)) * 16) + 8 * (s16 & 1);
 
-    const float c = p.scale_log2;
-
-    // one 32-key subtile of the current tile for this wave's 64 rows
-    auto subtile = [&](const char *tk, const char *tv, int key_base, auto mask_tag) {
-        constexpr bool kMask = decltype(mask_tag)::value;
-        // ---- S^T = K . Q^T: operand reads run two k-steps ahead of the products ----
-        f32x16 s[2];
+    // one 32-key subtile of the current tile for this wave's 32 rows
+    auto subtile = [&](const char *tk, const char *tv, int key_base, bool need_mask) {
+        // ---- S^T = K . Q^T ----
+        f32x16 s;
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt)
+        for (int i = 0; i < 16; ++i) s[i] = 0.f;
+        constexpr int KG = KS < 4 ? KS : 4;  // operand reads are issued in groups of 4 k-steps
 #pragma unroll
-            for (int i = 0; i < 16; ++i) s[nt][i] = 0.f;
-        X8 ka[KS];
+        for (int k0 = 0; k0 < KS; k0 += KG) {
+            X8 ka[KG];
 #pragma unroll
-        for (int ks = 0; ks < KS && ks < 2; ++ks)
-            ka[ks] = __builtin_bit_cast(X8, *reinterpret_cast<const uint4 *>(tk + k_ofs[ks]));
+            for (int ks = 0; ks < KG; ++ks)
+                ka[ks] = __builtin_bit_cast(X8, *reinterpret_cast<const uint4 *>(tk + k_ofs[k0 + ks]));
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            if (ks + 2 < KS) ka[ks + 2] = __builtin_bit_cast(X8, *reinterpret_cast<const uint4 *>(tk + k_ofs[ks + 2]));
-            s[0] = M::mma(ka[ks], qreg[0][ks], s[0]);
-            s[1] = M::mma(ka[ks], qreg[1][ks], s[1]);
+            for (int ks = 0; ks < KG; ++ks) s = M::mma(ka[ks], qreg[k0 + ks], s);
         }
-        // first V^T operands are requested before the softmax arithmetic
+        // V^T operands of the first k-step are requested before the softmax arithmetic
         X4 vlo[DT], vhi[DT];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -231,49 +228,41 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) 
             vhi[dt] = M::tr_read(tv + v_ofs[dt] + 8 * G::RB);
         }
         // ---- online softmax per row (= per lane); P^T is packed in place ----
-        uint32_t pp[2][8];
+        if (need_mask) {  // uniform
+            const int limit = min(ctx_len - 1, prefix + row0 + col) - key_base - 4 * half;  // last visible key
 #pragma unroll
-        for (int nt = 0; nt < 2; ++nt) {
-            if (kMask) {
-                const int limit = min(ctx_len - 1, prefix + row0 + 32 * nt + col) - key_base - 4 * half;
-#pragma unroll
-                for (int i = 0; i < 16; ++i) s[nt][i] = 8 * (i >> 2) + (i & 3) <= limit ? s[nt][i] : -INFINITY;
-            }
-            float mx = fmaxf(s[nt][0], s[nt][1]);
-#pragma unroll
-            for (int i = 2; i < 16; ++i) mx = fmaxf(mx, s[nt][i]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m_raw[nt]) != 0, 0)) {
-                const float m_new = fmaxf(m_raw[nt], mx);
-                const float alpha = __builtin_amdgcn_exp2f((m_raw[nt] - m_new) * c);
-                l_run[nt] *= alpha;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int i = 0; i < 16; ++i) o[nt][dt][i] *= alpha;
-                m_raw[nt] = m_new;
-                m_sc[nt] = m_new * c;
-            }
-            float sum = 0.f;
-#pragma unroll
-            for (int i = 0; i < 16; i += 2) {
-                const float p0 = __builtin_amdgcn_exp2f(fmaf(s[nt][i], c, -m_sc[nt]));
-                const float p1 = __builtin_amdgcn_exp2f(fmaf(s[nt][i + 1], c, -m_sc[nt]));
-                sum += p0 + p1;
-                pp[nt][i >> 1] = M::pack(p0, p1);
-            }
-            l_run[nt] += sum;
+            for (int i = 0; i < 16; ++i) s[i] = 8 * (i >> 2) + (i & 3) <= limit ? s[i] : -INFINITY;
         }
+        float mx = fmaxf(s[0], s[1]);
+#pragma unroll
+        for (int i = 2; i < 16; ++i) mx = fmaxf(mx, s[i]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m_raw) != 0, 0)) {  // rare once the maxima settle
+            const float m_new = fmaxf(m_raw, mx);
+            const float alpha = __builtin_amdgcn_exp2f((m_raw - m_new) * c);
+            l_run *= alpha;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
+            m_raw = m_new;
+            m_sc = m_new * c;
+        }
+        uint32_t pp[8];
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; i += 2) {
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(s[i], c, -m_sc));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(s[i + 1], c, -m_sc));
+            sum += p0 + p1;
+            pp[i >> 1] = M::pack(p0, p1);
+        }
+        l_run += sum;
         // ---- O^T += V^T . P^T.  k-step ks2 uses result rows 8*ks2..8*ks2+7 of the lane, i.e. keys
         //      key_base + 16*ks2 + 8*(e/4) + 4*half + e%4 for operand element e ----
 #pragma unroll
         for (int ks2 = 0; ks2 < 2; ++ks2) {
-            X8 pb[2];
-#pragma unroll
-            for (int nt = 0; nt < 2; ++nt) {
-                const uint4 raw = uint4{pp[nt][4 * ks2], pp[nt][4 * ks2 + 1], pp[nt][4 * ks2 + 2], pp[nt][4 * ks2 + 3]};
-                pb[nt] = __builtin_bit_cast(X8, raw);
-            }
+            const X8 pb = __builtin_bit_cast(X8, uint4{pp[4 * ks2], pp[4 * ks2 + 1], pp[4 * ks2 + 2], pp[4 * ks2 + 3]});
             X8 va[DT];
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
@@ -287,10 +276,7 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) 
                 }
             }
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                o[0][dt] = M::mma(va[dt], pb[0], o[0][dt]);
-                o[1][dt] = M::mma(va[dt], pb[1], o[1][dt]);
-            }
+            for (int dt = 0; dt < DT; ++dt) o[dt] = M::mma(va[dt], pb, o[dt]);
         }
     };
 
@@ -305,35 +291,27 @@ __global__ __launch_bounds__(256) void prefill_mfma_kernel(const RowwiseArgs a) 
         // masking is needed only where the tile reaches past the first row's causal limit or the context end
         const bool need_mask = key0 + kPfKeys > prefix + row0 + 1 || key0 + kPfKeys > ctx_len;
         const char *tk = &s_buf[buf][0][0], *tv = &s_buf[buf][1][0];
-        if (need_mask) {
-            subtile(tk, tv, key0, std::true_type{});
-            subtile(tk + 32 * G::RB, tv + 32 * G::RB, key0 + 32, std::true_type{});
-        } else {
-            subtile(tk, tv, key0, std::false_type{});
-            subtile(tk + 32 * G::RB, tv + 32 * G::RB, key0 + 32, std::false_type{});
-        }
+#pragma unroll 1
+        for (int kt = 0; kt < 2; ++kt)
+            subtile(tk + kt * 32 * G::RB, tv + kt * 32 * G::RB, key0 + 32 * kt, need_mask);
     }
 
-    // ---- normalise and write: lane owns row (row0+32*nt+col), d = 32*dt + 4*half + 8*g + j ----
+    // ---- normalise and write: lane owns row (row0+col), d = 32*dt + 4*half + 8*g + j ----
     if (!live) return;
-    T *obase = reinterpret_cast<T *>(a.out) + ((int64_t)a.q_starts[b] * p.hq + qh) * D;
+    const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    const int row = row0 + col;
+    if (row >= q_len) return;
+    T *orow = reinterpret_cast<T *>(a.out) + (((int64_t)a.q_starts[b] + row) * p.hq + qh) * D;
 #pragma unroll
-    for (int nt = 0; nt < 2; ++nt) {
-        const float l_tot = l_run[nt] + __shfl_xor(l_run[nt], 32, 64);
-        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-        const int row = row0 + 32 * nt + col;
-        if (row >= q_len) continue;
-        T *orow = obase + (int64_t)row * p.hq * D;
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-        for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                uint2 w;
-                w.x = M::pack(o[nt][dt][4 * g] * inv, o[nt][dt][4 * g + 1] * inv);
-                w.y = M::pack(o[nt][dt][4 * g + 2] * inv, o[nt][dt][4 * g + 3] * inv);
-                *reinterpret_cast<uint2 *>(orow + 32 * dt + 4 * half + 8 * g) = w;
-            }
-    }
+        for (int g = 0; g < 4; ++g) {
+            uint2 w;
+            w.x = M::pack(o[dt][4 * g] * inv, o[dt][4 * g + 1] * inv);
+            w.y = M::pack(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
+            *reinterpret_cast<uint2 *>(orow + 32 * dt + 4 * half + 8 * g) = w;
+        }
 }
 
 typedef void (*prefill_mfma_fn)(const RowwiseArgs);
