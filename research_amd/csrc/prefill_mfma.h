@@ -95,7 +95,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     using G = PfTile<D>;
     constexpr int KS = D / 16;  // k-steps of the first product
     constexpr int DT = D / 32;  // 32-wide d tiles of the second product
-    __shared__ __attribute__((aligned(1024))) char s_buf[2][2][G::BYTES];  // [buffer][K, V][tile]
+    // Two K/V tile buffers as four separate LDS objects: the compiler then knows that a direct load into one
+    // buffer cannot alias the operand reads from the other and does not make the reads wait for the load.
+    __shared__ __attribute__((aligned(1024))) char s_k0[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char s_v0[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char s_k1[G::BYTES];
+    __shared__ __attribute__((aligned(1024))) char s_v1[G::BYTES];
 
     const PoolArgs &p = a.p;
     const int tid = threadIdx.x;
@@ -154,27 +159,42 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     const char *pool_k = reinterpret_cast<const char *>(p.k) + (int64_t)kvh * D * 2;
     const char *pool_v = reinterpret_cast<const char *>(p.v) + (int64_t)kvh * D * 2;
     const int ld_row = lane / G::CPR, ld_slot = lane % G::CPR;
-    auto issue = [&](int tile, int buf) {
+    constexpr int NLW = (G::LOADS + kPfWaves - 1) / kPfWaves;  // direct loads per wave, tile and tensor
+    // Block ids are looked up one tile ahead of the loads that use them, so that the table read (and its
+    // latency) never sits between the barrier and the products: bid_next[] holds the ids for the tile that
+    // the next call of issue() will load.
+    int bid_next[NLW];  // kept as loaded: any arithmetic on it here would wait for the load
+    auto lookup = [&](int tile) {
 #pragma unroll
-        for (int l0 = 0; l0 < G::LOADS; l0 += kPfWaves) {
-            const int l = l0 + wave;  // uniform
+        for (int n = 0; n < NLW; ++n) {
+            const int l = n * kPfWaves + wave;  // uniform
+            bid_next[n] = -1;
+            if (l >= G::LOADS) continue;
+            int blk;
+            if (BS16) {
+                blk = tile * 4 + (l * G::RPL) / 16;  // uniform: the load's rows lie in one pool block
+            } else {
+                const int key = tile * kPfKeys + l * G::RPL + ld_row;
+                blk = key < ctx_len ? key / p.bs : -1;
+            }
+            // The index is laundered through a VGPR so that this becomes a vector load: a scalar load would
+            // share its completion counter with the LDS operand reads and stall the first of them.
+            asm volatile("" : "+v"(blk));
+            if (blk >= 0 && blk < p.bt_stride && tile * kPfKeys < ctx_len) bid_next[n] = bt_row[blk];
+        }
+    };
+    auto issue = [&](int tile, char *buf_k, char *buf_v) {
+#pragma unroll
+        for (int n = 0; n < NLW; ++n) {
+            const int l = n * kPfWaves + wave;  // uniform
             if (l >= G::LOADS) break;
             const int row = l * G::RPL + ld_row;  // row of the tile this lane fills
             const int key = tile * kPfKeys + row;
-            int64_t bid = -1;
-            int tok = 0;
-            if (BS16) {
-                const int blk = tile * 4 + (l * G::RPL) / 16;  // uniform: the load's rows lie in one pool block
-                bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
-                tok = (l * G::RPL) % 16 + ld_row;
-            } else if (key < ctx_len) {
-                const int blk = key / p.bs;
-                bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
-                tok = key - blk * p.bs;
-            }
+            const int64_t bid = bid_next[n];  // sign-extended only now, one tile after the load was issued
+            const int tok = BS16 ? (l * G::RPL) % 16 + ld_row : key % p.bs;
             const bool ok = key < ctx_len && bid >= 0 && bid < p.num_blocks;
-            char *dst_k = &s_buf[buf][0][l * G::RPL * G::RB];  // uniform; lane i lands at +16*i
-            char *dst_v = &s_buf[buf][1][l * G::RPL * G::RB];
+            char *dst_k = buf_k + l * G::RPL * G::RB;  // uniform; lane i lands at +16*i
+            char *dst_v = buf_v + l * G::RPL * G::RB;
             if (ok) {
                 const int64_t off = (bid * p.bs + tok) * tok_stride;
                 __builtin_amdgcn_global_load_lds(
@@ -280,20 +300,29 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         }
     };
 
-    issue(0, 0);
-    for (int tile = 0; tile < n_tiles; ++tile) {
-        const int buf = tile & 1;
+    // one K/V tile: wait for it, start the next one into the other buffer, multiply
+    auto do_tile = [&](int tile, char *cur_k, char *cur_v, char *nxt_k, char *nxt_v) {
         __builtin_amdgcn_s_waitcnt(0);  // this wave's direct loads and zero fills of `tile` have landed
         __syncthreads();                // ... and everyone's; everyone is also done reading the other buffer
-        if (tile + 1 < n_tiles) issue(tile + 1, buf ^ 1);
+        if (tile + 1 < n_tiles) {
+            issue(tile + 1, nxt_k, nxt_v);
+            lookup(tile + 2);  // consumed by the next tile's issue()
+        }
         const int key0 = tile * kPfKeys;
-        if (key0 >= my_keys) continue;  // this wave's rows end before this tile (uniform per wave)
-        // masking is needed only where the tile reaches past the first row's causal limit or the context end
-        const bool need_mask = key0 + kPfKeys > prefix + row0 + 1 || key0 + kPfKeys > ctx_len;
-        const char *tk = &s_buf[buf][0][0], *tv = &s_buf[buf][1][0];
-#pragma unroll 1
-        for (int kt = 0; kt < 2; ++kt)
-            subtile(tk + kt * 32 * G::RB, tv + kt * 32 * G::RB, key0 + 32 * kt, need_mask);
+        if (key0 < my_keys) {  // else this wave's rows end before this tile (uniform per wave)
+            // masking is needed only where the tile reaches past the first row's causal limit or the context end
+            const bool need_mask = key0 + kPfKeys > prefix + row0 + 1 || key0 + kPfKeys > ctx_len;
+#pragma unroll
+            for (int kt = 0; kt < 2; ++kt)
+                subtile(cur_k + kt * 32 * G::RB, cur_v + kt * 32 * G::RB, key0 + 32 * kt, need_mask);
+        }
+    };
+    lookup(0);
+    issue(0, s_k0, s_v0);
+    lookup(1);
+    for (int tile = 0; tile < n_tiles; tile += 2) {
+        do_tile(tile, s_k0, s_v0, s_k1, s_v1);
+        if (tile + 1 < n_tiles) do_tile(tile + 1, s_k1, s_v1, s_k0, s_v0);
     }
 
     // ---- normalise and write: lane owns row (row0+col), d = 32*dt + 4*half + 8*g + j ----
