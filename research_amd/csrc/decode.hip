@@ -145,9 +145,7 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
         PA_CHECK_LAUNCH("pa_decode split pass");
     }
     if (phases & kPhaseReduce) {
-        int red_threads = head_dim < 64 ? 64 : head_dim;
-        if (red_threads > 256) red_threads = 256;
-        ks.reduce<<<dim3((unsigned)(batch * num_q_heads)), dim3(red_threads), 0, s>>>(a);
+        ks.reduce<<<dim3((unsigned)(batch * num_q_heads)), dim3(kThreads), 0, s>>>(a);
         PA_CHECK_LAUNCH("pa_decode reduction pass");
     }
     return PA_OK;

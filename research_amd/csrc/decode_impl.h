@@ -245,7 +245,10 @@ namespace pa_decode_detail {
 // fp32 loop.  Returns the row-group state in the generic form merge_rows takes.
 template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
     using S = RowShape<KV, D>;
-    static constexpr bool kPacked = sizeof(KV) == 2 && std::is_same<KV, QT>::value && (D == 64 || D == 128);
+    // packed loop: 16-bit pools with head_dim 64/128, fp8 pools (16-bit queries) with head_dim 64/128/256
+    static constexpr bool kPacked =
+        (sizeof(KV) == 2 && std::is_same<KV, QT>::value && (D == 64 || D == 128)) ||
+        (sizeof(KV) == 1 && sizeof(QT) == 2 && (D == 64 || D == 128 || D == 256));
 
     static __device__ __forceinline__ RowState<NREP, S::EPL> run(const PoolArgs &p, const QT *qrow,
                                                                   const int32_t *bt_row, int L, int blk_begin,
@@ -253,25 +256,30 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
                                                                   int lane, int kvh, int rep0) {
         RowState<NREP, S::EPL> out;
         if constexpr (kPacked) {
-            using HS = HeadScatter<NREP, D / 8>;
-            uint32_t qpk[NREP][4];
+            using HS = HeadScatter<NREP, S::LPR>;
+            constexpr int NW = S::EPL / 2;  // packed pairs per lane
+            uint32_t qpk[NREP][NW];
 #pragma unroll
             for (int r = 0; r < NREP; ++r) {
                 const bool live = rep0 + r < p.n_rep;
-                const uint4 raw = live ? ld16(qrow + ((int64_t)kvh * p.n_rep + rep0 + r) * D + role.d0)
-                                       : uint4{0, 0, 0, 0};
-                qpk[r][0] = raw.x; qpk[r][1] = raw.y; qpk[r][2] = raw.z; qpk[r][3] = raw.w;
+                const QT *qp = qrow + ((int64_t)kvh * p.n_rep + rep0 + r) * D + role.d0;
+#pragma unroll
+                for (int i = 0; i < NW; i += 4) {
+                    const uint4 raw = live ? ld16(qp + 2 * i) : uint4{0, 0, 0, 0};
+                    qpk[r][i] = raw.x; qpk[r][i + 1] = raw.y; qpk[r][i + 2] = raw.z; qpk[r][i + 3] = raw.w;
+                }
             }
-            PkState<NREP, HS::VPL> st;
+            PkState<NREP, HS::VPL, S::EPL> st;
             st.init();
-            const int lane_voff = role.tok_local * (p.hkv * D * 2) + kvh * (D * 2) + role.lir * 16;
-            attend_blocks_pk<KV, D, NREP, U>(st, qpk, p, bt_row, L, blk_begin, blk_end, blk_step, lane, lane_voff,
-                                             role.tok_local == 0);
+            const int lane_voff =
+                role.tok_local * (p.hkv * D * (int)sizeof(KV)) + kvh * (D * (int)sizeof(KV)) + role.lir * 16;
+            attend_blocks_pk<KV, QT, D, NREP, U>(st, qpk, p, bt_row, L, blk_begin, blk_end, blk_step, lane, lane_voff,
+                                                 kvh, role.tok_local == 0);
             StaticFor<NREP>::run([&](auto h) {
                 out.m[h.value] = HS::template bcast<h.value>(st.m);
                 out.l[h.value] = HS::template bcast<h.value>(st.l);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) out.acc[h.value][e] = st.acc[h.value][e];
+                for (int e = 0; e < S::EPL; ++e) out.acc[h.value][e] = st.acc[h.value][e];
             });
             out.zero_keys = st.zero_keys;
         } else {
@@ -447,11 +455,16 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
     }
 }
 
-// Reduction pass: one workgroup per (sequence, query head), thread d owns
-// out[d].  Rows the split pass finished in place are skipped; empty sequences
-// get their zeros (or the all-zero-keys result) here.
+// Reduction pass: one workgroup of 4 waves per (sequence, query head).  The
+// pieces of the sequence are dealt round-robin to the waves (a long sequence in
+// a small batch has one piece per workgroup of the split pass), each wave
+// merges its pieces online with lanes across d, and the four wave results are
+// merged through LDS.  Rows the split pass finished in place are skipped;
+// empty sequences get their zeros here.
 template <typename QT, int D, int NREP>
-__global__ void decode_reduce_kernel(const DecodeArgs a) {
+__global__ __launch_bounds__(kThreads) void decode_reduce_kernel(const DecodeArgs a) {
+    constexpr int DPL = (D + PA_WAVE - 1) / PA_WAVE;  // d values per lane
+    __shared__ float s_w[kWaves][D + 2];
     const PoolArgs &p = a.p;
     const int hq = p.hq;
     const int b = blockIdx.x / hq;
@@ -464,9 +477,10 @@ __global__ void decode_reduce_kernel(const DecodeArgs a) {
     const int64_t total = per_plane * p.n_hgroups * p.n_rgroups;
     const int nblk = a.block_prefix[b + 1] - a.block_prefix[b];
     const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
+    const int lane = threadIdx.x & (PA_WAVE - 1), wave = threadIdx.x / PA_WAVE;
     QT *orow = reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * D;
     if (nblk == 0) {
-        for (int d = threadIdx.x; d < D; d += blockDim.x) pa_scalar<QT>::store(orow + d, 0.f);
+        for (int d = threadIdx.x; d < D; d += kThreads) pa_scalar<QT>::store(orow + d, 0.f);
         return;
     }
     const int64_t u0 = plane * per_plane + a.block_prefix[b];
@@ -479,19 +493,42 @@ __global__ void decode_reduce_kernel(const DecodeArgs a) {
         return unit_begin(w, total, a.split_grid) < unit_begin((int64_t)w + 1, total, a.split_grid) &&
                w + key < a.slot_cap;
     };
-    float M = kNegBig;
-    for (int w = w0; w <= w1; ++w)
-        if (has_piece(w)) M = fmaxf(M, a.part_ml[(w + key) * stride_ml + idx * 2]);
-    for (int d = threadIdx.x; d < D; d += blockDim.x) {
-        float num = 0.f, den = 0.f;
-        for (int w = w0; w <= w1; ++w) {
-            if (!has_piece(w)) continue;
-            const int64_t slot = w + key;
-            const float wgt = __builtin_amdgcn_exp2f(a.part_ml[slot * stride_ml + idx * 2] - M);
-            num = fmaf(wgt, a.part_acc[slot * stride_acc + idx * D + d], num);
-            den = fmaf(wgt, a.part_ml[slot * stride_ml + idx * 2 + 1], den);
+    float M = kNegBig, den = 0.f, num[DPL];
+#pragma unroll
+    for (int k = 0; k < DPL; ++k) num[k] = 0.f;
+    for (int w = w0 + wave; w <= w1; w += kWaves) {
+        if (!has_piece(w)) continue;
+        const int64_t slot = w + key;
+        const float m = a.part_ml[slot * stride_ml + idx * 2], l = a.part_ml[slot * stride_ml + idx * 2 + 1];
+        const float mn = fmaxf(M, m);
+        const float so = __builtin_amdgcn_exp2f(M - mn), sn = __builtin_amdgcn_exp2f(m - mn);
+        den = den * so + l * sn;
+#pragma unroll
+        for (int k = 0; k < DPL; ++k) {
+            const int d = lane + PA_WAVE * k;
+            const float x = d < D ? a.part_acc[slot * stride_acc + idx * D + d] : 0.f;
+            num[k] = num[k] * so + x * sn;
         }
-        pa_scalar<QT>::store(orow + d, finish_row(num, M, den, ez));
+        M = mn;
+    }
+#pragma unroll
+    for (int k = 0; k < DPL; ++k)
+        if (lane + PA_WAVE * k < D) s_w[wave][lane + PA_WAVE * k] = num[k];
+    if (lane == 0) {
+        s_w[wave][D] = M;
+        s_w[wave][D + 1] = den;
+    }
+    __syncthreads();
+    for (int d = threadIdx.x; d < D; d += kThreads) {
+        float Mt = kNegBig;
+        for (int w = 0; w < kWaves; ++w) Mt = fmaxf(Mt, s_w[w][D]);
+        float n = 0.f, dn = 0.f;
+        for (int w = 0; w < kWaves; ++w) {
+            const float wgt = __builtin_amdgcn_exp2f(s_w[w][D] - Mt);
+            n = fmaf(wgt, s_w[w][d], n);
+            dn = fmaf(wgt, s_w[w][D + 1], dn);
+        }
+        pa_scalar<QT>::store(orow + d, finish_row(n, Mt, dn, ez));
     }
 }
 

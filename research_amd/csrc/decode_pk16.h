@@ -1,5 +1,8 @@
-// Packed 16-bit inner loop of single-query-row paged attention (bf16 / fp16
-// pools, head_dim 64 or 128) for gfx950.
+// Packed inner loop of single-query-row paged attention for gfx950: bf16 / fp16
+// pools (head_dim 64, 128) and fp8-e4m3 pools with bf16 / fp16 queries
+// (head_dim 64, 128, 256).  An fp8 pool is widened two elements at a time to
+// the query type (v_cvt_scalef32_pk_*_fp8, exact) and then runs the same
+// 16-bit arithmetic; its per-(block, head) scales multiply the logit and p.
 //
 // The generic loop converts every K/V element to fp32 and spends most of its
 // issue slots on conversions, per-head cross-lane sums and redundant softmax
@@ -50,6 +53,35 @@ template <> struct Pk16<pa_f16> {
     }
 };
 
+// How the 16 bytes a lane loads turn into packed pairs of the arithmetic type AT.
+template <typename KV, typename AT> struct PoolWords;
+template <typename AT> struct PoolWords<AT, AT> {  // 16-bit pool: the raw dwords are the pairs
+    static constexpr int NW = 4;
+    static __device__ __forceinline__ void unpack(const pa_u4 &raw, uint32_t (&w)[NW]) {
+        w[0] = raw[0]; w[1] = raw[1]; w[2] = raw[2]; w[3] = raw[3];
+    }
+};
+template <> struct PoolWords<pa_fp8, pa_bf16> {
+    static constexpr int NW = 8;
+    static __device__ __forceinline__ void unpack(const pa_u4 &raw, uint32_t (&w)[NW]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            w[2 * i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw[i], 1.0f, false));
+            w[2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw[i], 1.0f, true));
+        }
+    }
+};
+template <> struct PoolWords<pa_fp8, pa_f16> {
+    static constexpr int NW = 8;
+    static __device__ __forceinline__ void unpack(const pa_u4 &raw, uint32_t (&w)[NW]) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            w[2 * i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[i], 1.0f, false));
+            w[2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[i], 1.0f, true));
+        }
+    }
+};
+
 template <int CTRL, int BANKS = 0xf> __device__ __forceinline__ float dpp_mov(float old, float x) {
     return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, old),
                                                                  __builtin_bit_cast(int, x), CTRL, 0xf, BANKS, false));
@@ -62,7 +94,7 @@ template <int CTRL> __device__ __forceinline__ uint32_t dpp_mov_u(uint32_t x) {
 // After reduce(): a lane at quad position c = lane & 3 owns VPL totals, those
 // of heads head_base(c) .. head_base(c)+VPL-1.
 template <int NREP, int LPR> struct HeadScatter {
-    static_assert(LPR == 8 || LPR == 16, "rows of 8 or 16 lanes");
+    static_assert(LPR == 4 || LPR == 8 || LPR == 16, "rows of 4, 8 or 16 lanes");
     static constexpr int SC = NREP >= 4 ? 2 : (NREP == 2 ? 1 : 0);  // scatter steps (xor 1, xor 2)
     static constexpr int VPL = NREP >> SC;                            // values a lane keeps
 
@@ -99,7 +131,7 @@ template <int NREP, int LPR> struct HeadScatter {
             if (LPR == 16) {
                 out[i] += dpp_mov<0x124>(0.f, out[i]);  // row_ror:4
                 out[i] += dpp_mov<0x128>(0.f, out[i]);  // row_ror:8
-            } else {
+            } else if (LPR == 8) {
                 // partner quad inside the row of 8: from 4 lanes below for banks 1,3, from 4 lanes above for banks 0,2
                 float other = dpp_mov<0x114, 0xa>(0.f, out[i]);   // row_shr:4
                 other = dpp_mov<0x104, 0x5>(other, out[i]);       // row_shl:4
@@ -124,9 +156,9 @@ template <int NREP, int LPR> struct HeadScatter {
     }
 };
 
-template <int NREP, int VPL> struct PkState {
+template <int NREP, int VPL, int EPL> struct PkState {
     float m[VPL], l[VPL];
-    float acc[NREP][8];
+    float acc[NREP][EPL];
     int zero_keys;
     __device__ __forceinline__ void init() {
 #pragma unroll
@@ -134,7 +166,7 @@ template <int NREP, int VPL> struct PkState {
 #pragma unroll
         for (int r = 0; r < NREP; ++r)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[r][e] = 0.f;
+            for (int e = 0; e < EPL; ++e) acc[r][e] = 0.f;
         zero_keys = 0;
     }
 };
@@ -150,18 +182,22 @@ template <> struct StaticFor<0> {
 };
 
 // Attend keys [0, L) of blocks blk_begin, blk_begin+blk_step, ... < blk_end.
-// qpk[r][i]: raw 16-bit pairs of this lane's 8 query elements of head r.
-template <typename KV, int D, int NREP, int U>
-__device__ __forceinline__ void attend_blocks_pk(PkState<NREP, HeadScatter<NREP, D / 8>::VPL> &st,
-                                                 const uint32_t (&qpk)[NREP][4], const PoolArgs &p,
-                                                 const int32_t *bt_row, int L, int blk_begin, int blk_end,
-                                                 int blk_step, int lane, int lane_voff, bool count_zero_keys) {
+// qpk[r][i]: packed pairs of this lane's query elements of head r (raw bits of the query type AT).
+// lane_kvh: the kv head this lane's row belongs to (selects the fp8 scales).
+template <typename KV, typename AT, int D, int NREP, int U>
+__device__ __forceinline__ void attend_blocks_pk(
+    PkState<NREP, HeadScatter<NREP, D * (int)sizeof(KV) / 16>::VPL, 2 * PoolWords<KV, AT>::NW> &st,
+    const uint32_t (&qpk)[NREP][PoolWords<KV, AT>::NW], const PoolArgs &p, const int32_t *bt_row, int L, int blk_begin,
+    int blk_end, int blk_step, int lane, int lane_voff, int lane_kvh, bool count_zero_keys) {
     static_assert(U % 2 == 0, "tokens are consumed in pairs");
-    constexpr int LPR = D / 8;
+    constexpr int LPR = D * (int)sizeof(KV) / 16;
+    constexpr bool kFp8 = sizeof(KV) == 1;
     using HS = HeadScatter<NREP, LPR>;
-    using PK = Pk16<KV>;
+    using PK = Pk16<AT>;
+    using PW = PoolWords<KV, AT>;
+    constexpr int NW = PW::NW;
     constexpr int VPL = HS::VPL;
-    const int tok_stride = p.hkv * D * 2;  // bytes between tokens
+    const int tok_stride = p.hkv * D * (int)sizeof(KV);  // bytes between tokens
     const int tok_local = (lane / LPR) / p.hpw;
 
     for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
@@ -177,6 +213,11 @@ __device__ __forceinline__ void attend_blocks_pk(PkState<NREP, HeadScatter<NREP,
             (void *)(reinterpret_cast<const char *>(p.k) + block_off), 0, ntok * tok_stride, 0x00020000);
         const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
             (void *)(reinterpret_cast<const char *>(p.v) + block_off), 0, ntok * tok_stride, 0x00020000);
+        float k_sc = p.scale_log2, v_sc = 1.f;  // logit scale (with the K scale folded in) and V scale of this block
+        if (kFp8) {
+            k_sc *= p.k_scale[bid * p.hkv + lane_kvh];
+            v_sc = p.v_scale[bid * p.hkv + lane_kvh];
+        }
 
         for (int t0 = 0; t0 < ntok; t0 += p.tpw * U) {
             pa_u4 kraw[U], vraw[U];
@@ -192,17 +233,19 @@ __device__ __forceinline__ void attend_blocks_pk(PkState<NREP, HeadScatter<NREP,
             const bool partial = ntok - t0 < p.tpw * U;  // uniform
 #pragma unroll
             for (int u = 0; u < U; ++u) {
+                uint32_t kw[NW];
+                PW::unpack(kraw[u], kw);
                 float s[NREP];
 #pragma unroll
                 for (int r = 0; r < NREP; ++r) {
-                    float d = PK::dot2(kraw[u][0], qpk[r][0], 0.f);
-                    d = PK::dot2(kraw[u][1], qpk[r][1], d);
-                    d = PK::dot2(kraw[u][2], qpk[r][2], d);
-                    s[r] = PK::dot2(kraw[u][3], qpk[r][3], d);
+                    float d = PK::dot2(kw[0], qpk[r][0], 0.f);
+#pragma unroll
+                    for (int i = 1; i < NW; ++i) d = PK::dot2(kw[i], qpk[r][i], d);
+                    s[r] = d;
                 }
                 HS::reduce(s, sv[u], lane);
 #pragma unroll
-                for (int j = 0; j < VPL; ++j) sv[u][j] *= p.scale_log2;
+                for (int j = 0; j < VPL; ++j) sv[u][j] *= k_sc;
                 if (partial) {
                     const bool ok = t0 + u * p.tpw + tok_local < ntok;
 #pragma unroll
@@ -230,7 +273,7 @@ __device__ __forceinline__ void attend_blocks_pk(PkState<NREP, HeadScatter<NREP,
                 StaticFor<NREP>::run([&](auto h) {
                     const float a = HS::template bcast<h.value>(alpha);
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) st.acc[h.value][e] *= a;
+                    for (int e = 0; e < 2 * NW; ++e) st.acc[h.value][e] *= a;
                 });
             }
             // ---- p.v, two tokens per step ----------------------------------
@@ -242,18 +285,21 @@ __device__ __forceinline__ void attend_blocks_pk(PkState<NREP, HeadScatter<NREP,
                     const float p0 = __builtin_amdgcn_exp2f(sv[u][j] - st.m[j]);  // 0 for masked tokens
                     const float p1 = __builtin_amdgcn_exp2f(sv[u + 1][j] - st.m[j]);
                     st.l[j] += p0 + p1;
-                    ppk[j] = PK::pack(p0, p1);
+                    ppk[j] = kFp8 ? PK::pack(p0 * v_sc, p1 * v_sc) : PK::pack(p0, p1);
                 }
-                uint32_t lo[4], hi[4];  // (v_t0[2i], v_t1[2i]) and (v_t0[2i+1], v_t1[2i+1])
+                uint32_t v0[NW], v1[NW];
+                PW::unpack(vraw[u], v0);
+                PW::unpack(vraw[u + 1], v1);
+                uint32_t lo[NW], hi[NW];  // (v_t0[2i], v_t1[2i]) and (v_t0[2i+1], v_t1[2i+1])
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    lo[i] = __builtin_amdgcn_perm(vraw[u + 1][i], vraw[u][i], 0x05040100u);
-                    hi[i] = __builtin_amdgcn_perm(vraw[u + 1][i], vraw[u][i], 0x07060302u);
+                for (int i = 0; i < NW; ++i) {
+                    lo[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x05040100u);
+                    hi[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x07060302u);
                 }
                 StaticFor<NREP>::run([&](auto h) {
                     const uint32_t pb = HS::template bcast_u<h.value>(ppk);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
+                    for (int i = 0; i < NW; ++i) {
                         st.acc[h.value][2 * i] = PK::dot2(lo[i], pb, st.acc[h.value][2 * i]);
                         st.acc[h.value][2 * i + 1] = PK::dot2(hi[i], pb, st.acc[h.value][2 * i + 1]);
                     }
