@@ -68,7 +68,8 @@ template <> struct Mfma16<pa_f16> {
     static __device__ __forceinline__ uint32_t pack(float lo, float hi) { return Pk16<pa_f16>::pack(lo, hi); }
 };
 
-constexpr int kPfKeys = 64;   // keys per K/V tile
+constexpr int kPfKeys = 128;  // keys per K/V tile
+constexpr int kPfSub = kPfKeys / 32;  // 32-key subtiles per tile
 constexpr int kPfRows = 32;   // query rows per wave
 constexpr int kPfWaves = 8;
 constexpr int kPfThreads = kPfWaves * 64;
@@ -78,7 +79,7 @@ template <int D> struct PfTile {
     static constexpr int RB = D * 2;            // row bytes
     static constexpr int CPR = D / 8;           // 16-byte chunks per row
     static constexpr int RPL = 64 / CPR;        // rows one wave-wide direct load covers
-    static constexpr int LOADS = CPR;           // wave-wide direct loads per tile and tensor
+    static constexpr int LOADS = kPfKeys / RPL;  // wave-wide direct loads per tile and tensor
     static constexpr int BYTES = kPfKeys * RB;  // one tensor's tile
     static constexpr int RDIV = 16 / CPR;       // rows that share a 256-byte bank line
     // K: 16 consecutive rows read the same chunk -> 16 distinct 16-byte bank groups
@@ -172,7 +173,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
             if (l >= G::LOADS) continue;
             int blk;
             if (BS16) {
-                blk = tile * 4 + (l * G::RPL) / 16;  // uniform: the load's rows lie in one pool block
+                blk = tile * (kPfKeys / 16) + (l * G::RPL) / 16;  // uniform: the load's rows lie in one pool block
             } else {
                 const int key = tile * kPfKeys + l * G::RPL + ld_row;
                 blk = key < ctx_len ? key / p.bs : -1;
@@ -224,9 +225,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     for (int dt = 0; dt < DT; ++dt)
         v_ofs[dt] = v_key * G::RB + ((((4 * dt) ^ G::swz_v(v_key)) + 2 * (g16 & 1) + ((s16 & 3) >> 1)) * 16) + 8 * (s16 & 1);
 
-    // one 32-key subtile of the current tile for this wave's 32 rows
-    auto subtile = [&](const char *tk, const char *tv, int key_base, bool need_mask) {
-        // ---- S^T = K . Q^T ----
+    // S^T = K . Q^T for one 32-key subtile (this wave's 32 rows)
+    auto s_phase = [&](const char *tk) {
         f32x16 s;
 #pragma unroll
         for (int i = 0; i < 16; ++i) s[i] = 0.f;
@@ -240,6 +240,13 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
 #pragma unroll
             for (int ks = 0; ks < KG; ++ks) s = M::mma(ka[ks], qreg[k0 + ks], s);
         }
+        return s;
+    };
+
+    // Softmax and O^T update of one subtile whose S^T is `s`.  When there is a next subtile in the tile its
+    // S^T products are issued here, between the running-maximum step and the exponentials, so that the matrix
+    // unit works while this wave's vector ALU does the exp / sum / pack arithmetic.
+    auto subtile = [&](f32x16 s, const char *tk_next, const char *tv, int key_base, bool need_mask, bool has_next) {
         // V^T operands of the first k-step are requested before the softmax arithmetic
         X4 vlo[DT], vhi[DT];
 #pragma unroll
@@ -268,6 +275,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
             m_raw = m_new;
             m_sc = m_new * c;
         }
+        f32x16 s_next = s;
+        if (has_next) s_next = s_phase(tk_next);
         uint32_t pp[8];
         float sum = 0.f;
 #pragma unroll
@@ -298,6 +307,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) o[dt] = M::mma(va[dt], pb, o[dt]);
         }
+        return s_next;
     };
 
     // one K/V tile: wait for it, start the next one into the other buffer, multiply
@@ -312,9 +322,11 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         if (key0 < my_keys) {  // else this wave's rows end before this tile (uniform per wave)
             // masking is needed only where the tile reaches past the first row's causal limit or the context end
             const bool need_mask = key0 + kPfKeys > prefix + row0 + 1 || key0 + kPfKeys > ctx_len;
+            f32x16 s = s_phase(cur_k);
 #pragma unroll
-            for (int kt = 0; kt < 2; ++kt)
-                subtile(cur_k + kt * 32 * G::RB, cur_v + kt * 32 * G::RB, key0 + 32 * kt, need_mask);
+            for (int kt = 0; kt < kPfSub; ++kt)
+                s = subtile(s, cur_k + (kt + 1) * 32 * G::RB, cur_v + kt * 32 * G::RB, key0 + 32 * kt, need_mask,
+                            kt + 1 < kPfSub);
         }
     };
     lookup(0);
