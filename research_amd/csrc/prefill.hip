@@ -47,7 +47,7 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     if (mfma) {
         PA_REQUIRE(pa_aligned16(q) && pa_aligned16(out), "q and out must be 16-byte aligned");
         const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
-        const int groups = (row_blocks * a.p.n_rep + kPfWaves - 1) / kPfWaves;
+        const int groups = (row_blocks * a.p.n_rep + kPfTasks - 1) / kPfTasks;
         PA_REQUIRE(groups <= 65535, "max_q_len=%d is too long for one launch", max_q_len);
         mfma<<<dim3((unsigned)num_kv_heads, (unsigned)groups, (unsigned)batch), dim3(kPfThreads), 0, s>>>(a);
         PA_CHECK_LAUNCH("pa_prefill_paged (matrix-core kernel)");
