@@ -68,8 +68,9 @@ template <> struct Mfma16<pa_f16> {
     static __device__ __forceinline__ uint32_t pack(float lo, float hi) { return Pk16<pa_f16>::pack(lo, hi); }
 };
 
-constexpr int kPfKeys = 128;  // keys per K/V tile
+constexpr int kPfKeys = 64;   // keys per K/V tile
 constexpr int kPfSub = kPfKeys / 32;  // 32-key subtiles per tile
+constexpr int kPfStages = 4;  // K/V tiles held in LDS (a ring)
 constexpr int kPfRows = 32;   // query rows per task (one MFMA column tile)
 constexpr int kPfCols = 2;    // tasks (column tiles) per wave
 constexpr int kPfWaves = 4;
@@ -99,9 +100,40 @@ __device__ __forceinline__ const char *pf_scalar_ptr(const char *ptr) {
     return reinterpret_cast<const char *>(((uint64_t)hi << 32) | lo);
 }
 
+// Direct global -> LDS load of 16 bytes per lane: lane i's bytes land at LDS address lds_dst + 16*i.
+// Issued as inline assembly on purpose.  The compiler cannot tell which LDS bytes such a load writes when
+// the destination is computed, and would make every later LDS read wait for all loads in flight - the
+// opposite of prefetching.  The kernel below waits for these loads itself (pf_wait_loads) before the
+// barrier that publishes a tile.
+__device__ __forceinline__ void pf_dma16(uint32_t lds_dst, const char *scalar_base, uint32_t lane_ofs) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_dst), "v"(lane_ofs), "s"(scalar_base)
+                 : "memory", "m0");
+}
+__device__ __forceinline__ void pf_dma16(uint32_t lds_dst, const char *lane_ptr) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_dst), "v"(lane_ptr) : "memory", "m0");
+}
+// One table entry per lane, loaded behind the compiler's back like the tile loads (a load the compiler knows
+// about would make it wait for ALL loads in flight wherever it cannot prove the value has arrived); the
+// caller waits with pf_wait_loads<0>() before the value is used.
+__device__ __forceinline__ int pf_load_i32(const int32_t *lane_ptr) {
+    int v;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(lane_ptr) : "memory");
+    return v;
+}
+// Wait until at most N of this wave's vector memory loads are outstanding (they complete in order).
+template <int N> __device__ __forceinline__ void pf_wait_loads() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));  // expcnt / lgkmcnt: no wait
+}
+
+template <bool B> struct PfBool { static constexpr bool value = B; };
+
 // Nothing may be moved across this point by the instruction scheduler: the order of the groups of matrix,
 // vector and LDS instructions written below is the order they issue in.
 #define PF_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define PF_INLINE __attribute__((always_inline))
 
 template <typename T, int D, bool BS16>
 __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseArgs a) {
@@ -112,12 +144,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     constexpr int KS = D / 16;  // k-steps of the first product
     constexpr int DT = D / 32;  // 32-wide d tiles of the second product
     constexpr int NC = kPfCols;
-    // Two K/V tile buffers as four separate LDS objects: the compiler then knows that a direct load into one
-    // buffer cannot alias the operand reads from the other and does not make the reads wait for the load.
-    __shared__ __attribute__((aligned(1024))) char s_k0[G::BYTES];
-    __shared__ __attribute__((aligned(1024))) char s_v0[G::BYTES];
-    __shared__ __attribute__((aligned(1024))) char s_k1[G::BYTES];
-    __shared__ __attribute__((aligned(1024))) char s_v1[G::BYTES];
+    typedef __attribute__((address_space(3))) char lds_char;
+    // Ring of kPfStages K/V tiles: stage s holds K at s*2*BYTES and V behind it.
+    __shared__ __attribute__((aligned(1024))) char s_kv[kPfStages * 2 * G::BYTES];
+    const uint32_t lds_base = (uint32_t)(size_t)(lds_char *)s_kv;
 
     const PoolArgs &p = a.p;
     const int tid = threadIdx.x;
@@ -150,6 +180,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         my_keys[c] = live[c] ? min(ctx_len, prefix + min(q_len, row0[c] + kPfRows)) : 0;  // keys [0, my_keys)
     }
     const int wave_keys = max(my_keys[0], my_keys[1]);
+    const int n_sub = (wave_keys + 31) / 32;  // 32-key subtiles this wave multiplies
+    const int mask_from = min(prefix + min(row0[0], row0[1]) + 1, ctx_len);  // subtiles reaching past this key are masked
     const int last_task = min(n_tasks, task0 + kPfTasks) - 1;
     const int wg_keys = min(ctx_len, prefix + min(q_len, (last_task / p.n_rep) * kPfRows + kPfRows));
     const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys;
@@ -168,6 +200,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         }
     }
 
+    // (used here, so that the compiler waits for them here and knows inside the loop that they have arrived)
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qreg[c][ks]));  // (product operands live in AGPRs)
+
     f32x16 o[NC][DT];
 #pragma unroll
     for (int c = 0; c < NC; ++c)
@@ -175,13 +213,13 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) o[c][dt][i] = 0.f;
-    // running maximum of the raw (unscaled) logits, the same times scale*log2e, and the running sum
-    const float sc = p.scale_log2;
+    // Running maximum of the raw (unscaled) logits, the same times scale*log2e, and the running sum.
     // The reference maximum of a row is allowed to lag behind the true running maximum by up to 2^kPfSlack
     // (as a factor on the probabilities): sums and accumulators are rescaled only when a row's maximum grows
     // by more than that, which it rarely does, instead of on nearly every subtile.  The result is the same
     // quotient either way; probabilities stay below 2^kPfSlack, far inside the range of fp32 sums and of the
     // 16-bit operand types.
+    const float sc = p.scale_log2;
     const float slack_raw = kPfSlack / sc;
     float m_raw[NC], m_sc[NC], m_thr[NC], l_run[NC];
 #pragma unroll
@@ -194,15 +232,13 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     const char *pool_v = reinterpret_cast<const char *>(p.v) + (int64_t)kvh * D * 2;
     const int ld_row = lane / G::CPR, ld_slot = lane % G::CPR;
     constexpr int NLW = (G::LOADS + kPfWaves - 1) / kPfWaves;  // direct loads per wave, tile and tensor
-    // Block ids are looked up one tile ahead of the loads that use them, so that the table read (and its
-    // latency) never sits between the barrier and the products.
-    //
+    static_assert(G::LOADS % kPfWaves == 0, "every wave issues the same number of loads");
     // Pools of 16-token blocks: a wave-wide load lies inside one pool block, and the position of a lane's
     // 16 bytes inside that block (token, swizzled chunk) is the same for every load the wave issues.  The
-    // address is then a scalar block base plus one per-lane constant, and the block ids of a tile are one
-    // vector register (lane i holds block i of the tile) read out with v_readlane.
-    constexpr int BPT = kPfKeys / 16;  // pool blocks per tile
-    int bid_vec = -1;
+    // address is then a scalar block base plus one per-lane constant.  Block ids come from a window of 64
+    // table entries (16 tiles) held one per lane and read out with v_readlane.
+    constexpr int BPT = kPfKeys / 16;     // pool blocks per tile
+    constexpr int WIN = 64 / BPT;         // tiles per block-id window
     const int64_t block_bytes = 16 * tok_stride;
     uint32_t lane_k = 0, lane_v = 0;
     if (BS16) {
@@ -211,82 +247,62 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         lane_k = tok_ofs + (uint32_t)((ld_slot ^ G::swz_k(row)) * 16);
         lane_v = tok_ofs + (uint32_t)((ld_slot ^ G::swz_v(row)) * 16);
     }
-    // Other block sizes: per-lane block ids and addresses.
-    int bid_next[BS16 ? 1 : NLW];  // kept as loaded: any arithmetic on it here would wait for the load
-    auto lookup = [&](int tile) __attribute__((always_inline)) {
+    int bid_win = -1;
+    // Loads of one tile into its ring stage.  Returns true if the wave issued exactly 2*NLW direct loads and no
+    // other vector memory operation after them (what the load-count waits below rely on).
+    auto issue = [&](int tile) PF_INLINE -> bool {
+        const uint32_t dst0 = lds_base + (uint32_t)(tile % kPfStages) * 2 * G::BYTES;
         if (BS16) {
-            const int idx = tile * BPT + lane;
-            bid_vec = -1;
-            if (lane < BPT && idx < p.bt_stride && tile * kPfKeys < ctx_len) bid_vec = bt_row[idx];
-            return;
-        }
-#pragma unroll
-        for (int n = 0; n < NLW; ++n) {
-            const int l = n * kPfWaves + wave;  // uniform
-            bid_next[BS16 ? 0 : n] = -1;
-            if (l >= G::LOADS) continue;
-            const int key = tile * kPfKeys + l * G::RPL + ld_row;
-            const int blk = key < ctx_len ? key / p.bs : -1;
-            if (blk >= 0 && blk < p.bt_stride) bid_next[BS16 ? 0 : n] = bt_row[blk];
-        }
-    };
-    auto load_rows = [&](const char *src_k, const char *src_v, char *dst_k, char *dst_v) __attribute__((always_inline)) {
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src_k,
-                                         (__attribute__((address_space(3))) void *)dst_k, 16, 0, 0);
-        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src_v,
-                                         (__attribute__((address_space(3))) void *)dst_v, 16, 0, 0);
-    };
-    auto zero_rows = [&](char *dst_k, char *dst_v) __attribute__((always_inline)) {
-        // past the context end or a missing block: all-zero key and value rows
-        *reinterpret_cast<uint4 *>(dst_k + lane * 16) = uint4{0, 0, 0, 0};
-        *reinterpret_cast<uint4 *>(dst_v + lane * 16) = uint4{0, 0, 0, 0};
-    };
-    auto issue = [&](int tile, char *buf_k, char *buf_v) __attribute__((always_inline)) {
-        if (BS16) {
-            // whole tile inside the context and every block present (the common case): straight-line loads
-            const bool in_pool = lane >= BPT || (bid_vec >= 0 && bid_vec < p.num_blocks);
-            if ((tile + 1) * kPfKeys <= ctx_len && __builtin_amdgcn_ballot_w64(!in_pool) == 0) {
+            if (tile % WIN == 0) {  // next window of block ids (once per 16 tiles: its latency is not hidden)
+                const int idx = tile * BPT + lane;
+                int v = -1;
+                if (idx < p.bt_stride) v = pf_load_i32(bt_row + idx);
+                pf_wait_loads<0>();
+                asm volatile("" : "+v"(v));
+                bid_win = v;
+            }
+            const int first = (tile % WIN) * BPT;  // lane of the window that holds the tile's first block
+            const bool mine = lane >= first && lane < first + BPT;
+            const bool bad = mine && !(bid_win >= 0 && bid_win < p.num_blocks);
+            if ((tile + 1) * kPfKeys <= ctx_len && __builtin_amdgcn_ballot_w64(bad) == 0) {
+                // whole tile inside the context and every block present (the common case): straight-line loads
                 uint32_t lk = lane_k, lv = lane_v;
-                asm volatile("" : "+v"(lk), "+v"(lv));  // 32-bit lane offsets at the point of use: scalar base + offset loads
+                asm volatile("" : "+v"(lk), "+v"(lv));
 #pragma unroll
                 for (int n = 0; n < NLW; ++n) {
                     const int l = n * kPfWaves + wave;  // uniform
-                    if (G::LOADS % kPfWaves != 0 && l >= G::LOADS) break;
-                    const uint32_t bid = (uint32_t)__builtin_amdgcn_readlane(bid_vec, (l * G::RPL) / 16);
+                    const uint32_t bid = (uint32_t)__builtin_amdgcn_readlane(bid_win, first + (l * G::RPL) / 16);
                     const uint64_t ofs = (uint64_t)bid * (uint32_t)block_bytes;  // 32 x 32 -> 64 bits on the scalar unit
-                    // (read back through the scalar unit so that the base stays apart from the lane offset)
-                    const char *base_k = pf_scalar_ptr(pool_k + ofs);
-                    const char *base_v = pf_scalar_ptr(pool_v + ofs);
-                    load_rows(base_k + lk, base_v + lv, buf_k + l * G::RPL * G::RB, buf_v + l * G::RPL * G::RB);
+                    pf_dma16(dst0 + l * G::RPL * G::RB, pf_scalar_ptr(pool_k + ofs), lk);
+                    pf_dma16(dst0 + G::BYTES + l * G::RPL * G::RB, pf_scalar_ptr(pool_v + ofs), lv);
                 }
-                return;
+                return true;
             }
         }
+        // tile with rows past the context end or missing blocks, or another block size: per-lane addresses
 #pragma unroll
         for (int n = 0; n < NLW; ++n) {
             const int l = n * kPfWaves + wave;  // uniform
-            if (l >= G::LOADS) break;
-            char *dst_k = buf_k + l * G::RPL * G::RB;  // uniform; lane i lands at +16*i
-            char *dst_v = buf_v + l * G::RPL * G::RB;
+            const uint32_t dst_k = dst0 + l * G::RPL * G::RB, dst_v = dst_k + G::BYTES;
             const int row = l * G::RPL + ld_row;  // row of the tile this lane fills
             const int key = tile * kPfKeys + row;
+            int64_t bid = -1;
             if (BS16) {
-                const int64_t bid = __builtin_amdgcn_readlane(bid_vec, (l * G::RPL) / 16);  // uniform
-                if (key < ctx_len && bid >= 0 && bid < p.num_blocks)
-                    load_rows(pool_k + bid * block_bytes + lane_k, pool_v + bid * block_bytes + lane_v, dst_k, dst_v);
-                else
-                    zero_rows(dst_k, dst_v);
+                bid = __builtin_amdgcn_readlane(bid_win, (tile % WIN) * BPT + (l * G::RPL) / 16);
+            } else if (key < ctx_len && key / p.bs < p.bt_stride) {
+                bid = bt_row[key / p.bs];
+            }
+            if (key < ctx_len && bid >= 0 && bid < p.num_blocks) {
+                const int64_t off = (bid * p.bs + key % p.bs) * tok_stride;
+                pf_dma16(dst_k, pool_k + off + ((ld_slot ^ G::swz_k(row)) * 16));
+                pf_dma16(dst_v, pool_v + off + ((ld_slot ^ G::swz_v(row)) * 16));
             } else {
-                const int64_t bid = bid_next[BS16 ? 0 : n];  // sign-extended only now, one tile after it was loaded
-                if (key < ctx_len && bid >= 0 && bid < p.num_blocks) {
-                    const int64_t off = (bid * p.bs + key % p.bs) * tok_stride;
-                    load_rows(pool_k + off + ((ld_slot ^ G::swz_k(row)) * 16), pool_v + off + ((ld_slot ^ G::swz_v(row)) * 16),
-                              dst_k, dst_v);
-                } else {
-                    zero_rows(dst_k, dst_v);
-                }
+                // past the context end or a missing block: all-zero key and value rows
+                *reinterpret_cast<uint4 *>(s_kv + (dst_k - lds_base) + lane * 16) = uint4{0, 0, 0, 0};
+                *reinterpret_cast<uint4 *>(s_kv + (dst_v - lds_base) + lane * 16) = uint4{0, 0, 0, 0};
             }
         }
+        return false;
     };
 
     // ---- per-lane byte offsets of the operand reads inside a tile ----
@@ -302,19 +318,28 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     for (int dt = 0; dt < DT; ++dt)
         v_ofs[dt] = v_key * G::RB + ((((4 * dt) ^ G::swz_v(v_key)) + 2 * (g16 & 1) + ((s16 & 3) >> 1)) * 16) + 8 * (s16 & 1);
 
-    // LDS addresses are handled as 32-bit integers: a tile's base is added to the per-lane offsets once per
-    // tile, and every operand read of the tile is that register plus an immediate offset.
-    typedef __attribute__((address_space(3))) char lds_char;
-    auto lds_addr = [&](char *ptr) __attribute__((always_inline)) { return (uint32_t)(size_t)(lds_char *)ptr; };
-    // K operands of the 32-key subtile `kt` (shared by the wave's column tiles)
-    auto read_k = [&](const uint32_t (&k_adr)[KS], int kt, X8 (&ka)[KS]) __attribute__((always_inline)) {
+    // LDS addresses are 32-bit integers: a tile's stage base is added to the per-lane offsets once per tile,
+    // and every operand read of the tile is that register plus an immediate offset.
+    uint32_t k_adr[KS], v_adr[DT];
+    auto set_k_tile = [&](int tile) PF_INLINE {
+        const uint32_t base = lds_base + (uint32_t)(tile % kPfStages) * 2 * G::BYTES;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) { k_adr[ks] = base + k_ofs[ks]; asm volatile("" : "+v"(k_adr[ks])); }
+    };
+    auto set_v_tile = [&](int tile) PF_INLINE {
+        const uint32_t base = lds_base + (uint32_t)(tile % kPfStages) * 2 * G::BYTES + G::BYTES;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) { v_adr[dt] = base + v_ofs[dt]; asm volatile("" : "+v"(v_adr[dt])); }
+    };
+    // K operands of the 32-key subtile `kt` of the tile k_adr points at (shared by the wave's column tiles)
+    auto read_k = [&](int kt, X8 (&ka)[KS]) PF_INLINE {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
             ka[ks] = __builtin_bit_cast(X8, *reinterpret_cast<const __attribute__((address_space(3))) uint4 *>(
                                                 (const lds_char *)(size_t)k_adr[ks] + kt * 32 * G::RB));
     };
-    // V^T operands of k-step ks2 of subtile kt (keys 32*kt + 16*ks2 .. +16)
-    auto read_v = [&](const uint32_t (&v_adr)[DT], int kt, int ks2, X8 (&va)[DT]) __attribute__((always_inline)) {
+    // V^T operands of k-step ks2 of subtile kt (keys 32*kt + 16*ks2 .. +16) of the tile v_adr points at
+    auto read_v = [&](int kt, int ks2, X8 (&va)[DT]) PF_INLINE {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
             const lds_char *base = (const lds_char *)(size_t)v_adr[dt] + (32 * kt + 16 * ks2) * G::RB;
@@ -326,7 +351,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         }
     };
     // causal / context-end mask of S^T
-    auto mask_s = [&](f32x16 (&s)[NC], int key_base) __attribute__((always_inline)) {
+    auto mask_s = [&](f32x16 (&s)[NC], int key_base) PF_INLINE {
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int limit = min(ctx_len - 1, prefix + row0[c] + col) - key_base - 4 * half;  // last visible key
@@ -337,7 +362,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     // Row maximum over a subtile's 32 keys, in two pieces (the empty asm statements pin each piece between the
     // scheduling fences around it): the first folds values 0..7, the second values 8..15 and the half of the
     // keys that the other half-wave holds.
-    auto max_piece = [&](f32x16 &s, int h, float &mx) __attribute__((always_inline)) {
+    auto max_piece = [&](f32x16 &s, int h, float &mx) PF_INLINE {
         asm volatile("" : "+v"(s));
         float m = fmaxf(s[8 * h], s[8 * h + 1]);
 #pragma unroll
@@ -352,168 +377,193 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         }
         asm volatile("" : "+v"(mx));
     };
-
-    // One K/V tile.  Per 32-key subtile the issue order is
-    //   (a) S^T products of the NEXT subtile, with the first half of this subtile's exponentials between them,
-    //   (b) first k-step of this subtile's O^T products, with the second half of the exponentials,
-    //   (c) second k-step of the O^T products, with the next subtile's row maxima,
-    // so that the matrix unit always has a product queued while the vector ALU does the softmax arithmetic,
-    // and every LDS operand is requested at least one stage before the product that consumes it.
-    auto do_tile = [&](int tile, char *cur_k, char *cur_v, char *nxt_k, char *nxt_v) __attribute__((always_inline)) {
-        __builtin_amdgcn_s_waitcnt(0);  // this wave's direct loads and zero fills of `tile` have landed
-        __syncthreads();                // ... and everyone's; everyone is also done reading the other buffer
-        if (tile + 1 < n_tiles) {
-            issue(tile + 1, nxt_k, nxt_v);
-            lookup(tile + 2);  // consumed by the next tile's issue()
-        }
-        const int key0 = tile * kPfKeys;
-        if (key0 >= wave_keys) return;  // this wave's rows end before this tile (uniform per wave)
-        // masking is needed only where the tile reaches past a first row's causal limit or the context end
-        const bool need_mask = key0 + kPfKeys > prefix + min(row0[0], row0[1]) + 1 || key0 + kPfKeys > ctx_len;
-
-        uint32_t k_adr[KS], v_adr[DT];
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) { k_adr[ks] = lds_addr(cur_k) + k_ofs[ks]; asm volatile("" : "+v"(k_adr[ks])); }
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) { v_adr[dt] = lds_addr(cur_v) + v_ofs[dt]; asm volatile("" : "+v"(v_adr[dt])); }
-
-        X8 ka[KS], va0[DT], va1[DT];
-        f32x16 s_nx[NC];
-        float mx[NC];
-        // prologue: S^T of the first subtile
-        read_k(k_adr, 0, ka);
-        read_v(v_adr, 0, 0, va0);
-        PF_FENCE();
+    auto s_products = [&](const X8 (&ka)[KS], f32x16 (&s)[NC]) PF_INLINE {
 #pragma unroll
         for (int c = 0; c < NC; ++c)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) s_nx[c][i] = 0.f;
+            for (int i = 0; i < 16; ++i) s[c][i] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-            for (int c = 0; c < NC; ++c) s_nx[c] = M::mma(ka[ks], qreg[c][ks], s_nx[c]);
-        PF_FENCE();
-        read_k(k_adr, 1, ka);
-        PF_FENCE();
-        if (need_mask) mask_s(s_nx, key0);
-#pragma unroll
-        for (int c = 0; c < NC; ++c) { max_piece(s_nx[c], 0, mx[c]); max_piece(s_nx[c], 1, mx[c]); }
-        PF_FENCE();
+            for (int c = 0; c < NC; ++c) s[c] = M::mma(ka[ks], qreg[c][ks], s[c]);
+    };
 
+    // ---- fill the ring: tiles 0 .. kPfStages-2 ----
+    bool counted[kPfStages - 1];  // loads of the tiles in flight, oldest first: issued as a full group of direct loads?
+#pragma unroll
+    for (int i = 0; i < kPfStages - 1; ++i) counted[i] = i < n_tiles ? issue(i) : false;
+    if (counted[1] && counted[2]) pf_wait_loads<4 * NLW>(); else __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();  // tile 0 is visible
+
+    // Software pipeline over the wave's 32-key subtiles g = 0 .. n_sub-1 (tile g/2).  While subtile g is
+    // exponentiated and multiplied into O^T, the S^T products of subtile g+1 run on the matrix unit:
+    //   (a) S^T products of subtile g+1, with the first half of subtile g's exponentials between them,
+    //   (b) first k-step of subtile g's O^T products, with the second half of the exponentials,
+    //   (c) second k-step of the O^T products, with subtile g+1's row maxima.
+    // Every LDS operand is requested at least one stage before the product that consumes it.  Tile t+1 is
+    // published (loads waited for, barrier) in the middle of tile t's first subtile, and the loads of tile
+    // t+3 are issued behind that barrier into the stage tile t-1 occupied.
+    X8 ka[KS], va0[DT], va1[DT];
+    f32x16 sb[2][NC];  // S^T of the current and of the next subtile, swapping roles every subtile
+    float mx[NC] = {kNegBig, kNegBig};
+    if (n_sub > 0) {
+        set_k_tile(0);
+        set_v_tile(0);
+        read_k(0, ka);
+        read_v(0, 0, va0);
+        PF_FENCE();
+        s_products(ka, sb[0]);
+        PF_FENCE();
+        if (n_sub > 1) read_k(1, ka);
+        PF_FENCE();
+        if (32 > mask_from) mask_s(sb[0], 0);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) { max_piece(sb[0][c], 0, mx[c]); max_piece(sb[0][c], 1, mx[c]); }
+        PF_FENCE();
+    }
+
+    // One tile.  STEADY: every subtile of the tile, the one after it and the operand reads for the one after
+    // that exist for this wave, so the body is straight-line code (the compiler then places its LDS waits
+    // exactly; with the run-time conditions below it has to assume the worst over all paths).
+    auto do_tile = [&](int tile, auto steady_tag) PF_INLINE {
+        constexpr bool STEADY = decltype(steady_tag)::value;
 #pragma unroll
         for (int kt = 0; kt < kPfSub; ++kt) {
-            const bool has_next = kt + 1 < kPfSub;
-            f32x16 s[NC];
-#pragma unroll
-            for (int c = 0; c < NC; ++c) s[c] = s_nx[c];
-            // ---- a row's maximum outgrew its reference by more than the slack (rare): rescale ----
-            if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx[0] > m_thr[0] || mx[1] > m_thr[1]) != 0, 0)) {
-#pragma unroll
-                for (int c = 0; c < NC; ++c) {
-                    const float m_new = fmaxf(m_raw[c], mx[c]);
-                    const float alpha = __builtin_amdgcn_exp2f((m_raw[c] - m_new) * sc);
-                    l_run[c] *= alpha;
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) o[c][dt][i] *= alpha;
-                    m_raw[c] = m_new;
-                    m_thr[c] = m_new + slack_raw;
-                    m_sc[c] = m_new * sc;
-                }
-            }
-            PF_FENCE();
-            read_v(v_adr, kt, 1, va1);  // second k-step's V^T: consumed in (c)
-            PF_FENCE();
+            const int g = tile * kPfSub + kt;
+            const bool act = STEADY || g < n_sub;            // uniform per wave
+            const bool has_next = STEADY || g + 1 < n_sub;
+            const bool mask_next = 32 * (g + 2) > mask_from;  // subtile g+1 reaches past the first causal limit
+            static_assert(kPfSub == 2, "the two S^T buffers swap roles once per subtile of a tile");
+            f32x16(&s)[NC] = sb[kt & 1];
+            f32x16(&s_nx)[NC] = sb[(kt + 1) & 1];
             uint32_t pp[NC][8];
             float sum[NC] = {0.f, 0.f};
             // exponentials of the pair of S^T values 2*j, 2*j+1 of column tile c, packed as a P^T operand word
             // (pinned like the maxima above: otherwise the compiler gathers all exponentials behind the products)
-            auto exp_pair = [&](int c, int j) __attribute__((always_inline)) {
-                float x0 = s[c][2 * j], x1 = s[c][2 * j + 1];
-                asm volatile("" : "+v"(x0), "+v"(x1));
-                const float p0 = __builtin_amdgcn_exp2f(fmaf(x0, sc, -m_sc[c]));
-                const float p1 = __builtin_amdgcn_exp2f(fmaf(x1, sc, -m_sc[c]));
+            auto exp_pair = [&](int c, int j) PF_INLINE {
+                float scl = sc;
+                asm volatile("" : "+s"(scl));  // a scalar copy defined here: the arithmetic cannot start earlier
+                const float p0 = __builtin_amdgcn_exp2f(fmaf(s[c][2 * j], scl, -m_sc[c]));
+                const float p1 = __builtin_amdgcn_exp2f(fmaf(s[c][2 * j + 1], scl, -m_sc[c]));
                 sum[c] += p0 + p1;
                 uint32_t w = M::pack(p0, p1);
                 asm volatile("" : "+v"(w), "+v"(sum[c]));
                 pp[c][j] = w;
             };
             // piece n of 16: pieces 0..7 make the operand words of the first k-step, 8..15 of the second
-            auto exp_piece = [&](int n) __attribute__((always_inline)) { exp_pair(n & 1, (n >> 1)); };
-            // ---- (a) ----
-            constexpr int PA = 8 / KS;  // pieces per k-step
-            if (has_next) {
+            auto exp_piece = [&](int n) PF_INLINE { exp_pair(n & 1, (n >> 1)); };
+            if (act) {
+                // ---- a row's maximum outgrew its reference by more than the slack (rare): rescale ----
+                if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx[0] > m_thr[0] || mx[1] > m_thr[1]) != 0, 0)) {
 #pragma unroll
-                for (int c = 0; c < NC; ++c)
+                    for (int c = 0; c < NC; ++c) {
+                        const float m_new = fmaxf(m_raw[c], mx[c]);
+                        const float alpha = __builtin_amdgcn_exp2f((m_raw[c] - m_new) * sc);
+                        l_run[c] *= alpha;
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) s_nx[c][i] = 0.f;
+                        for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int ks = 0; ks < KS; ++ks) {
+                            for (int i = 0; i < 16; ++i) o[c][dt][i] *= alpha;
+                        m_raw[c] = m_new;
+                        m_thr[c] = m_new + slack_raw;
+                        m_sc[c] = m_new * sc;
+                    }
+                }
+                PF_FENCE();
+                read_v(kt, 1, va1);  // second k-step's V^T: consumed in (c)
+                PF_FENCE();
+                // ---- (a) ----
+                constexpr int PA = 8 / KS;  // pieces per k-step
+                if (has_next) {
 #pragma unroll
-                    for (int c = 0; c < NC; ++c) s_nx[c] = M::mma(ka[ks], qreg[c][ks], s_nx[c]);
+                    for (int c = 0; c < NC; ++c)
 #pragma unroll
-                    for (int n = 0; n < PA; ++n) exp_piece(ks * PA + n);
+                        for (int i = 0; i < 16; ++i) s_nx[c][i] = 0.f;
+#pragma unroll
+                    for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+                        for (int c = 0; c < NC; ++c) s_nx[c] = M::mma(ka[ks], qreg[c][ks], s_nx[c]);
+#pragma unroll
+                        for (int n = 0; n < PA; ++n) exp_piece(ks * PA + n);
+                        PF_FENCE();
+                    }
+                } else {
+#pragma unroll
+                    for (int n = 0; n < 8; ++n) exp_piece(n);
                     PF_FENCE();
                 }
-                if (kt + 2 < kPfSub) read_k(k_adr, kt + 2, ka);  // consumed in (a) of the next subtile
-                PF_FENCE();
-            } else {
-#pragma unroll
-                for (int n = 0; n < 8; ++n) exp_piece(n);
-                PF_FENCE();
             }
-            // ---- (b) O^T += V^T . P^T, first k-step: result rows 0..7 of a lane, i.e. keys
-            //      key_base + 8*(e/4) + 4*half + e%4 for operand element e ----
-            constexpr int PB = 8 / (DT * NC);  // pieces per product
-            {
-                X8 pb[NC];
-#pragma unroll
-                for (int c = 0; c < NC; ++c) pb[c] = __builtin_bit_cast(X8, uint4{pp[c][0], pp[c][1], pp[c][2], pp[c][3]});
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int c = 0; c < NC; ++c) {
-                        o[c][dt] = M::mma(va0[dt], pb[c], o[c][dt]);
-#pragma unroll
-                        for (int n = 0; n < PB; ++n) exp_piece(8 + (dt * NC + c) * PB + n);
-                        PF_FENCE();
-                    }
-            }
-            if (has_next) read_v(v_adr, kt + 1, 0, va0);  // first k-step's V^T of the next subtile
-            if (has_next && need_mask) mask_s(s_nx, key0 + 32 * (kt + 1));
-            PF_FENCE();
-            // ---- (c) second k-step (keys +16), with the next subtile's row maxima ----
-            {
-                X8 pb[NC];
-#pragma unroll
-                for (int c = 0; c < NC; ++c) pb[c] = __builtin_bit_cast(X8, uint4{pp[c][4], pp[c][5], pp[c][6], pp[c][7]});
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int c = 0; c < NC; ++c) {
-                        o[c][dt] = M::mma(va1[dt], pb[c], o[c][dt]);
-                        const int g = dt * NC + c;  // products issued so far in this stage
-                        if (has_next && g < 2 * NC) max_piece(s_nx[g / 2], g % 2, mx[g / 2]);
-                        PF_FENCE();
-                    }
-                if (has_next && DT * NC < 2 * NC) {  // head_dim 32: fewer products than pieces
-#pragma unroll
-                    for (int g = DT * NC; g < 2 * NC; ++g) max_piece(s_nx[g / 2], g % 2, mx[g / 2]);
+            if (kt == 0) {
+                // ---- publish tile+1; start the loads of tile+3 into the stage of tile-1 (all waves) ----
+                if (STEADY || tile + 1 < n_tiles) {
+                    // loads in flight, oldest first: tile+1, tile+2
+                    if (counted[1]) pf_wait_loads<2 * NLW>(); else __builtin_amdgcn_s_waitcnt(0);
+                    __syncthreads();
                 }
+                counted[0] = counted[1];
+                counted[1] = counted[2];
+                counted[2] = tile + 3 < n_tiles ? issue(tile + 3) : false;
+                PF_FENCE();
             }
-#pragma unroll
-            for (int c = 0; c < NC; ++c) l_run[c] += sum[c];
+            // K operands of subtile g+2 (first subtile of the next tile when kt == 0): consumed in (a) of g+1
+            if (STEADY || g + 2 < n_sub) {
+                if (kt == 0) set_k_tile(tile + 1);
+                read_k(kt == 0 ? 0 : 1, ka);
+            }
             PF_FENCE();
+            if (act) {
+                // ---- (b) O^T += V^T . P^T, first k-step: result rows 0..7 of a lane, i.e. keys
+                //      key_base + 8*(e/4) + 4*half + e%4 for operand element e ----
+                constexpr int PB = 8 / (DT * NC);  // pieces per product
+                {
+                    X8 pb[NC];
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) pb[c] = __builtin_bit_cast(X8, uint4{pp[c][0], pp[c][1], pp[c][2], pp[c][3]});
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int c = 0; c < NC; ++c) {
+                            o[c][dt] = M::mma(va0[dt], pb[c], o[c][dt]);
+#pragma unroll
+                            for (int n = 0; n < PB; ++n) exp_piece(8 + (dt * NC + c) * PB + n);
+                            PF_FENCE();
+                        }
+                }
+                if (has_next) {  // first k-step's V^T of the next subtile
+                    if (kt == kPfSub - 1) set_v_tile(tile + 1);
+                    read_v(kt == kPfSub - 1 ? 0 : kt + 1, 0, va0);
+                    if (mask_next) mask_s(s_nx, 32 * (g + 1));
+                }
+                PF_FENCE();
+                // ---- (c) second k-step (keys +16), with the next subtile's row maxima ----
+                {
+                    X8 pb[NC];
+#pragma unroll
+                    for (int c = 0; c < NC; ++c) pb[c] = __builtin_bit_cast(X8, uint4{pp[c][4], pp[c][5], pp[c][6], pp[c][7]});
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                        for (int c = 0; c < NC; ++c) {
+                            o[c][dt] = M::mma(va1[dt], pb[c], o[c][dt]);
+                            const int i = dt * NC + c;  // products issued so far in this stage
+                            if (has_next && i < 2 * NC) max_piece(s_nx[i / 2], i % 2, mx[i / 2]);
+                            PF_FENCE();
+                        }
+                    if (has_next && DT * NC < 2 * NC) {  // head_dim 32: fewer products than pieces
+#pragma unroll
+                        for (int i = DT * NC; i < 2 * NC; ++i) max_piece(s_nx[i / 2], i % 2, mx[i / 2]);
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < NC; ++c) l_run[c] += sum[c];
+                PF_FENCE();
+            }
         }
     };
-    lookup(0);
-    issue(0, s_k0, s_v0);
-    lookup(1);
-    for (int tile = 0; tile < n_tiles; tile += 2) {
-        do_tile(tile, s_k0, s_v0, s_k1, s_v1);
-        if (tile + 1 < n_tiles) do_tile(tile + 1, s_k1, s_v1, s_k0, s_v0);
-    }
+    const int steady_tiles = max(0, (n_sub - 2) / kPfSub);  // tiles whose subtiles g all have g + 2 < n_sub
+    int tile = 0;
+    for (; tile < steady_tiles; ++tile) do_tile(tile, PfBool<true>{});
+    for (; tile < n_tiles; ++tile) do_tile(tile, PfBool<false>{});
 
     // ---- normalise and write: lane owns row (row0+col), d = 32*dt + 4*half + 8*g + j ----
 #pragma unroll
