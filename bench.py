@@ -38,6 +38,9 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--preheat-s", type=float, default=0.5,
+                    help="seconds of untimed steps before the warmup steps: an idle GPU sits at its lowest clocks "
+                         "and takes a few hundred milliseconds of work to leave them")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -83,6 +86,15 @@ def cpu_baseline(w, budget_s: float):
                   f"cycling ({done_tokens} keys), per-sequence index gather + torch SDPA on {threads} threads, "
                   f"{dt:.1f} s",
     }
+
+
+def preheat(fn, seconds):
+    """Untimed calls of `fn` for about `seconds`, so that the timed region does not start on idle clocks."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
 
 
 def timed_ms(fn, steps):
@@ -139,6 +151,7 @@ def bench_prefill_c3(args, dev) -> int:
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+    preheat(step, args.preheat_s)
     for _ in range(args.warmup):
         step()
     ms_step = timed_ms(step, args.steps)
@@ -149,7 +162,7 @@ def bench_prefill_c3(args, dev) -> int:
     result = {
         "metric": "prefill-attn TFLOP/s", "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
         "tokens_per_s": S * C / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "c3 shared-prefix chunked prefill + KV append, 32 x (2048 + 256), bf16",
                    "num_seqs": S, "prefix_len": P, "chunk_len": C, "num_q_heads": w.num_q_heads,
@@ -237,6 +250,7 @@ def main() -> int:
         dst.copy_(src)  # reads 1 GiB, writes 1 GiB
         torch.cuda.synchronize()
         del src, dst
+    preheat(step, args.preheat_s)
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
@@ -258,6 +272,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "preheat_s": args.preheat_s,
         "ms_per_step": ms_step,
         "wall_ms_per_step": wall * 1e3 / args.steps,
         "higher_is_better": True,
