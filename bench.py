@@ -27,9 +27,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, vendor figure
 
-# HBM traffic of one decode_split_kernel launch on workload c4, from
+# HBM traffic of one launch of the dominant kernel (c4: decode_split_kernel, c3: prefill_mfma_kernel), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/); None until measured.
-MEASURED_TRAFFIC_BYTES = {"c4": 3455256371}  # profiles/decode_c4_bf16.md: fetch 3 447 663 616 + write 7 592 755
+# c4: fetch 3 447 663 616 + write 7 592 755; c3: fetch 131 099 238 + write 67 108 864 (the output)
+MEASURED_TRAFFIC_BYTES = {"c4": 3455256371, "c3": 198208102}
 
 
 def parse_args():
@@ -170,26 +171,28 @@ def bench_prefill_c3(args, dev) -> int:
                    "attention_flops": flops, "append_bytes": w.append_bytes(), "seed": 1003},
         "roofline": {"bound": "mfma", "kernel": "prefill_mfma_kernel", "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "kernel_ms": ms_prefill},
+                     "traffic": MEASURED_TRAFFIC_BYTES.get("c3"), "kernel_ms": ms_prefill},
         "append": {"kernel": "kv_scatter_kernel", "kernel_ms": ms_append,
                    "achieved_gbps": w.append_bytes() / (ms_append * 1e-3) / 1e9, "peak_gbps": HBM_PEAK_GBPS},
     }
     if not args.no_cpu_baseline:
         threads = torch.get_num_threads()
-        n = 4  # sequences of the sample
         kcc, vcc = kc.cpu(), vc.cpu()
+        n = 0  # sequence passes of the sample (cycling over the batch)
         t0 = time.perf_counter()
-        for s in range(n):
+        while time.perf_counter() - t0 < args.cpu_seconds:
+            s = n % S
             blocks = np.asarray(w.block_tables[s])
             pos = np.arange(P + C)
             idx = torch.from_numpy(blocks[pos // w.block_size] * w.block_size + pos % w.block_size)
             k_full, v_full = kcc[idx][None], vcc[idx][None]
             q_full = torch.cat([torch.zeros(P, w.num_q_heads, w.head_dim, dtype=w.dtype), w.q[s]])[None]
             po.prefill_literal(q_full, k_full, v_full, w.scale)
+            n += 1
         dt = time.perf_counter() - t0
         result["cpu_baseline"] = {
             "value": flops / S * n / dt / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
-            "sample": f"{n} of {S} sequences: index gather of prefix+chunk, then the reference's full-sequence causal "
+            "sample": f"{n} sequence passes over the {S} sequences (cycling): index gather of prefix+chunk, then the reference's full-sequence causal "
                       f"SDPA over {P + C} tokens (rows {P}..{P + C - 1} are the chunk), {threads} threads, {dt:.1f} s; "
                       "FLOPs counted for the chunk rows only",
         }
