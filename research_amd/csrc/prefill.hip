@@ -39,8 +39,9 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     a.batch = batch; a.max_q_len = max_q_len;
     hipStream_t s = (hipStream_t)stream;
     // bf16 / fp16 with head_dim 32, 64, 128 run on the matrix cores; PA_PREFILL_ROWWISE=1 forces the
-    // vector kernel (used to cross-check the two paths).
-    static const bool force_rowwise = [] { const char *e = getenv("PA_PREFILL_ROWWISE"); return e && e[0] == '1'; }();
+    // vector kernel (used to cross-check the two paths; read on every call so a test can switch it).
+    const char *env_rowwise = getenv("PA_PREFILL_ROWWISE");
+    const bool force_rowwise = env_rowwise && env_rowwise[0] == '1';
     // (its softmax takes the running maximum of the unscaled logits, which needs scale > 0)
     const prefill_mfma_fn mfma =
         force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);

@@ -1,0 +1,152 @@
+"""The BASELINE configurations at full size on the GPU.
+
+The CPU checker cannot attend 840 000 keys x 32 heads in test time, so the
+full-size runs are checked three ways: the checker on a sample of sequences
+(on a compacted copy of their blocks - block ids do not matter, a property
+the checker itself is pinned on), a size-independent property over EVERY
+sequence (with q = 0 attention is uniform, so each output row is the mean of
+the sequence's V rows, computed here with plain torch indexing), and - for
+prefill - two independent kernels against each other on every output.
+"""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_oracle as po
+from research_amd import ops
+from research_amd.workloads import make_decode, make_prefill_c3
+from tests.gpu_helpers import DEV, announce, assert_close, tables_to_device
+
+pytestmark = pytest.mark.gpu
+
+
+def _compact(w, seqs, k_pool, v_pool):
+    """Pools holding only the blocks of `seqs`, renumbered 0.., and the matching tables."""
+    bs = w.block_size
+    blocks = np.concatenate([np.asarray(w.block_tables[b]) for b in seqs])
+    slots = torch.from_numpy((blocks[:, None] * bs + np.arange(bs)[None, :]).reshape(-1))
+    tables, at = [], 0
+    for b in seqs:
+        n = len(w.block_tables[b])
+        tables.append(list(range(at, at + n)))
+        at += n
+    return k_pool[slots], v_pool[slots], tables
+
+
+def _sample(w, n_random, seed):
+    order = np.argsort(w.seq_lens)
+    rng = np.random.default_rng(seed)
+    picks = {int(order[0]), int(order[-1]), *rng.choice(w.batch, n_random, replace=False).tolist()}
+    return sorted(picks)
+
+
+def _mean_of_v_rows(w, v_pool_dev, dequant=None):
+    """float32 [B, Hkv, D]: mean over each sequence's V rows, by torch indexing on the device."""
+    bs = w.block_size
+    out = torch.zeros(w.batch, w.num_kv_heads, w.head_dim, dtype=torch.float32, device=DEV)
+    for b in range(w.batch):
+        n = int(w.seq_lens[b])
+        if n == 0:
+            continue
+        blocks = torch.from_numpy(np.asarray(w.block_tables[b], dtype=np.int64)).to(DEV)
+        pos = torch.arange(n, device=DEV)
+        blk = blocks[pos // bs]
+        rows = v_pool_dev[blk * bs + pos % bs].float()
+        if dequant is not None:
+            rows = rows * dequant[blk][:, :, None]
+        out[b] = rows.mean(0)
+    return out
+
+
+def _assert_mean(got, want, rel, floor, what):
+    """|got - want| <= rel*|want| + floor: `rel` is the rounding of the 16-bit output, `floor` what a sum of
+    thousands of fp32 terms may lose; a dropped or doubled 16-key block of a 2000-key sequence moves the mean
+    of N(0,1) rows by about 2e-3."""
+    got, want = got.double().cpu().numpy(), want.double().cpu().numpy()
+    assert np.isfinite(got).all(), f"{what}: non-finite output"
+    excess = np.abs(got - want) - rel * np.abs(want)
+    assert excess.max() <= floor, f"{what}: {excess.max():.3e} over the bar at {np.unravel_index(excess.argmax(), excess.shape)}"
+
+
+def test_c4_full_size():
+    """BASELINE config 4: B=256, 840 539 keys in 52 656 blocks, bf16."""
+    announce("decode c4 full size")
+    w = make_decode("c4")
+    assert w.batch == 256 and w.total_tokens == 840539
+    q, kp, vp = w.q.to(DEV), w.k_pool.to(DEV), w.v_pool.to(DEV)
+    tables = tables_to_device(w.block_tables)
+    lens = torch.from_numpy(w.seq_lens.astype(np.int32)).to(DEV)
+    ws = ops.decode_workspace(q, kp)
+    got = ops.decode(q, kp, vp, tables, lens, w.block_size, w.scale, ws).float().cpu()
+    # the checker on the shortest, the longest and 6 other sequences
+    seqs = _sample(w, 6, 4)
+    kc, vc, tc = _compact(w, seqs, w.k_pool, w.v_pool)
+    want = po.paged_decode(w.q[seqs], kc, vc, tc, w.seq_lens[seqs], w.block_size, w.scale)
+    assert_close(got[seqs], want, 2e-2, "c4 sample against the checker")
+    # every sequence: uniform attention = mean of its V rows
+    uni = ops.decode(torch.zeros_like(q), kp, vp, tables, lens, w.block_size, w.scale, ws).float()
+    mean = _mean_of_v_rows(w, vp).repeat_interleave(w.num_q_heads // w.num_kv_heads, dim=1)
+    _assert_mean(uni, mean, 2.0 ** -8, 2e-4, "c4 uniform attention over all 256 sequences")
+    # the same launch again gives the same bits (no dependence on workspace contents or timing)
+    again = ops.decode(q, kp, vp, tables, lens, w.block_size, w.scale, ws).float().cpu()
+    assert torch.equal(got, again)
+
+
+def test_c5_full_size_fp8():
+    """BASELINE config 5: B=8, 802 997 keys, fp8-e4m3 pool with per-(block, kv head) scales."""
+    announce("decode c5 full size")
+    w = make_decode("c5")
+    assert w.batch == 8 and w.total_tokens == 802997
+    q = w.q.to(DEV)
+    k8, ks = ops.quantize_kv_e4m3(w.k_pool.to(DEV), w.block_size)
+    v8, vs = ops.quantize_kv_e4m3(w.v_pool.to(DEV), w.block_size)
+    tables = tables_to_device(w.block_tables)
+    lens = torch.from_numpy(w.seq_lens.astype(np.int32)).to(DEV)
+    ws = ops.decode_workspace(q, k8)
+    got = ops.decode(q, k8, v8, tables, lens, w.block_size, w.scale, ws, k_scale=ks, v_scale=vs).float().cpu()
+    # the checker (dequantise, then attend) on two sequences
+    seqs = _sample(w, 0, 5)
+    bs = w.block_size
+    kq, vq, tc = _compact(w, seqs, k8.cpu().view(torch.uint8), v8.cpu().view(torch.uint8))
+    blocks = np.concatenate([np.asarray(w.block_tables[b]) for b in seqs])
+    kd = po.dequantize_kv_e4m3(kq, ks.cpu()[blocks], bs)
+    vd = po.dequantize_kv_e4m3(vq, vs.cpu()[blocks], bs)
+    want = po.paged_decode(w.q[seqs], kd, vd, tc, w.seq_lens[seqs], bs, w.scale)
+    assert_close(got[seqs], want, 6e-2, "c5 sample against the checker")
+    uni = ops.decode(torch.zeros_like(q), k8, v8, tables, lens, bs, w.scale, ws, k_scale=ks, v_scale=vs).float()
+    mean = _mean_of_v_rows(w, v8, dequant=vs).repeat_interleave(w.num_q_heads // w.num_kv_heads, dim=1)
+    # (the kernel rounds p * v_scale to the 16-bit query type once per block: 2^-9 relative, same sign per block)
+    _assert_mean(uni, mean, 2.0 ** -7, 2e-4, "c5 uniform attention over all 8 sequences")
+
+
+def test_c3_full_size_two_kernels_and_sample():
+    """BASELINE config 3: 32 x (2048 shared + 256 own) tokens; matrix-core kernel against the vector kernel on
+    every output element, and against the checker on three sequences."""
+    announce("prefill c3 full size")
+    w = make_prefill_c3()
+    S, C, P = w.num_seqs, w.chunk_len, w.prefix_len
+    shape = (w.num_blocks * w.block_size, w.num_kv_heads, w.head_dim)
+    kc = torch.zeros(shape, dtype=w.dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    ops.kv_scatter(kc, vc, w.k_prefix.to(DEV), w.v_prefix.to(DEV), torch.from_numpy(w.prefix_slots()).to(DEV))
+    ops.kv_scatter(kc, vc, w.k_chunk.reshape(S * C, *shape[1:]).to(DEV), w.v_chunk.reshape(S * C, *shape[1:]).to(DEV),
+                   torch.from_numpy(w.chunk_slots()).to(DEV))
+    q = w.q.reshape(S * C, w.num_q_heads, w.head_dim).to(DEV)
+    tables = tables_to_device(w.block_tables)
+    i32 = lambda x: torch.tensor(list(x), dtype=torch.int32, device=DEV)
+    args = (q, kc, vc, tables, i32([P + C] * S), i32([C] * S), i32(np.arange(S) * C), C, w.block_size, w.scale)
+    assert os.environ.get("PA_PREFILL_ROWWISE", "0") != "1"
+    mfma = ops.prefill_paged(*args).float().cpu()
+    os.environ["PA_PREFILL_ROWWISE"] = "1"
+    try:
+        rowwise = ops.prefill_paged(*args).float().cpu()
+    finally:
+        del os.environ["PA_PREFILL_ROWWISE"]
+    assert_close(mfma, rowwise, 2e-2, "matrix-core kernel against the vector kernel, all 32 x 256 x 32 rows")
+    seqs = [0, 17, 31]
+    want = po.paged_prefill_chunk(w.q[seqs], kc.cpu(), vc.cpu(), [w.block_tables[s] for s in seqs], [P] * 3, [C] * 3,
+                                  w.block_size, w.scale)
+    assert_close(mfma.reshape(S, C, w.num_q_heads, w.head_dim)[seqs], want, 2e-2, "c3 sample against the checker")
