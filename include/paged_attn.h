@@ -184,6 +184,27 @@ int pa_quantize_kv_e4m3(const void *src, void *dst, float *scale, int64_t num_bl
                         int block_size, int num_kv_heads, int head_dim, int src_dtype,
                         void *stream);
 
+/*
+ * Append rows to an fp8-e4m3 pool (no counterpart in the reference: its _store_kv, flex_backend.py:116-142,
+ * copies rows of the pool's own type).  Policy, per (block, kv head) tile: "re-round on growth".
+ *   - rows of the tile below the lowest offset this call writes are its content so far; a call that writes
+ *     offset 0 starts the tile over (recycled blocks need no clearing);
+ *   - a_old = scale * max|stored value| over the content, a_new = max|x| over the rows written by this call;
+ *   - a_new <= a_old: scale unchanged; otherwise scale' = a_new/448 (1 if a_new = 0) and every content byte
+ *     becomes e4m3fn_rne(float(byte) * (scale / scale'));
+ *   - new rows are stored as e4m3fn_rne(x / scale').
+ *   slots          : int64[n_tokens], slot = block*block_size + offset; negative or out-of-pool slots are skipped;
+ *                    of two tokens with the same slot the later one is stored
+ *   touched_blocks : int32[n_touched], the distinct blocks the slots fall in (extra entries are harmless,
+ *                    a block must not appear twice)
+ *   k_src, v_src   : [n_tokens][num_kv_heads][head_dim] in src_dtype (F32/BF16/F16)
+ *   k_scale,v_scale: float[num_blocks][num_kv_heads], updated in place
+ */
+int pa_kv_append_e4m3(void *k_cache, void *v_cache, float *k_scale, float *v_scale, const void *k_src,
+                      const void *v_src, const int64_t *slots, int64_t n_tokens,
+                      const int32_t *touched_blocks, int n_touched, int64_t num_blocks, int block_size,
+                      int num_kv_heads, int head_dim, int src_dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

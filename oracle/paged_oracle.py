@@ -35,6 +35,12 @@ How each function is pinned (see tests/test_oracle.py):
   quantize_kv_e4m3      torch.float8_e4m3fn conversion (library definition of
                         OCP e4m3fn, round to nearest even), known values
                         464 -> 448, 2**-10 -> 0, max 448
+  append_kv_e4m3        (a policy of this build, the reference has no fp8 pool)
+                        appending a whole block in one call equals
+                        quantize_kv_e4m3 of that block bit for bit; rows of
+                        non-increasing magnitude leave earlier bytes and the
+                        scale untouched; after any append order the dequantised
+                        pool is within two e4m3 roundings of the input
 Parity unpinned by any test of the reference itself: decode values, the
 gather and ragged batches (the reference only asserts shapes there).
 """
@@ -313,3 +319,46 @@ def dequantize_kv_e4m3(bits: torch.Tensor, scale: torch.Tensor, block_size: int)
     nb = slots // block_size
     x = bits.view(torch.float8_e4m3fn).to(torch.float32).reshape(nb, block_size, hkv, d)
     return (x * scale[:, None, :, None]).reshape(slots, hkv, d)
+
+
+def append_kv_e4m3(bits: torch.Tensor, scale: torch.Tensor, src: torch.Tensor, slots, block_size: int) -> None:
+    """Append rows to an fp8 pool in place, "re-round on growth" (not a reference function: the reference has no
+    fp8 pool; this states the policy the HIP entry point pa_kv_append_e4m3 documents, tile by tile in fp32).
+
+    bits ``uint8 [total_slots, Hkv, D]``, scale ``float32 [num_blocks, Hkv]``, src ``[N, Hkv, D]``.  Per (block,
+    kv head) tile: rows below the lowest offset written by this call are the content so far;
+    a_old = scale*max|content|, a_new = max|new rows|; if a_new > a_old (or offset 0 is written) the scale becomes
+    a_new/448 (1 for 0) and the content is re-rounded as e4m3(float(byte)*(scale/scale')); new rows are
+    e4m3(x/scale').  Pinned by: appending a whole block at once equals quantize_kv_e4m3 of that block; appending
+    rows of non-increasing magnitude never changes earlier bytes; the dequantised error bound in the tests.
+    """
+    f8 = torch.float8_e4m3fn
+    slots = np.asarray(slots, dtype=np.int64)
+    total_slots, hkv, d = bits.shape
+    nb = total_slots // block_size
+    x = src.to(torch.float32)
+    c448 = torch.tensor(448.0, dtype=torch.float32)
+    by_block = {}
+    for t, s in enumerate(slots):
+        if 0 <= s < nb * block_size:
+            by_block.setdefault(int(s // block_size), {})[int(s % block_size)] = t  # later token wins
+    for blk, offs in by_block.items():
+        first = min(offs)
+        rows = sorted(offs)
+        toks = [offs[o] for o in rows]
+        for h in range(hkv):
+            s_old = scale[blk, h].clone()
+            content = bits[blk * block_size : blk * block_size + first, h].view(f8).to(torch.float32)
+            new = x[toks, h]
+            a_new = new.abs().amax() if new.numel() else torch.tensor(0.0)
+            a_old = s_old * content.abs().amax() if first > 0 else torch.tensor(0.0)
+            s_new = s_old
+            if first == 0 or a_new > a_old:
+                s_new = a_new / c448 if a_new > 0 else torch.tensor(1.0, dtype=torch.float32)
+            if first > 0 and s_new != s_old:
+                ratio = s_old / s_new
+                bits[blk * block_size : blk * block_size + first, h] = (content * ratio).to(f8).view(torch.uint8)
+            enc = (new / s_new).to(f8).view(torch.uint8)
+            for i, o in enumerate(rows):
+                bits[blk * block_size + o, h] = enc[i]
+            scale[blk, h] = s_new

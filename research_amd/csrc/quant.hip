@@ -40,7 +40,115 @@ __global__ __launch_bounds__(kQThreads) void quantize_e4m3_kernel(const T *__res
     }
 }
 
+// Append to an fp8 pool ("re-round on growth"): one workgroup per (touched block, kv head) tile.
+//   rows of the tile below the lowest offset this call writes are the tile's content so far; rows from there
+//   on are new or not yet written (a recycled block starts over when its offset 0 is written);
+//   a_old = scale * max|byte value| over the content, a_new = max|x| over the rows this call writes;
+//   a_new <= a_old: the scale stays and only the new rows are encoded;
+//   otherwise scale' = a_new / 448 and the content is re-rounded: byte' = e4m3(float(byte) * (scale / scale')).
+constexpr int kMaxBlockTokens = 256;
+
+template <typename T>
+__global__ __launch_bounds__(kQThreads) void append_e4m3_kernel(const T *__restrict__ src, uint8_t *__restrict__ dst,
+                                                                 float *__restrict__ scale,
+                                                                 const int64_t *__restrict__ slots, int64_t n_tokens,
+                                                                 const int32_t *__restrict__ touched, int64_t num_blocks,
+                                                                 int block_size, int hkv, int d) {
+    __shared__ int s_token[kMaxBlockTokens];  // token of this call that writes offset i (-1: none); highest index wins
+    __shared__ float s_max[2][kQThreads / PA_WAVE];
+    const int64_t blk = touched[blockIdx.x];
+    const int h = blockIdx.y;
+    if (blk < 0 || blk >= num_blocks) return;  // uniform
+    for (int i = threadIdx.x; i < block_size; i += kQThreads) s_token[i] = -1;
+    __syncthreads();
+    const int64_t slot0 = blk * block_size;
+    for (int64_t t = threadIdx.x; t < n_tokens; t += kQThreads) {
+        const int64_t off = slots[t] - slot0;
+        if (off >= 0 && off < block_size) atomicMax(&s_token[off], (int)t);
+    }
+    __syncthreads();
+    int first = block_size;  // lowest offset written
+    for (int i = 0; i < block_size; ++i)
+        if (s_token[i] >= 0) { first = i; break; }
+    if (first == block_size) return;  // uniform: the block is not touched after all
+
+    const int64_t tok_stride = (int64_t)hkv * d;
+    const int64_t tile0 = (slot0 * hkv + h) * (int64_t)d;
+    const float s_old = scale[blk * hkv + h];
+    // content so far: rows [0, first)
+    float q_max = 0.f, a_new = 0.f;
+    for (int i = threadIdx.x; i < first * d; i += kQThreads) {
+        const int t = i / d, e = i - t * d;
+        q_max = fmaxf(q_max, fabsf(__builtin_amdgcn_cvt_f32_fp8((int)dst[tile0 + t * tok_stride + e], 0)));
+    }
+    for (int i = threadIdx.x; i < (block_size - first) * d; i += kQThreads) {
+        const int t = first + i / d, e = i % d;
+        const int tok = s_token[t];
+        if (tok >= 0) a_new = fmaxf(a_new, fabsf(pa_scalar<T>::load(src + ((int64_t)tok * hkv + h) * d + e)));
+    }
+    for (int off = 32; off > 0; off >>= 1) {
+        q_max = fmaxf(q_max, __shfl_xor(q_max, off, 64));
+        a_new = fmaxf(a_new, __shfl_xor(a_new, off, 64));
+    }
+    if ((threadIdx.x & 63) == 0) { s_max[0][threadIdx.x >> 6] = q_max; s_max[1][threadIdx.x >> 6] = a_new; }
+    __syncthreads();
+    q_max = fmaxf(fmaxf(s_max[0][0], s_max[0][1]), fmaxf(s_max[0][2], s_max[0][3]));
+    a_new = fmaxf(fmaxf(s_max[1][0], s_max[1][1]), fmaxf(s_max[1][2], s_max[1][3]));
+    const float a_old = first > 0 ? s_old * q_max : 0.f;
+    float s_new = s_old;
+    if (first == 0 || a_new > a_old) s_new = a_new > 0.f ? a_new / 448.0f : 1.0f;
+    if (first > 0 && s_new != s_old) {  // uniform: re-round the content to the new scale
+        const float ratio = s_old / s_new;
+        for (int i = threadIdx.x; i < first * d; i += kQThreads) {
+            const int t = i / d, e = i - t * d;
+            const float x = __builtin_amdgcn_cvt_f32_fp8((int)dst[tile0 + t * tok_stride + e], 0) * ratio;
+            dst[tile0 + t * tok_stride + e] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(x, 0.f, 0, false) & 0xff);
+        }
+    }
+    for (int i = threadIdx.x; i < (block_size - first) * d; i += kQThreads) {
+        const int t = first + i / d, e = i % d;
+        const int tok = s_token[t];
+        if (tok < 0) continue;
+        const float x = pa_scalar<T>::load(src + ((int64_t)tok * hkv + h) * d + e) / s_new;
+        dst[tile0 + t * tok_stride + e] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(x, 0.f, 0, false) & 0xff);
+    }
+    if (threadIdx.x == 0) scale[blk * hkv + h] = s_new;
+}
+
 }  // namespace
+
+extern "C" int pa_kv_append_e4m3(void *k_cache, void *v_cache, float *k_scale, float *v_scale, const void *k_src,
+                                 const void *v_src, const int64_t *slots, int64_t n_tokens,
+                                 const int32_t *touched_blocks, int n_touched, int64_t num_blocks, int block_size,
+                                 int num_kv_heads, int head_dim, int src_dtype, void *stream) {
+    pa_clear_error();
+    PA_REQUIRE(n_tokens >= 0 && n_touched >= 0, "n_tokens=%lld / n_touched=%d is negative", (long long)n_tokens, n_touched);
+    PA_REQUIRE(block_size > 0 && block_size <= kMaxBlockTokens, "block_size=%d outside 1..%d", block_size, kMaxBlockTokens);
+    PA_REQUIRE(num_kv_heads > 0 && num_kv_heads <= 65535 && head_dim > 0, "num_kv_heads / head_dim out of range");
+    PA_REQUIRE(src_dtype == PA_F32 || src_dtype == PA_BF16 || src_dtype == PA_F16, "src_dtype=%d is not F32, BF16 or F16",
+               src_dtype);
+    PA_REQUIRE(n_tokens <= 0x7fffffffll, "n_tokens above 2^31-1");
+    if (n_tokens == 0 || n_touched == 0) return PA_OK;
+    PA_REQUIRE(k_cache && v_cache && k_scale && v_scale && k_src && v_src && slots && touched_blocks, "NULL pointer argument");
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((unsigned)n_touched, (unsigned)num_kv_heads), block(kQThreads);
+    for (int which = 0; which < 2; ++which) {
+        uint8_t *dst = (uint8_t *)(which ? v_cache : k_cache);
+        float *sc = which ? v_scale : k_scale;
+        const void *src = which ? v_src : k_src;
+        if (src_dtype == PA_F32)
+            append_e4m3_kernel<float><<<grid, block, 0, s>>>((const float *)src, dst, sc, slots, n_tokens, touched_blocks,
+                                                             num_blocks, block_size, num_kv_heads, head_dim);
+        else if (src_dtype == PA_BF16)
+            append_e4m3_kernel<pa_bf16><<<grid, block, 0, s>>>((const pa_bf16 *)src, dst, sc, slots, n_tokens,
+                                                               touched_blocks, num_blocks, block_size, num_kv_heads, head_dim);
+        else
+            append_e4m3_kernel<pa_f16><<<grid, block, 0, s>>>((const pa_f16 *)src, dst, sc, slots, n_tokens, touched_blocks,
+                                                              num_blocks, block_size, num_kv_heads, head_dim);
+        PA_CHECK_LAUNCH("pa_kv_append_e4m3");
+    }
+    return PA_OK;
+}
 
 extern "C" int pa_quantize_kv_e4m3(const void *src, void *dst, float *scale, int64_t num_blocks,
                                    int block_size, int num_kv_heads, int head_dim, int src_dtype,

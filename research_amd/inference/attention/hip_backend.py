@@ -42,12 +42,12 @@ _COMPUTE_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
 class _StepTensors:
     """Device copies of one context's integer fields, built once per step."""
 
-    __slots__ = ("ctx", "slots", "tables", "bt_stride", "seq_lens", "extra_zero", "ctx_lens", "q_lens", "q_starts",
-                 "max_q_len")
+    __slots__ = ("ctx", "slots", "touched", "tables", "bt_stride", "seq_lens", "extra_zero", "ctx_lens", "q_lens",
+                 "q_starts", "max_q_len")
 
     def __init__(self, ctx: InferenceContext) -> None:
         self.ctx = ctx  # keeps id(ctx) alive while the entry is cached
-        self.slots = self.tables = self.seq_lens = self.extra_zero = None
+        self.slots = self.touched = self.tables = self.seq_lens = self.extra_zero = None
         self.ctx_lens = self.q_lens = self.q_starts = None
         self.bt_stride = self.max_q_len = 0
 
@@ -167,8 +167,6 @@ class HipPagedAttentionBackend:
                   _step: Optional[_StepTensors] = None) -> None:
         """``cache[layer, slot] = row`` for every non-negative slot (flex_backend.py:116-142)."""
         cfg = self.config
-        if self._fp8:
-            raise NotImplementedError("appending to an fp8 pool: quantise a filled pool with quantize_from()")
         k_flat = k.reshape(-1, cfg.num_kv_heads, cfg.head_dim)
         v_flat = v.reshape(-1, cfg.num_kv_heads, cfg.head_dim)
         n = len(slot_mapping)
@@ -178,7 +176,10 @@ class HipPagedAttentionBackend:
                 f"The shape of the mask [{n}] at index 0 does not match the shape of the indexed tensor "
                 f"{list(k_flat.shape)} at index 0"
             )
-        if k_flat.dtype != self.k_cache.dtype or v_flat.dtype != self.v_cache.dtype:
+        if self._fp8:
+            if k_flat.dtype not in (torch.float32, torch.bfloat16, torch.float16) or v_flat.dtype != k_flat.dtype:
+                raise RuntimeError("an fp8 pool takes fp32, bf16 or fp16 rows (k and v of the same type)")
+        elif k_flat.dtype != self.k_cache.dtype or v_flat.dtype != self.v_cache.dtype:
             raise RuntimeError("Index put requires the source and destination dtypes match")
         if n == 0:
             return
@@ -195,6 +196,17 @@ class HipPagedAttentionBackend:
                 _step.slots = slots
         k_flat, v_flat = k_flat.contiguous(), v_flat.contiguous()
         kc, vc = self._layer(layer_idx)
+        if self._fp8:
+            # rows are encoded with the tile's scale; a row that raises a tile's absmax re-rounds the tile
+            if _step is not None and _step.touched is not None:
+                touched = _step.touched
+            else:
+                touched = ops.touched_blocks(slots, cfg.block_size, cfg.num_blocks)
+                if _step is not None:
+                    _step.touched = touched
+            ops.kv_append_e4m3(kc, vc, self.k_scale[layer_idx], self.v_scale[layer_idx], k_flat, v_flat, slots,
+                               cfg.block_size, touched)
+            return
         ops.kv_scatter(kc, vc, k_flat, v_flat, slots)
 
     # ------------------------------------------------------------------ gather

@@ -111,3 +111,27 @@ def quantize_kv_e4m3(pool: Tensor, block_size: int) -> Tuple[Tensor, Tensor]:
     _run("pa_quantize_kv_e4m3", _ptr(pool), _ptr(dst), _ptr(scale), num_blocks, block_size, hkv, d,
          PA_DTYPE[pool.dtype], _stream(pool))
     return dst, scale
+
+
+def touched_blocks(slots: Tensor, block_size: int, num_blocks: int) -> Tensor:
+    """Distinct blocks (int32, on the device) that the non-negative, in-pool slots fall in."""
+    blocks = torch.div(slots, block_size, rounding_mode="floor")
+    blocks = blocks[(slots >= 0) & (blocks < num_blocks)]
+    return torch.unique(blocks).to(torch.int32)
+
+
+def kv_append_e4m3(k_cache: Tensor, v_cache: Tensor, k_scale: Tensor, v_scale: Tensor, k_src: Tensor, v_src: Tensor,
+                   slots: Tensor, block_size: int, touched: Optional[Tensor] = None) -> None:
+    """Append rows to an fp8-e4m3 pool with the "re-round on growth" policy of ``pa_kv_append_e4m3``.
+
+    k_cache/v_cache ``[total_slots, Hkv, D]`` float8_e4m3fn, scales ``float32 [num_blocks, Hkv]`` (updated in
+    place), k_src/v_src ``[N, Hkv, D]`` fp32/bf16/fp16, slots ``int64 [N]``.  ``touched`` (the distinct target
+    blocks) is computed with torch when not given.
+    """
+    total_slots, hkv, d = k_cache.shape
+    num_blocks = total_slots // block_size
+    if touched is None:
+        touched = touched_blocks(slots, block_size, num_blocks)
+    _run("pa_kv_append_e4m3", _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale), _ptr(k_src), _ptr(v_src),
+         _ptr(slots), slots.numel(), _ptr(touched), touched.numel(), num_blocks, block_size, hkv, d,
+         PA_DTYPE[k_src.dtype], _stream(k_cache))

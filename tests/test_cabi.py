@@ -133,6 +133,19 @@ def test_prefill_and_quantize_argument_errors():
     assert rc == _lib.PA_ERR_INVALID_ARG and "src_dtype" in msg
     rc, msg = _status("pa_quantize_kv_e4m3", None, FAKE, FAKE, 4, 16, 8, 128, _lib.PA_F32, None)
     assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
+    append = [FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 5, FAKE, 2, 64, 16, 8, 128, _lib.PA_BF16, None]
+    bad = list(append); bad[14] = _lib.PA_FP8_E4M3
+    rc, msg = _status("pa_kv_append_e4m3", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "src_dtype" in msg
+    bad = list(append); bad[11] = 1024
+    rc, msg = _status("pa_kv_append_e4m3", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "block_size" in msg
+    bad = list(append); bad[8] = None
+    rc, msg = _status("pa_kv_append_e4m3", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
+    bad = list(append); bad[7] = 0  # nothing to append: fine even with no device
+    rc, msg = _status("pa_kv_append_e4m3", *bad)
+    assert rc == _lib.PA_OK
 
 
 def test_error_text_is_cleared_by_a_good_call():

@@ -189,3 +189,46 @@ def test_fp8_backend_decode():
     kd = po.dequantize_kv_e4m3(backend.k_cache[0].cpu().view(torch.uint8), backend.k_scale[0].cpu(), 16)
     vd = po.dequantize_kv_e4m3(backend.v_cache[0].cpu().view(torch.uint8), backend.v_scale[0].cpu(), 16)
     assert_close(out[:, 0], po.paged_decode(w.q, kd, vd, tables, lens, 16, w.scale), 6e-2, "fp8 backend")
+
+
+def test_fp8_backend_prefill_then_decode_appends():
+    """A prompt and 10 decode steps written through the backend into an fp8 pool: stored bytes and scales equal
+    the checker's append policy, and the decode output equals dequantise-then-attend."""
+    announce("backend fp8 append + decode")
+    g = torch.Generator().manual_seed(31)
+    hq, hkv, d, bs = 8, 2, 64, 16
+    config = CacheConfig(num_layers=2, num_kv_heads=hkv, head_dim=d, num_blocks=16, block_size=bs, device="cuda",
+                         kv_format="fp8_e4m3")
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(hq)
+    cache = PagedKVCache(config.num_blocks, bs)
+    layer = 1
+    bits = torch.zeros(16 * bs, hkv, d, dtype=torch.uint8)
+    vbits = bits.clone()
+    ks, vs = torch.ones(16, hkv), torch.ones(16, hkv)
+    tokens = list(range(100, 137))
+    k = (torch.randn(1, len(tokens), hkv, d, generator=g)).to(torch.bfloat16)
+    v = (torch.randn(1, len(tokens), hkv, d, generator=g)).to(torch.bfloat16)
+    q = torch.randn(1, len(tokens), hq, d, generator=g).to(torch.bfloat16)
+    ctx, _ = allocate_and_build_context(cache, seq_id=7, token_ids=tokens)
+    backend.forward(q.cuda(), k.cuda(), v.cuda(), layer, ctx)
+    po.append_kv_e4m3(bits, ks, k[0], ctx.slot_mapping, bs)
+    po.append_kv_e4m3(vbits, vs, v[0], ctx.slot_mapping, bs)
+    n = len(tokens)
+    for step in range(10):  # stays inside the prompt's last block (the allocator twin keeps the reference's quirks)
+        kn = (torch.randn(1, 1, hkv, d, generator=g) * (1 + 0.3 * step)).to(torch.bfloat16)
+        vn = torch.randn(1, 1, hkv, d, generator=g).to(torch.bfloat16)
+        qn = torch.randn(1, 1, hq, d, generator=g).to(torch.bfloat16)
+        ctx = extend_and_build_context(cache, seq_id=7, new_token=500 + step, current_len=n)
+        assert min(ctx.slot_mapping) >= 0
+        out = backend.forward(qn.cuda(), kn.cuda(), vn.cuda(), layer, ctx)
+        po.append_kv_e4m3(bits, ks, kn[0], ctx.slot_mapping, bs)
+        po.append_kv_e4m3(vbits, vs, vn[0], ctx.slot_mapping, bs)
+        n += 1
+        assert torch.equal(backend.k_cache[layer].cpu().view(torch.uint8), bits), f"step {step}: K bytes"
+        assert torch.equal(backend.v_cache[layer].cpu().view(torch.uint8), vbits), f"step {step}: V bytes"
+        assert torch.equal(backend.k_scale[layer].cpu(), ks) and torch.equal(backend.v_scale[layer].cpu(), vs)
+        kd, vd = po.dequantize_kv_e4m3(bits, ks, bs), po.dequantize_kv_e4m3(vbits, vs, bs)
+        want = po.paged_decode(qn[:, 0], kd, vd, ctx.block_tables, ctx.seq_lens, bs, backend.scale)
+        assert_close(out[:, 0], want, 6e-2, f"decode step {step}")
+    assert (backend.k_cache[0].view(torch.uint8) == 0).all()  # the other layer was not touched

@@ -117,3 +117,69 @@ def test_gather_short_table_and_bad_ids_read_as_zero():
     bad = torch.tensor([[3, 99, -5]], dtype=torch.int32, device=DEV)
     kg, _ = ops.kv_gather(kc.to(DEV), vc.to(DEV), bad, torch.tensor([12], dtype=torch.int32, device=DEV), 12, bs)
     assert torch.equal(kg[0, :4].cpu(), kc[12:16]) and not kg[0, 4:].any()
+
+
+# ---------------------------------------------------------------- fp8 append
+def _fp8_pool(nb, bs, hkv, d):
+    bits = torch.zeros(nb * bs, hkv, d, dtype=torch.uint8)
+    scale = torch.ones(nb, hkv, dtype=torch.float32)
+    return bits, scale
+
+
+def _append_both(bits, scale, src, slots, bs):
+    """The same append on the device (through the C ABI) and in the checker; returns the device result."""
+    kb = bits.clone().to(DEV).view(torch.float8_e4m3fn)
+    vb = bits.clone().to(DEV).view(torch.float8_e4m3fn)
+    ks, vs = scale.clone().to(DEV), scale.clone().to(DEV)
+    sl = torch.from_numpy(np.asarray(slots, dtype=np.int64)).to(DEV)
+    ops.kv_append_e4m3(kb, vb, ks, vs, src.to(DEV), (src * 0.5).to(DEV), sl, bs)
+    po.append_kv_e4m3(bits, scale, src, slots, bs)
+    assert torch.equal(kb.view(torch.uint8).cpu(), bits), "K bytes differ from the checker"
+    assert torch.equal(ks.cpu(), scale), "K scales differ from the checker"
+    return kb, vb, ks, vs
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_fp8_append_bit_exact_token_by_token_and_in_chunks(dtype):
+    announce(f"fp8 append {dtype}")
+    g = torch.Generator().manual_seed(21)
+    nb, bs, hkv, d = 6, 16, 8, 128
+    bits, scale = _fp8_pool(nb, bs, hkv, d)
+    # a prompt of 37 tokens into blocks 4, 1, 5 in one call, then 20 decode steps one token at a time with
+    # growing magnitude (every step re-rounds the last block), then a chunk that crosses into a new block
+    table = [4, 1, 5, 0, 2]
+    pos_slot = lambda p: table[p // bs] * bs + p % bs
+    prompt = (torch.randn(37, hkv, d, generator=g) * 0.3).to(dtype)
+    _append_both(bits, scale, prompt, [pos_slot(p) for p in range(37)], bs)
+    for i in range(20):
+        row = (torch.randn(1, hkv, d, generator=g) * (0.3 + 0.2 * i)).to(dtype)
+        _append_both(bits, scale, row, [pos_slot(37 + i)], bs)
+    chunk = (torch.randn(11, hkv, d, generator=g) * 3).to(dtype)
+    _append_both(bits, scale, chunk, [pos_slot(57 + i) for i in range(11)], bs)
+    # the V pool of the same calls holds half the values: same bytes, half the scale (powers of two are exact)
+    # and the dequantised pool is close to what was appended
+    everything = prompt.float()
+    back = po.dequantize_kv_e4m3(bits, scale, bs)
+    got = torch.stack([back[pos_slot(p)] for p in range(37)])
+    assert ((got - everything).abs() <= 0.5 * everything.abs() + 0.05).all()
+
+
+def test_fp8_append_v_pool_and_edge_cases():
+    announce("fp8 append edge cases")
+    g = torch.Generator().manual_seed(22)
+    nb, bs, hkv, d = 4, 16, 2, 64
+    bits, scale = _fp8_pool(nb, bs, hkv, d)
+    src = torch.randn(5, hkv, d, generator=g).to(torch.bfloat16)
+    # negative and out-of-pool slots are skipped, a duplicated slot keeps the later token
+    kb, vb, ks, vs = _append_both(bits, scale, src, [3 * bs, -1, nb * bs + 7, 3 * bs + 1, 3 * bs + 1], bs)
+    # the V rows of these calls are half the K rows: same bytes, half the scale (exact), other tiles untouched
+    assert torch.equal(vb.view(torch.uint8).cpu(), bits)
+    assert torch.equal(vs.cpu()[3], scale[3] * 0.5) and (vs.cpu()[:3] == 1).all() and (scale[:3] == 1).all()
+    # whole blocks at once equal the block quantiser
+    full = torch.randn(2 * bs, hkv, d, generator=g)
+    bits2, scale2 = _fp8_pool(nb, bs, hkv, d)
+    _append_both(bits2, scale2, full, list(range(bs, 3 * bs)), bs)
+    want_bits, want_scale = po.quantize_kv_e4m3(full, bs)
+    assert torch.equal(bits2[bs : 3 * bs], want_bits) and torch.equal(scale2[1:3], want_scale)
+    # nothing to do
+    ops.kv_append_e4m3(kb, vb, ks, vs, src[:0].to(DEV), src[:0].to(DEV), torch.zeros(0, dtype=torch.int64, device=DEV), bs)

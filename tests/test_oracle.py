@@ -349,3 +349,67 @@ def test_fp8_decode_oracle_is_dequantise_then_attend():
     exact = po.paged_decode(w.q, w.k_pool, w.v_pool, tables, w.seq_lens, w.block_size, w.scale)
     assert np.abs(approx - exact).max() < 6e-2  # the quantisation error itself sits inside the fp8 tolerance
     assert np.abs(approx - exact).max() > 1e-4
+
+
+# ---------------------------------------------------------------- fp8 append policy
+def _empty_fp8_pool(nb, bs, hkv, d):
+    return torch.zeros(nb * bs, hkv, d, dtype=torch.uint8), torch.ones(nb, hkv, dtype=torch.float32)
+
+
+def test_fp8_append_of_whole_blocks_equals_block_quantisation():
+    g = torch.Generator().manual_seed(11)
+    nb, bs, hkv, d = 5, 16, 3, 32
+    src = torch.randn(nb * bs, hkv, d, generator=g) * torch.logspace(-2, 1, nb * bs)[:, None, None]
+    bits, scale = _empty_fp8_pool(nb, bs, hkv, d)
+    perm = torch.randperm(nb * bs, generator=g).numpy()  # token t goes to slot perm[t]: every block completely
+    po.append_kv_e4m3(bits, scale, src, perm, bs)
+    pool = torch.empty_like(src)
+    pool[perm] = src
+    want_bits, want_scale = po.quantize_kv_e4m3(pool, bs)
+    assert torch.equal(bits, want_bits) and torch.equal(scale, want_scale)
+
+
+def test_fp8_append_token_by_token_policy():
+    g = torch.Generator().manual_seed(12)
+    bs, hkv, d = 16, 2, 64
+    bits, scale = _empty_fp8_pool(2, bs, hkv, d)
+    # block 0: magnitudes shrink -> the first row fixes the scale, earlier bytes never change
+    rows = torch.randn(bs, hkv, d, generator=g) * torch.linspace(4.0, 0.5, bs)[:, None, None]
+    rows = rows.clamp(-19.0, 19.0)
+    rows[0, :, 0] = 20.0  # the tile maximum sits in the first row
+    history = []
+    for t in range(bs):
+        po.append_kv_e4m3(bits, scale, rows[t : t + 1], [t], bs)
+        history.append((bits[: t + 1].clone(), scale[0].clone()))
+    for t in range(1, bs):
+        assert torch.equal(history[t][0][:t], history[t - 1][0]) and torch.equal(history[t][1], history[0][1])
+    assert torch.equal(scale[0], torch.full((hkv,), 20.0) / 448.0)
+    # block 1: magnitudes grow -> the scale follows the running maximum and earlier rows are re-rounded
+    rows = torch.randn(bs, hkv, d, generator=g) * torch.linspace(0.5, 4.0, bs)[:, None, None]
+    for t in range(bs):
+        po.append_kv_e4m3(bits, scale, rows[t : t + 1], [bs + t], bs)
+        amax = rows[: t + 1].abs().amax(dim=(0, 2))
+        assert torch.equal(scale[1], amax / 448.0)
+    back = po.dequantize_kv_e4m3(bits, scale, bs)[bs:]
+    # a row is rounded once when it is written and once more each time the tile maximum grows afterwards; every
+    # rounding is within half an e4m3 step (2^-4 relative, 2^-10 of the scale grid for subnormals)
+    run_max = torch.stack([rows[: t + 1].abs().amax(dim=(0, 2)) for t in range(bs)])  # [bs, hkv]
+    grew = torch.cat([torch.zeros(1, hkv, dtype=torch.bool), run_max[1:] > run_max[:-1]])
+    n_round = 1 + torch.stack([grew[t + 1 :].sum(0) for t in range(bs)])  # [bs, hkv]
+    err = (back - rows).abs()
+    bound = n_round[:, :, None] * (2.0 ** -4 * 1.01 * rows.abs() + scale[1][None, :, None] * 2.0 ** -9)
+    assert (err <= bound).all(), float((err - bound).max())
+    assert (n_round[0] > 3).all()  # the case does exercise repeated re-rounding
+
+
+def test_fp8_append_restarts_a_recycled_block_and_skips_bad_slots():
+    bs, hkv, d = 4, 1, 8
+    bits, scale = _empty_fp8_pool(2, bs, hkv, d)
+    po.append_kv_e4m3(bits, scale, torch.full((3, hkv, d), 100.0), [0, 1, 2], bs)
+    assert float(scale[0, 0]) == float(np.float32(100.0) / np.float32(448.0))
+    # the block is handed to another sequence: offset 0 is written again, the old rows do not count
+    po.append_kv_e4m3(bits, scale, torch.full((2, hkv, d), 2.0), [0, -1], bs)
+    assert float(scale[0, 0]) == float(np.float32(2.0) / np.float32(448.0))
+    assert (bits[0].view(torch.float8_e4m3fn).to(torch.float32) == 448.0).all()
+    po.append_kv_e4m3(bits, scale, torch.full((1, hkv, d), 1.0), [99], bs)  # outside the pool: ignored
+    assert float(scale[1, 0]) == 1.0 and int(bits[bs:].max()) == 0
