@@ -118,6 +118,12 @@ size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads, i
  *                   zero-pads ragged batches to the longest sequence without a
  *                   mask (:253-264, :227-229); passing max_len - seq_lens[b]
  *                   reproduces it.
+ *   window        : 0, or a sliding window: only the last `window` keys of each sequence are attended
+ *                   (j >= seq_lens[b] - window), the rule of the reference's causal_sliding_window_mask
+ *                   (attention/mask.py:83-89: q_idx - kv_idx < window_size) for the query at position
+ *                   seq_lens[b]-1; blocks wholly before the window are never read.  The reference's own
+ *                   decode applies a window only through a caller-built ctx.block_mask
+ *                   (flex_backend.py:220-225).  Not combinable with extra_zero_keys.
  *   batch         : at most 8192 sequences per call
  *   workspace     : pa_decode_workspace_bytes(...) bytes
  *   A sequence of length 0 yields zeros.
@@ -126,7 +132,7 @@ int pa_decode(const void *q, const void *k_cache, const void *v_cache, void *out
               const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
               const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale,
               int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-              int64_t num_blocks, float scale, int q_dtype, int kv_dtype, void *workspace,
+              int64_t num_blocks, float scale, int window, int q_dtype, int kv_dtype, void *workspace,
               size_t workspace_bytes, void *stream);
 
 /*
@@ -140,13 +146,13 @@ int pa_decode_split(const void *q, const void *k_cache, const void *v_cache, voi
                     const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
                     const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale,
                     int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-                    int64_t num_blocks, float scale, int q_dtype, int kv_dtype, void *workspace,
+                    int64_t num_blocks, float scale, int window, int q_dtype, int kv_dtype, void *workspace,
                     size_t workspace_bytes, void *stream);
 int pa_decode_reduce(const void *q, const void *k_cache, const void *v_cache, void *out,
                      const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
                      const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale,
                      int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-                     int64_t num_blocks, float scale, int q_dtype, int kv_dtype, void *workspace,
+                     int64_t num_blocks, float scale, int window, int q_dtype, int kv_dtype, void *workspace,
                      size_t workspace_bytes, void *stream);
 
 /*
@@ -164,12 +170,15 @@ int pa_decode_reduce(const void *q, const void *k_cache, const void *v_cache, vo
  *              PA_F32 (vector path)
  *   ctx_lens, q_lens, q_starts : int32[batch]
  *   max_q_len: upper bound of q_lens (grid sizing)
+ *   window   : 0, or the sliding window of CacheConfig.sliding_window (attention/config.py:31): row i at
+ *              position p = ctx_lens[b] - q_lens[b] + i attends keys p - window < j <= p
+ *              (attention/mask.py:83-89).  Windowed calls run on the vector path.
  */
 int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, void *out,
                      const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
                      const int32_t *q_lens, const int32_t *q_starts, int batch, int max_q_len,
                      int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-                     int64_t num_blocks, float scale, int dtype, void *stream);
+                     int64_t num_blocks, float scale, int window, int dtype, void *stream);
 
 /*
  * fp8-e4m3 pool construction (no counterpart in the reference; its oracle is

@@ -32,6 +32,11 @@ How each function is pinned (see tests/test_oracle.py):
                         of the reference's test (test_kv_cache.py:321-342)
   paged_prefill_chunk   rows [P:P+C] of dense_prefill over the whole sequence;
                         P=0 equals dense_prefill
+  window= (decode, prefill)
+                        torch SDPA with the explicit boolean mask
+                        q_idx >= kv_idx and q_idx - kv_idx < window, the
+                        recipe of the reference's debug_swa.py; window >= length
+                        equals no window; decode equals the last prefill row
   quantize_kv_e4m3      torch.float8_e4m3fn conversion (library definition of
                         OCP e4m3fn, round to nearest even), known values
                         464 -> 448, 2**-10 -> 0, max 448
@@ -137,18 +142,23 @@ def kv_gather_loop(k_cache, v_cache, block_tables, seq_lens, block_size: int):
 
 
 def _attend_rows(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, n_zero: int = 0,
-                 causal_offset: Optional[int] = None) -> np.ndarray:
+                 causal_offset: Optional[int] = None, window: int = 0) -> np.ndarray:
     """softmax(scale * q k^T) v for one kv head group.
 
     q ``[R, n_rep, D]``, k/v ``[L, D]`` -> ``[R, n_rep, D]``.  ``n_zero`` extra
     all-zero keys (logit 0, value 0) join the softmax.  ``causal_offset``: row
-    r may only see keys ``j <= causal_offset + r``.
+    r sits at position ``causal_offset + r`` and may only see keys
+    ``j <= causal_offset + r``; with ``window`` > 0 also only keys with
+    ``position - j < window`` (attention/mask.py:83-89).
     """
     logits = scale * np.einsum("rhd,ld->rhl", q, k)  # [R, n_rep, L]
     if causal_offset is not None:
         rows = np.arange(q.shape[0])[:, None, None]
         cols = np.arange(k.shape[0])[None, None, :]
-        logits = np.where(cols <= causal_offset + rows, logits, -np.inf)
+        seen = cols <= causal_offset + rows
+        if window > 0:
+            seen &= (causal_offset + rows) - cols < window
+        logits = np.where(seen, logits, -np.inf)
     m = logits.max(axis=-1, keepdims=True) if logits.shape[-1] else np.full(logits.shape[:-1] + (1,), -np.inf)
     if n_zero > 0:
         m = np.maximum(m, 0.0)
@@ -161,7 +171,7 @@ def _attend_rows(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, n_ze
 
 
 def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, block_size: int, scale: float,
-                 pad_zero_keys: bool = False) -> np.ndarray:
+                 pad_zero_keys: bool = False, window: int = 0) -> np.ndarray:
     """Decode attention at exact lengths (flex_backend.py:187-231 with a length mask).
 
     q ``[B, Hq, D]``; caches ``[total_slots, Hkv, D]``; returns float64 ``[B, Hq, D]``.
@@ -170,7 +180,9 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, block_size: int, s
     table are all-zero keys, as in the reference's gather (:274).  With
     ``pad_zero_keys`` every sequence additionally sees ``max(seq_lens) - len``
     zero keys: the reference's unmasked attention over the zero-padded batch.
-    A sequence with no keys at all yields zeros.
+    A sequence with no keys at all yields zeros.  ``window`` > 0: the query (at
+    position len-1) sees only keys ``j`` with ``len-1 - j < window``
+    (attention/mask.py:83-89 applied to the decode row).
     """
     q, kc, vc = to_f64(q), to_f64(k_cache), to_f64(v_cache)
     batch, hq, d = q.shape
@@ -182,17 +194,19 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, block_size: int, s
         n = int(seq_lens[b])
         blocks = np.asarray(block_tables[b], dtype=np.int64)
         n_ok = max(0, min(n, len(blocks) * block_size))
-        pos = np.arange(n_ok)
+        first = max(0, n - window) if window > 0 else 0
+        pos = np.arange(min(first, n_ok), n_ok)
         slots = blocks[pos // block_size] * block_size + pos % block_size
-        n_zero = (n - n_ok) + (max_len - n if pad_zero_keys else 0)
+        n_zero = (n - max(n_ok, first)) + (max_len - n if pad_zero_keys else 0)
         for g in range(hkv):
             qg = q[b, g * n_rep : (g + 1) * n_rep][None]  # [1, n_rep, D]
             out[b, g * n_rep : (g + 1) * n_rep] = _attend_rows(qg, kc[slots, g], vc[slots, g], scale, n_zero)[0]
     return out
 
 
-def dense_prefill(q, k, v, scale: float) -> np.ndarray:
-    """Causal attention over the step's own K/V (flex_backend.py:144-185, SDPA is_causal=True).
+def dense_prefill(q, k, v, scale: float, window: int = 0) -> np.ndarray:
+    """Causal attention over the step's own K/V (flex_backend.py:144-185, SDPA is_causal=True; with
+    ``window`` the flex_attention path under causal_sliding_window_mask, attention/mask.py:56-100).
 
     q ``[B, T, Hq, D]``, k/v ``[B, T, Hkv, D]`` -> float64 ``[B, T, Hq, D]``.
     """
@@ -204,12 +218,12 @@ def dense_prefill(q, k, v, scale: float) -> np.ndarray:
     for b in range(batch):
         for g in range(hkv):
             sl = slice(g * n_rep, (g + 1) * n_rep)
-            out[b, :, sl] = _attend_rows(q[b, :, sl], k[b, :, g], v[b, :, g], scale, causal_offset=0)
+            out[b, :, sl] = _attend_rows(q[b, :, sl], k[b, :, g], v[b, :, g], scale, causal_offset=0, window=window)
     return out
 
 
 def paged_prefill_chunk(q, k_cache, v_cache, block_tables, prefix_lens, chunk_lens, block_size: int,
-                        scale: float) -> np.ndarray:
+                        scale: float, window: int = 0) -> np.ndarray:
     """Chunked prefill over a cached prefix (composition; not a reference function).
 
     Defined as: gather keys ``0 .. P+C-1`` through the block table
@@ -230,7 +244,8 @@ def paged_prefill_chunk(q, k_cache, v_cache, block_tables, prefix_lens, chunk_le
         slots = blocks[pos // block_size] * block_size + pos % block_size
         for g in range(hkv):
             sl = slice(g * n_rep, (g + 1) * n_rep)
-            out[b, :c, sl] = _attend_rows(q[b, :c, sl], kc[slots, g], vc[slots, g], scale, causal_offset=p)
+            out[b, :c, sl] = _attend_rows(q[b, :c, sl], kc[slots, g], vc[slots, g], scale, causal_offset=p,
+                                          window=window)
     return out
 
 

@@ -41,14 +41,14 @@ SIGNATURES = {
     "pa_decode": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,
-         c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p, c_size_t, c_void_p],
+         c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "pa_decode_split": None,   # same signature as pa_decode, filled in below
     "pa_decode_reduce": None,
     "pa_prefill_paged": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
-         c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_void_p],
+         c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p],
     ),
     "pa_quantize_kv_e4m3": (
         c_int,

@@ -94,13 +94,15 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
                   const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
                   const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale, int batch,
                   int num_q_heads, int num_kv_heads, int head_dim, int block_size, int64_t num_blocks, float scale,
-                  int q_dtype, int kv_dtype, void *workspace, size_t workspace_bytes, void *stream) {
+                  int window, int q_dtype, int kv_dtype, void *workspace, size_t workspace_bytes, void *stream) {
     pa_clear_error();
     PA_REQUIRE(batch >= 0, "batch=%d is negative", batch);
     PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, "head counts / head_dim must be positive");
     PA_REQUIRE(num_q_heads % num_kv_heads == 0, "num_q_heads=%d is not a multiple of num_kv_heads=%d",
                num_q_heads, num_kv_heads);
     PA_REQUIRE(block_size > 0, "block_size=%d must be positive", block_size);
+    PA_REQUIRE(window >= 0, "window=%d is negative (0 = no sliding window)", window);
+    PA_REQUIRE(window == 0 || !extra_zero_keys, "a sliding window cannot be combined with extra_zero_keys");
     PA_REQUIRE(num_blocks >= 0 && bt_stride >= 0, "num_blocks / bt_stride must be non-negative");
     PA_REQUIRE(num_blocks * (int64_t)block_size < (1ll << 40), "pool of %lld blocks is too large", (long long)num_blocks);
     PA_REQUIRE((int64_t)block_size * num_kv_heads * head_dim * 4 < (1ll << 31),
@@ -128,6 +130,7 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     a.p.k_scale = k_scale; a.p.v_scale = v_scale;
     a.p.bs = block_size; a.p.num_blocks = num_blocks;
     a.p.scale_log2 = scale * 1.4426950408889634f;
+    a.p.window = window;
     a.q = q; a.out = out; a.seq_lens = seq_lens; a.extra_zero = extra_zero_keys;
     a.batch = batch;
     a.slot_cap = w.slots;
@@ -174,12 +177,12 @@ extern "C" size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_
     const void *q, const void *k_cache, const void *v_cache, void *out, const int32_t *block_tables,          \
         int64_t bt_stride, const int32_t *seq_lens, const int32_t *extra_zero_keys, const float *k_scale,      \
         const float *v_scale, int batch, int num_q_heads, int num_kv_heads, int head_dim, int block_size,      \
-        int64_t num_blocks, float scale, int q_dtype, int kv_dtype, void *workspace, size_t workspace_bytes,   \
-        void *stream
+        int64_t num_blocks, float scale, int window, int q_dtype, int kv_dtype, void *workspace,                \
+        size_t workspace_bytes, void *stream
 #define PA_DECODE_ARGS                                                                                         \
     q, k_cache, v_cache, out, block_tables, bt_stride, seq_lens, extra_zero_keys, k_scale, v_scale, batch,     \
-        num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, q_dtype, kv_dtype, workspace,      \
-        workspace_bytes, stream
+        num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, window, q_dtype, kv_dtype,         \
+        workspace, workspace_bytes, stream
 
 extern "C" int pa_decode(PA_DECODE_PARAMS) { return decode_launch(kPhaseSplit | kPhaseReduce, PA_DECODE_ARGS); }
 extern "C" int pa_decode_split(PA_DECODE_PARAMS) { return decode_launch(kPhaseSplit, PA_DECODE_ARGS); }

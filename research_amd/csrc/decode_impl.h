@@ -49,6 +49,7 @@ struct PoolArgs {
     int hq, hkv, n_rep, bs;
     int64_t num_blocks;
     float scale_log2;  // softmax scale * log2(e)
+    int window;        // sliding window: a query at position i sees keys j with i - j < window (0 = all keys)
     int hpw, tpw, n_hgroups, n_rgroups;
 };
 
@@ -76,6 +77,11 @@ struct RowwiseArgs {
 };
 
 __device__ __forceinline__ uint4 ld16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }
+
+// First key a query at position n_keys-1 sees under the sliding window (0 without one).
+__device__ __forceinline__ int window_first_key(const PoolArgs &p, int n_keys) {
+    return p.window > 0 ? max(0, n_keys - p.window) : 0;
+}
 
 // 16-byte load of pool data: used once, so it carries the non-temporal hint.
 __device__ __forceinline__ uint4 ld16_stream(const void *p) {
@@ -149,12 +155,12 @@ __device__ __forceinline__ void load_q(float (&qf)[NREP][EPL], const QT *qrow, c
     }
 }
 
-// Attend keys [0, L) restricted to blocks blk_begin, blk_begin+blk_step, ... < blk_end
+// Attend keys [k_lo, L) restricted to blocks blk_begin, blk_begin+blk_step, ... < blk_end
 // of the block-table row `bt_row`, for kv head `kvh`.
 template <typename KV, int D, int NREP, int U>
 __device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EPL> &st,
                                               const float (&qf)[NREP][RowShape<KV, D>::EPL], const PoolArgs &p,
-                                              const int32_t *bt_row, int L, int blk_begin, int blk_end,
+                                              const int32_t *bt_row, int k_lo, int L, int blk_begin, int blk_end,
                                               int blk_step, const LaneRole &role, int kvh) {
     using S = RowShape<KV, D>;
     constexpr int EPL = S::EPL;
@@ -163,9 +169,10 @@ __device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EP
 
     for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
         const int ntok = min(p.bs, L - blk * p.bs);
+        const int tlo = max(0, k_lo - blk * p.bs);  // tokens below it lie before the window
         const int64_t bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
         if (bid < 0 || bid >= p.num_blocks) {
-            if (role.tok_local == 0) st.zero_keys += ntok;
+            if (role.tok_local == 0) st.zero_keys += max(0, ntok - tlo);
             continue;
         }
         const int64_t base = ((bid * p.bs) * p.hkv + kvh) * (int64_t)(D * sizeof(KV)) + (int64_t)role.lir * 16;
@@ -182,7 +189,7 @@ __device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EP
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int t = t0 + u * p.tpw + role.tok_local;
-                ok[u] = t < ntok;
+                ok[u] = t < ntok && t >= tlo;
                 kraw[u] = ok[u] ? ld16_stream(kp + t * tok_stride) : uint4{0, 0, 0, 0};
             }
 #pragma unroll
@@ -251,9 +258,9 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
         (sizeof(KV) == 1 && sizeof(QT) == 2 && (D == 64 || D == 128 || D == 256));
 
     static __device__ __forceinline__ RowState<NREP, S::EPL> run(const PoolArgs &p, const QT *qrow,
-                                                                  const int32_t *bt_row, int L, int blk_begin,
-                                                                  int blk_end, int blk_step, const LaneRole &role,
-                                                                  int lane, int kvh, int rep0) {
+                                                                  const int32_t *bt_row, int k_lo, int L,
+                                                                  int blk_begin, int blk_end, int blk_step,
+                                                                  const LaneRole &role, int lane, int kvh, int rep0) {
         RowState<NREP, S::EPL> out;
         if constexpr (kPacked) {
             using HS = HeadScatter<NREP, S::LPR>;
@@ -273,8 +280,8 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
             st.init();
             const int lane_voff =
                 role.tok_local * (p.hkv * D * (int)sizeof(KV)) + kvh * (D * (int)sizeof(KV)) + role.lir * 16;
-            attend_blocks_pk<KV, QT, D, NREP, U>(st, qpk, p, bt_row, L, blk_begin, blk_end, blk_step, lane, lane_voff,
-                                                 kvh, role.tok_local == 0);
+            attend_blocks_pk<KV, QT, D, NREP, U>(st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step, lane,
+                                                 lane_voff, kvh, role.tok_local == 0);
             StaticFor<NREP>::run([&](auto h) {
                 out.m[h.value] = HS::template bcast<h.value>(st.m);
                 out.l[h.value] = HS::template bcast<h.value>(st.l);
@@ -286,7 +293,7 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
             float qf[NREP][S::EPL];
             load_q<QT, D, NREP, S::EPL>(qf, qrow, p, kvh, rep0, role.d0);
             out.init();
-            attend_blocks<KV, D, NREP, U>(out, qf, p, bt_row, L, blk_begin, blk_end, blk_step, role, kvh);
+            attend_blocks<KV, D, NREP, U>(out, qf, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step, role, kvh);
         }
         return out;
     }
@@ -376,7 +383,11 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
     {
         const int per = (B + kThreads - 1) / kThreads;
         const int lo = min(B, tid * per), hi = min(B, lo + per);
-        auto blocks_of = [&](int b) { return (max(0, a.seq_lens[b]) + p.bs - 1) / p.bs; };
+        // blocks of sequence b that hold visible keys: [first_key(b) / bs, ceil(L / bs))
+        auto blocks_of = [&](int b) {
+            const int len = max(0, a.seq_lens[b]);
+            return (len + p.bs - 1) / p.bs - window_first_key(p, len) / p.bs;
+        };
         int sum = 0;
         for (int b = lo; b < hi; ++b) sum += blocks_of(b);
         s_scan[tid] = sum;
@@ -422,10 +433,12 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
         const int kvh = hg * p.hpw + role.head_local;
         const int rep0 = rg * NREP;
         const int L = a.seq_lens[b];
+        const int k_lo = window_first_key(p, L);  // the query sits at position L-1
+        const int fb = k_lo / p.bs;               // first block with a visible key
 
         RowState<NREP, S::EPL> st = Attender<KV, QT, D, NREP, U>::run(
-            p, reinterpret_cast<const QT *>(a.q) + (int64_t)b * p.hq * D, p.bt + (int64_t)b * p.bt_stride, L,
-            blk0 + wave, blk1, kWaves, role, lane, kvh, rep0);
+            p, reinterpret_cast<const QT *>(a.q) + (int64_t)b * p.hq * D, p.bt + (int64_t)b * p.bt_stride, k_lo, L,
+            fb + blk0 + wave, fb + blk1, kWaves, role, lane, kvh, rep0);
         if (blk0 == 0 && blk1 == nblk) {
             // the whole sequence is ours: write the output row
             const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
@@ -555,9 +568,10 @@ __global__ __launch_bounds__(kThreads) void prefill_rowwise_kernel(const Rowwise
     const int64_t qrow = (int64_t)a.q_starts[b] + i;
 
     const int nblk = L > 0 ? (L + p.bs - 1) / p.bs : 0;
+    const int k_lo = window_first_key(p, max(L, 0));  // the row sits at position L-1
     RowState<NREP, S::EPL> st = Attender<KV, QT, D, NREP, U>::run(
-        p, reinterpret_cast<const QT *>(a.q) + qrow * p.hq * D, p.bt + (int64_t)b * p.bt_stride, L, wave, nblk,
-        kWaves, role, lane, kvh, rep0);
+        p, reinterpret_cast<const QT *>(a.q) + qrow * p.hq * D, p.bt + (int64_t)b * p.bt_stride, k_lo, L,
+        k_lo / p.bs + wave, nblk, kWaves, role, lane, kvh, rep0);
     QT *orow = reinterpret_cast<QT *>(a.out) + qrow * p.hq * D;
     merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
                             [&](int qh, int d, float num, float M, float den) {

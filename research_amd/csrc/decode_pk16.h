@@ -181,14 +181,14 @@ template <> struct StaticFor<0> {
     template <typename F> static __device__ __forceinline__ void run(F &&) {}
 };
 
-// Attend keys [0, L) of blocks blk_begin, blk_begin+blk_step, ... < blk_end.
+// Attend keys [k_lo, L) of blocks blk_begin, blk_begin+blk_step, ... < blk_end.
 // qpk[r][i]: packed pairs of this lane's query elements of head r (raw bits of the query type AT).
 // lane_kvh: the kv head this lane's row belongs to (selects the fp8 scales).
 template <typename KV, typename AT, int D, int NREP, int U>
 __device__ __forceinline__ void attend_blocks_pk(
     PkState<NREP, HeadScatter<NREP, D * (int)sizeof(KV) / 16>::VPL, 2 * PoolWords<KV, AT>::NW> &st,
-    const uint32_t (&qpk)[NREP][PoolWords<KV, AT>::NW], const PoolArgs &p, const int32_t *bt_row, int L, int blk_begin,
-    int blk_end, int blk_step, int lane, int lane_voff, int lane_kvh, bool count_zero_keys) {
+    const uint32_t (&qpk)[NREP][PoolWords<KV, AT>::NW], const PoolArgs &p, const int32_t *bt_row, int k_lo, int L,
+    int blk_begin, int blk_end, int blk_step, int lane, int lane_voff, int lane_kvh, bool count_zero_keys) {
     static_assert(U % 2 == 0, "tokens are consumed in pairs");
     constexpr int LPR = D * (int)sizeof(KV) / 16;
     constexpr bool kFp8 = sizeof(KV) == 1;
@@ -202,9 +202,10 @@ __device__ __forceinline__ void attend_blocks_pk(
 
     for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
         const int ntok = min(p.bs, L - blk * p.bs);
+        const int tlo = max(0, k_lo - blk * p.bs);  // tokens below it lie before the window (first block only)
         const int64_t bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
         if (bid < 0 || bid >= p.num_blocks) {
-            if (count_zero_keys) st.zero_keys += ntok;
+            if (count_zero_keys) st.zero_keys += max(0, ntok - tlo);
             continue;
         }
         // descriptor of the valid part of this block: reads past it return 0
@@ -230,7 +231,7 @@ __device__ __forceinline__ void attend_blocks_pk(
 
             // ---- logits: one (token, head) per lane -----------------------
             float sv[U][VPL];
-            const bool partial = ntok - t0 < p.tpw * U;  // uniform
+            const bool partial = ntok - t0 < p.tpw * U || t0 < tlo;  // uniform
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 uint32_t kw[NW];
@@ -247,7 +248,8 @@ __device__ __forceinline__ void attend_blocks_pk(
 #pragma unroll
                 for (int j = 0; j < VPL; ++j) sv[u][j] *= k_sc;
                 if (partial) {
-                    const bool ok = t0 + u * p.tpw + tok_local < ntok;
+                    const int tt = t0 + u * p.tpw + tok_local;
+                    const bool ok = tt < ntok && tt >= tlo;
 #pragma unroll
                     for (int j = 0; j < VPL; ++j) sv[u][j] = ok ? sv[u][j] : -INFINITY;
                 }

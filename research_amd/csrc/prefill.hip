@@ -9,13 +9,14 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
                                 const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
                                 const int32_t *q_lens, const int32_t *q_starts, int batch, int max_q_len,
                                 int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-                                int64_t num_blocks, float scale, int dtype, void *stream) {
+                                int64_t num_blocks, float scale, int window, int dtype, void *stream) {
     pa_clear_error();
     PA_REQUIRE(batch >= 0 && max_q_len >= 0, "batch=%d max_q_len=%d must be non-negative", batch, max_q_len);
     PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, "head counts / head_dim must be positive");
     PA_REQUIRE(num_q_heads % num_kv_heads == 0, "num_q_heads=%d is not a multiple of num_kv_heads=%d",
                num_q_heads, num_kv_heads);
     PA_REQUIRE(block_size > 0, "block_size=%d must be positive", block_size);
+    PA_REQUIRE(window >= 0, "window=%d is negative (0 = no sliding window)", window);
     PA_REQUIRE(num_blocks >= 0 && bt_stride >= 0, "num_blocks / bt_stride must be non-negative");
     PA_REQUIRE(num_blocks * (int64_t)block_size < (1ll << 40), "pool of %lld blocks is too large", (long long)num_blocks);
     PA_REQUIRE(dtype == PA_F32 || dtype == PA_BF16 || dtype == PA_F16, "dtype=%d is not F32, BF16 or F16", dtype);
@@ -35,6 +36,7 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     a.p.k_scale = nullptr; a.p.v_scale = nullptr;
     a.p.bs = block_size; a.p.num_blocks = num_blocks;
     a.p.scale_log2 = scale * 1.4426950408889634f;
+    a.p.window = window;
     a.q = q; a.out = out; a.ctx_lens = ctx_lens; a.q_lens = q_lens; a.q_starts = q_starts;
     a.batch = batch; a.max_q_len = max_q_len;
     hipStream_t s = (hipStream_t)stream;
@@ -44,7 +46,7 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     const bool force_rowwise = env_rowwise && env_rowwise[0] == '1';
     // (its softmax takes the running maximum of the unscaled logits, which needs scale > 0)
     const prefill_mfma_fn mfma =
-        force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
+        force_rowwise || !(scale > 0.f) || window > 0 ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
     if (mfma) {
         PA_REQUIRE(pa_aligned16(q) && pa_aligned16(out), "q and out must be 16-byte aligned");
         const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;

@@ -19,7 +19,14 @@ Differences from the reference, all deliberate:
 * ``ctx.prefix_lens`` (an added, optional context field) selects chunked
   prefill: the chunk's queries attend the cached prefix and the chunk itself,
   both read from the pool through the block table.
-* ``ctx.block_mask`` objects and ``config.sliding_window`` are not supported
+* ``config.sliding_window`` is applied inside the kernels (a row at position p
+  sees keys ``p - window < j <= p``, attention/mask.py:83-89) instead of through
+  a FlexAttention ``BlockMask``; ``get_block_mask`` therefore returns ``None``.
+  Prefill applies it as the reference does.  Decode in the reference applies a
+  window only when the caller passes ``ctx.block_mask`` (flex_backend.py:220-225)
+  and otherwise attends the whole cache; ``window_in_decode=False`` keeps that,
+  the default ``True`` attends the last ``window`` keys, consistent with prefill.
+* ``ctx.block_mask`` objects (arbitrary FlexAttention masks) are not supported
   and raise ``NotImplementedError`` instead of being ignored.
 """
 
@@ -62,12 +69,18 @@ def _padded_tables(block_tables: Sequence[Sequence[int]]) -> np.ndarray:
 
 
 class HipPagedAttentionBackend:
-    def __init__(self, config: CacheConfig, pad_zero_keys: bool = False) -> None:
+    def __init__(self, config: CacheConfig, pad_zero_keys: bool = False, window_in_decode: bool = True) -> None:
         self._lib = _lib.load()  # raises if the HIP library has not been built
         self.config = config
         self.num_heads_per_kv = 1  # until set_num_heads(), as in the reference (flex_backend.py:31,43-45)
         self.scale = config.head_dim**-0.5
         self.pad_zero_keys = pad_zero_keys
+        if config.sliding_window is not None and config.sliding_window <= 0:
+            raise ValueError(f"sliding_window={config.sliding_window} must be positive")
+        self._window = int(config.sliding_window or 0)
+        self.window_in_decode = window_in_decode
+        if self._window and pad_zero_keys and window_in_decode:
+            raise ValueError("pad_zero_keys cannot be combined with a sliding window in decode")
         self._mask_cache: dict = {}
         self._step_cache: "OrderedDict[int, _StepTensors]" = OrderedDict()
         self._workspace: Optional[Tensor] = None
@@ -92,9 +105,8 @@ class HipPagedAttentionBackend:
         self.num_heads_per_kv = num_heads // self.config.num_kv_heads
 
     def get_block_mask(self, batch_size: int, seq_len: int) -> object:
-        if self.config.sliding_window is None:
-            return None  # plain causal needs no mask object (flex_backend.py:62-63)
-        raise NotImplementedError("sliding_window masks are not supported by the HIP backend")
+        # plain causal needs no mask object (flex_backend.py:62-63); the sliding window is applied by the kernels
+        return None
 
     def clear_mask_cache(self) -> None:
         self._mask_cache.clear()
@@ -245,7 +257,7 @@ class HipPagedAttentionBackend:
         ksc = self.k_scale[layer_idx] if self._fp8 else None
         vsc = self.v_scale[layer_idx] if self._fp8 else None
         out = ops.decode(q3, kc, vc, step.tables, step.seq_lens, cfg.block_size, self.scale, ws, step.extra_zero,
-                         ksc, vsc)
+                         ksc, vsc, window=self._window if self.window_in_decode else 0)
         return out.view(batch, 1, num_heads, head_dim)
 
     # ------------------------------------------------------------------ prefill
@@ -255,8 +267,8 @@ class HipPagedAttentionBackend:
         The dense ``[B, T, Hkv, D]`` inputs are handed to the paged kernel as a
         pool of ``B`` blocks of ``T`` tokens with the identity block table.
         """
-        if ctx.block_mask is not None or self.config.sliding_window is not None:
-            raise NotImplementedError("block_mask / sliding_window are not supported by the HIP backend")
+        if ctx.block_mask is not None:
+            raise NotImplementedError("block_mask objects are not supported by the HIP backend")
         batch, seq_len, num_heads, head_dim = q.shape
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         if out.numel() == 0:
@@ -273,13 +285,13 @@ class HipPagedAttentionBackend:
             k.contiguous().view(batch * seq_len, num_kv, head_dim),
             v.contiguous().view(batch * seq_len, num_kv, head_dim),
             ar.reshape(batch, 1).contiguous(), lens, lens, ar * seq_len, seq_len, seq_len, self.scale,
-            out=out.view(batch * seq_len, num_heads, head_dim))
+            out=out.view(batch * seq_len, num_heads, head_dim), window=self._window)
         return out
 
     def _prefill_paged(self, q: Tensor, layer_idx: int, ctx: InferenceContext) -> Tensor:
         """Chunked prefill: ``q[b]`` holds the last ``T`` positions of a context of ``seq_lens[b]`` keys."""
-        if ctx.block_mask is not None or self.config.sliding_window is not None:
-            raise NotImplementedError("block_mask / sliding_window are not supported by the HIP backend")
+        if ctx.block_mask is not None:
+            raise NotImplementedError("block_mask objects are not supported by the HIP backend")
         if ctx.block_tables is None or ctx.seq_lens is None:
             raise ValueError("Chunked prefill requires block_tables and seq_lens in context")
         if self._fp8:
@@ -305,7 +317,7 @@ class HipPagedAttentionBackend:
         kc, vc = self._layer(layer_idx)
         ops.prefill_paged(q.contiguous().view(batch * seq_len, num_heads, head_dim), kc, vc, step.tables,
                           step.ctx_lens, step.q_lens, step.q_starts, step.max_q_len, cfg.block_size, self.scale,
-                          out=out.view(batch * seq_len, num_heads, head_dim))
+                          out=out.view(batch * seq_len, num_heads, head_dim), window=self._window)
         return out
 
     # ------------------------------------------------------------------ fp8 pool

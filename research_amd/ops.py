@@ -72,10 +72,11 @@ def decode_workspace(q: Tensor, k_cache: Tensor) -> Tensor:
 def decode(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, seq_lens: Tensor, block_size: int,
            scale: float, workspace: Tensor, extra_zero_keys: Optional[Tensor] = None,
            k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None, out: Optional[Tensor] = None,
-           entry: str = "pa_decode") -> Tensor:
+           entry: str = "pa_decode", window: int = 0) -> Tensor:
     """Paged decode attention; q ``[B, Hq, D]`` -> out ``[B, Hq, D]`` (same dtype).
 
-    ``entry`` may name ``pa_decode_split`` or ``pa_decode_reduce`` to run one pass only.
+    ``entry`` may name ``pa_decode_split`` or ``pa_decode_reduce`` to run one pass only; ``window`` > 0
+    restricts every sequence to its last ``window`` keys.
     """
     batch, hq, d = q.shape
     total_slots, hkv, _ = k_cache.shape
@@ -83,22 +84,24 @@ def decode(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, se
         out = torch.empty_like(q)
     _run(entry, _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_tables), block_tables.shape[1],
          _ptr(seq_lens), _ptr(extra_zero_keys), _ptr(k_scale), _ptr(v_scale), batch, hq, hkv, d, block_size,
-         total_slots // block_size, float(scale), PA_DTYPE[q.dtype], PA_DTYPE[k_cache.dtype], _ptr(workspace),
+         total_slots // block_size, float(scale), int(window), PA_DTYPE[q.dtype], PA_DTYPE[k_cache.dtype],
+         _ptr(workspace),
          workspace.numel() * workspace.element_size(), _stream(q))
     return out
 
 
 def prefill_paged(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, ctx_lens: Tensor,
                   q_lens: Tensor, q_starts: Tensor, max_q_len: int, block_size: int, scale: float,
-                  out: Optional[Tensor] = None) -> Tensor:
-    """Causal prefill over a paged context; q ``[total_q, Hq, D]`` packed rows."""
+                  out: Optional[Tensor] = None, window: int = 0) -> Tensor:
+    """Causal prefill over a paged context; q ``[total_q, Hq, D]`` packed rows; ``window`` > 0 adds the
+    sliding window (a row at position p sees keys p - window < j <= p)."""
     _, hq, d = q.shape
     total_slots, hkv, _ = k_cache.shape
     if out is None:
         out = torch.empty_like(q)
     _run("pa_prefill_paged", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_tables),
          block_tables.shape[1], _ptr(ctx_lens), _ptr(q_lens), _ptr(q_starts), block_tables.shape[0], max_q_len, hq,
-         hkv, d, block_size, total_slots // block_size, float(scale), PA_DTYPE[q.dtype], _stream(q))
+         hkv, d, block_size, total_slots // block_size, float(scale), int(window), PA_DTYPE[q.dtype], _stream(q))
     return out
 
 

@@ -95,8 +95,12 @@ def test_out_of_range_slot_is_an_index_error():
 
 def test_unsupported_features_raise():
     be = HipPagedAttentionBackend(_cfg(sliding_window=4))
-    with pytest.raises(NotImplementedError):
-        be.get_block_mask(1, 8)
+    assert be.get_block_mask(1, 8) is None  # the window is applied inside the kernels, no mask object
+    with pytest.raises(ValueError):
+        HipPagedAttentionBackend(_cfg(sliding_window=0))
+    with pytest.raises(ValueError):
+        HipPagedAttentionBackend(_cfg(sliding_window=4), pad_zero_keys=True)
+    assert HipPagedAttentionBackend(_cfg(sliding_window=4), pad_zero_keys=True, window_in_decode=False)
     with pytest.raises(ValueError):
         HipPagedAttentionBackend(_cfg(kv_format="int4"))
     with pytest.raises(ValueError):

@@ -74,11 +74,11 @@ def test_gather_argument_errors():
 
 def _decode_args(**kw):
     a = dict(q=FAKE, k=FAKE, v=FAKE, out=FAKE, bt=FAKE, bt_stride=4, lens=FAKE, ez=None, ks=None, vs=None,
-             batch=2, hq=32, hkv=8, d=128, bs=16, nb=64, scale=0.088, qd=_lib.PA_BF16, kvd=_lib.PA_BF16,
+             batch=2, hq=32, hkv=8, d=128, bs=16, nb=64, scale=0.088, window=0, qd=_lib.PA_BF16, kvd=_lib.PA_BF16,
              ws=FAKE, ws_bytes=1 << 30, stream=None)
     a.update(kw)
     return [a[k] for k in ("q", "k", "v", "out", "bt", "bt_stride", "lens", "ez", "ks", "vs", "batch", "hq", "hkv",
-                           "d", "bs", "nb", "scale", "qd", "kvd", "ws", "ws_bytes", "stream")]
+                           "d", "bs", "nb", "scale", "window", "qd", "kvd", "ws", "ws_bytes", "stream")]
 
 
 def test_decode_argument_errors():
@@ -121,7 +121,7 @@ def test_decode_workspace_arithmetic():
 
 
 def test_prefill_and_quantize_argument_errors():
-    args = [FAKE, FAKE, FAKE, FAKE, FAKE, 4, FAKE, FAKE, FAKE, 2, 16, 32, 8, 128, 16, 64, 0.088, _lib.PA_FP8_E4M3,
+    args = [FAKE, FAKE, FAKE, FAKE, FAKE, 4, FAKE, FAKE, FAKE, 2, 16, 32, 8, 128, 16, 64, 0.088, 0, _lib.PA_FP8_E4M3,
             None]
     rc, msg = _status("pa_prefill_paged", *args)
     assert rc == _lib.PA_ERR_INVALID_ARG and "dtype" in msg

@@ -232,3 +232,34 @@ def test_fp8_backend_prefill_then_decode_appends():
         want = po.paged_decode(qn[:, 0], kd, vd, ctx.block_tables, ctx.seq_lens, bs, backend.scale)
         assert_close(out[:, 0], want, 6e-2, f"decode step {step}")
     assert (backend.k_cache[0].view(torch.uint8) == 0).all()  # the other layer was not touched
+
+
+def test_sliding_window_through_the_backend():
+    """CacheConfig.sliding_window: prefill as the reference masks it, decode over the last `window` keys
+    (or, with window_in_decode=False, over everything, as the reference's decode without a block_mask)."""
+    announce("backend sliding window")
+    g = torch.Generator().manual_seed(51)
+    hq, hkv, d, bs, window = 8, 2, 64, 16, 6
+    config = CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=8, block_size=bs, device="cuda",
+                         sliding_window=window)
+    outs = {}
+    for in_decode in (True, False):
+        backend = FlexAttentionBackend(config, window_in_decode=in_decode)
+        backend.set_num_heads(hq)
+        cache = PagedKVCache(8, bs)
+        n = 21
+        q = torch.randn(1, n, hq, d, generator=g).to(torch.bfloat16)
+        k = torch.randn(1, n, hkv, d, generator=g).to(torch.bfloat16)
+        v = torch.randn(1, n, hkv, d, generator=g).to(torch.bfloat16)
+        ctx, _ = allocate_and_build_context(cache, seq_id=0, token_ids=list(range(n)))
+        out = backend.forward(q.cuda(), k.cuda(), v.cuda(), 0, ctx)
+        assert_close(out, po.dense_prefill(q, k, v, backend.scale, window=window), 2e-2, "windowed prefill")
+        q1 = torch.randn(1, 1, hq, d, generator=g).to(torch.bfloat16)
+        k1 = torch.randn(1, 1, hkv, d, generator=g).to(torch.bfloat16)
+        v1 = torch.randn(1, 1, hkv, d, generator=g).to(torch.bfloat16)
+        ctx = extend_and_build_context(cache, seq_id=0, new_token=99, current_len=n)
+        out = backend.forward(q1.cuda(), k1.cuda(), v1.cuda(), 0, ctx)
+        want = po.paged_decode(q1[:, 0], backend.k_cache[0].cpu(), backend.v_cache[0].cpu(), ctx.block_tables,
+                               ctx.seq_lens, bs, backend.scale, window=window if in_decode else 0)
+        assert_close(out[:, 0], want, 2e-2, f"decode, window_in_decode={in_decode}")
+        outs[in_decode] = out

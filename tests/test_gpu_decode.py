@@ -12,7 +12,7 @@ import torch
 from oracle import paged_oracle as po
 from research_amd import ops
 from research_amd.workloads import make_decode
-from tests.gpu_helpers import DEV, announce, assert_close, run_decode
+from tests.gpu_helpers import DEV, announce, assert_close, run_decode, tables_to_device
 
 pytestmark = pytest.mark.gpu
 
@@ -187,3 +187,65 @@ def test_c5_fp8_reduced():
     got = run_decode(w.q.to(DEV), kb, vb, _lists(w), w.seq_lens, w.block_size, w.scale, k_scale=ks, v_scale=vs)
     assert_close(got, want, 6e-2, "c5 fp8")
     assert_close(got, want, 2e-2, "c5 fp8 (the arithmetic itself is as tight as bf16)")
+
+
+@pytest.mark.parametrize("window", [1, 16, 17, 100, 1000, 5000])
+def test_sliding_window_decode(window):
+    """Only the last `window` keys count; blocks wholly before the window are not visited."""
+    announce(f"decode window {window}")
+    w = make_decode("c4", batch=9, len_range=(1, 3000), seed=13)
+    q, kp, vp = w.q.to(DEV), w.k_pool.to(DEV), w.v_pool.to(DEV)
+    tables = tables_to_device(_lists(w))
+    lens = torch.from_numpy(w.seq_lens.astype(np.int32)).to(DEV)
+    ws = ops.decode_workspace(q, kp)
+    got = ops.decode(q, kp, vp, tables, lens, w.block_size, w.scale, ws, window=window)
+    want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, w.block_size, w.scale, window=window)
+    assert_close(got, want, 2e-2, f"window {window}")
+    if window >= int(w.seq_lens.max()):
+        assert torch.equal(got, ops.decode(q, kp, vp, tables, lens, w.block_size, w.scale, ws))
+
+
+def test_sliding_window_decode_other_types_and_garbage_before_the_window():
+    announce("decode window fp32 / fp8 / poisoned prefix")
+    w = make_decode("c1")
+    lists = _lists(w)
+    got = run_decode(w.q.to(DEV), w.k_pool.to(DEV), w.v_pool.to(DEV), lists, w.seq_lens, w.block_size, w.scale)
+    q, kp, vp = w.q.to(DEV), w.k_pool.to(DEV), w.v_pool.to(DEV)
+    tables = tables_to_device(lists)
+    lens = torch.from_numpy(w.seq_lens.astype(np.int32)).to(DEV)
+    ws = ops.decode_workspace(q, kp)
+    for window in (3, 20):
+        got = ops.decode(q, kp, vp, tables, lens, w.block_size, w.scale, ws, window=window)
+        want = po.paged_decode(w.q, w.k_pool, w.v_pool, lists, w.seq_lens, w.block_size, w.scale, window=window)
+        assert_close(got, want, 1e-5, f"c1 window {window}")
+    w = make_decode("c5", batch=3, len_range=(200, 900))
+    k8, ks = ops.quantize_kv_e4m3(w.k_pool.to(DEV), w.block_size)
+    v8, vs = ops.quantize_kv_e4m3(w.v_pool.to(DEV), w.block_size)
+    q = w.q.to(DEV)
+    tables = tables_to_device(_lists(w))
+    lens = torch.from_numpy(w.seq_lens.astype(np.int32)).to(DEV)
+    ws = ops.decode_workspace(q, k8)
+    got = ops.decode(q, k8, v8, tables, lens, w.block_size, w.scale, ws, k_scale=ks, v_scale=vs, window=77)
+    kd = po.dequantize_kv_e4m3(k8.cpu().view(torch.uint8), ks.cpu(), w.block_size)
+    vd = po.dequantize_kv_e4m3(v8.cpu().view(torch.uint8), vs.cpu(), w.block_size)
+    assert_close(got, po.paged_decode(w.q, kd, vd, _lists(w), w.seq_lens, w.block_size, w.scale, window=77), 6e-2,
+                 "fp8 window")
+    # blocks wholly before the window may hold anything, including NaN: they are never read; older keys inside
+    # the window's first block are real keys of the sequence (finite) and are masked out by selection
+    w = make_decode("c2", batch=2, len_range=(300, 400), seed=3)
+    kp, vp = w.k_pool.clone(), w.v_pool.clone()
+    window = 50
+    for b in range(2):
+        n = int(w.seq_lens[b])
+        first_block = (n - window) // 16
+        for pos in range(n - window):
+            slot = int(w.block_tables[b][pos // 16]) * 16 + pos % 16
+            kp[slot] = float("nan") if pos // 16 < first_block else 1.0e4
+            vp[slot] = float("nan") if pos // 16 < first_block else -1.0e4
+    q = w.q.to(DEV)
+    tables = tables_to_device(_lists(w))
+    lens = torch.from_numpy(w.seq_lens.astype(np.int32)).to(DEV)
+    got = ops.decode(q, kp.to(DEV), vp.to(DEV), tables, lens, 16, w.scale, ops.decode_workspace(q, kp.to(DEV)),
+                     window=window)
+    want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, 16, w.scale, window=window)
+    assert_close(got, want, 2e-2, "poisoned keys before the window")

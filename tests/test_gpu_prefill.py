@@ -97,3 +97,33 @@ def test_c3_reduced_shared_prefix():
                             torch.cat([w.k_prefix, w.k_chunk[s]])[None], torch.cat([w.v_prefix, w.v_chunk[s]])[None],
                             w.scale)
     assert_close(got[s], full[0, 512:], 2e-2, "rows of the full-sequence prefill")
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+def test_sliding_window_prefill(dtype, tol):
+    """Chunked and dense prefill under a sliding window (the vector kernel runs windowed calls)."""
+    announce(f"prefill window {dtype}")
+    w = make_prefill_c3(num_seqs=3, prefix_len=96, chunk_len=40, num_q_heads=8, num_kv_heads=2, head_dim=64,
+                        dtype=dtype)
+    shape = (w.num_blocks * w.block_size, w.num_kv_heads, w.head_dim)
+    kc = torch.zeros(shape, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    ops.kv_scatter(kc, vc, w.k_prefix.to(DEV), w.v_prefix.to(DEV), torch.from_numpy(w.prefix_slots()).to(DEV))
+    ops.kv_scatter(kc, vc, w.k_chunk.reshape(-1, *shape[1:]).to(DEV), w.v_chunk.reshape(-1, *shape[1:]).to(DEV),
+                   torch.from_numpy(w.chunk_slots()).to(DEV))
+    S, C, P = w.num_seqs, w.chunk_len, w.prefix_len
+    q = w.q.reshape(S * C, w.num_q_heads, w.head_dim).to(DEV)
+    tables = tables_to_device(w.block_tables)
+    for window in (1, 7, 40, 41, 130, 1000):
+        got = ops.prefill_paged(q, kc, vc, tables, _i32([P + C] * S), _i32([C] * S), _i32(np.arange(S) * C), C,
+                                w.block_size, w.scale, window=window).reshape(S, C, w.num_q_heads, w.head_dim)
+        want = po.paged_prefill_chunk(w.q, kc.cpu(), vc.cpu(), w.block_tables, [P] * S, [C] * S, w.block_size,
+                                      w.scale, window=window)
+        assert_close(got, want, tol, f"chunked window {window}")
+    # dense: the step's own K/V as a pool of S blocks of C tokens
+    k = w.k_chunk.reshape(S * C, *shape[1:]).to(DEV)
+    v = w.v_chunk.reshape(S * C, *shape[1:]).to(DEV)
+    ident = torch.arange(S, dtype=torch.int32, device=DEV).reshape(S, 1).contiguous()
+    got = ops.prefill_paged(q, k, v, ident, _i32([C] * S), _i32([C] * S), _i32(np.arange(S) * C), C, C, w.scale,
+                            window=9).reshape(S, C, w.num_q_heads, w.head_dim)
+    assert_close(got, po.dense_prefill(w.q, w.k_chunk, w.v_chunk, w.scale, window=9), tol, "dense window 9")

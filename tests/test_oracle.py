@@ -413,3 +413,63 @@ def test_fp8_append_restarts_a_recycled_block_and_skips_bad_slots():
     assert (bits[0].view(torch.float8_e4m3fn).to(torch.float32) == 448.0).all()
     po.append_kv_e4m3(bits, scale, torch.full((1, hkv, d), 1.0), [99], bs)  # outside the pool: ignored
     assert float(scale[1, 0]) == 1.0 and int(bits[bs:].max()) == 0
+
+
+# ---------------------------------------------------------------- sliding window
+def _swa_sdpa(q, k, v, scale, window):
+    """The recipe of the reference's debug_swa.py (:56-82): tril mask AND (row - col) < window, SDPA with the
+    explicit -inf mask.  q [B,T,Hq,D], k/v [B,T,Hkv,D] float32."""
+    t = q.shape[1]
+    n_rep = q.shape[2] // k.shape[2]
+    row = torch.arange(t)[:, None]
+    col = torch.arange(t)[None, :]
+    keep = torch.tril(torch.ones(t, t, dtype=torch.bool)) & ((row - col) < window)
+    mask = torch.where(keep, 0.0, float("-inf"))[None, None]
+    qt = q.transpose(1, 2)
+    kt = k.transpose(1, 2).repeat_interleave(n_rep, dim=1)
+    vt = v.transpose(1, 2).repeat_interleave(n_rep, dim=1)
+    return torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, attn_mask=mask, scale=scale).transpose(1, 2)
+
+
+def test_window_prefill_matches_the_reference_recipe():
+    g = torch.Generator().manual_seed(41)
+    b, t, hq, hkv, d = 2, 16, 4, 2, 8  # debug_swa.py uses seq_len 16, window 4
+    q, k, v = (torch.randn(b, t, h, d, generator=g) for h in (hq, hkv, hkv))
+    scale = d ** -0.5
+    for window in (1, 4, 7):
+        want = _swa_sdpa(q, k, v, scale, window)
+        np.testing.assert_allclose(po.dense_prefill(q, k, v, scale, window=window), want.numpy(), rtol=1e-4, atol=1e-4)
+    # a window that covers the sequence is plain causal attention (debug_swa.py:131-150)
+    np.testing.assert_allclose(po.dense_prefill(q, k, v, scale, window=t + 1), po.dense_prefill(q, k, v, scale),
+                               rtol=0, atol=1e-12)
+    assert not np.allclose(po.dense_prefill(q, k, v, scale, window=4), po.dense_prefill(q, k, v, scale))
+
+
+def test_window_decode_is_the_last_row_of_windowed_prefill():
+    g = torch.Generator().manual_seed(42)
+    hq, hkv, d, bs, nb = 4, 2, 8, 4, 12
+    lens = [13, 5, 1, 9]
+    perm = torch.randperm(nb, generator=g).tolist()
+    tables = [perm[0:4], perm[4:6], perm[6:7], perm[7:10]]
+    kc = torch.randn(nb * bs, hkv, d, generator=g)
+    vc = torch.randn(nb * bs, hkv, d, generator=g)
+    q = torch.randn(len(lens), hq, d, generator=g)
+    scale = 0.3
+    for window in (1, 3, 6, 100):
+        got = po.paged_decode(q, kc, vc, tables, lens, bs, scale, window=window)
+        for b, n in enumerate(lens):
+            slots = [tables[b][p // bs] * bs + p % bs for p in range(n)]
+            qf = torch.zeros(1, n, hq, d)
+            qf[0, -1] = q[b]
+            want = _swa_sdpa(qf, kc[slots][None], vc[slots][None], scale, window)[0, -1]
+            np.testing.assert_allclose(got[b], want.numpy(), rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(po.paged_decode(q, kc, vc, tables, lens, bs, scale, window=100),
+                               po.paged_decode(q, kc, vc, tables, lens, bs, scale), rtol=0, atol=1e-12)
+    # chunked prefill: rows [P:P+C] of the windowed dense result
+    p_len, c_len, window = 7, 6, 5
+    slots = [tables[0][p // bs] * bs + p % bs for p in range(p_len + c_len)]
+    qc = torch.randn(1, c_len, hq, d, generator=g)
+    qf = torch.cat([torch.zeros(1, p_len, hq, d), qc], 1)
+    want = _swa_sdpa(qf, kc[slots][None], vc[slots][None], scale, window)[:, p_len:]
+    got = po.paged_prefill_chunk(qc, kc, vc, [tables[0]], [p_len], [c_len], bs, scale, window=window)
+    np.testing.assert_allclose(got, want.numpy(), rtol=1e-4, atol=1e-5)
