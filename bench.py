@@ -3,7 +3,7 @@
 
 One step = one ``pa_decode`` call (split-K pass + reduction pass) over one
 batch of the synthetic workload, inputs resident in HBM.  The headline
-workload is BASELINE configuration 4 (Llama-3-8B shape, B=256, bf16 pool,
+workload is workload c4 (Llama-3-8B shape, B=256, bf16 pool,
 lognormal context lengths, seed 1004).  Prints one JSON line.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1]

@@ -27,7 +27,7 @@ def _gpu_decode(w, **kw):
 
 
 def test_c1_fp32_masked_and_pad_zero_keys():
-    """BASELINE config 1 in both semantics; the padded one against the literal restatement too."""
+    """workload c1 in both semantics; the padded one against the literal restatement too."""
     announce("decode c1 fp32")
     w = make_decode("c1")
     want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, w.block_size, w.scale)
@@ -42,7 +42,7 @@ def test_c1_fp32_masked_and_pad_zero_keys():
 
 
 def test_c2_bf16_full_size():
-    """BASELINE config 2 at full size (B=64, 141 622 keys)."""
+    """workload c2 at full size (B=64, 141 622 keys)."""
     announce("decode c2 bf16 full")
     w = make_decode("c2")
     assert w.total_tokens == 141622
@@ -51,7 +51,7 @@ def test_c2_bf16_full_size():
 
 
 def test_c4_shape_reduced_batch():
-    """BASELINE config 4's shape (Hq=32, Hkv=8, D=128, lognormal lengths) on 24 sequences."""
+    """workload c4's shape (Hq=32, Hkv=8, D=128, lognormal lengths) on 24 sequences."""
     announce("decode c4 reduced")
     w = make_decode("c4", batch=24, len_range=(64, 6000))
     want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, w.block_size, w.scale)
@@ -176,7 +176,7 @@ def test_quantize_matches_torch_e4m3_bit_for_bit():
 
 
 def test_c5_fp8_reduced():
-    """BASELINE config 5's shape with shorter contexts: e4m3 pool, per-(block, head) scales, bf16 q."""
+    """workload c5's shape with shorter contexts: e4m3 pool, per-(block, head) scales, bf16 q."""
     announce("decode c5 fp8 reduced")
     w = make_decode("c5", batch=4, len_range=(3000, 9000))
     kb, ks = ops.quantize_kv_e4m3(w.k_pool.to(DEV), w.block_size)

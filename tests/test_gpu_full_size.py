@@ -1,4 +1,4 @@
-"""The BASELINE configurations at full size on the GPU.
+"""The benchmark workloads (research_amd/workloads.py) at full size on the GPU.
 
 The CPU checker cannot attend 840 000 keys x 32 heads in test time, so the
 full-size runs are checked three ways: the checker on a sample of sequences
@@ -72,7 +72,7 @@ def _assert_mean(got, want, rel, floor, what):
 
 
 def test_c4_full_size():
-    """BASELINE config 4: B=256, 840 539 keys in 52 656 blocks, bf16."""
+    """workload c4: B=256, 840 539 keys in 52 656 blocks, bf16."""
     announce("decode c4 full size")
     w = make_decode("c4")
     assert w.batch == 256 and w.total_tokens == 840539
@@ -96,7 +96,7 @@ def test_c4_full_size():
 
 
 def test_c5_full_size_fp8():
-    """BASELINE config 5: B=8, 802 997 keys, fp8-e4m3 pool with per-(block, kv head) scales."""
+    """workload c5: B=8, 802 997 keys, fp8-e4m3 pool with per-(block, kv head) scales."""
     announce("decode c5 full size")
     w = make_decode("c5")
     assert w.batch == 8 and w.total_tokens == 802997
@@ -123,7 +123,7 @@ def test_c5_full_size_fp8():
 
 
 def test_c3_full_size_two_kernels_and_sample():
-    """BASELINE config 3: 32 x (2048 shared + 256 own) tokens; matrix-core kernel against the vector kernel on
+    """workload c3: 32 x (2048 shared + 256 own) tokens; matrix-core kernel against the vector kernel on
     every output element, and against the checker on three sequences."""
     announce("prefill c3 full size")
     w = make_prefill_c3()

@@ -67,7 +67,7 @@ def test_scatter_rows_not_multiple_of_16_bytes():
 
 
 def test_scatter_c3_append_full_size():
-    """BASELINE config 3 append: 32 x 256 new tokens into a 640-block pool next to a shared prefix."""
+    """workload c3 append: 32 x 256 new tokens into a 640-block pool next to a shared prefix."""
     announce("scatter c3 full size")
     w = make_prefill_c3()
     shape = (w.num_blocks * w.block_size, w.num_kv_heads, w.head_dim)

@@ -85,7 +85,7 @@ def test_chunked_prefill_ragged_chunks_and_prefixes():
 
 
 def test_c3_reduced_shared_prefix():
-    """BASELINE config 3's head shape with 4 sequences sharing a 512-token prefix, 64-token chunks."""
+    """workload c3's head shape with 4 sequences sharing a 512-token prefix, 64-token chunks."""
     announce("chunked prefill c3 reduced")
     w = make_prefill_c3(num_seqs=4, prefix_len=512, chunk_len=64)
     got, kc, vc = _run_chunked(w)
