@@ -248,6 +248,21 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         lane_v = tok_ofs + (uint32_t)((ld_slot ^ G::swz_v(row)) * 16);
     }
     int bid_win = -1;
+    // Other block sizes (dense prefill hands over whole sequences as single blocks): the loads of a wave walk
+    // the context 64 keys per tile, so (table entry, offset in the block) of each of the wave's loads is
+    // advanced incrementally; block ids come from a window of 64 table entries starting at win_base.  A tile is
+    // regular for the wave when its rows exist, no load straddles a block boundary and every block is present.
+    const uint32_t lane_g = (uint32_t)(ld_row * tok_stride);  // + the swizzled chunk, per tensor, below
+    int g_blk[NLW], g_off[NLW];  // of the next tile this wave issues
+    int win_base = -(1 << 30);
+    if (!BS16) {
+#pragma unroll
+        for (int n = 0; n < NLW; ++n) {
+            const int key_first = (n * kPfWaves + wave) * G::RPL;
+            g_blk[n] = key_first / p.bs;
+            g_off[n] = key_first % p.bs;
+        }
+    }
     // Loads of one tile into its ring stage.  Returns true if the wave issued exactly 2*NLW direct loads and no
     // other vector memory operation after them (what the load-count waits below rely on).
     auto issue = [&](int tile) PF_INLINE -> bool {
@@ -278,8 +293,55 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
                 }
                 return true;
             }
+        } else {
+            bool regular = (tile + 1) * kPfKeys <= ctx_len && g_blk[NLW - 1] < p.bt_stride &&
+                           g_blk[NLW - 1] - g_blk[0] < 64 && (int64_t)p.num_blocks * p.bs <= 0xffffffffll;
+            if (regular && (g_blk[0] < win_base || g_blk[NLW - 1] >= win_base + 64)) {  // move the id window
+                win_base = g_blk[0];
+                const int idx = win_base + lane;
+                int v = -1;
+                if (idx < p.bt_stride) v = pf_load_i32(bt_row + idx);
+                pf_wait_loads<0>();
+                asm volatile("" : "+v"(v));
+                bid_win = v;
+            }
+            uint32_t g_row[NLW];  // pool row (slot) of the first row of each load
+#pragma unroll
+            for (int n = 0; n < NLW; ++n) {
+                g_row[n] = 0;
+                if (regular) {
+                    const int64_t bid = __builtin_amdgcn_readlane(bid_win, g_blk[n] - win_base);
+                    regular = g_off[n] + G::RPL <= p.bs && bid >= 0 && bid < p.num_blocks;
+                    g_row[n] = (uint32_t)(bid * p.bs + g_off[n]);
+                }
+            }
+            // advance to the next tile (tiles are issued in increasing order, each exactly once)
+#pragma unroll
+            for (int n = 0; n < NLW; ++n) {
+                g_off[n] += kPfKeys;
+                if (p.bs >= kPfKeys) {
+                    if (g_off[n] >= p.bs) { g_off[n] -= p.bs; g_blk[n] += 1; }
+                } else {
+                    g_blk[n] += g_off[n] / p.bs;
+                    g_off[n] %= p.bs;
+                }
+            }
+            if (regular) {
+#pragma unroll
+                for (int n = 0; n < NLW; ++n) {
+                    const int l = n * kPfWaves + wave;  // uniform
+                    const int row = l * G::RPL + ld_row;  // row of the tile this lane fills (its swizzle)
+                    const uint64_t ofs = (uint64_t)g_row[n] * (uint32_t)tok_stride;  // 32 x 32 -> 64 bits, scalar
+                    uint32_t lk = lane_g + (uint32_t)((ld_slot ^ G::swz_k(row)) * 16);
+                    uint32_t lv = lane_g + (uint32_t)((ld_slot ^ G::swz_v(row)) * 16);
+                    asm volatile("" : "+v"(lk), "+v"(lv));
+                    pf_dma16(dst0 + l * G::RPL * G::RB, pf_scalar_ptr(pool_k + ofs), lk);
+                    pf_dma16(dst0 + G::BYTES + l * G::RPL * G::RB, pf_scalar_ptr(pool_v + ofs), lv);
+                }
+                return true;
+            }
         }
-        // tile with rows past the context end or missing blocks, or another block size: per-lane addresses
+        // tile with rows past the context end, missing blocks or loads across block boundaries: per-lane addresses
 #pragma unroll
         for (int n = 0; n < NLW; ++n) {
             const int l = n * kPfWaves + wave;  // uniform
