@@ -127,3 +127,34 @@ def test_sliding_window_prefill(dtype, tol):
     got = ops.prefill_paged(q, k, v, ident, _i32([C] * S), _i32([C] * S), _i32(np.arange(S) * C), C, C, w.scale,
                             window=9).reshape(S, C, w.num_q_heads, w.head_dim)
     assert_close(got, po.dense_prefill(w.q, w.k_chunk, w.v_chunk, w.scale, window=9), tol, "dense window 9")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("d", [32, 64, 128])
+@pytest.mark.parametrize("hq,hkv", [(4, 4), (6, 2), (8, 1)])
+def test_matrix_core_kernel_shapes_and_block_sizes(dtype, d, hq, hkv):
+    """The matrix-core kernel over ragged chunks and prefixes for block sizes that take the scalar-base loads
+    (16; 8, 64, 96 via the incremental walk) and one that makes loads straddle blocks (5), with group sizes
+    1, 3 (odd: a wave's two column tiles are different row blocks) and 8."""
+    announce(f"prefill mfma shapes {dtype} d={d} hq={hq} hkv={hkv}")
+    rng = np.random.default_rng(100 + d + hq)
+    for bs in (16, 8, 5, 64, 96):
+        prefix = [0, 130, 67, 300, 1]
+        chunk = [70, 33, 129, 1, 64]
+        cmax = max(chunk)
+        need = [-(-(p + c) // bs) for p, c in zip(prefix, chunk)]
+        nb = sum(need) + 3
+        perm = rng.permutation(nb)
+        tables, at = [], 0
+        for n in need:
+            tables.append(perm[at : at + n].tolist())
+            at += n
+        kc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
+        vc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
+        q = torch.from_numpy(rng.standard_normal((len(chunk), cmax, hq, d)).astype(np.float32)).to(dtype)
+        want = po.paged_prefill_chunk(q, kc, vc, tables, prefix, chunk, bs, d ** -0.5)
+        out = torch.zeros(len(chunk) * cmax, hq, d, device=DEV, dtype=dtype)
+        ops.prefill_paged(q.reshape(-1, hq, d).to(DEV), kc.to(DEV), vc.to(DEV), tables_to_device(tables),
+                          _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk), _i32(np.arange(len(chunk)) * cmax),
+                          cmax, bs, d ** -0.5, out=out)
+        assert_close(out.reshape(len(chunk), cmax, hq, d), want, 2e-2, f"block_size {bs}")
