@@ -172,7 +172,7 @@ int pa_decode_reduce(const void *q, const void *k_cache, const void *v_cache, vo
  *   max_q_len: upper bound of q_lens (grid sizing)
  *   window   : 0, or the sliding window of CacheConfig.sliding_window (attention/config.py:31): row i at
  *              position p = ctx_lens[b] - q_lens[b] + i attends keys p - window < j <= p
- *              (attention/mask.py:83-89).  Windowed calls run on the vector path.
+ *              (attention/mask.py:83-89); tiles wholly before the window of a workgroup's rows are not loaded.
  */
 int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, void *out,
                      const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,

@@ -46,7 +46,7 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     const bool force_rowwise = env_rowwise && env_rowwise[0] == '1';
     // (its softmax takes the running maximum of the unscaled logits, which needs scale > 0)
     const prefill_mfma_fn mfma =
-        force_rowwise || !(scale > 0.f) || window > 0 ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
+        force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
     if (mfma) {
         PA_REQUIRE(pa_aligned16(q) && pa_aligned16(out), "q and out must be 16-byte aligned");
         const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;

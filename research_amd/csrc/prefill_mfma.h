@@ -185,6 +185,14 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     const int last_task = min(n_tasks, task0 + kPfTasks) - 1;
     const int wg_keys = min(ctx_len, prefix + min(q_len, (last_task / p.n_rep) * kPfRows + kPfRows));
     const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys;
+    // Sliding window: a row at position pos sees keys j > pos - window.  The workgroup starts at the tile that
+    // holds the first key its first row block can see (earlier tiles are never loaded); keys below a row's own
+    // bound are masked.  Waves whose rows start later see a fully masked first subtile, which contributes nothing.
+    const int win = p.window;
+    const int wg_first_key = win > 0 ? max(0, prefix + (task0 / p.n_rep) * kPfRows - win + 1) : 0;
+    const int t0 = wg_first_key / kPfKeys;  // first tile of the workgroup
+    // subtiles that start below this key hold keys that some row of the wave cannot see any more
+    const int lo_mask_until = win > 0 ? prefix + max(row0[0], row0[1]) + kPfRows - win + 1 : 0;
 
     // ---- Q^T operands: row = row0 + col, d = 16*ks + 8*half .. +8 ----
     X8 qreg[NC][KS];
@@ -258,7 +266,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     if (!BS16) {
 #pragma unroll
         for (int n = 0; n < NLW; ++n) {
-            const int key_first = (n * kPfWaves + wave) * G::RPL;
+            const int key_first = t0 * kPfKeys + (n * kPfWaves + wave) * G::RPL;
             g_blk[n] = key_first / p.bs;
             g_off[n] = key_first % p.bs;
         }
@@ -268,8 +276,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     auto issue = [&](int tile) PF_INLINE -> bool {
         const uint32_t dst0 = lds_base + (uint32_t)(tile % kPfStages) * 2 * G::BYTES;
         if (BS16) {
-            if (tile % WIN == 0) {  // next window of block ids (once per 16 tiles: its latency is not hidden)
-                const int idx = tile * BPT + lane;
+            if (tile % WIN == 0 || tile == t0) {  // next window of block ids (once per 16 tiles: latency not hidden)
+                const int idx = (tile - tile % WIN) * BPT + lane;
                 int v = -1;
                 if (idx < p.bt_stride) v = pf_load_i32(bt_row + idx);
                 pf_wait_loads<0>();
@@ -417,8 +425,17 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int limit = min(ctx_len - 1, prefix + row0[c] + col) - key_base - 4 * half;  // last visible key
+            if (win > 0) {  // uniform
+                const int first = prefix + row0[c] + col - win + 1 - key_base - 4 * half;  // first visible key
 #pragma unroll
-            for (int i = 0; i < 16; ++i) s[c][i] = 8 * (i >> 2) + (i & 3) <= limit ? s[c][i] : -INFINITY;
+                for (int i = 0; i < 16; ++i) {
+                    const int idx = 8 * (i >> 2) + (i & 3);
+                    s[c][i] = idx <= limit && idx >= first ? s[c][i] : -INFINITY;
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) s[c][i] = 8 * (i >> 2) + (i & 3) <= limit ? s[c][i] : -INFINITY;
+            }
         }
     };
     // Row maximum over a subtile's 32 keys, in two pieces (the empty asm statements pin each piece between the
@@ -450,12 +467,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
             for (int c = 0; c < NC; ++c) s[c] = M::mma(ka[ks], qreg[c][ks], s[c]);
     };
 
-    // ---- fill the ring: tiles 0 .. kPfStages-2 ----
+    // ---- fill the ring: tiles t0 .. t0 + kPfStages-2 ----
     bool counted[kPfStages - 1];  // loads of the tiles in flight, oldest first: issued as a full group of direct loads?
 #pragma unroll
-    for (int i = 0; i < kPfStages - 1; ++i) counted[i] = i < n_tiles ? issue(i) : false;
+    for (int i = 0; i < kPfStages - 1; ++i) counted[i] = t0 + i < n_tiles ? issue(t0 + i) : false;
     if (counted[1] && counted[2]) pf_wait_loads<4 * NLW>(); else __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();  // tile 0 is visible
+    __syncthreads();  // tile t0 is visible
 
     // Software pipeline over the wave's 32-key subtiles g = 0 .. n_sub-1 (tile g/2).  While subtile g is
     // exponentiated and multiplied into O^T, the S^T products of subtile g+1 run on the matrix unit:
@@ -468,17 +485,18 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     X8 ka[KS], va0[DT], va1[DT];
     f32x16 sb[2][NC];  // S^T of the current and of the next subtile, swapping roles every subtile
     float mx[NC] = {kNegBig, kNegBig};
-    if (n_sub > 0) {
-        set_k_tile(0);
-        set_v_tile(0);
+    const int g0 = t0 * kPfSub;  // first subtile
+    if (n_sub > g0) {
+        set_k_tile(t0);
+        set_v_tile(t0);
         read_k(0, ka);
         read_v(0, 0, va0);
         PF_FENCE();
         s_products(ka, sb[0]);
         PF_FENCE();
-        if (n_sub > 1) read_k(1, ka);
+        if (n_sub > g0 + 1) read_k(1, ka);
         PF_FENCE();
-        if (32 > mask_from) mask_s(sb[0], 0);
+        if (32 * (g0 + 1) > mask_from || 32 * g0 < lo_mask_until) mask_s(sb[0], 32 * g0);
 #pragma unroll
         for (int c = 0; c < NC; ++c) { max_piece(sb[0][c], 0, mx[c]); max_piece(sb[0][c], 1, mx[c]); }
         PF_FENCE();
@@ -494,7 +512,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
             const int g = tile * kPfSub + kt;
             const bool act = STEADY || g < n_sub;            // uniform per wave
             const bool has_next = STEADY || g + 1 < n_sub;
-            const bool mask_next = 32 * (g + 2) > mask_from;  // subtile g+1 reaches past the first causal limit
+            // subtile g+1 reaches past the first causal limit, or starts below the last window bound
+            const bool mask_next = 32 * (g + 2) > mask_from || 32 * (g + 1) < lo_mask_until;
             static_assert(kPfSub == 2, "the two S^T buffers swap roles once per subtile of a tile");
             f32x16(&s)[NC] = sb[kt & 1];
             f32x16(&s_nx)[NC] = sb[(kt + 1) & 1];
@@ -623,7 +642,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         }
     };
     const int steady_tiles = max(0, (n_sub - 2) / kPfSub);  // tiles whose subtiles g all have g + 2 < n_sub
-    int tile = 0;
+    int tile = t0;
     for (; tile < steady_tiles; ++tile) do_tile(tile, PfBool<true>{});
     for (; tile < n_tiles; ++tile) do_tile(tile, PfBool<false>{});
 

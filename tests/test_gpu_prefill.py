@@ -158,3 +158,31 @@ def test_matrix_core_kernel_shapes_and_block_sizes(dtype, d, hq, hkv):
                           _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk), _i32(np.arange(len(chunk)) * cmax),
                           cmax, bs, d ** -0.5, out=out)
         assert_close(out.reshape(len(chunk), cmax, hq, d), want, 2e-2, f"block_size {bs}")
+
+
+def test_sliding_window_prefill_long_prefix_on_the_matrix_core_kernel():
+    """Windows much shorter than the prefix: workgroups start deep inside the context (ring and block-id window
+    start at an arbitrary tile), for 16-token blocks and for whole-sequence blocks."""
+    announce("prefill window, long prefix")
+    rng = np.random.default_rng(77)
+    hq, hkv, d = 8, 2, 128
+    for bs in (16, 2048):
+        prefix, chunk = [1500, 1111, 0], [300, 77, 260]
+        cmax = max(chunk)
+        need = [-(-(p + c) // bs) for p, c in zip(prefix, chunk)]
+        nb = sum(need) + 1
+        perm = rng.permutation(nb)
+        tables, at = [], 0
+        for n in need:
+            tables.append(perm[at : at + n].tolist())
+            at += n
+        kc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+        vc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+        q = torch.from_numpy(rng.standard_normal((3, cmax, hq, d)).astype(np.float32)).to(torch.bfloat16)
+        for window in (64, 65, 200, 513, 1100):
+            want = po.paged_prefill_chunk(q, kc, vc, tables, prefix, chunk, bs, d ** -0.5, window=window)
+            out = torch.zeros(3 * cmax, hq, d, device=DEV, dtype=torch.bfloat16)
+            ops.prefill_paged(q.reshape(-1, hq, d).to(DEV), kc.to(DEV), vc.to(DEV), tables_to_device(tables),
+                              _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk), _i32(np.arange(3) * cmax),
+                              cmax, bs, d ** -0.5, out=out, window=window)
+            assert_close(out.reshape(3, cmax, hq, d), want, 2e-2, f"block_size {bs} window {window}")
