@@ -162,9 +162,27 @@ class HipPagedAttentionBackend:
         return torch.from_numpy(array).to(self.k_cache.device)
 
     def _tables(self, step: _StepTensors, block_tables) -> None:
+        """Device copy of the block tables.  The reference's tuple-of-tuples costs a Python-level pass over every
+        block id (tens of ms at 256 sequences x 2000 blocks); a 2-D int32 array or tensor padded with -1 is
+        taken as it is."""
         if step.tables is None:
-            padded = _padded_tables(block_tables)
-            step.tables, step.bt_stride = self._to_device(padded), padded.shape[1]
+            if isinstance(block_tables, Tensor):
+                if block_tables.dim() != 2:
+                    raise ValueError("block_tables tensor must be [num_seqs, width], padded with -1")
+                step.tables = block_tables.to(device=self.k_cache.device, dtype=torch.int32).contiguous()
+            elif isinstance(block_tables, np.ndarray):
+                if block_tables.ndim != 2:
+                    raise ValueError("block_tables array must be [num_seqs, width], padded with -1")
+                step.tables = self._to_device(np.ascontiguousarray(block_tables, dtype=np.int32))
+            else:
+                step.tables = self._to_device(_padded_tables(block_tables))
+            step.bt_stride = step.tables.shape[1]
+
+    def _lens(self, values, batch: int) -> np.ndarray:
+        """Host int64 copy of a per-sequence integer field (tuple, array or tensor)."""
+        if isinstance(values, Tensor):
+            values = values.detach().cpu().numpy()
+        return np.asarray(values, dtype=np.int64)[:batch]
 
     def _workspace_for(self, nbytes: int) -> Tensor:
         if self._workspace is None or self._workspace.numel() < nbytes:
@@ -197,7 +215,15 @@ class HipPagedAttentionBackend:
             return
         if _step is not None and _step.slots is not None:
             slots = _step.slots
+        elif isinstance(slot_mapping, Tensor) and slot_mapping.device.type == "cuda":
+            # already on the device: used as it is (out-of-range slots are dropped by the kernel, not reported)
+            self._require_device(k_flat, v_flat, self.k_cache)
+            slots = slot_mapping.to(torch.int64).contiguous()
+            if _step is not None:
+                _step.slots = slots
         else:
+            if isinstance(slot_mapping, Tensor):
+                slot_mapping = slot_mapping.numpy()
             host = np.asarray(slot_mapping, dtype=np.int64)
             if host.max() >= cfg.total_slots:
                 raise IndexError(
@@ -245,7 +271,7 @@ class HipPagedAttentionBackend:
         self._require_device(q, self.k_cache)
         step = self._step(ctx)
         if step.seq_lens is None:
-            lens = np.asarray(ctx.seq_lens, dtype=np.int64)[:batch]
+            lens = self._lens(ctx.seq_lens, batch)
             self._tables(step, ctx.block_tables[:batch])
             step.seq_lens = self._to_device(lens.astype(np.int32))
             if self.pad_zero_keys and batch > 0:
@@ -304,8 +330,8 @@ class HipPagedAttentionBackend:
         self._require_device(q, self.k_cache)
         step = self._step(ctx)
         if step.ctx_lens is None:
-            totals = np.asarray(ctx.seq_lens, dtype=np.int64)[:batch]
-            chunk = totals - np.asarray(ctx.prefix_lens, dtype=np.int64)[:batch]
+            totals = self._lens(ctx.seq_lens, batch)
+            chunk = totals - self._lens(ctx.prefix_lens, batch)
             if (chunk < 0).any() or (chunk > seq_len).any():
                 raise ValueError("prefix_lens / seq_lens do not describe chunks of at most q.shape[1] tokens")
             self._tables(step, ctx.block_tables[:batch])

@@ -263,3 +263,34 @@ def test_sliding_window_through_the_backend():
                                ctx.seq_lens, bs, backend.scale, window=window if in_decode else 0)
         assert_close(out[:, 0], want, 2e-2, f"decode, window_in_decode={in_decode}")
         outs[in_decode] = out
+
+
+def test_context_fields_as_arrays_and_tensors():
+    """block_tables / seq_lens / slot_mapping may be int arrays or tensors instead of the reference's tuples."""
+    announce("backend array / tensor context fields")
+    w = make_decode("c2", batch=6, len_range=(20, 300), seed=8)
+    config = CacheConfig(num_layers=1, num_kv_heads=8, head_dim=128, num_blocks=w.num_blocks, block_size=16,
+                         device="cuda", dtype=torch.bfloat16)
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(16)
+    backend.k_cache[0].copy_(w.k_pool.cuda())
+    backend.v_cache[0].copy_(w.v_pool.cuda())
+    tuples = tuple(tuple(int(b) for b in t) for t in w.block_tables)
+    lens = tuple(int(n) for n in w.seq_lens)
+    q = w.q[:, None].cuda()
+    base = backend.forward(q, None, None, 0, InferenceContext(is_prefill=False, block_tables=tuples, seq_lens=lens))
+    padded = w.padded_tables().astype(np.int32)
+    for tables, ln in ((padded, np.asarray(lens)), (torch.from_numpy(padded), torch.tensor(lens)),
+                       (torch.from_numpy(padded).cuda(), torch.tensor(lens, dtype=torch.int32).cuda())):
+        got = backend.forward(q, None, None, 0, InferenceContext(is_prefill=False, block_tables=tables, seq_lens=ln))
+        assert torch.equal(got, base)
+    # slot mapping as a device tensor: same rows land in the pool
+    k = torch.randn(6, 1, 8, 128, device="cuda", dtype=torch.bfloat16)
+    slots = [int(tuples[b][lens[b] // 16 if lens[b] // 16 < len(tuples[b]) else -1]) * 16 + lens[b] % 16
+             if lens[b] // 16 < len(tuples[b]) else -1 for b in range(6)]
+    ctx = InferenceContext(is_prefill=False, slot_mapping=torch.tensor(slots, device="cuda"), block_tables=padded,
+                           seq_lens=np.asarray(lens))
+    backend.forward(q, k, k, 0, ctx)
+    for b, s in enumerate(slots):
+        if s >= 0:
+            assert torch.equal(backend.k_cache[0, s], k[b, 0])
