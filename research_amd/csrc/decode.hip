@@ -148,7 +148,12 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
         PA_CHECK_LAUNCH("pa_decode split pass");
     }
     if (phases & kPhaseReduce) {
-        ks.reduce<<<dim3((unsigned)(batch * num_q_heads)), dim3(kThreads), 0, s>>>(a);
+        // Many rows and therefore few pieces per sequence: one wave per row.
+        const int64_t rows = (int64_t)batch * num_q_heads;
+        if (rows >= 4 * (int64_t)grid)
+            ks.reduce_wave<<<dim3((unsigned)((rows + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(a);
+        else
+            ks.reduce<<<dim3((unsigned)rows), dim3(kThreads), 0, s>>>(a);
         PA_CHECK_LAUNCH("pa_decode reduction pass");
     }
     return PA_OK;

@@ -545,6 +545,84 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_kernel(const DecodeArg
     }
 }
 
+// Reduction pass for large batches: one wave per (sequence, query head), four
+// heads per workgroup.  With many sequences a sequence has few pieces, so one
+// wave merges them all (loads of four pieces in flight at a time) and no LDS
+// merge or barrier is needed; a quarter of the workgroups of the kernel above.
+template <typename QT, int D, int NREP>
+__global__ __launch_bounds__(kThreads) void decode_reduce_wave_kernel(const DecodeArgs a) {
+    constexpr int DPL = (D + PA_WAVE - 1) / PA_WAVE;  // d values per lane
+    constexpr int PIPE = 4;
+    const PoolArgs &p = a.p;
+    const int hq = p.hq;
+    const int lane = threadIdx.x & (PA_WAVE - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / PA_WAVE);
+    const int row = blockIdx.x * kWaves + wave;
+    if (row >= a.batch * hq) return;
+    const int b = row / hq;
+    const int qh = row - b * hq;
+    const int kv = qh / p.n_rep, rep = qh - kv * p.n_rep;
+    const int hg = kv / p.hpw, rg = rep / NREP;
+    const int plane = rg * p.n_hgroups + hg;
+    const int idx = (kv - hg * p.hpw) * NREP + (rep - rg * NREP);
+    const int64_t per_plane = a.block_prefix[a.batch];
+    const int64_t total = per_plane * p.n_hgroups * p.n_rgroups;
+    const int nblk = a.block_prefix[b + 1] - a.block_prefix[b];
+    const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
+    QT *orow = reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * D;
+    if (nblk == 0) {
+        for (int d = lane; d < D; d += PA_WAVE) pa_scalar<QT>::store(orow + d, 0.f);
+        return;
+    }
+    const int64_t u0 = plane * per_plane + a.block_prefix[b];
+    const int w0 = owner_of(u0, total, a.split_grid), w1 = owner_of(u0 + nblk - 1, total, a.split_grid);
+    if (w0 == w1) return;  // finished by the split pass
+    const int64_t key = (int64_t)plane * a.batch + b;
+    const int stride_acc = p.hpw * NREP * D, stride_ml = p.hpw * NREP * 2;
+    auto has_piece = [&](int w) {
+        return w <= w1 && unit_begin(w, total, a.split_grid) < unit_begin((int64_t)w + 1, total, a.split_grid) &&
+               w + key < a.slot_cap;
+    };
+    float M = kNegBig, den = 0.f, num[DPL];
+#pragma unroll
+    for (int k = 0; k < DPL; ++k) num[k] = 0.f;
+    for (int w = w0; w <= w1; w += PIPE) {
+        float m[PIPE], l[PIPE], x[PIPE][DPL];
+#pragma unroll
+        for (int j = 0; j < PIPE; ++j) {
+            const bool have = has_piece(w + j);
+            const int64_t slot = have ? w + j + key : w0 + key;
+            m[j] = have ? a.part_ml[slot * stride_ml + idx * 2] : kNegBig;
+            l[j] = have ? a.part_ml[slot * stride_ml + idx * 2 + 1] : 0.f;
+#pragma unroll
+            for (int k = 0; k < DPL; ++k) {
+                const int d = lane + PA_WAVE * k;
+                x[j][k] = have && d < D ? a.part_acc[slot * stride_acc + idx * D + d] : 0.f;
+            }
+        }
+        float mn = M;
+#pragma unroll
+        for (int j = 0; j < PIPE; ++j) mn = fmaxf(mn, m[j]);
+        const float so = __builtin_amdgcn_exp2f(M - mn);
+        den *= so;
+#pragma unroll
+        for (int k = 0; k < DPL; ++k) num[k] *= so;
+#pragma unroll
+        for (int j = 0; j < PIPE; ++j) {
+            const float sn = __builtin_amdgcn_exp2f(m[j] - mn);
+            den = fmaf(l[j], sn, den);
+#pragma unroll
+            for (int k = 0; k < DPL; ++k) num[k] = fmaf(x[j][k], sn, num[k]);
+        }
+        M = mn;
+    }
+#pragma unroll
+    for (int k = 0; k < DPL; ++k) {
+        const int d = lane + PA_WAVE * k;
+        if (d < D) pa_scalar<QT>::store(orow + d, finish_row(num[k], M, den, ez));
+    }
+}
+
 // Causal prefill, one workgroup per (sequence, query row, head group, rep
 // group): query row i of sequence b attends keys [0, ctx_len - q_len + i].
 template <typename KV, typename QT, int D, int NREP, int U>
@@ -586,6 +664,7 @@ typedef void (*rowwise_fn)(const RowwiseArgs);
 struct KernelSet {
     split_fn split = nullptr;
     reduce_fn reduce = nullptr;
+    reduce_fn reduce_wave = nullptr;  // for batches with few pieces per sequence
     rowwise_fn rowwise = nullptr;
 };
 
@@ -593,10 +672,10 @@ template <typename KV, typename QT, int D> KernelSet kernels_for_d(int nrep_t) {
     constexpr int U = sizeof(KV) == 1 ? 4 : 8;
     KernelSet k;
     switch (nrep_t) {
-    case 1: k.reduce = decode_reduce_kernel<QT, D, 1>; k.split = decode_split_kernel<KV, QT, D, 1, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 1, U>; break;
-    case 2: k.reduce = decode_reduce_kernel<QT, D, 2>; k.split = decode_split_kernel<KV, QT, D, 2, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 2, U>; break;
-    case 4: k.reduce = decode_reduce_kernel<QT, D, 4>; k.split = decode_split_kernel<KV, QT, D, 4, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 4, U>; break;
-    case 8: k.reduce = decode_reduce_kernel<QT, D, 8>; k.split = decode_split_kernel<KV, QT, D, 8, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 8, U>; break;
+    case 1: k.reduce = decode_reduce_kernel<QT, D, 1>; k.reduce_wave = decode_reduce_wave_kernel<QT, D, 1>; k.split = decode_split_kernel<KV, QT, D, 1, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 1, U>; break;
+    case 2: k.reduce = decode_reduce_kernel<QT, D, 2>; k.reduce_wave = decode_reduce_wave_kernel<QT, D, 2>; k.split = decode_split_kernel<KV, QT, D, 2, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 2, U>; break;
+    case 4: k.reduce = decode_reduce_kernel<QT, D, 4>; k.reduce_wave = decode_reduce_wave_kernel<QT, D, 4>; k.split = decode_split_kernel<KV, QT, D, 4, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 4, U>; break;
+    case 8: k.reduce = decode_reduce_kernel<QT, D, 8>; k.reduce_wave = decode_reduce_wave_kernel<QT, D, 8>; k.split = decode_split_kernel<KV, QT, D, 8, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 8, U>; break;
     }
     return k;
 }
