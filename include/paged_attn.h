@@ -173,12 +173,18 @@ int pa_decode_reduce(const void *q, const void *k_cache, const void *v_cache, vo
  *   window   : 0, or the sliding window of CacheConfig.sliding_window (attention/config.py:31): row i at
  *              position p = ctx_lens[b] - q_lens[b] + i attends keys p - window < j <= p
  *              (attention/mask.py:83-89); tiles wholly before the window of a workgroup's rows are not loaded.
+ *   row_first_key : NULL, or int32[total_q] indexed like the rows of q: the first key position (in the
+ *              row's own sequence) the row attends, on top of the causal bound -- the packed-document mask
+ *              of create_document_mask (attention/mask.py:141-191: same document and q_idx >= kv_idx) with
+ *              row_first_key = start of the row's document.  Must not decrease along a sequence; values
+ *              are clamped to [0, position of the row], so a row always sees itself.  Combines with window
+ *              (the later of the two bounds applies).
  */
 int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, void *out,
                      const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
-                     const int32_t *q_lens, const int32_t *q_starts, int batch, int max_q_len,
-                     int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-                     int64_t num_blocks, float scale, int window, int dtype, void *stream);
+                     const int32_t *q_lens, const int32_t *q_starts, const int32_t *row_first_key,
+                     int batch, int max_q_len, int num_q_heads, int num_kv_heads, int head_dim,
+                     int block_size, int64_t num_blocks, float scale, int window, int dtype, void *stream);
 
 /*
  * fp8-e4m3 pool construction (no counterpart in the reference; its oracle is

@@ -37,6 +37,10 @@ How each function is pinned (see tests/test_oracle.py):
                         q_idx >= kv_idx and q_idx - kv_idx < window, the
                         recipe of the reference's debug_swa.py; window >= length
                         equals no window; decode equals the last prefill row
+  doc_lens= (prefill)   torch SDPA with the explicit boolean mask evaluated by a
+                        scalar restatement of document_mask's loop
+                        (attention/mask.py:173-186) entry by entry; equals
+                        independent causal attention on each document alone
   quantize_kv_e4m3      torch.float8_e4m3fn conversion (library definition of
                         OCP e4m3fn, round to nearest even), known values
                         464 -> 448, 2**-10 -> 0, max 448
@@ -141,15 +145,34 @@ def kv_gather_loop(k_cache, v_cache, block_tables, seq_lens, block_size: int):
 # --------------------------------------------------------------------------- attention (float64, explicit)
 
 
+def document_of(boundaries: Sequence[int], idx: np.ndarray) -> np.ndarray:
+    """Document index of each position: the number of document ends at or before it
+    (attention/mask.py:176-185: ``doc = i + 1`` for the last boundary with ``idx >= boundary``);
+    positions past the last document therefore form one more document."""
+    ends = np.asarray(list(boundaries)[1:], dtype=np.int64)
+    return (np.asarray(idx)[..., None] >= ends).sum(axis=-1)
+
+
+def document_boundaries(seq_lens: Sequence[int]) -> List[int]:
+    """Running sums of the document lengths, starting at 0 (attention/mask.py:168-171)."""
+    bounds = [0]
+    for n in seq_lens:
+        bounds.append(bounds[-1] + int(n))
+    return bounds
+
+
 def _attend_rows(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, n_zero: int = 0,
-                 causal_offset: Optional[int] = None, window: int = 0) -> np.ndarray:
+                 causal_offset: Optional[int] = None, window: int = 0,
+                 boundaries: Optional[Sequence[int]] = None) -> np.ndarray:
     """softmax(scale * q k^T) v for one kv head group.
 
     q ``[R, n_rep, D]``, k/v ``[L, D]`` -> ``[R, n_rep, D]``.  ``n_zero`` extra
     all-zero keys (logit 0, value 0) join the softmax.  ``causal_offset``: row
     r sits at position ``causal_offset + r`` and may only see keys
     ``j <= causal_offset + r``; with ``window`` > 0 also only keys with
-    ``position - j < window`` (attention/mask.py:83-89).
+    ``position - j < window`` (attention/mask.py:83-89); with ``boundaries``
+    (document starts and the final end) also only keys of the row's own
+    document (attention/mask.py:173-186).
     """
     logits = scale * np.einsum("rhd,ld->rhl", q, k)  # [R, n_rep, L]
     if causal_offset is not None:
@@ -158,6 +181,8 @@ def _attend_rows(q: np.ndarray, k: np.ndarray, v: np.ndarray, scale: float, n_ze
         seen = cols <= causal_offset + rows
         if window > 0:
             seen &= (causal_offset + rows) - cols < window
+        if boundaries is not None:
+            seen &= document_of(boundaries, causal_offset + rows) == document_of(boundaries, cols)
         logits = np.where(seen, logits, -np.inf)
     m = logits.max(axis=-1, keepdims=True) if logits.shape[-1] else np.full(logits.shape[:-1] + (1,), -np.inf)
     if n_zero > 0:
@@ -204,9 +229,10 @@ def paged_decode(q, k_cache, v_cache, block_tables, seq_lens, block_size: int, s
     return out
 
 
-def dense_prefill(q, k, v, scale: float, window: int = 0) -> np.ndarray:
+def dense_prefill(q, k, v, scale: float, window: int = 0, doc_lens: Optional[Sequence[int]] = None) -> np.ndarray:
     """Causal attention over the step's own K/V (flex_backend.py:144-185, SDPA is_causal=True; with
-    ``window`` the flex_attention path under causal_sliding_window_mask, attention/mask.py:56-100).
+    ``window`` the flex_attention path under causal_sliding_window_mask, attention/mask.py:56-100; with
+    ``doc_lens`` under the packed-document mask of create_document_mask, attention/mask.py:141-191).
 
     q ``[B, T, Hq, D]``, k/v ``[B, T, Hkv, D]`` -> float64 ``[B, T, Hq, D]``.
     """
@@ -215,28 +241,32 @@ def dense_prefill(q, k, v, scale: float, window: int = 0) -> np.ndarray:
     hkv = k.shape[2]
     n_rep = hq // hkv
     out = np.zeros_like(q)
+    bounds = document_boundaries(doc_lens) if doc_lens is not None else None
     for b in range(batch):
         for g in range(hkv):
             sl = slice(g * n_rep, (g + 1) * n_rep)
-            out[b, :, sl] = _attend_rows(q[b, :, sl], k[b, :, g], v[b, :, g], scale, causal_offset=0, window=window)
+            out[b, :, sl] = _attend_rows(q[b, :, sl], k[b, :, g], v[b, :, g], scale, causal_offset=0, window=window,
+                                         boundaries=bounds)
     return out
 
 
 def paged_prefill_chunk(q, k_cache, v_cache, block_tables, prefix_lens, chunk_lens, block_size: int,
-                        scale: float, window: int = 0) -> np.ndarray:
+                        scale: float, window: int = 0, doc_lens: Optional[Sequence[int]] = None) -> np.ndarray:
     """Chunked prefill over a cached prefix (composition; not a reference function).
 
     Defined as: gather keys ``0 .. P+C-1`` through the block table
     (flex_backend.py:233-279) and attend with a bottom-right aligned causal
     mask, i.e. chunk row i (absolute position P+i) sees keys ``j <= P+i``.
     The chunk's own K/V must already be in the cache.  q ``[B, Cmax, Hq, D]``;
-    rows past ``chunk_lens[b]`` give zeros.
+    rows past ``chunk_lens[b]`` give zeros.  ``doc_lens``: documents packed
+    into every sequence by absolute position (attention/mask.py:141-191).
     """
     q, kc, vc = to_f64(q), to_f64(k_cache), to_f64(v_cache)
     batch, cmax, hq, d = q.shape
     hkv = kc.shape[1]
     n_rep = hq // hkv
     out = np.zeros_like(q)
+    bounds = document_boundaries(doc_lens) if doc_lens is not None else None
     for b in range(batch):
         p, c = int(prefix_lens[b]), int(chunk_lens[b])
         blocks = np.asarray(block_tables[b], dtype=np.int64)
@@ -245,7 +275,7 @@ def paged_prefill_chunk(q, k_cache, v_cache, block_tables, prefix_lens, chunk_le
         for g in range(hkv):
             sl = slice(g * n_rep, (g + 1) * n_rep)
             out[b, :c, sl] = _attend_rows(q[b, :c, sl], kc[slots, g], vc[slots, g], scale, causal_offset=p,
-                                          window=window)
+                                          window=window, boundaries=bounds)
     return out
 
 

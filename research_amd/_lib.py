@@ -47,8 +47,8 @@ SIGNATURES = {
     "pa_decode_reduce": None,
     "pa_prefill_paged": (
         c_int,
-        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
-         c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p],
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+         c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p],
     ),
     "pa_quantize_kv_e4m3": (
         c_int,

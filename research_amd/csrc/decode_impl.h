@@ -72,6 +72,7 @@ struct RowwiseArgs {
     const void *q;
     void *out;
     const int32_t *ctx_lens, *q_lens, *q_starts;
+    const int32_t *row_lo;  // per query row: first key it sees (NULL = none); non-decreasing along a sequence
     int batch;
     int max_q_len;
 };
@@ -646,7 +647,9 @@ __global__ __launch_bounds__(kThreads) void prefill_rowwise_kernel(const Rowwise
     const int64_t qrow = (int64_t)a.q_starts[b] + i;
 
     const int nblk = L > 0 ? (L + p.bs - 1) / p.bs : 0;
-    const int k_lo = window_first_key(p, max(L, 0));  // the row sits at position L-1
+    int k_lo = window_first_key(p, max(L, 0));  // the row sits at position L-1
+    if (a.row_lo) k_lo = max(k_lo, min(a.row_lo[qrow], L - 1));
+    k_lo = max(k_lo, 0);
     RowState<NREP, S::EPL> st = Attender<KV, QT, D, NREP, U>::run(
         p, reinterpret_cast<const QT *>(a.q) + qrow * p.hq * D, p.bt + (int64_t)b * p.bt_stride, k_lo, L,
         k_lo / p.bs + wave, nblk, kWaves, role, lane, kvh, rep0);

@@ -7,9 +7,10 @@ using namespace pa_decode_detail;
 
 extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, void *out,
                                 const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
-                                const int32_t *q_lens, const int32_t *q_starts, int batch, int max_q_len,
-                                int num_q_heads, int num_kv_heads, int head_dim, int block_size,
-                                int64_t num_blocks, float scale, int window, int dtype, void *stream) {
+                                const int32_t *q_lens, const int32_t *q_starts, const int32_t *row_first_key,
+                                int batch, int max_q_len, int num_q_heads, int num_kv_heads, int head_dim,
+                                int block_size, int64_t num_blocks, float scale, int window, int dtype,
+                                void *stream) {
     pa_clear_error();
     PA_REQUIRE(batch >= 0 && max_q_len >= 0, "batch=%d max_q_len=%d must be non-negative", batch, max_q_len);
     PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, "head counts / head_dim must be positive");
@@ -38,6 +39,7 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     a.p.scale_log2 = scale * 1.4426950408889634f;
     a.p.window = window;
     a.q = q; a.out = out; a.ctx_lens = ctx_lens; a.q_lens = q_lens; a.q_starts = q_starts;
+    a.row_lo = row_first_key;
     a.batch = batch; a.max_q_len = max_q_len;
     hipStream_t s = (hipStream_t)stream;
     // bf16 / fp16 with head_dim 32, 64, 128 run on the matrix cores; PA_PREFILL_ROWWISE=1 forces the

@@ -185,14 +185,28 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     const int last_task = min(n_tasks, task0 + kPfTasks) - 1;
     const int wg_keys = min(ctx_len, prefix + min(q_len, (last_task / p.n_rep) * kPfRows + kPfRows));
     const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys;
-    // Sliding window: a row at position pos sees keys j > pos - window.  The workgroup starts at the tile that
-    // holds the first key its first row block can see (earlier tiles are never loaded); keys below a row's own
-    // bound are masked.  Waves whose rows start later see a fully masked first subtile, which contributes nothing.
+    // Lower bounds.  Sliding window: a row at position pos sees keys j > pos - window.  Per-row first keys (packed
+    // documents): row i sees keys j >= row_lo[i].  Both bounds are non-decreasing along a sequence, so the
+    // workgroup starts at the tile that holds the first key its first row can see (earlier tiles are never
+    // loaded); keys below a row's own bound are masked.  Waves whose rows start later see a fully masked first
+    // subtile, which contributes nothing.
     const int win = p.window;
-    const int wg_first_key = win > 0 ? max(0, prefix + (task0 / p.n_rep) * kPfRows - win + 1) : 0;
+    const int32_t *rlo = a.row_lo ? a.row_lo + a.q_starts[b] : nullptr;
+    const bool bounded = win > 0 || rlo != nullptr;  // uniform
+    // a row's first visible key, clamped so that the row always sees its own position
+    auto row_first = [&](int row) PF_INLINE {
+        const int pos = prefix + row;
+        int lo = win > 0 ? pos - win + 1 : 0;
+        if (rlo) lo = max(lo, rlo[min(row, q_len - 1)]);
+        return min(max(lo, 0), min(pos, ctx_len - 1));
+    };
+    const int wg_first_key = bounded ? row_first((task0 / p.n_rep) * kPfRows) : 0;
     const int t0 = wg_first_key / kPfKeys;  // first tile of the workgroup
     // subtiles that start below this key hold keys that some row of the wave cannot see any more
-    const int lo_mask_until = win > 0 ? prefix + max(row0[0], row0[1]) + kPfRows - win + 1 : 0;
+    const int lo_mask_until = bounded ? row_first(min(q_len, max(row0[0], row0[1]) + kPfRows) - 1) : 0;
+    int lo_row[NC];  // this lane's rows
+#pragma unroll
+    for (int c = 0; c < NC; ++c) lo_row[c] = bounded ? row_first(row0[c] + col) : 0;
 
     // ---- Q^T operands: row = row0 + col, d = 16*ks + 8*half .. +8 ----
     X8 qreg[NC][KS];
@@ -425,8 +439,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
             const int limit = min(ctx_len - 1, prefix + row0[c] + col) - key_base - 4 * half;  // last visible key
-            if (win > 0) {  // uniform
-                const int first = prefix + row0[c] + col - win + 1 - key_base - 4 * half;  // first visible key
+            if (bounded) {
+                const int first = lo_row[c] - key_base - 4 * half;  // first visible key
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int idx = 8 * (i >> 2) + (i & 3);

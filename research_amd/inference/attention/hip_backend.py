@@ -21,13 +21,18 @@ Differences from the reference, all deliberate:
   both read from the pool through the block table.
 * ``config.sliding_window`` is applied inside the kernels (a row at position p
   sees keys ``p - window < j <= p``, attention/mask.py:83-89) instead of through
-  a FlexAttention ``BlockMask``; ``get_block_mask`` therefore returns ``None``.
+  a FlexAttention ``BlockMask``; ``get_block_mask`` returns the ``PagedMask``
+  description of it (``None`` without a window, as in the reference).
   Prefill applies it as the reference does.  Decode in the reference applies a
   window only when the caller passes ``ctx.block_mask`` (flex_backend.py:220-225)
   and otherwise attends the whole cache; ``window_in_decode=False`` keeps that,
   the default ``True`` attends the last ``window`` keys, consistent with prefill.
-* ``ctx.block_mask`` objects (arbitrary FlexAttention masks) are not supported
-  and raise ``NotImplementedError`` instead of being ignored.
+* ``ctx.block_mask`` takes the ``PagedMask`` objects of ``attention/mask.py``
+  (causal, sliding window, packed documents): a window becomes the kernels'
+  ``window`` argument and documents become one first key per query row.  Any
+  other object (a FlexAttention ``BlockMask``, an arbitrary predicate) raises
+  ``NotImplementedError`` instead of being ignored.  A document mask describes
+  packed prefill rows; in decode it raises as well.
 """
 
 from __future__ import annotations
@@ -42,6 +47,7 @@ from torch import Tensor
 from ... import _lib, ops
 from ..types import InferenceContext
 from .config import CacheConfig
+from .mask import PagedMask, create_attention_mask
 
 _COMPUTE_DTYPES = (torch.float32, torch.bfloat16, torch.float16)
 
@@ -50,12 +56,12 @@ class _StepTensors:
     """Device copies of one context's integer fields, built once per step."""
 
     __slots__ = ("ctx", "slots", "touched", "tables", "bt_stride", "seq_lens", "extra_zero", "ctx_lens", "q_lens",
-                 "q_starts", "max_q_len")
+                 "q_starts", "max_q_len", "row_first_key")
 
     def __init__(self, ctx: InferenceContext) -> None:
         self.ctx = ctx  # keeps id(ctx) alive while the entry is cached
         self.slots = self.touched = self.tables = self.seq_lens = self.extra_zero = None
-        self.ctx_lens = self.q_lens = self.q_starts = None
+        self.ctx_lens = self.q_lens = self.q_starts = self.row_first_key = None
         self.bt_stride = self.max_q_len = 0
 
 
@@ -105,8 +111,42 @@ class HipPagedAttentionBackend:
         self.num_heads_per_kv = num_heads // self.config.num_kv_heads
 
     def get_block_mask(self, batch_size: int, seq_len: int) -> object:
-        # plain causal needs no mask object (flex_backend.py:62-63); the sliding window is applied by the kernels
-        return None
+        """The configured mask for a step of this shape (flex_backend.py:47-83): ``None`` for plain causal,
+        else the sliding-window description, cached per shape with the reference's bound of 100 entries."""
+        if self.config.sliding_window is None:
+            return None
+        key = (batch_size, seq_len)
+        mask = self._mask_cache.get(key)
+        if mask is None:
+            mask = create_attention_mask(batch_size=batch_size, seq_len=seq_len,
+                                         sliding_window=self.config.sliding_window,
+                                         block_size=self.config.block_size, device=self.config.device)
+            if len(self._mask_cache) < 100:
+                self._mask_cache[key] = mask
+        return mask
+
+    def _mask_window(self, mask: object, default: int) -> int:
+        """The ``window`` kernel argument under ``ctx.block_mask`` (which replaces the configured mask, as in
+        flex_backend.py:170-173)."""
+        if mask is None:
+            return default
+        if not isinstance(mask, PagedMask):
+            raise NotImplementedError(
+                f"block_mask of type {type(mask).__name__}: the HIP backend takes the PagedMask objects of "
+                "attention/mask.py (causal, sliding window, documents), not arbitrary mask objects")
+        return int(mask.window or 0)
+
+    def _mask_first_keys(self, mask: object, step: _StepTensors, batch: int, seq_len: int,
+                         prefix: Optional[np.ndarray]) -> Optional[Tensor]:
+        """Per-row first keys (int32 ``[batch * seq_len]``) of a document mask, None for the other masks.
+        Row t of sequence b sits at position ``prefix[b] + t``."""
+        if not isinstance(mask, PagedMask) or mask.boundaries is None:
+            return None
+        if step.row_first_key is None:
+            pos = np.arange(seq_len, dtype=np.int64)[None, :] + (
+                prefix[:, None] if prefix is not None else np.zeros((batch, 1), dtype=np.int64))
+            step.row_first_key = self._to_device(np.ascontiguousarray(mask.first_keys(pos)).reshape(-1))
+        return step.row_first_key
 
     def clear_mask_cache(self) -> None:
         self._mask_cache.clear()
@@ -265,8 +305,11 @@ class HipPagedAttentionBackend:
         assert seq_len == 1, "Decode should have seq_len=1"
         if ctx.block_tables is None or ctx.seq_lens is None:
             raise ValueError("Decode requires block_tables and seq_lens in context")
-        if ctx.block_mask is not None:
-            raise NotImplementedError("block_mask objects are not supported by the HIP backend")
+        window = self._mask_window(ctx.block_mask, self._window if self.window_in_decode else 0)
+        if isinstance(ctx.block_mask, PagedMask) and ctx.block_mask.boundaries is not None:
+            raise NotImplementedError("a document mask describes packed prefill rows, not a decode step")
+        if window and self.pad_zero_keys:
+            raise ValueError("pad_zero_keys cannot be combined with a sliding window in decode")
         cfg = self.config
         self._require_device(q, self.k_cache)
         step = self._step(ctx)
@@ -283,7 +326,7 @@ class HipPagedAttentionBackend:
         ksc = self.k_scale[layer_idx] if self._fp8 else None
         vsc = self.v_scale[layer_idx] if self._fp8 else None
         out = ops.decode(q3, kc, vc, step.tables, step.seq_lens, cfg.block_size, self.scale, ws, step.extra_zero,
-                         ksc, vsc, window=self._window if self.window_in_decode else 0)
+                         ksc, vsc, window=window)
         return out.view(batch, 1, num_heads, head_dim)
 
     # ------------------------------------------------------------------ prefill
@@ -293,13 +336,13 @@ class HipPagedAttentionBackend:
         The dense ``[B, T, Hkv, D]`` inputs are handed to the paged kernel as a
         pool of ``B`` blocks of ``T`` tokens with the identity block table.
         """
-        if ctx.block_mask is not None:
-            raise NotImplementedError("block_mask objects are not supported by the HIP backend")
+        window = self._mask_window(ctx.block_mask, self._window)
         batch, seq_len, num_heads, head_dim = q.shape
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         if out.numel() == 0:
             return out
         dev = self._require_device(q, k, v)
+        first = self._mask_first_keys(ctx.block_mask, self._step(ctx), batch, seq_len, None)
         num_kv = k.shape[2]
         if num_heads != num_kv * self.num_heads_per_kv:
             raise RuntimeError(
@@ -311,13 +354,12 @@ class HipPagedAttentionBackend:
             k.contiguous().view(batch * seq_len, num_kv, head_dim),
             v.contiguous().view(batch * seq_len, num_kv, head_dim),
             ar.reshape(batch, 1).contiguous(), lens, lens, ar * seq_len, seq_len, seq_len, self.scale,
-            out=out.view(batch * seq_len, num_heads, head_dim), window=self._window)
+            out=out.view(batch * seq_len, num_heads, head_dim), window=window, row_first_key=first)
         return out
 
     def _prefill_paged(self, q: Tensor, layer_idx: int, ctx: InferenceContext) -> Tensor:
         """Chunked prefill: ``q[b]`` holds the last ``T`` positions of a context of ``seq_lens[b]`` keys."""
-        if ctx.block_mask is not None:
-            raise NotImplementedError("block_mask objects are not supported by the HIP backend")
+        window = self._mask_window(ctx.block_mask, self._window)
         if ctx.block_tables is None or ctx.seq_lens is None:
             raise ValueError("Chunked prefill requires block_tables and seq_lens in context")
         if self._fp8:
@@ -339,11 +381,14 @@ class HipPagedAttentionBackend:
             step.q_lens = self._to_device(chunk.astype(np.int32))
             step.q_starts = self._to_device((np.arange(batch, dtype=np.int64) * seq_len).astype(np.int32))
             step.max_q_len = int(chunk.max()) if batch else 0
+        first = None
+        if isinstance(ctx.block_mask, PagedMask) and ctx.block_mask.boundaries is not None:
+            first = self._mask_first_keys(ctx.block_mask, step, batch, seq_len, self._lens(ctx.prefix_lens, batch))
         out.zero_()  # rows past a sequence's chunk length are padding and stay zero
         kc, vc = self._layer(layer_idx)
         ops.prefill_paged(q.contiguous().view(batch * seq_len, num_heads, head_dim), kc, vc, step.tables,
                           step.ctx_lens, step.q_lens, step.q_starts, step.max_q_len, cfg.block_size, self.scale,
-                          out=out.view(batch * seq_len, num_heads, head_dim), window=self._window)
+                          out=out.view(batch * seq_len, num_heads, head_dim), window=window, row_first_key=first)
         return out
 
     # ------------------------------------------------------------------ fp8 pool

@@ -59,6 +59,37 @@ def test_decode_error_conventions():
                                                      block_mask=object()))
 
 
+def test_mask_objects():
+    """The factory functions keep the reference's names and arguments (attention/mask.py) and describe the
+    same predicate: mask_mod is compared entry by entry with the range form the kernels receive."""
+    from research_amd.inference.attention import (create_attention_mask, create_causal_block_mask,
+                                                  create_document_mask, create_sliding_window_causal_mask)
+    import numpy as np
+
+    causal = create_causal_block_mask(2, 12, block_size=128, device="cpu")
+    swa = create_sliding_window_causal_mask(2, 12, window_size=5)
+    assert create_attention_mask(2, 12, sliding_window=None) == causal
+    assert create_attention_mask(2, 12, sliding_window=5) == swa
+    docs = create_document_mask(1, (3, 0, 4, 2), 12)  # an empty document, and 3 positions past the last one
+    assert docs.boundaries == (0, 3, 3, 7, 9) and docs.kind == "document"
+    assert (causal.kind, swa.kind) == ("causal", "sliding_window")
+    with pytest.raises(ValueError):
+        create_sliding_window_causal_mask(1, 8, 0)
+    for mask in (causal, swa, docs):
+        first = np.maximum(mask.first_keys(np.arange(12)),
+                           np.arange(12) - (mask.window or 12) + 1).clip(min=0)
+        for qi in range(12):
+            for ki in range(12):
+                assert mask.mask_mod(0, 0, qi, ki) == (first[qi] <= ki <= qi), (mask.kind, qi, ki)
+    assert docs.first_keys(np.arange(12)).tolist() == [0, 0, 0, 3, 3, 3, 3, 7, 7, 9, 9, 9]
+    be = HipPagedAttentionBackend(_cfg())
+    be.set_num_heads(8)
+    q1 = torch.zeros(1, 1, 8, 32, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="document"):
+        be._decode_attention(q1, 0, InferenceContext(is_prefill=False, block_tables=((0,),), seq_lens=(1,),
+                                                     block_mask=docs))
+
+
 def test_store_kv_error_conventions():
     be = HipPagedAttentionBackend(_cfg())
     k = torch.zeros(1, 4, 4, 32, dtype=torch.bfloat16)
@@ -95,7 +126,10 @@ def test_out_of_range_slot_is_an_index_error():
 
 def test_unsupported_features_raise():
     be = HipPagedAttentionBackend(_cfg(sliding_window=4))
-    assert be.get_block_mask(1, 8) is None  # the window is applied inside the kernels, no mask object
+    mask = be.get_block_mask(1, 8)  # a description of the window, cached per shape (flex_backend.py:47-83)
+    assert mask.kind == "sliding_window" and mask.window == 4 and be.get_block_mask(1, 8) is mask
+    be.clear_mask_cache()
+    assert be.get_block_mask(1, 8) is not mask
     with pytest.raises(ValueError):
         HipPagedAttentionBackend(_cfg(sliding_window=0))
     with pytest.raises(ValueError):

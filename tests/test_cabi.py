@@ -121,12 +121,12 @@ def test_decode_workspace_arithmetic():
 
 
 def test_prefill_and_quantize_argument_errors():
-    args = [FAKE, FAKE, FAKE, FAKE, FAKE, 4, FAKE, FAKE, FAKE, 2, 16, 32, 8, 128, 16, 64, 0.088, 0, _lib.PA_FP8_E4M3,
-            None]
+    args = [FAKE, FAKE, FAKE, FAKE, FAKE, 4, FAKE, FAKE, FAKE, None, 2, 16, 32, 8, 128, 16, 64, 0.088, 0,
+            _lib.PA_FP8_E4M3, None]
     rc, msg = _status("pa_prefill_paged", *args)
     assert rc == _lib.PA_ERR_INVALID_ARG and "dtype" in msg
     args[-2] = _lib.PA_BF16
-    args[13] = 80
+    args[14] = 80
     rc, msg = _status("pa_prefill_paged", *args)
     assert rc == _lib.PA_ERR_UNSUPPORTED
     rc, msg = _status("pa_quantize_kv_e4m3", FAKE, FAKE, FAKE, 4, 16, 8, 128, _lib.PA_FP8_E4M3, None)

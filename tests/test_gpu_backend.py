@@ -294,3 +294,45 @@ def test_context_fields_as_arrays_and_tensors():
     for b, s in enumerate(slots):
         if s >= 0:
             assert torch.equal(backend.k_cache[0, s], k[b, 0])
+
+
+def test_block_mask_objects_through_the_backend():
+    """ctx.block_mask with the mask objects of attention/mask.py: documents and a window in prefill (replacing
+    the configured mask, flex_backend.py:170-173), a window in decode (flex_backend.py:220-225)."""
+    from research_amd.inference.attention import (create_causal_block_mask, create_document_mask,
+                                                  create_sliding_window_causal_mask)
+
+    announce("backend block_mask objects")
+    g = torch.Generator().manual_seed(52)
+    hq, hkv, d, bs = 8, 2, 64, 16
+    config = CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=16, block_size=bs, device="cuda",
+                         sliding_window=9)
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(hq)
+    b, t = 2, 100
+    q = torch.randn(b, t, hq, d, generator=g).to(torch.bfloat16)
+    k = torch.randn(b, t, hkv, d, generator=g).to(torch.bfloat16)
+    v = torch.randn(b, t, hkv, d, generator=g).to(torch.bfloat16)
+    doc_lens = (17, 40, 33)
+    cases = ((create_document_mask(b, doc_lens, t), dict(doc_lens=doc_lens)),
+             (create_sliding_window_causal_mask(b, t, 5), dict(window=5)),
+             (create_causal_block_mask(b, t), dict()),
+             (None, dict(window=9)))
+    for mask, kw in cases:
+        ctx = InferenceContext(is_prefill=True, block_mask=mask)
+        out = backend.forward(q.cuda(), k.cuda(), v.cuda(), 0, ctx)
+        assert_close(out, po.dense_prefill(q, k, v, backend.scale, **kw), 2e-2, f"prefill under {kw}")
+    # decode: the pool holds sequence 0 of the step above in blocks 3, 1, 4, 9, 2, 6, 5
+    blocks = (3, 1, 4, 9, 2, 6, 5)
+    slots = tuple(blocks[p // bs] * bs + p % bs for p in range(t))
+    backend._store_kv(k[:1].cuda(), v[:1].cuda(), 0, slots)
+    q1 = torch.randn(1, 1, hq, d, generator=g).to(torch.bfloat16)
+    for mask, window in ((create_sliding_window_causal_mask(1, t, 20), 20), (create_causal_block_mask(1, t), 0),
+                         (None, 9)):
+        ctx = InferenceContext(is_prefill=False, block_tables=(blocks,), seq_lens=(t,), block_mask=mask)
+        out = backend.forward(q1.cuda(), None, None, 0, ctx)
+        want = po.paged_decode(q1[:, 0], backend.k_cache[0].cpu(), backend.v_cache[0].cpu(), (blocks,), (t,), bs,
+                               backend.scale, window=window)
+        assert_close(out[:, 0], want, 2e-2, f"decode under window {window}")
+    with pytest.raises(NotImplementedError):
+        backend.forward(q.cuda(), k.cuda(), v.cuda(), 0, InferenceContext(is_prefill=True, block_mask=object()))

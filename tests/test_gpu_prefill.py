@@ -186,3 +186,55 @@ def test_sliding_window_prefill_long_prefix_on_the_matrix_core_kernel():
                               _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk), _i32(np.arange(3) * cmax),
                               cmax, bs, d ** -0.5, out=out, window=window)
             assert_close(out.reshape(3, cmax, hq, d), want, 2e-2, f"block_size {bs} window {window}")
+
+
+@pytest.mark.parametrize("dtype,tol,d", [(torch.bfloat16, 2e-2, 128), (torch.float16, 2e-2, 64),
+                                         (torch.float32, 1e-5, 64)])
+def test_packed_documents_prefill(dtype, tol, d):
+    """Per-row first keys: packed documents (attention/mask.py:141-191) in dense rows, with boundaries inside
+    32-row blocks and 64-key tiles, an empty document, positions past the last document, alone and under a
+    sliding window; bf16 / fp16 run on the matrix cores, fp32 on the vector kernel."""
+    announce(f"prefill documents {dtype}")
+    rng = np.random.default_rng(300 + d)
+    hq, hkv, b, t = 8, 2, 2, 700
+    q, k, v = (torch.from_numpy(rng.standard_normal((b, t, h, d)).astype(np.float32)).to(dtype)
+               for h in (hq, hkv, hkv))
+    ident = torch.arange(b, dtype=torch.int32, device=DEV).reshape(b, 1).contiguous()
+    lens = _i32([t] * b)
+    for doc_lens in ((700,), (1, 31, 32, 0, 64, 65, 300, 150), (333, 300), (5,) * 100):
+        bounds = np.asarray(po.document_boundaries(doc_lens))
+        first = bounds[np.searchsorted(bounds[1:], np.arange(t), side="right")].astype(np.int32)
+        first = torch.from_numpy(np.tile(first, b)).to(DEV)
+        for window in (0, 40):
+            got = ops.prefill_paged(q.reshape(b * t, hq, d).to(DEV), k.reshape(b * t, hkv, d).to(DEV),
+                                    v.reshape(b * t, hkv, d).to(DEV), ident, lens, lens, _i32(np.arange(b) * t), t, t,
+                                    d ** -0.5, window=window, row_first_key=first)
+            want = po.dense_prefill(q, k, v, d ** -0.5, window=window, doc_lens=doc_lens)
+            assert_close(got.reshape(b, t, hq, d), want, tol, f"documents {doc_lens[:4]}.. window {window}")
+
+
+def test_packed_documents_chunked_prefill_over_a_prefix():
+    """Documents by absolute position in chunked prefill: the chunk's rows start inside a document that began
+    in the cached prefix, 16-token blocks."""
+    announce("prefill documents, chunked")
+    rng = np.random.default_rng(311)
+    hq, hkv, d, bs = 8, 2, 128, 16
+    prefix, chunk = [500, 129], [200, 260]
+    cmax = max(chunk)
+    need = [-(-(p + c) // bs) for p, c in zip(prefix, chunk)]
+    nb = sum(need) + 2
+    perm = rng.permutation(nb)
+    tables = [perm[: need[0]].tolist(), perm[need[0] : need[0] + need[1]].tolist()]
+    kc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+    vc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+    q = torch.from_numpy(rng.standard_normal((2, cmax, hq, d)).astype(np.float32)).to(torch.bfloat16)
+    doc_lens = (90, 350, 130, 47, 33, 200)
+    bounds = np.asarray(po.document_boundaries(doc_lens))
+    pos = np.asarray(prefix)[:, None] + np.arange(cmax)[None, :]
+    first = bounds[np.searchsorted(bounds[1:], pos, side="right")].astype(np.int32)
+    want = po.paged_prefill_chunk(q, kc, vc, tables, prefix, chunk, bs, d ** -0.5, doc_lens=doc_lens)
+    out = torch.zeros(2 * cmax, hq, d, device=DEV, dtype=torch.bfloat16)
+    ops.prefill_paged(q.reshape(-1, hq, d).to(DEV), kc.to(DEV), vc.to(DEV), tables_to_device(tables),
+                      _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk), _i32(np.arange(2) * cmax), cmax, bs,
+                      d ** -0.5, out=out, row_first_key=torch.from_numpy(first.reshape(-1)).to(DEV))
+    assert_close(out.reshape(2, cmax, hq, d), want, 2e-2, "chunked documents")

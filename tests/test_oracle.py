@@ -473,3 +473,60 @@ def test_window_decode_is_the_last_row_of_windowed_prefill():
     want = _swa_sdpa(qf, kc[slots][None], vc[slots][None], scale, window)[:, p_len:]
     got = po.paged_prefill_chunk(qc, kc, vc, [tables[0]], [p_len], [c_len], bs, scale, window=window)
     np.testing.assert_allclose(got, want.numpy(), rtol=1e-4, atol=1e-5)
+
+
+def _reference_document_entry(boundaries, q_idx, kv_idx):
+    """The loop of document_mask (attention/mask.py:173-186), one entry at a time."""
+    q_doc = 0
+    kv_doc = 0
+    for i, boundary in enumerate(boundaries[1:]):
+        if q_idx >= boundary:
+            q_doc = i + 1
+        if kv_idx >= boundary:
+            kv_doc = i + 1
+    return (q_doc == kv_doc) and (q_idx >= kv_idx)
+
+
+def test_document_prefill_matches_the_explicit_mask_and_separate_documents():
+    g = torch.Generator().manual_seed(43)
+    b, t, hq, hkv, d = 2, 23, 4, 2, 8
+    doc_lens = (5, 1, 0, 9, 4)  # sums to 19: positions 19..22 form one more document
+    bounds = po.document_boundaries(doc_lens)
+    assert bounds == [0, 5, 6, 6, 15, 19]
+    assert po.document_of(bounds, np.arange(t)).tolist() == [0] * 5 + [1] + [3] * 9 + [4] * 4 + [5] * 4
+    q, k, v = (torch.randn(b, t, h, d, generator=g) for h in (hq, hkv, hkv))
+    scale = d ** -0.5
+    keep = torch.tensor([[_reference_document_entry(bounds, r, c) for c in range(t)] for r in range(t)])
+    mask = torch.where(keep, 0.0, float("-inf"))[None, None]
+    n_rep = hq // hkv
+    want = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(1, 2), k.transpose(1, 2).repeat_interleave(n_rep, dim=1),
+        v.transpose(1, 2).repeat_interleave(n_rep, dim=1), attn_mask=mask, scale=scale).transpose(1, 2)
+    got = po.dense_prefill(q, k, v, scale, doc_lens=doc_lens)
+    np.testing.assert_allclose(got, want.numpy(), rtol=1e-4, atol=1e-5)
+    # every document alone, plain causal
+    for lo, hi in zip(bounds + [t], (bounds + [t])[1:]):
+        if hi > lo:
+            alone = po.dense_prefill(q[:, lo:hi], k[:, lo:hi], v[:, lo:hi], scale)
+            np.testing.assert_allclose(got[:, lo:hi], alone, rtol=0, atol=1e-12)
+    assert not np.allclose(got, po.dense_prefill(q, k, v, scale))
+    # with a window on top: both bounds apply
+    keep_w = keep & ((torch.arange(t)[:, None] - torch.arange(t)[None, :]) < 3)
+    want_w = torch.nn.functional.scaled_dot_product_attention(
+        q.transpose(1, 2), k.transpose(1, 2).repeat_interleave(n_rep, dim=1),
+        v.transpose(1, 2).repeat_interleave(n_rep, dim=1),
+        attn_mask=torch.where(keep_w, 0.0, float("-inf"))[None, None], scale=scale).transpose(1, 2)
+    np.testing.assert_allclose(po.dense_prefill(q, k, v, scale, window=3, doc_lens=doc_lens), want_w.numpy(),
+                               rtol=1e-4, atol=1e-5)
+    # chunked: rows [P:P+C] of the packed result, documents by absolute position
+    bs, p_len, c_len = 4, 9, 11
+    nb = 6
+    perm = torch.randperm(nb, generator=g).tolist()
+    kc = torch.zeros(nb * bs, hkv, d)
+    vc = torch.zeros(nb * bs, hkv, d)
+    slots = [perm[p // bs] * bs + p % bs for p in range(p_len + c_len)]
+    kc[slots] = k[0, : p_len + c_len]
+    vc[slots] = v[0, : p_len + c_len]
+    got_c = po.paged_prefill_chunk(q[:1, p_len : p_len + c_len], kc, vc, [perm], [p_len], [c_len], bs, scale,
+                                   doc_lens=doc_lens)
+    np.testing.assert_allclose(got_c, got[:1, p_len : p_len + c_len], rtol=0, atol=1e-12)
