@@ -158,6 +158,28 @@ def bench_prefill_c3(args, dev) -> int:
     ms_step = timed_ms(step, args.steps)
     ms_prefill = timed_ms(prefill, args.steps)
     ms_append = timed_ms(append, args.steps)
+    # The same append with the rotary embedding of q and k fused in (the step a model runs right before this
+    # path), beside the two-pass form: rotation into dense buffers, then the scatter.
+    pos = (torch.arange(C, dtype=torch.int32, device=dev) + P).repeat(S)
+    inv_freq = 1.0 / (10000.0 ** (torch.arange(0, w.head_dim, 2, device=dev).float() / w.head_dim))
+    angles = torch.arange(P + C, device=dev).float()[:, None] * inv_freq[None, :]
+    cos_t = torch.cat((angles, angles), dim=-1).cos().to(w.dtype)
+    sin_t = torch.cat((angles, angles), dim=-1).sin().to(w.dtype)
+    q_rot, k_rot = torch.empty_like(q), torch.empty_like(k_new)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)  # scratch pool: the timed pool keeps its unrotated rows
+
+    def rope_fused():
+        ops.rope_kv_append(q, k_new, v_new, cos_t, sin_t, kc2, vc2, slots, positions=pos, q_out=q_rot)
+
+    def rope_two_pass():
+        ops.rope_kv_append(q, k_new, v_new, cos_t, sin_t, None, None, None, positions=pos, q_out=q_rot, k_out=k_rot)
+        ops.kv_scatter(kc2, vc2, k_rot, v_new, slots)
+
+    preheat(rope_fused, 0.1)
+    ms_rope = timed_ms(rope_fused, args.steps)
+    ms_rope2 = timed_ms(rope_two_pass, args.steps)
+    eb = q.element_size()
+    rope_bytes = (2 * q.numel() + 4 * k_new.numel()) * eb + 2 * S * C * w.head_dim * eb + S * C * 12
     flops = w.attention_flops()
     achieved = flops / (ms_prefill * 1e-3) / 1e12
     result = {
@@ -174,6 +196,9 @@ def bench_prefill_c3(args, dev) -> int:
                      "traffic": MEASURED_TRAFFIC_BYTES.get("c3"), "kernel_ms": ms_prefill},
         "append": {"kernel": "kv_scatter_kernel", "kernel_ms": ms_append,
                    "achieved_gbps": w.append_bytes() / (ms_append * 1e-3) / 1e9, "peak_gbps": HBM_PEAK_GBPS},
+        "rope_append": {"kernel": "rope_kv_append_kernel", "kernel_ms": ms_rope, "bytes": rope_bytes,
+                        "achieved_gbps": rope_bytes / (ms_rope * 1e-3) / 1e9, "peak_gbps": HBM_PEAK_GBPS,
+                        "two_pass_ms": ms_rope2},
     }
     if not args.no_cpu_baseline:
         threads = torch.get_num_threads()

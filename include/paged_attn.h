@@ -220,6 +220,43 @@ int pa_kv_append_e4m3(void *k_cache, void *v_cache, float *k_scale, float *v_sca
                       const int32_t *touched_blocks, int n_touched, int64_t num_blocks, int block_size,
                       int num_kv_heads, int head_dim, int src_dtype, void *stream);
 
+/*
+ * Rotary position embedding fused with the KV append: the step a model runs immediately before this path
+ * (rollouts/tools/functional_extractor/llama_functional.py:203 applies apply_rotary_pos_emb, :75-98, right
+ * before attention, :210) merged with FlexAttentionBackend._store_kv (attention/flex_backend.py:116-142), so
+ * the step's new K rows are read once and written once.  For every token i, with r = positions[i] (or i):
+ *     x_embed = (x * cos[r]) + (rotate_half(x) * sin[r]),   rotate_half(x) = cat(-x[D/2:], x[:D/2])
+ * for every head of q (written to q_out, which may be q itself) and of k; the rotated k row goes to
+ * k_cache[slots[i]] (and to k_out[i] when k_out is given), the v row to v_cache[slots[i]].  Every product and
+ * the sum are rounded to `dtype`, as when the statement is evaluated on tensors of that type: results equal
+ * that evaluation bit for bit.
+ *   q, q_out     : [n_tokens][num_q_heads][head_dim]
+ *   k_src, v_src : [n_tokens][num_kv_heads][head_dim];  k_out: same shape or NULL
+ *   k_cache, v_cache : [total_slots][num_kv_heads][head_dim] of the same dtype
+ *   cos, sin     : [rope_rows][head_dim] of the same dtype (both halves are read, as the statement does)
+ *   positions    : int32[n_tokens] rows of cos/sin, clamped to the table; NULL: token i uses row i
+ *                  (tables laid out per token, the (batch, seq_len, head_dim) form of llama_functional.py:101-136)
+ *   slots        : int64[n_tokens]; negative or out-of-pool slots skip the cache write; NULL: no cache write
+ *                  (then k_out is required)
+ * head_dim/2 elements must fill whole 16-byte vectors (head_dim % 16 == 0 for 16-bit types).
+ */
+int pa_rope_kv_append(const void *q, void *q_out, const void *k_src, const void *v_src, void *k_out,
+                      void *k_cache, void *v_cache, const void *cos, const void *sin, const int32_t *positions,
+                      int64_t rope_rows, const int64_t *slots, int64_t n_tokens, int64_t total_slots,
+                      int num_q_heads, int num_kv_heads, int head_dim, int dtype, void *stream);
+
+/*
+ * The same for an fp8-e4m3 pool: q is rotated to q_out, the k rows are rotated as pa_rope_kv_append does
+ * (rounded to src_dtype) while pa_kv_append_e4m3's append reads them, and the v rows are appended as they are.
+ * Arguments as in pa_rope_kv_append and pa_kv_append_e4m3; the result equals pa_rope_kv_append into a dense
+ * k_out followed by pa_kv_append_e4m3 of k_out, bit for bit.
+ */
+int pa_rope_kv_append_e4m3(const void *q, void *q_out, const void *k_src, const void *v_src, void *k_cache,
+                           void *v_cache, float *k_scale, float *v_scale, const void *cos, const void *sin,
+                           const int32_t *positions, int64_t rope_rows, const int64_t *slots, int64_t n_tokens,
+                           const int32_t *touched_blocks, int n_touched, int64_t num_blocks, int block_size,
+                           int num_q_heads, int num_kv_heads, int head_dim, int src_dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -41,6 +41,12 @@ How each function is pinned (see tests/test_oracle.py):
                         scalar restatement of document_mask's loop
                         (attention/mask.py:173-186) entry by entry; equals
                         independent causal attention on each document alone
+  rope_tables           closed form angle = pos * theta**(-2i/D) in float64; cos^2 +
+                        sin^2 = 1; both halves of a row equal; position 0 -> (1, 0)
+  rope_literal          rope_exact (complex multiplication in float64) within the
+                        rounding of the type; position 0 is the identity; norms of
+                        (x_i, x_{i+D/2}) pairs kept; q.k after rotation depends only
+                        on the distance between the two positions
   quantize_kv_e4m3      torch.float8_e4m3fn conversion (library definition of
                         OCP e4m3fn, round to nearest even), known values
                         464 -> 448, 2**-10 -> 0, max 448
@@ -277,6 +283,39 @@ def paged_prefill_chunk(q, k_cache, v_cache, block_tables, prefix_lens, chunk_le
             out[b, :c, sl] = _attend_rows(q[b, :c, sl], kc[slots, g], vc[slots, g], scale, causal_offset=p,
                                           window=window, boundaries=bounds)
     return out
+
+
+# --------------------------------------------------------------------------- rotary embedding
+# (rollouts/tools/functional_extractor/llama_functional.py; the step a model runs right before attention)
+
+
+def rope_tables(positions: torch.Tensor, head_dim: int, theta: float = 10000.0,
+                dtype: torch.dtype = torch.bfloat16) -> Tuple[torch.Tensor, torch.Tensor]:
+    """cos / sin tables, statement by statement (llama_functional.py:101-136): ``inv_freq[i] =
+    theta**(-2i/D)`` in float32, angles = position * inv_freq, both halves of a row hold the same
+    angles, cosine and sine taken in float32 and cast once.  positions ``[B, T]`` -> ``[B, T, D]`` each."""
+    inv_freq = 1.0 / (theta ** (torch.arange(0, head_dim, 2).float() / head_dim))
+    freqs = (inv_freq[None, :, None] @ positions[:, None, :].float()).transpose(1, 2)
+    emb = torch.cat((freqs, freqs), dim=-1)
+    return emb.cos().to(dtype), emb.sin().to(dtype)
+
+
+def rope_literal(x: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor) -> torch.Tensor:
+    """``(x * cos) + (rotate_half(x) * sin)`` with the same tensor operations, in the tensors' own type
+    (llama_functional.py:68-72, :96-97).  x ``[N, H, D]``, cos/sin ``[N, D]`` (one row per token)."""
+    half = x.shape[-1] // 2
+    rotated = torch.cat((-x[..., half:], x[..., :half]), dim=-1)
+    return (x * cos[:, None, :]) + (rotated * sin[:, None, :])
+
+
+def rope_exact(x, angles: np.ndarray) -> np.ndarray:
+    """What the statement above computes, in float64 and in complex form: element i and element i + D/2 of a
+    head are the real and imaginary part of a number that is multiplied by ``exp(1j * angle_i)``.
+    x ``[N, H, D]``, angles ``[N, D/2]`` -> float64 ``[N, H, D]``."""
+    x = to_f64(x)
+    half = x.shape[-1] // 2
+    z = (x[..., :half] + 1j * x[..., half:]) * np.exp(1j * np.asarray(angles, dtype=np.float64))[:, None, :]
+    return np.concatenate([z.real, z.imag], axis=-1)
 
 
 # --------------------------------------------------------------------------- literal restatement (torch)

@@ -25,6 +25,12 @@ void pa_clear_error();
             return pa_fail(PA_ERR_HIP, "%s: %s", what, hipGetErrorString(e_));     \
     } while (0)
 
+// Shared by the rotary entry points (rope.hip): argument checks, and the rotation of q alone (no K/V work).
+int pa_rope_check(const char *what, int64_t n_tokens, int64_t rope_rows, const int32_t *positions, int num_q_heads,
+                  int num_kv_heads, int head_dim, int dtype);
+int pa_rope_q_only(const void *q, void *q_out, const void *cos, const void *sin, const int32_t *positions,
+                   int64_t rope_rows, int64_t n_tokens, int num_q_heads, int head_dim, int dtype, void *stream);
+
 static inline bool pa_aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 // -------------------------------------------------------------- device side

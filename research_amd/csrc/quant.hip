@@ -48,12 +48,43 @@ __global__ __launch_bounds__(kQThreads) void quantize_e4m3_kernel(const T *__res
 //   otherwise scale' = a_new / 448 and the content is re-rounded: byte' = e4m3(float(byte) * (scale / scale')).
 constexpr int kMaxBlockTokens = 256;
 
-template <typename T>
+// Rotary tables of a fused append: the rows are rotated as they are read, x' = (x*cos) + (rotate_half(x)*sin)
+// with every product and the sum rounded to the rows' type T (the rounding of that statement evaluated in T).
+struct RopeTables {
+    const void *cos, *sin;     // [rope_rows][d] of T
+    const int32_t *positions;  // row per token, or NULL: the token's own index
+    int64_t rope_rows;
+};
+
+template <typename T> __device__ __forceinline__ float round_to(float x) {
+    T t;
+    pa_scalar<T>::store(&t, x);
+    return pa_scalar<T>::load(&t);
+}
+
+template <typename T, bool ROPE>
+__device__ __forceinline__ float load_src_elem(const T *src, const RopeTables &rt, int tok, int hkv, int h, int d, int e) {
+#pragma clang fp contract(off)
+    const T *row = src + ((int64_t)tok * hkv + h) * d;
+    const float x = pa_scalar<T>::load(row + e);
+    if (!ROPE) return x;
+    int64_t r = rt.positions ? (int64_t)rt.positions[tok] : tok;
+    r = r < 0 ? 0 : (r >= rt.rope_rows ? rt.rope_rows - 1 : r);
+    const int half = d / 2;
+    const float other = e < half ? -pa_scalar<T>::load(row + e + half) : pa_scalar<T>::load(row + e - half);
+    const float c = pa_scalar<T>::load((const T *)rt.cos + r * d + e);
+    const float sn = pa_scalar<T>::load((const T *)rt.sin + r * d + e);
+    const float a = round_to<T>(x * c);
+    const float b = round_to<T>(other * sn);
+    return round_to<T>(a + b);
+}
+
+template <typename T, bool ROPE>
 __global__ __launch_bounds__(kQThreads) void append_e4m3_kernel(const T *__restrict__ src, uint8_t *__restrict__ dst,
                                                                  float *__restrict__ scale,
                                                                  const int64_t *__restrict__ slots, int64_t n_tokens,
                                                                  const int32_t *__restrict__ touched, int64_t num_blocks,
-                                                                 int block_size, int hkv, int d) {
+                                                                 int block_size, int hkv, int d, const RopeTables rt) {
     __shared__ int s_token[kMaxBlockTokens];  // token of this call that writes offset i (-1: none); highest index wins
     __shared__ float s_max[2][kQThreads / PA_WAVE];
     const int64_t blk = touched[blockIdx.x];
@@ -84,7 +115,7 @@ __global__ __launch_bounds__(kQThreads) void append_e4m3_kernel(const T *__restr
     for (int i = threadIdx.x; i < (block_size - first) * d; i += kQThreads) {
         const int t = first + i / d, e = i % d;
         const int tok = s_token[t];
-        if (tok >= 0) a_new = fmaxf(a_new, fabsf(pa_scalar<T>::load(src + ((int64_t)tok * hkv + h) * d + e)));
+        if (tok >= 0) a_new = fmaxf(a_new, fabsf(load_src_elem<T, ROPE>(src, rt, tok, hkv, h, d, e)));
     }
     for (int off = 32; off > 0; off >>= 1) {
         q_max = fmaxf(q_max, __shfl_xor(q_max, off, 64));
@@ -109,10 +140,37 @@ __global__ __launch_bounds__(kQThreads) void append_e4m3_kernel(const T *__restr
         const int t = first + i / d, e = i % d;
         const int tok = s_token[t];
         if (tok < 0) continue;
-        const float x = pa_scalar<T>::load(src + ((int64_t)tok * hkv + h) * d + e) / s_new;
+        const float x = load_src_elem<T, ROPE>(src, rt, tok, hkv, h, d, e) / s_new;
         dst[tile0 + t * tok_stride + e] = (uint8_t)(__builtin_amdgcn_cvt_pk_fp8_f32(x, 0.f, 0, false) & 0xff);
     }
     if (threadIdx.x == 0) scale[blk * hkv + h] = s_new;
+}
+
+// Appends one of K / V; `rt` non-NULL rotates the rows on the way (K of a fused rotary append).
+template <bool ROPE>
+void launch_append(const void *src, uint8_t *dst, float *sc, const int64_t *slots, int64_t n_tokens,
+                   const int32_t *touched, int n_touched, int64_t num_blocks, int block_size, int hkv, int d,
+                   int src_dtype, const RopeTables &rt, hipStream_t s) {
+    const dim3 grid((unsigned)n_touched, (unsigned)hkv), block(kQThreads);
+    if (src_dtype == PA_F32)
+        append_e4m3_kernel<float, ROPE><<<grid, block, 0, s>>>((const float *)src, dst, sc, slots, n_tokens, touched,
+                                                                num_blocks, block_size, hkv, d, rt);
+    else if (src_dtype == PA_BF16)
+        append_e4m3_kernel<pa_bf16, ROPE><<<grid, block, 0, s>>>((const pa_bf16 *)src, dst, sc, slots, n_tokens, touched,
+                                                                  num_blocks, block_size, hkv, d, rt);
+    else
+        append_e4m3_kernel<pa_f16, ROPE><<<grid, block, 0, s>>>((const pa_f16 *)src, dst, sc, slots, n_tokens, touched,
+                                                                 num_blocks, block_size, hkv, d, rt);
+}
+
+int check_append(int64_t n_tokens, int n_touched, int block_size, int num_kv_heads, int head_dim, int src_dtype) {
+    PA_REQUIRE(n_tokens >= 0 && n_touched >= 0, "n_tokens=%lld / n_touched=%d is negative", (long long)n_tokens, n_touched);
+    PA_REQUIRE(block_size > 0 && block_size <= kMaxBlockTokens, "block_size=%d outside 1..%d", block_size, kMaxBlockTokens);
+    PA_REQUIRE(num_kv_heads > 0 && num_kv_heads <= 65535 && head_dim > 0, "num_kv_heads / head_dim out of range");
+    PA_REQUIRE(src_dtype == PA_F32 || src_dtype == PA_BF16 || src_dtype == PA_F16, "src_dtype=%d is not F32, BF16 or F16",
+               src_dtype);
+    PA_REQUIRE(n_tokens <= 0x7fffffffll, "n_tokens above 2^31-1");
+    return PA_OK;
 }
 
 }  // namespace
@@ -122,31 +180,47 @@ extern "C" int pa_kv_append_e4m3(void *k_cache, void *v_cache, float *k_scale, f
                                  const int32_t *touched_blocks, int n_touched, int64_t num_blocks, int block_size,
                                  int num_kv_heads, int head_dim, int src_dtype, void *stream) {
     pa_clear_error();
-    PA_REQUIRE(n_tokens >= 0 && n_touched >= 0, "n_tokens=%lld / n_touched=%d is negative", (long long)n_tokens, n_touched);
-    PA_REQUIRE(block_size > 0 && block_size <= kMaxBlockTokens, "block_size=%d outside 1..%d", block_size, kMaxBlockTokens);
-    PA_REQUIRE(num_kv_heads > 0 && num_kv_heads <= 65535 && head_dim > 0, "num_kv_heads / head_dim out of range");
-    PA_REQUIRE(src_dtype == PA_F32 || src_dtype == PA_BF16 || src_dtype == PA_F16, "src_dtype=%d is not F32, BF16 or F16",
-               src_dtype);
-    PA_REQUIRE(n_tokens <= 0x7fffffffll, "n_tokens above 2^31-1");
+    if (int rc = check_append(n_tokens, n_touched, block_size, num_kv_heads, head_dim, src_dtype)) return rc;
     if (n_tokens == 0 || n_touched == 0) return PA_OK;
     PA_REQUIRE(k_cache && v_cache && k_scale && v_scale && k_src && v_src && slots && touched_blocks, "NULL pointer argument");
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid((unsigned)n_touched, (unsigned)num_kv_heads), block(kQThreads);
-    for (int which = 0; which < 2; ++which) {
-        uint8_t *dst = (uint8_t *)(which ? v_cache : k_cache);
-        float *sc = which ? v_scale : k_scale;
-        const void *src = which ? v_src : k_src;
-        if (src_dtype == PA_F32)
-            append_e4m3_kernel<float><<<grid, block, 0, s>>>((const float *)src, dst, sc, slots, n_tokens, touched_blocks,
-                                                             num_blocks, block_size, num_kv_heads, head_dim);
-        else if (src_dtype == PA_BF16)
-            append_e4m3_kernel<pa_bf16><<<grid, block, 0, s>>>((const pa_bf16 *)src, dst, sc, slots, n_tokens,
-                                                               touched_blocks, num_blocks, block_size, num_kv_heads, head_dim);
-        else
-            append_e4m3_kernel<pa_f16><<<grid, block, 0, s>>>((const pa_f16 *)src, dst, sc, slots, n_tokens, touched_blocks,
-                                                              num_blocks, block_size, num_kv_heads, head_dim);
-        PA_CHECK_LAUNCH("pa_kv_append_e4m3");
-    }
+    const RopeTables none{};
+    launch_append<false>(k_src, (uint8_t *)k_cache, k_scale, slots, n_tokens, touched_blocks, n_touched, num_blocks,
+                         block_size, num_kv_heads, head_dim, src_dtype, none, s);
+    PA_CHECK_LAUNCH("pa_kv_append_e4m3");
+    launch_append<false>(v_src, (uint8_t *)v_cache, v_scale, slots, n_tokens, touched_blocks, n_touched, num_blocks,
+                         block_size, num_kv_heads, head_dim, src_dtype, none, s);
+    PA_CHECK_LAUNCH("pa_kv_append_e4m3");
+    return PA_OK;
+}
+
+extern "C" int pa_rope_kv_append_e4m3(const void *q, void *q_out, const void *k_src, const void *v_src, void *k_cache,
+                                      void *v_cache, float *k_scale, float *v_scale, const void *cos, const void *sin,
+                                      const int32_t *positions, int64_t rope_rows, const int64_t *slots,
+                                      int64_t n_tokens, const int32_t *touched_blocks, int n_touched,
+                                      int64_t num_blocks, int block_size, int num_q_heads, int num_kv_heads,
+                                      int head_dim, int src_dtype, void *stream) {
+    pa_clear_error();
+    if (int rc = check_append(n_tokens, n_touched, block_size, num_kv_heads, head_dim, src_dtype)) return rc;
+    if (int rc = pa_rope_check("pa_rope_kv_append_e4m3", n_tokens, rope_rows, positions, num_q_heads, num_kv_heads,
+                               head_dim, src_dtype))
+        return rc;
+    if (n_tokens == 0) return PA_OK;
+    PA_REQUIRE(q && q_out && cos && sin, "NULL q / q_out / cos / sin");
+    PA_REQUIRE(pa_aligned16(q) && pa_aligned16(q_out) && pa_aligned16(cos) && pa_aligned16(sin),
+               "q, q_out, cos and sin must be 16-byte aligned");
+    if (int rc = pa_rope_q_only(q, q_out, cos, sin, positions, rope_rows, n_tokens, num_q_heads, head_dim, src_dtype, stream))
+        return rc;
+    if (n_touched == 0) return PA_OK;
+    PA_REQUIRE(k_cache && v_cache && k_scale && v_scale && k_src && v_src && slots && touched_blocks, "NULL pointer argument");
+    hipStream_t s = (hipStream_t)stream;
+    const RopeTables rt{cos, sin, positions, rope_rows};
+    launch_append<true>(k_src, (uint8_t *)k_cache, k_scale, slots, n_tokens, touched_blocks, n_touched, num_blocks,
+                        block_size, num_kv_heads, head_dim, src_dtype, rt, s);
+    PA_CHECK_LAUNCH("pa_rope_kv_append_e4m3");
+    launch_append<false>(v_src, (uint8_t *)v_cache, v_scale, slots, n_tokens, touched_blocks, n_touched, num_blocks,
+                         block_size, num_kv_heads, head_dim, src_dtype, RopeTables{}, s);
+    PA_CHECK_LAUNCH("pa_rope_kv_append_e4m3");
     return PA_OK;
 }
 

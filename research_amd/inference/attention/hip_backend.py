@@ -168,13 +168,69 @@ class HipPagedAttentionBackend:
         """
         if ctx.slot_mapping is not None:
             self._store_kv(k, v, layer_idx, ctx.slot_mapping, _step=self._step(ctx))
+        return self._attend(q, k, v, layer_idx, ctx)
+
+    __call__ = forward
+
+    def _attend(self, q: Tensor, k: Tensor, v: Tensor, layer_idx: int, ctx: InferenceContext) -> Tensor:
         if ctx.is_prefill:
             if getattr(ctx, "prefix_lens", None) is not None:  # absent on the reference's own context type
                 return self._prefill_paged(q, layer_idx, ctx)
             return self._prefill_attention(q, k, v, ctx)
         return self._decode_attention(q, layer_idx, ctx)
 
-    __call__ = forward
+    def forward_rope(self, q: Tensor, k: Tensor, v: Tensor, cos: Tensor, sin: Tensor, layer_idx: int,
+                     ctx: InferenceContext, positions: Optional[Tensor] = None) -> Tensor:
+        """``forward`` on the rotary-embedded q and k, with the rotation fused into the KV append.
+
+        Equals ``q, k = apply_rotary_pos_emb(q, k, cos, sin)`` (rollouts/tools/functional_extractor/
+        llama_functional.py:75-98, evaluated in the tensors' dtype) followed by ``forward(q, k, v, layer_idx,
+        ctx)``, but the new K rows are read once and written once: one kernel rotates q and k and writes the
+        rotated k and v to their slots.  q ``[B, T, Hq, D]``, k/v ``[B, T, Hkv, D]``; cos/sin ``[B, T, D]`` (one
+        row per token) or, with ``positions`` (int ``[B, T]``), a table ``[rows, D]`` indexed by position.
+        q and k are not modified.
+        """
+        cfg = self.config
+        batch, seq_len, num_heads, head_dim = q.shape
+        n = batch * seq_len
+        self._require_device(q, k, v, cos, sin, self.k_cache)
+        q3 = q.contiguous().view(n, num_heads, head_dim)
+        k3 = k.reshape(n, cfg.num_kv_heads, head_dim).contiguous()
+        v3 = v.reshape(n, cfg.num_kv_heads, head_dim).contiguous()
+        cos2 = cos.reshape(-1, head_dim).contiguous()
+        sin2 = sin.reshape(-1, head_dim).contiguous()
+        pos = None
+        if positions is not None:
+            pos = positions.reshape(-1).to(device=q.device, dtype=torch.int32).contiguous()
+            if pos.numel() != n:
+                raise ValueError("positions must hold one entry per token")
+        elif cos2.shape[0] != n:
+            raise ValueError("cos / sin must hold one row per token when no positions are given")
+        q_rot = torch.empty_like(q3)
+        if n == 0:
+            return q_rot.view(q.shape)
+        slots = None
+        if ctx.slot_mapping is not None:
+            step = self._step(ctx)
+            slots = self._device_slots(ctx.slot_mapping, n, step)
+        dense = ctx.is_prefill and getattr(ctx, "prefix_lens", None) is None  # attends the step's own K/V
+        kc, vc = self._layer(layer_idx)
+        if self._fp8 and slots is not None:
+            if dense:
+                raise NotImplementedError("dense prefill attends the step's own K; use an fp8 pool with chunked prefill")
+            if step.touched is None:
+                step.touched = ops.touched_blocks(slots, cfg.block_size, cfg.num_blocks)
+            ops.rope_kv_append_e4m3(q3, k3, v3, cos2, sin2, kc, vc, self.k_scale[layer_idx], self.v_scale[layer_idx],
+                                    slots, cfg.block_size, positions=pos, q_out=q_rot, touched=step.touched)
+            k_rot = None
+        else:
+            if slots is not None and k3.dtype != self.k_cache.dtype:
+                raise RuntimeError("Index put requires the source and destination dtypes match")
+            k_rot = torch.empty_like(k3) if dense or slots is None else None
+            ops.rope_kv_append(q3, k3, v3, cos2, sin2, kc if slots is not None else None,
+                               vc if slots is not None else None, slots, positions=pos, q_out=q_rot, k_out=k_rot)
+        k_att = k_rot.view(batch, seq_len, cfg.num_kv_heads, head_dim) if k_rot is not None else k
+        return self._attend(q_rot.view(q.shape), k_att, v, layer_idx, ctx)
 
     # ------------------------------------------------------------------ helpers
     def _require_device(self, *tensors: Tensor) -> torch.device:
@@ -232,6 +288,33 @@ class HipPagedAttentionBackend:
     def _layer(self, layer_idx: int) -> Tuple[Tensor, Tensor]:
         return self.k_cache[layer_idx], self.v_cache[layer_idx]
 
+    def _device_slots(self, slot_mapping, n: int, step: Optional[_StepTensors], *tensors: Tensor) -> Tensor:
+        """int64 device copy of a slot mapping (cached on the step), with the reference's error for a slot
+        past the pool."""
+        cfg = self.config
+        if len(slot_mapping) != n:
+            raise IndexError(
+                f"The shape of the mask [{len(slot_mapping)}] at index 0 does not match the shape of the indexed "
+                f"tensor [{n}, {cfg.num_kv_heads}, {cfg.head_dim}] at index 0")
+        if step is not None and step.slots is not None:
+            return step.slots
+        if isinstance(slot_mapping, Tensor) and slot_mapping.device.type == "cuda":
+            # already on the device: used as it is (out-of-range slots are dropped by the kernel, not reported)
+            self._require_device(*tensors, self.k_cache)
+            slots = slot_mapping.to(torch.int64).contiguous()
+        else:
+            if isinstance(slot_mapping, Tensor):
+                slot_mapping = slot_mapping.numpy()
+            host = np.asarray(slot_mapping, dtype=np.int64)
+            if host.size and host.max() >= cfg.total_slots:
+                raise IndexError(
+                    f"index {int(host.max())} is out of bounds for dimension 0 with size {cfg.total_slots}")
+            self._require_device(*tensors, self.k_cache)
+            slots = self._to_device(host)
+        if step is not None:
+            step.slots = slots
+        return slots
+
     # ------------------------------------------------------------------ KV append
     def _store_kv(self, k: Tensor, v: Tensor, layer_idx: int, slot_mapping: Tuple[int, ...],
                   _step: Optional[_StepTensors] = None) -> None:
@@ -253,25 +336,7 @@ class HipPagedAttentionBackend:
             raise RuntimeError("Index put requires the source and destination dtypes match")
         if n == 0:
             return
-        if _step is not None and _step.slots is not None:
-            slots = _step.slots
-        elif isinstance(slot_mapping, Tensor) and slot_mapping.device.type == "cuda":
-            # already on the device: used as it is (out-of-range slots are dropped by the kernel, not reported)
-            self._require_device(k_flat, v_flat, self.k_cache)
-            slots = slot_mapping.to(torch.int64).contiguous()
-            if _step is not None:
-                _step.slots = slots
-        else:
-            if isinstance(slot_mapping, Tensor):
-                slot_mapping = slot_mapping.numpy()
-            host = np.asarray(slot_mapping, dtype=np.int64)
-            if host.max() >= cfg.total_slots:
-                raise IndexError(
-                    f"index {int(host.max())} is out of bounds for dimension 0 with size {cfg.total_slots}")
-            self._require_device(k_flat, v_flat, self.k_cache)
-            slots = self._to_device(host)
-            if _step is not None:
-                _step.slots = slots
+        slots = self._device_slots(slot_mapping, n, _step, k_flat, v_flat)
         k_flat, v_flat = k_flat.contiguous(), v_flat.contiguous()
         kc, vc = self._layer(layer_idx)
         if self._fp8:

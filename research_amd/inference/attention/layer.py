@@ -21,3 +21,9 @@ class Attention(nn.Module):
 
     def forward(self, q: Tensor, k: Tensor, v: Tensor, ctx: InferenceContext) -> Tensor:
         return self.backend.forward(q, k, v, self.layer_idx, ctx)
+
+    def forward_rope(self, q: Tensor, k: Tensor, v: Tensor, cos: Tensor, sin: Tensor, ctx: InferenceContext,
+                     positions=None) -> Tensor:
+        """``forward`` on rotary-embedded q and k with the rotation fused into the KV append (an addition: the
+        reference's blocks rotate q and k themselves, llama_functional.py:203, and then call ``forward``)."""
+        return self.backend.forward_rope(q, k, v, cos, sin, self.layer_idx, ctx, positions=positions)

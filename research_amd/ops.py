@@ -142,3 +142,55 @@ def kv_append_e4m3(k_cache: Tensor, v_cache: Tensor, k_scale: Tensor, v_scale: T
     _run("pa_kv_append_e4m3", _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale), _ptr(k_src), _ptr(v_src),
          _ptr(slots), slots.numel(), _ptr(touched), touched.numel(), num_blocks, block_size, hkv, d,
          PA_DTYPE[k_src.dtype], _stream(k_cache))
+
+
+def rope_kv_append(q: Tensor, k_src: Tensor, v_src: Tensor, cos: Tensor, sin: Tensor, k_cache: Optional[Tensor],
+                   v_cache: Optional[Tensor], slots: Optional[Tensor], positions: Optional[Tensor] = None,
+                   q_out: Optional[Tensor] = None, k_out: Optional[Tensor] = None) -> Tensor:
+    """Rotary embedding of q and k fused with the KV append (``pa_rope_kv_append``).
+
+    q ``[N, Hq, D]``, k_src/v_src ``[N, Hkv, D]``, cos/sin ``[R, D]`` of the same dtype; ``positions`` int32 ``[N]``
+    picks the table row per token (None: row i for token i).  The rotated k and v go to the caches at ``slots``
+    (int64 ``[N]``; None: no cache write) and the rotated k also to ``k_out`` when given.  Returns rotated q
+    (``q_out``, or q itself rotated in place when ``q_out`` is None).
+    """
+    n, hq, d = q.shape
+    hkv = k_src.shape[1]
+    if q_out is None:
+        q_out = q
+    for t in (k_src, v_src, cos, sin):
+        if t.dtype != q.dtype:
+            raise RuntimeError("q, k, v, cos and sin must have the same dtype")
+    if positions is not None and positions.dtype != torch.int32:
+        raise ValueError("positions must be int32")
+    if cos.shape != sin.shape or cos.dim() != 2 or cos.shape[1] != d:
+        raise ValueError("cos / sin must be [rows, head_dim]")
+    total_slots = k_cache.shape[0] if k_cache is not None else 0
+    _run("pa_rope_kv_append", _ptr(q), _ptr(q_out), _ptr(k_src), _ptr(v_src), _ptr(k_out), _ptr(k_cache),
+         _ptr(v_cache), _ptr(cos), _ptr(sin), _ptr(positions), cos.shape[0], _ptr(slots), n, total_slots, hq, hkv, d,
+         PA_DTYPE[q.dtype], _stream(q))
+    return q_out
+
+
+def rope_kv_append_e4m3(q: Tensor, k_src: Tensor, v_src: Tensor, cos: Tensor, sin: Tensor, k_cache: Tensor,
+                        v_cache: Tensor, k_scale: Tensor, v_scale: Tensor, slots: Tensor, block_size: int,
+                        positions: Optional[Tensor] = None, q_out: Optional[Tensor] = None,
+                        touched: Optional[Tensor] = None) -> Tensor:
+    """``rope_kv_append`` into an fp8-e4m3 pool (``pa_rope_kv_append_e4m3``): k is rotated while the fp8 append
+    reads it; arguments as in ``rope_kv_append`` and ``kv_append_e4m3``."""
+    n, hq, d = q.shape
+    total_slots, hkv, _ = k_cache.shape
+    num_blocks = total_slots // block_size
+    if q_out is None:
+        q_out = q
+    for t in (k_src, v_src, cos, sin):
+        if t.dtype != q.dtype:
+            raise RuntimeError("q, k, v, cos and sin must have the same dtype")
+    if positions is not None and positions.dtype != torch.int32:
+        raise ValueError("positions must be int32")
+    if touched is None:
+        touched = touched_blocks(slots, block_size, num_blocks)
+    _run("pa_rope_kv_append_e4m3", _ptr(q), _ptr(q_out), _ptr(k_src), _ptr(v_src), _ptr(k_cache), _ptr(v_cache),
+         _ptr(k_scale), _ptr(v_scale), _ptr(cos), _ptr(sin), _ptr(positions), cos.shape[0], _ptr(slots), n,
+         _ptr(touched), touched.numel(), num_blocks, block_size, hq, hkv, d, PA_DTYPE[q.dtype], _stream(q))
+    return q_out

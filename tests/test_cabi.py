@@ -148,6 +148,37 @@ def test_prefill_and_quantize_argument_errors():
     assert rc == _lib.PA_OK
 
 
+def test_rope_argument_errors():
+    rope = [FAKE, FAKE, FAKE, FAKE, None, FAKE, FAKE, FAKE, FAKE, None, 8, FAKE, 4, 64, 32, 8, 128, _lib.PA_BF16, None]
+    bad = list(rope); bad[17] = _lib.PA_FP8_E4M3
+    rc, msg = _status("pa_rope_kv_append", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "dtype" in msg
+    bad = list(rope); bad[16] = 24  # half a head = 12 bf16 = 24 bytes
+    rc, msg = _status("pa_rope_kv_append", *bad)
+    assert rc == _lib.PA_ERR_UNSUPPORTED and "16 bytes" in msg
+    bad = list(rope); bad[10] = 3  # 3 table rows for 4 tokens and no positions
+    rc, msg = _status("pa_rope_kv_append", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "positions" in msg
+    bad = list(rope); bad[11] = None  # no slots and no k_out
+    rc, msg = _status("pa_rope_kv_append", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "nowhere" in msg
+    bad = list(rope); bad[0] = None
+    rc, msg = _status("pa_rope_kv_append", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
+    bad = list(rope); bad[12] = 0
+    assert _status("pa_rope_kv_append", *bad)[0] == _lib.PA_OK
+    fp8 = [FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, None, 8, FAKE, 4, FAKE, 1, 64, 16, 32, 8, 128,
+           _lib.PA_BF16, None]
+    bad = list(fp8); bad[17] = 1024
+    rc, msg = _status("pa_rope_kv_append_e4m3", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "block_size" in msg
+    bad = list(fp8); bad[11] = 2
+    rc, msg = _status("pa_rope_kv_append_e4m3", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "positions" in msg
+    bad = list(fp8); bad[13] = 0
+    assert _status("pa_rope_kv_append_e4m3", *bad)[0] == _lib.PA_OK
+
+
 def test_error_text_is_cleared_by_a_good_call():
     _status("pa_kv_scatter", FAKE, FAKE, FAKE, FAKE, FAKE, -1, 64, 8, 128, 2, None)
     assert _lib.last_error() != ""

@@ -530,3 +530,48 @@ def test_document_prefill_matches_the_explicit_mask_and_separate_documents():
     got_c = po.paged_prefill_chunk(q[:1, p_len : p_len + c_len], kc, vc, [perm], [p_len], [c_len], bs, scale,
                                    doc_lens=doc_lens)
     np.testing.assert_allclose(got_c, got[:1, p_len : p_len + c_len], rtol=0, atol=1e-12)
+
+
+def test_rope_tables_closed_form():
+    d, theta = 16, 10000.0
+    pos = torch.tensor([[0, 1, 2, 77], [5, 4096, 3, 9]])
+    cos, sin = po.rope_tables(pos, d, theta, torch.float32)
+    assert cos.shape == (2, 4, d)
+    angle = pos.numpy()[..., None].astype(np.float64) * theta ** (-np.arange(0, d, 2, dtype=np.float64) / d)
+    np.testing.assert_allclose(cos[..., : d // 2].numpy(), np.cos(angle), atol=5e-4)  # float32 angles at 4096 rad
+    np.testing.assert_allclose(sin[..., : d // 2].numpy(), np.sin(angle), atol=5e-4)
+    small = pos.numpy() < 100
+    np.testing.assert_allclose(cos[..., : d // 2].numpy()[small], np.cos(angle)[small], atol=1e-5)
+    assert torch.equal(cos[..., : d // 2], cos[..., d // 2 :]) and torch.equal(sin[..., : d // 2], sin[..., d // 2 :])
+    np.testing.assert_allclose((cos ** 2 + sin ** 2).numpy(), 1.0, atol=1e-6)
+    assert torch.equal(cos[0, 0], torch.ones(d)) and torch.equal(sin[0, 0], torch.zeros(d))
+    cb, _ = po.rope_tables(pos, d, theta, torch.bfloat16)
+    assert cb.dtype == torch.bfloat16 and torch.equal(cb, cos.to(torch.bfloat16))  # cast once, at the end
+
+
+def test_rope_literal_is_a_rotation():
+    g = torch.Generator().manual_seed(44)
+    n, h, d, theta = 9, 3, 16, 10000.0
+    x = torch.randn(n, h, d, generator=g)
+    pos = torch.tensor([[0, 1, 2, 3, 10, 50, 7, 7, 123]])
+    cos, sin = (t[0] for t in po.rope_tables(pos, d, theta, torch.float32))
+    angle = pos[0].numpy()[:, None].astype(np.float64) * theta ** (-np.arange(0, d, 2, dtype=np.float64) / d)
+    got = po.rope_literal(x, cos, sin)
+    np.testing.assert_allclose(got.numpy(), po.rope_exact(x, angle), atol=2e-5)
+    assert torch.equal(got[0], x[0])  # position 0
+    pair_norm = lambda t: (t[..., : d // 2] ** 2 + t[..., d // 2 :] ** 2)
+    np.testing.assert_allclose(pair_norm(got).numpy(), pair_norm(x).numpy(), rtol=1e-5, atol=1e-6)
+    # a sign or half mix-up fails this: rotating by +angle then by -angle is the identity
+    back = po.rope_literal(got, cos, -sin)
+    np.testing.assert_allclose(back.numpy(), x.numpy(), atol=1e-5)
+    # relative positions: <rope(q, m), rope(k, n)> depends on m - n only
+    q, k = torch.randn(1, 1, d, generator=g), torch.randn(1, 1, d, generator=g)
+    def dot(m, nn):
+        c, s = (t[0] for t in po.rope_tables(torch.tensor([[m, nn]]), d, theta, torch.float32))
+        return float((po.rope_literal(q, c[:1], s[:1]) * po.rope_literal(k, c[1:], s[1:])).sum())
+    assert abs(dot(5, 2) - dot(40, 37)) < 1e-4 and abs(dot(5, 2) - dot(2, 5)) > 1e-3
+    # bf16: every product and the sum rounded to bf16 -> within a few bf16 ulps of the exact rotation
+    xb = x.to(torch.bfloat16)
+    gb = po.rope_literal(xb, cos.to(torch.bfloat16), sin.to(torch.bfloat16))
+    assert gb.dtype == torch.bfloat16
+    np.testing.assert_allclose(gb.float().numpy(), po.rope_exact(xb, angle), atol=0.06, rtol=0.02)
