@@ -336,3 +336,52 @@ def test_block_mask_objects_through_the_backend():
         assert_close(out[:, 0], want, 2e-2, f"decode under window {window}")
     with pytest.raises(NotImplementedError):
         backend.forward(q.cuda(), k.cuda(), v.cuda(), 0, InferenceContext(is_prefill=True, block_mask=object()))
+
+
+def test_prefix_reuse_through_the_radix_cache():
+    """Rollouts of one prompt: the first prefills everything, the others find the prompt's full blocks in the
+    tree and prefill only their own suffix over the shared blocks; every result equals dense causal attention
+    over the whole sequence, and decode afterwards reads the shared blocks through each block table."""
+    from research_amd.inference.cache import RadixKVCache
+    from research_amd.inference.context import build_chunked_prefill_context, build_decode_context
+
+    announce("backend + radix cache prefix reuse")
+    g = torch.Generator().manual_seed(71)
+    hq, hkv, d, bs = 8, 2, 64, 16
+    config = CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=32, block_size=bs, device="cuda")
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(hq)
+    cache = RadixKVCache(32, bs)
+    prompt_len, n_rollouts = 70, 4  # 4 full blocks + 6 tokens
+    prompt = list(range(prompt_len))
+    qp, kp, vp = (torch.randn(1, prompt_len, h, d, generator=g).to(torch.bfloat16) for h in (hq, hkv, hkv))
+    full_q, full_k, full_v = [], [], []
+    for r in range(n_rollouts):
+        own = 5 + 3 * r
+        toks = prompt + [1000 * (r + 1) + i for i in range(own)]
+        qo, ko, vo = (torch.randn(1, own, h, d, generator=g).to(torch.bfloat16) for h in (hq, hkv, hkv))
+        q, k, v = torch.cat([qp, qo], 1), torch.cat([kp, ko], 1), torch.cat([vp, vo], 1)
+        full_q.append(q), full_k.append(k), full_v.append(v)
+        blocks = cache.allocate(r, toks)
+        cached = cache.get_cached_tokens(r)
+        assert cached == (0 if r == 0 else 64)
+        ctx = build_chunked_prefill_context(cache, [r], [cached], [len(toks) - cached], [blocks])
+        out = backend.forward(q[:, cached:].cuda(), k[:, cached:].cuda(), v[:, cached:].cuda(), 0, ctx)
+        want = po.dense_prefill(q, k, v, backend.scale)[:, cached:]
+        assert_close(out, want, 2e-2, f"rollout {r}, {cached} cached tokens")
+    tables = [cache.get_block_ids(r) for r in range(n_rollouts)]
+    assert all(t[:4] == tables[0][:4] for t in tables) and len({t[4] for t in tables}) == n_rollouts
+    # one decode step for all rollouts at once
+    lens = [prompt_len + 5 + 3 * r + 1 for r in range(n_rollouts)]
+    q1, k1, v1 = (torch.randn(n_rollouts, 1, h, d, generator=g).to(torch.bfloat16) for h in (hq, hkv, hkv))
+    for r in range(n_rollouts):
+        cache.append_token(r, 7)
+    tables = [cache.get_block_ids(r) for r in range(n_rollouts)]
+    ctx = build_decode_context(cache, list(range(n_rollouts)), lens, tables)
+    out = backend.forward(q1.cuda(), k1.cuda(), v1.cuda(), 0, ctx)
+    for r in range(n_rollouts):
+        k_all = torch.cat([full_k[r], k1[r : r + 1]], 1)
+        v_all = torch.cat([full_v[r], v1[r : r + 1]], 1)
+        q_all = torch.cat([torch.zeros_like(full_q[r]), q1[r : r + 1]], 1)
+        want = po.dense_prefill(q_all, k_all, v_all, backend.scale)[:, -1]
+        assert_close(out[r], want, 2e-2, f"decode rollout {r}")

@@ -147,9 +147,10 @@ def test_allocate_errors():
         PagedKVCache(num_blocks=0)
 
 
-def test_radix_stub_raises():
-    with pytest.raises(NotImplementedError):
-        RadixKVCache(num_blocks=4)
+def test_radix_cache_constructs():
+    """The reference's RadixKVCache is a stub whose constructor raises (cache/radix.py:42-43); here it is built
+    (tests/test_radix_cache.py covers it)."""
+    assert RadixKVCache(num_blocks=4).num_free_blocks() == 4
 
 
 # ---- context builders ---------------------------------------------------------
