@@ -1,11 +1,12 @@
-"""Attention / KV-cache call surface (reference: rollouts/rollouts/inference/__init__.py).
+"""Inference package on the paged attention path (reference: rollouts/rollouts/inference/__init__.py).
 
-Exports the subset of the reference package's names that belong to the paged
-attention path; the engine, scheduler and sampling names are not part of it.
+Exports the reference package's names: the attention / KV-cache call surface and the engine, scheduler and
+sampling that drive it.
 """
 
-from .attention import Attention, AttentionBackend, CacheConfig, FlexAttentionBackend, HipPagedAttentionBackend
-from .cache import PagedKVCache
+from .attention import (Attention, AttentionBackend, CacheConfig, FlexAttentionBackend, HipPagedAttentionBackend,
+                        create_causal_block_mask)
+from .cache import PagedKVCache, RadixKVCache
 from .context import (
     allocate_and_build_context,
     build_chunked_prefill_context,
@@ -13,7 +14,12 @@ from .context import (
     build_prefill_context,
     extend_and_build_context,
 )
-from .types import InferenceContext
+from .engine import InferenceEngine
+from .model import ModelConfig, PagedLlama
+from .sampling import sample_with_logprobs
+from .scheduler import schedule
+from .types import (EngineConfig, InferenceContext, SamplingParams, SchedulerConfig, SchedulerOutput, Sequence,
+                    SequenceStatus, TrainingSample)
 
 __all__ = [
     "InferenceContext",
@@ -28,4 +34,18 @@ __all__ = [
     "FlexAttentionBackend",
     "Attention",
     "PagedKVCache",
+    "RadixKVCache",
+    "EngineConfig",
+    "SamplingParams",
+    "SchedulerConfig",
+    "SchedulerOutput",
+    "TrainingSample",
+    "Sequence",
+    "SequenceStatus",
+    "sample_with_logprobs",
+    "schedule",
+    "create_causal_block_mask",
+    "InferenceEngine",
+    "ModelConfig",
+    "PagedLlama",
 ]

@@ -1,7 +1,7 @@
 """Host-side block allocators (reference: rollouts/rollouts/inference/cache/__init__.py)."""
 
-from .paged import Block, PagedKVCache, compute_block_hash
+from .paged import Block, CountingPagedKVCache, PagedKVCache, compute_block_hash
 from .protocol import KVCacheManager
 from .radix import RadixKVCache
 
-__all__ = ["PagedKVCache", "RadixKVCache", "Block", "KVCacheManager", "compute_block_hash"]
+__all__ = ["PagedKVCache", "CountingPagedKVCache", "RadixKVCache", "Block", "KVCacheManager", "compute_block_hash"]

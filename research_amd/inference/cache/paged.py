@@ -176,3 +176,39 @@ class PagedKVCache:
     # names the reference uses for the two internals (paged.py:217, :226)
     _allocate_block = _take
     _deallocate_block = _release
+
+
+class CountingPagedKVCache(PagedKVCache):
+    """``PagedKVCache`` that grows by token count.
+
+    The reference's ``append_token`` hands out a block only when the last block was filled completely by
+    ``allocate`` (paged.py:194-201), so a sequence whose prompt is not a whole number of blocks never grows.
+    An engine that decodes past the first block boundary needs growth exactly when a token starts a new block;
+    this subclass counts tokens and does that, and leaves allocation, prefix reuse and release as they are.
+    """
+
+    def __init__(self, num_blocks: int, block_size: int = 16) -> None:
+        super().__init__(num_blocks, block_size)
+        self.seq_num_tokens: Dict[int, int] = {}
+
+    def allocate(self, seq_id: int, token_ids: List[int]) -> Tuple[int, ...]:
+        blocks = super().allocate(seq_id, token_ids)
+        self.seq_num_tokens[seq_id] = len(token_ids)
+        return blocks
+
+    def deallocate(self, seq_id: int) -> None:
+        super().deallocate(seq_id)
+        self.seq_num_tokens.pop(seq_id, None)
+
+    def append_token(self, seq_id: int, token_id: int) -> Optional[int]:
+        assert seq_id in self.seq_to_blocks
+        n = self.seq_num_tokens[seq_id]
+        fresh = None
+        if n % self.block_size == 0:
+            if not self.free_block_ids:
+                raise RuntimeError("No free blocks for token append")
+            fresh = self.free_block_ids[0]
+            self._take(fresh)
+            self.seq_to_blocks[seq_id].append(fresh)
+        self.seq_num_tokens[seq_id] = n + 1
+        return fresh

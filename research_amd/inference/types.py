@@ -1,17 +1,19 @@
-"""Per-step descriptor handed to every attention layer.
+"""Dataclasses of the inference package (reference: rollouts/rollouts/inference/types.py).
 
-Mirrors the field names, order and defaults of the reference's
-``InferenceContext`` (rollouts/rollouts/inference/types.py:72-107) so that
-code which builds a context for the reference backend builds one for this
-backend unchanged.  Only the type that the attention / KV-cache path consumes
-is restated here; the engine, sampling and scheduler dataclasses of the same
-reference file are not on that path.
+``InferenceContext`` (types.py:72-107) is the per-step descriptor handed to
+every attention layer; its field names, order and defaults are the
+reference's, so code which builds a context for the reference backend builds
+one for this backend unchanged.  The engine-side types (types.py:14-69,
+:110-171) keep their names, fields and defaults as well; ``EngineConfig``
+gains optional fields for what the reference's engine does not have yet: a KV
+pool size and an end-of-sequence token for engines built without a tokenizer.
 """
 
 from __future__ import annotations
 
 from dataclasses import dataclass
-from typing import Optional, Tuple
+from enum import Enum, auto
+from typing import FrozenSet, List, Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -42,3 +44,116 @@ class InferenceContext:
     max_seq_len: int = 0
     block_mask: Optional[object] = None
     prefix_lens: Optional[Tuple[int, ...]] = None
+
+
+# --------------------------------------------------------------------------- engine configuration (types.py:14-49)
+
+
+@dataclass(frozen=True)
+class EngineConfig:
+    """Engine configuration (types.py:14-24).  ``model_path`` names a local directory with ``config.json`` and
+    safetensors weights, or is ignored when the engine is handed a model object.  Added, optional:
+    ``num_kv_blocks`` (pool size; default: enough for ``max_batch_size`` sequences of ``max_model_len`` tokens,
+    capped at 65 536 blocks), ``eos_token_id`` (used when there is no tokenizer)."""
+
+    model_path: str
+    cache_type: str = "none"  # "paged" | "radix" | "none"
+    block_size: int = 16
+    max_batch_size: int = 256
+    max_model_len: int = 8192
+    gpu_memory_utilization: float = 0.9
+    tensor_parallel_size: int = 1
+    num_kv_blocks: Optional[int] = None
+    eos_token_id: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class SamplingParams:
+    """Sampling configuration (types.py:27-33)."""
+
+    temperature: float = 1.0
+    max_tokens: int = 256
+    stop_token_ids: FrozenSet[int] = frozenset()
+
+
+@dataclass(frozen=True)
+class SchedulerConfig:
+    """Scheduler limits (types.py:36-42)."""
+
+    max_batch_size: int
+    max_tokens_per_batch: int
+    block_size: int
+
+
+# --------------------------------------------------------------------------- outputs (types.py:50-69)
+
+
+@dataclass(frozen=True)
+class TrainingSample:
+    """One finished sequence for RL training (types.py:50-60)."""
+
+    prompt_tokens: Tuple[int, ...]
+    completion_tokens: Tuple[int, ...]
+    logprobs: Tuple[float, ...]
+    ref_logprobs: Optional[Tuple[float, ...]]
+    weight_version: int
+    finish_reason: str  # "stop" | "length"
+
+
+@dataclass(frozen=True)
+class SchedulerOutput:
+    """Sequence ids to prefill, decode and preempt in one step (types.py:63-69)."""
+
+    prefill_seqs: Tuple[int, ...]
+    decode_seqs: Tuple[int, ...]
+    preempted_seqs: Tuple[int, ...]
+
+
+# --------------------------------------------------------------------------- per-sequence state (types.py:115-171)
+
+
+class SequenceStatus(Enum):
+    WAITING = auto()
+    RUNNING = auto()
+    FINISHED = auto()
+
+
+@dataclass
+class Sequence:
+    """Mutable state of one request while it generates (types.py:121-171)."""
+
+    seq_id: int
+    token_ids: List[int]
+    block_ids: List[int]
+    num_prompt_tokens: int
+    status: SequenceStatus
+    temperature: float
+    max_tokens: int
+    stop_token_ids: FrozenSet[int]
+    output_logprobs: List[float]
+
+    def append_token(self, token_id: int, logprob: float) -> None:
+        assert self.status == SequenceStatus.RUNNING
+        self.token_ids.append(token_id)
+        self.output_logprobs.append(logprob)
+
+    @property
+    def num_generated(self) -> int:
+        return len(self.token_ids) - self.num_prompt_tokens
+
+    @property
+    def is_finished(self) -> bool:
+        return self.status == SequenceStatus.FINISHED
+
+    def to_training_sample(self, weight_version: int) -> TrainingSample:
+        assert self.status == SequenceStatus.FINISHED
+        n = self.num_prompt_tokens
+        stopped = self.token_ids[-1] in self.stop_token_ids
+        return TrainingSample(
+            prompt_tokens=tuple(self.token_ids[:n]),
+            completion_tokens=tuple(self.token_ids[n:]),
+            logprobs=tuple(self.output_logprobs),
+            ref_logprobs=None,
+            weight_version=weight_version,
+            finish_reason="stop" if stopped else "length",
+        )
