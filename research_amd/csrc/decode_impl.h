@@ -249,13 +249,13 @@ __device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EP
 namespace pa_decode_detail {
 
 // One wave's pass over its blocks of one query row: picks the packed 16-bit
-// loop where it applies (bf16/fp16 pool, head_dim 64 or 128), else the generic
+// loop where it applies (bf16/fp16 pool, head_dim 64, 128 or 256), else the generic
 // fp32 loop.  Returns the row-group state in the generic form merge_rows takes.
 template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
     using S = RowShape<KV, D>;
-    // packed loop: 16-bit pools with head_dim 64/128, fp8 pools (16-bit queries) with head_dim 64/128/256
+    // packed loop: 16-bit pools and fp8 pools (16-bit queries) with head_dim 64/128/256
     static constexpr bool kPacked =
-        (sizeof(KV) == 2 && std::is_same<KV, QT>::value && (D == 64 || D == 128)) ||
+        (sizeof(KV) == 2 && std::is_same<KV, QT>::value && (D == 64 || D == 128 || D == 256)) ||
         (sizeof(KV) == 1 && sizeof(QT) == 2 && (D == 64 || D == 128 || D == 256));
 
     static __device__ __forceinline__ RowState<NREP, S::EPL> run(const PoolArgs &p, const QT *qrow,

@@ -1,5 +1,5 @@
 // Packed inner loop of single-query-row paged attention for gfx950: bf16 / fp16
-// pools (head_dim 64, 128) and fp8-e4m3 pools with bf16 / fp16 queries
+// pools (head_dim 64, 128, 256) and fp8-e4m3 pools with bf16 / fp16 queries
 // (head_dim 64, 128, 256).  An fp8 pool is widened two elements at a time to
 // the query type (v_cvt_scalef32_pk_*_fp8, exact) and then runs the same
 // 16-bit arithmetic; its per-(block, head) scales multiply the logit and p.
@@ -94,7 +94,7 @@ template <int CTRL> __device__ __forceinline__ uint32_t dpp_mov_u(uint32_t x) {
 // After reduce(): a lane at quad position c = lane & 3 owns VPL totals, those
 // of heads head_base(c) .. head_base(c)+VPL-1.
 template <int NREP, int LPR> struct HeadScatter {
-    static_assert(LPR == 4 || LPR == 8 || LPR == 16, "rows of 4, 8 or 16 lanes");
+    static_assert(LPR == 4 || LPR == 8 || LPR == 16 || LPR == 32, "rows of 4, 8, 16 or 32 lanes");
     static constexpr int SC = NREP >= 4 ? 2 : (NREP == 2 ? 1 : 0);  // scatter steps (xor 1, xor 2)
     static constexpr int VPL = NREP >> SC;                            // values a lane keeps
 
@@ -128,9 +128,14 @@ template <int NREP, int LPR> struct HeadScatter {
         // remaining levels keep the quad position: every quad of the row gets the row total
 #pragma unroll
         for (int i = 0; i < VPL; ++i) {
-            if (LPR == 16) {
+            if (LPR >= 16) {
                 out[i] += dpp_mov<0x124>(0.f, out[i]);  // row_ror:4
                 out[i] += dpp_mov<0x128>(0.f, out[i]);  // row_ror:8
+                if (LPR == 32) {  // the row spans two groups of 16 lanes: add the partner group's total
+                    const uint32_t u = __builtin_bit_cast(uint32_t, out[i]);
+                    const auto sw = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+                    out[i] = __builtin_bit_cast(float, (uint32_t)sw[0]) + __builtin_bit_cast(float, (uint32_t)sw[1]);
+                }
             } else if (LPR == 8) {
                 // partner quad inside the row of 8: from 4 lanes below for banks 1,3, from 4 lanes above for banks 0,2
                 float other = dpp_mov<0x114, 0xa>(0.f, out[i]);   // row_shr:4

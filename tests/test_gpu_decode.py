@@ -108,6 +108,8 @@ def test_pool_permutation_and_constant_values():
     (8, 4, 32, torch.bfloat16),    # the reference script's shape (test_kv_cache.py:131-136)
     (6, 6, 128, torch.float16),    # MHA, 6 kv heads: two per wave load
     (3, 1, 256, torch.bfloat16),   # MQA, group of 3, D=256
+    (16, 8, 256, torch.bfloat16),  # Gemma-2-9B-like: D=256 rows span 32 lanes, two kv heads per wave load
+    (8, 2, 256, torch.float16),    # D=256, group of 4
     (32, 2, 128, torch.float32),   # group of 16: two passes of 8
     (5, 5, 64, torch.float32),     # odd head count: one kv head per wave load
 ])
