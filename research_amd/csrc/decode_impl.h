@@ -281,8 +281,12 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
             st.init();
             const int lane_voff =
                 role.tok_local * (p.hkv * D * (int)sizeof(KV)) + kvh * (D * (int)sizeof(KV)) + role.lir * 16;
-            attend_blocks_pk<KV, QT, D, NREP, U>(st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step, lane,
-                                                 lane_voff, kvh, role.tok_local == 0);
+            if (p.tpw * U > p.bs)  // uniform: few kv heads per wave load and short blocks
+                attend_blocks_pk<KV, QT, D, NREP, U, true>(st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step,
+                                                           lane, lane_voff, kvh, role.tok_local == 0);
+            else
+                attend_blocks_pk<KV, QT, D, NREP, U, false>(st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step,
+                                                            lane, lane_voff, kvh, role.tok_local == 0);
             StaticFor<NREP>::run([&](auto h) {
                 out.m[h.value] = HS::template bcast<h.value>(st.m);
                 out.l[h.value] = HS::template bcast<h.value>(st.l);

@@ -189,7 +189,10 @@ template <> struct StaticFor<0> {
 // Attend keys [k_lo, L) of blocks blk_begin, blk_begin+blk_step, ... < blk_end.
 // qpk[r][i]: packed pairs of this lane's query elements of head r (raw bits of the query type AT).
 // lane_kvh: the kv head this lane's row belongs to (selects the fp8 scales).
-template <typename KV, typename AT, int D, int NREP, int U>
+// SHORT: a token step of the wave (tpw tokens) times U exceeds the block, so whole steps can lie past the
+// block's end; they are skipped under uniform branches.  The straight-line form (SHORT = false) keeps the
+// loop free of branches for the layouts where every step of a full block is live.
+template <typename KV, typename AT, int D, int NREP, int U, bool SHORT>
 __device__ __forceinline__ void attend_blocks_pk(
     PkState<NREP, HeadScatter<NREP, D * (int)sizeof(KV) / 16>::VPL, 2 * PoolWords<KV, AT>::NW> &st,
     const uint32_t (&qpk)[NREP][PoolWords<KV, AT>::NW], const PoolArgs &p, const int32_t *bt_row, int k_lo, int L,
@@ -236,9 +239,15 @@ __device__ __forceinline__ void attend_blocks_pk(
 
             // ---- logits: one (token, head) per lane -----------------------
             float sv[U][VPL];
-            const bool partial = ntok - t0 < p.tpw * U || t0 < tlo;  // uniform
+            const int rem = ntok - t0;                         // tokens of the block from t0 on (uniform)
+            const bool partial = rem < p.tpw * U || t0 < tlo;  // uniform
 #pragma unroll
             for (int u = 0; u < U; ++u) {
+                if (SHORT && u * p.tpw >= rem) {  // uniform: the whole token step lies past the block
+#pragma unroll
+                    for (int j = 0; j < VPL; ++j) sv[u][j] = -INFINITY;
+                    continue;
+                }
                 uint32_t kw[NW];
                 PW::unpack(kraw[u], kw);
                 float s[NREP];
@@ -286,6 +295,7 @@ __device__ __forceinline__ void attend_blocks_pk(
             // ---- p.v, two tokens per step ----------------------------------
 #pragma unroll
             for (int u = 0; u < U; u += 2) {
+                if (SHORT && u * p.tpw >= rem) continue;  // uniform: both token steps lie past the block
                 uint32_t ppk[VPL];
 #pragma unroll
                 for (int j = 0; j < VPL; ++j) {
