@@ -257,6 +257,19 @@ int pa_rope_kv_append_e4m3(const void *q, void *q_out, const void *k_src, const 
                            const int32_t *touched_blocks, int n_touched, int64_t num_blocks, int block_size,
                            int num_q_heads, int num_kv_heads, int head_dim, int src_dtype, void *stream);
 
+/*
+ * Dequantise listed blocks of an fp8-e4m3 pool into a compact 16-bit pool (no counterpart in the reference):
+ * block j of dst = block block_ids[j] of the pool, every value float(byte) * scale[block][kv_head] rounded to
+ * dst_dtype (BF16/F16).  Used to run prefill over an fp8 pool on the matrix cores: dequantise the blocks the
+ * step's block tables name (each once, however many sequences share it), renumber the tables to positions in
+ * block_ids, and call pa_prefill_paged on dst.  Ids outside [0, num_blocks) give zero blocks.
+ *   cache : [num_blocks*block_size][num_kv_heads][head_dim] bytes;  scale: float[num_blocks][num_kv_heads]
+ *   dst   : [n_ids*block_size][num_kv_heads][head_dim] of dst_dtype;  head_dim % 16 == 0
+ */
+int pa_dequantize_blocks_e4m3(const void *cache, const float *scale, const int32_t *block_ids, int n_ids,
+                              void *dst, int64_t num_blocks, int block_size, int num_kv_heads, int head_dim,
+                              int dst_dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

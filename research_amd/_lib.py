@@ -59,6 +59,10 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64,
          c_int, c_int, c_int, c_int, c_void_p],
     ),
+    "pa_dequantize_blocks_e4m3": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p],
+    ),
     "pa_rope_kv_append": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,

@@ -146,6 +146,37 @@ __global__ __launch_bounds__(kQThreads) void append_e4m3_kernel(const T *__restr
     if (threadIdx.x == 0) scale[blk * hkv + h] = s_new;
 }
 
+// Dequantise listed blocks of an fp8 pool into a compact 16-bit pool: block j of dst = block ids[j] of src times
+// its scales.  One workgroup per (listed block, kv head) tile; a lane widens 16 bytes to 16 values (two 16-byte
+// stores).  Ids outside the pool give zero blocks.
+template <typename T>
+__global__ __launch_bounds__(kQThreads) void dequantize_blocks_kernel(const uint8_t *__restrict__ src,
+                                                                       const float *__restrict__ scale,
+                                                                       const int32_t *__restrict__ ids,
+                                                                       T *__restrict__ dst, int64_t num_blocks,
+                                                                       int block_size, int hkv, int d) {
+    const int j = blockIdx.x, h = blockIdx.y;
+    const int64_t bid = ids[j];
+    const bool ok = bid >= 0 && bid < num_blocks;
+    const float sc = ok ? scale[bid * hkv + h] : 0.f;
+    const int vecs_per_row = d / 16;
+    const int64_t tok_stride = (int64_t)hkv * d;
+    for (int i = threadIdx.x; i < block_size * vecs_per_row; i += kQThreads) {
+        const int t = i / vecs_per_row, e = (i - t * vecs_per_row) * 16;
+        float f[16];
+        if (ok) {
+            const uint4 raw = *reinterpret_cast<const uint4 *>(src + ((bid * block_size + t) * hkv + h) * (int64_t)d + e);
+            pa_vec16<pa_fp8>::unpack(raw, f);
+        } else {
+#pragma unroll
+            for (int k = 0; k < 16; ++k) f[k] = 0.f;
+        }
+        T *out = dst + (((int64_t)j * block_size + t) * tok_stride + (int64_t)h * d + e);
+#pragma unroll
+        for (int k = 0; k < 16; ++k) pa_scalar<T>::store(out + k, f[k] * sc);
+    }
+}
+
 // Appends one of K / V; `rt` non-NULL rotates the rows on the way (K of a fused rotary append).
 template <bool ROPE>
 void launch_append(const void *src, uint8_t *dst, float *sc, const int64_t *slots, int64_t n_tokens,
@@ -248,5 +279,29 @@ extern "C" int pa_quantize_kv_e4m3(const void *src, void *dst, float *scale, int
         quantize_e4m3_kernel<pa_f16><<<grid, block, 0, s>>>((const pa_f16 *)src, (uint8_t *)dst, scale, block_size,
                                                             num_kv_heads, head_dim);
     PA_CHECK_LAUNCH("pa_quantize_kv_e4m3");
+    return PA_OK;
+}
+
+extern "C" int pa_dequantize_blocks_e4m3(const void *cache, const float *scale, const int32_t *block_ids, int n_ids,
+                                         void *dst, int64_t num_blocks, int block_size, int num_kv_heads, int head_dim,
+                                         int dst_dtype, void *stream) {
+    pa_clear_error();
+    PA_REQUIRE(n_ids >= 0 && num_blocks >= 0, "n_ids=%d / num_blocks=%lld is negative", n_ids, (long long)num_blocks);
+    PA_REQUIRE(block_size > 0 && num_kv_heads > 0 && num_kv_heads <= 65535 && head_dim > 0,
+               "block_size / num_kv_heads / head_dim out of range");
+    PA_REQUIRE(head_dim % 16 == 0, "head_dim=%d is not a multiple of 16", head_dim);
+    PA_REQUIRE(dst_dtype == PA_BF16 || dst_dtype == PA_F16, "dst_dtype=%d is not BF16 or F16", dst_dtype);
+    if (n_ids == 0) return PA_OK;
+    PA_REQUIRE(cache && scale && block_ids && dst, "NULL pointer argument");
+    PA_REQUIRE(pa_aligned16(cache) && pa_aligned16(dst), "cache and dst must be 16-byte aligned");
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid((unsigned)n_ids, (unsigned)num_kv_heads), block(kQThreads);
+    if (dst_dtype == PA_BF16)
+        dequantize_blocks_kernel<pa_bf16><<<grid, block, 0, s>>>((const uint8_t *)cache, scale, block_ids, (pa_bf16 *)dst,
+                                                                 num_blocks, block_size, num_kv_heads, head_dim);
+    else
+        dequantize_blocks_kernel<pa_f16><<<grid, block, 0, s>>>((const uint8_t *)cache, scale, block_ids, (pa_f16 *)dst,
+                                                                num_blocks, block_size, num_kv_heads, head_dim);
+    PA_CHECK_LAUNCH("pa_dequantize_blocks_e4m3");
     return PA_OK;
 }

@@ -56,12 +56,13 @@ class _StepTensors:
     """Device copies of one context's integer fields, built once per step."""
 
     __slots__ = ("ctx", "slots", "touched", "tables", "bt_stride", "seq_lens", "extra_zero", "ctx_lens", "q_lens",
-                 "q_starts", "max_q_len", "row_first_key")
+                 "q_starts", "max_q_len", "row_first_key", "fp8_blocks", "fp8_tables")
 
     def __init__(self, ctx: InferenceContext) -> None:
         self.ctx = ctx  # keeps id(ctx) alive while the entry is cached
         self.slots = self.touched = self.tables = self.seq_lens = self.extra_zero = None
         self.ctx_lens = self.q_lens = self.q_starts = self.row_first_key = None
+        self.fp8_blocks = self.fp8_tables = None  # distinct blocks of the tables and the tables renumbered to them
         self.bt_stride = self.max_q_len = 0
 
 
@@ -427,8 +428,6 @@ class HipPagedAttentionBackend:
         window = self._mask_window(ctx.block_mask, self._window)
         if ctx.block_tables is None or ctx.seq_lens is None:
             raise ValueError("Chunked prefill requires block_tables and seq_lens in context")
-        if self._fp8:
-            raise NotImplementedError("chunked prefill over an fp8 pool")
         cfg = self.config
         batch, seq_len, num_heads, head_dim = q.shape
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
@@ -451,7 +450,21 @@ class HipPagedAttentionBackend:
             first = self._mask_first_keys(ctx.block_mask, step, batch, seq_len, self._lens(ctx.prefix_lens, batch))
         out.zero_()  # rows past a sequence's chunk length are padding and stay zero
         kc, vc = self._layer(layer_idx)
-        ops.prefill_paged(q.contiguous().view(batch * seq_len, num_heads, head_dim), kc, vc, step.tables,
+        tables = step.tables
+        if self._fp8:
+            # The matrix-core kernel reads 16-bit pools: dequantise the blocks the tables name into a compact
+            # pool (each block once, however many sequences share it) and renumber the tables to match.
+            if q.dtype not in (torch.bfloat16, torch.float16):
+                raise RuntimeError("prefill over an fp8 pool takes bf16 or fp16 queries")
+            if step.fp8_blocks is None:
+                uniq, inverse = torch.unique(step.tables.reshape(-1), return_inverse=True)
+                step.fp8_blocks = uniq.to(torch.int32)
+                step.fp8_tables = torch.where(step.tables.reshape(-1) < 0, -1, inverse).to(torch.int32).view(
+                    step.tables.shape).contiguous()
+            kc = ops.dequantize_blocks_e4m3(kc, self.k_scale[layer_idx], step.fp8_blocks, cfg.block_size, q.dtype)
+            vc = ops.dequantize_blocks_e4m3(vc, self.v_scale[layer_idx], step.fp8_blocks, cfg.block_size, q.dtype)
+            tables = step.fp8_tables
+        ops.prefill_paged(q.contiguous().view(batch * seq_len, num_heads, head_dim), kc, vc, tables,
                           step.ctx_lens, step.q_lens, step.q_starts, step.max_q_len, cfg.block_size, self.scale,
                           out=out.view(batch * seq_len, num_heads, head_dim), window=window, row_first_key=first)
         return out

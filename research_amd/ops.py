@@ -194,3 +194,16 @@ def rope_kv_append_e4m3(q: Tensor, k_src: Tensor, v_src: Tensor, cos: Tensor, si
          _ptr(k_scale), _ptr(v_scale), _ptr(cos), _ptr(sin), _ptr(positions), cos.shape[0], _ptr(slots), n,
          _ptr(touched), touched.numel(), num_blocks, block_size, hq, hkv, d, PA_DTYPE[q.dtype], _stream(q))
     return q_out
+
+
+def dequantize_blocks_e4m3(cache: Tensor, scale: Tensor, block_ids: Tensor, block_size: int,
+                           dtype: torch.dtype = torch.bfloat16) -> Tensor:
+    """Compact 16-bit pool ``[len(block_ids) * block_size, Hkv, D]`` holding the listed blocks of an fp8-e4m3
+    pool dequantised (``pa_dequantize_blocks_e4m3``); ``block_ids`` int32 on the device."""
+    total_slots, hkv, d = cache.shape
+    if block_ids.dtype != torch.int32:
+        raise ValueError("block_ids must be int32")
+    dst = torch.empty((block_ids.numel() * block_size, hkv, d), dtype=dtype, device=cache.device)
+    _run("pa_dequantize_blocks_e4m3", _ptr(cache), _ptr(scale), _ptr(block_ids), block_ids.numel(), _ptr(dst),
+         total_slots // block_size, block_size, hkv, d, PA_DTYPE[dtype], _stream(cache))
+    return dst

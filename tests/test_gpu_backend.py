@@ -385,3 +385,51 @@ def test_prefix_reuse_through_the_radix_cache():
         q_all = torch.cat([torch.zeros_like(full_q[r]), q1[r : r + 1]], 1)
         want = po.dense_prefill(q_all, k_all, v_all, backend.scale)[:, -1]
         assert_close(out[r], want, 2e-2, f"decode rollout {r}")
+
+
+def test_fp8_blocks_dequantise_bit_exact_and_chunked_prefill_over_an_fp8_pool():
+    """pa_dequantize_blocks_e4m3 against the checker's dequantisation (bytes x scale, rounded once to bf16), and
+    chunked prefill over shared prefix blocks of an fp8 pool = dequantise, then attend."""
+    from research_amd import ops
+    from research_amd.inference.context import build_chunked_prefill_context
+
+    announce("backend fp8 chunked prefill")
+    g = torch.Generator().manual_seed(81)
+    hq, hkv, d, bs, nb = 8, 2, 128, 16, 24
+    config = CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=nb, block_size=bs, device="cuda",
+                         kv_format="fp8_e4m3")
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(hq)
+    pool_k = torch.randn(nb * bs, hkv, d, generator=g).to(torch.bfloat16)
+    pool_v = (torch.randn(nb * bs, hkv, d, generator=g) * 3).to(torch.bfloat16)
+    backend.quantize_from(pool_k.cuda(), pool_v.cuda(), 0)
+    bits = backend.k_cache[0].cpu().view(torch.uint8)
+    scale = backend.k_scale[0].cpu()
+    ids = torch.tensor([5, 0, 23, -1, 7, 99, 5], dtype=torch.int32)
+    got = ops.dequantize_blocks_e4m3(backend.k_cache[0], backend.k_scale[0], ids.cuda(), bs).cpu()
+    full = po.dequantize_kv_e4m3(bits, scale, bs).to(torch.bfloat16).view(nb, bs, hkv, d)
+    for j, b in enumerate(ids.tolist()):
+        want = full[b] if 0 <= b < nb else torch.zeros(bs, hkv, d, dtype=torch.bfloat16)
+        assert torch.equal(got.view(-1, bs, hkv, d)[j].view(torch.int16), want.view(torch.int16)), f"block {b}"
+    # three sequences sharing 4 prefix blocks, ragged chunks appended through the backend
+    shared = [3, 9, 1, 20]
+    tables = [shared + [4, 5], shared + [6, 7], shared + [8]]
+    prefix, chunk = [64, 64, 64], [20, 32, 7]
+    cmax = max(chunk)
+    q = torch.randn(3, cmax, hq, d, generator=g).to(torch.bfloat16)
+    k = torch.randn(3, cmax, hkv, d, generator=g).to(torch.bfloat16)
+    v = torch.randn(3, cmax, hkv, d, generator=g).to(torch.bfloat16)
+    ctx = build_chunked_prefill_context(PagedKVCache(nb, bs), [0, 1, 2], prefix, chunk, tables)
+    slots = np.full((3, cmax), -1, dtype=np.int64)  # padded rows carry slot -1
+    at = 0
+    for b, c in enumerate(chunk):
+        slots[b, :c] = ctx.slot_mapping[at : at + c]
+        at += c
+    ctx = InferenceContext(is_prefill=True, slot_mapping=slots.reshape(-1), block_tables=ctx.block_tables,
+                           seq_lens=ctx.seq_lens, max_seq_len=ctx.max_seq_len, prefix_lens=ctx.prefix_lens)
+    out = backend.forward(q.cuda(), k.cuda(), v.cuda(), 0, ctx)
+    kd = po.dequantize_kv_e4m3(backend.k_cache[0].cpu().view(torch.uint8), backend.k_scale[0].cpu(), bs)
+    vd = po.dequantize_kv_e4m3(backend.v_cache[0].cpu().view(torch.uint8), backend.v_scale[0].cpu(), bs)
+    want = po.paged_prefill_chunk(q, kd, vd, tables, prefix, chunk, bs, backend.scale)
+    for b, c in enumerate(chunk):
+        assert_close(out[b, :c], want[b, :c], 6e-2, f"sequence {b}")

@@ -131,3 +131,23 @@ def test_bf16_generation_and_weight_update():
     with torch.no_grad():
         want = mo.logprobs_of(new_weights, CFG, list(s.prompt_tokens + s.completion_tokens), len(s.prompt_tokens))
     assert s.logprobs == pytest.approx(want, abs=0.08)
+
+
+def test_engine_on_an_fp8_pool():
+    """The same model with an fp8-e4m3 KV pool: rotary append into fp8 blocks, chunked prefill over dequantised
+    blocks, fp8 decode.  Teacher-forced log probabilities stay close to the full-precision checker."""
+    announce("engine fp8 pool")
+    backend = HipPagedAttentionBackend(CacheConfig(
+        num_layers=CFG.num_layers, num_kv_heads=CFG.num_kv_heads, head_dim=CFG.head_dim, num_blocks=64,
+        block_size=16, device="cuda", dtype=torch.bfloat16, kv_format="fp8_e4m3"))
+    torch.manual_seed(1)
+    model = PagedLlama(CFG, backend).to(torch.bfloat16).cuda().eval()
+    engine = InferenceEngine(EngineConfig(model_path="", cache_type="radix", max_batch_size=8, max_model_len=512),
+                             model=model)
+    weights = {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
+    samples = engine.generate(_prompts(), SamplingParams(temperature=0.0, max_tokens=12))
+    assert len(samples) == 6
+    for s in samples:
+        with torch.no_grad():
+            want = mo.logprobs_of(weights, CFG, list(s.prompt_tokens + s.completion_tokens), len(s.prompt_tokens))
+        assert s.logprobs == pytest.approx(want, abs=0.25)
