@@ -160,3 +160,30 @@ def test_forward_rope_through_the_backend():
     k1_r = po.rope_literal(k1[0], table_cos[n : n + 1], table_sin[n : n + 1])[None]
     out_p = plain.forward(q1_r.cuda(), k1_r.cuda(), v1.cuda(), 1, ctx_p)
     assert torch.equal(out_f, out_p) and torch.equal(fused.k_cache, plain.k_cache)
+
+
+def test_rope_append_at_full_size():
+    """The append of workload c3 (8 192 tokens, 32 q heads, 8 kv heads, D=128, positions 2048..2303 from a table)
+    and a decode-step append of workload c4's shape (256 tokens at positions up to 32 767): every output bit
+    against the elementwise statement on the CPU."""
+    announce("rope append, c3 / c4 sizes")
+    hq, hkv, d, bs = 32, 8, 128, 16
+    for n, max_pos, nb, seed in ((8192, 2304, 640, 1), (256, 32768, 4096, 2)):
+        g = torch.Generator().manual_seed(seed)
+        q = torch.randn(n, hq, d, generator=g).to(torch.bfloat16)
+        k = torch.randn(n, hkv, d, generator=g).to(torch.bfloat16)
+        v = torch.randn(n, hkv, d, generator=g).to(torch.bfloat16)
+        pos = torch.randint(max(0, max_pos - 256), max_pos, (n,), generator=g)
+        cos_t, sin_t = (t[0] for t in po.rope_tables(torch.arange(max_pos)[None], d, 10000.0, torch.bfloat16))
+        slots = torch.randperm(nb * bs, generator=g)[:n]
+        kc = torch.zeros(nb * bs, hkv, d, dtype=torch.bfloat16, device=DEV)
+        vc = torch.zeros_like(kc)
+        q_rot = ops.rope_kv_append(q.to(DEV), k.to(DEV), v.to(DEV), cos_t.to(DEV), sin_t.to(DEV), kc, vc, slots.to(DEV),
+                                   positions=pos.to(torch.int32).to(DEV), q_out=torch.empty(n, hq, d, dtype=torch.bfloat16, device=DEV))
+        want_q = po.rope_literal(q, cos_t[pos], sin_t[pos])
+        want_k = po.rope_literal(k, cos_t[pos], sin_t[pos])
+        assert torch.equal(_bits(q_rot.cpu()), _bits(want_q))
+        assert torch.equal(_bits(kc.cpu()[slots]), _bits(want_k)) and torch.equal(_bits(vc.cpu()[slots]), _bits(v))
+        untouched = torch.ones(nb * bs, dtype=torch.bool)
+        untouched[slots] = False
+        assert not kc.cpu()[untouched].any() and not vc.cpu()[untouched].any()
