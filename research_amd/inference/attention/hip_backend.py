@@ -216,20 +216,22 @@ class HipPagedAttentionBackend:
             slots = self._device_slots(ctx.slot_mapping, n, step)
         dense = ctx.is_prefill and getattr(ctx, "prefix_lens", None) is None  # attends the step's own K/V
         kc, vc = self._layer(layer_idx)
-        if self._fp8 and slots is not None:
-            if dense:
-                raise NotImplementedError("dense prefill attends the step's own K; use an fp8 pool with chunked prefill")
-            if step.touched is None:
-                step.touched = ops.touched_blocks(slots, cfg.block_size, cfg.num_blocks)
+        if self._fp8 and slots is not None and step.touched is None:
+            step.touched = ops.touched_blocks(slots, cfg.block_size, cfg.num_blocks)
+        if self._fp8 and slots is not None and not dense:
             ops.rope_kv_append_e4m3(q3, k3, v3, cos2, sin2, kc, vc, self.k_scale[layer_idx], self.v_scale[layer_idx],
                                     slots, cfg.block_size, positions=pos, q_out=q_rot, touched=step.touched)
             k_rot = None
         else:
-            if slots is not None and k3.dtype != self.k_cache.dtype:
+            to_pool = slots is not None and not self._fp8  # rows of the pool's own type go straight to their slots
+            if to_pool and k3.dtype != self.k_cache.dtype:
                 raise RuntimeError("Index put requires the source and destination dtypes match")
-            k_rot = torch.empty_like(k3) if dense or slots is None else None
-            ops.rope_kv_append(q3, k3, v3, cos2, sin2, kc if slots is not None else None,
-                               vc if slots is not None else None, slots, positions=pos, q_out=q_rot, k_out=k_rot)
+            k_rot = torch.empty_like(k3) if dense or not to_pool else None
+            ops.rope_kv_append(q3, k3, v3, cos2, sin2, kc if to_pool else None, vc if to_pool else None,
+                               slots if to_pool else None, positions=pos, q_out=q_rot, k_out=k_rot)
+            if self._fp8 and slots is not None:  # dense prefill keeps the rotated K: append it from there
+                ops.kv_append_e4m3(kc, vc, self.k_scale[layer_idx], self.v_scale[layer_idx], k_rot, v3, slots,
+                                   cfg.block_size, step.touched)
         k_att = k_rot.view(batch, seq_len, cfg.num_kv_heads, head_dim) if k_rot is not None else k
         return self._attend(q_rot.view(q.shape), k_att, v, layer_idx, ctx)
 

@@ -251,3 +251,59 @@ def test_sliding_window_decode_other_types_and_garbage_before_the_window():
                      window=window)
     want = po.paged_decode(w.q, w.k_pool, w.v_pool, _lists(w), w.seq_lens, 16, w.scale, window=window)
     assert_close(got, want, 2e-2, "poisoned keys before the window")
+
+
+def test_decode_step_in_a_hip_graph():
+    """The append + decode launches of one step, captured once and replayed: the entry points allocate nothing,
+    clear nothing with memsets and read lengths, slots and tables from device memory, so a serving loop can
+    update those buffers in place and replay.  Every replay is checked against the checker, with eager work
+    and synchronisations between the replays."""
+    announce("decode in a HIP graph")
+    rng = np.random.default_rng(91)
+    hq, hkv, d, bs, nb, batch = 8, 2, 128, 16, 64, 3
+    lens = np.array([37, 5, 60], dtype=np.int32)
+    tables = np.full((batch, 8), -1, dtype=np.int32)
+    perm = rng.permutation(nb)
+    for b in range(batch):
+        tables[b, :6] = perm[b * 6 : b * 6 + 6]  # room for 96 tokens each
+    kp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+    vp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+    kc, vc = kp.to(DEV), vp.to(DEV)
+    q = torch.zeros(batch, hq, d, dtype=torch.bfloat16, device=DEV)
+    k_new = torch.zeros(batch, hkv, d, dtype=torch.bfloat16, device=DEV)
+    v_new = torch.zeros_like(k_new)
+    lens_dev = torch.from_numpy(lens).to(DEV)
+    slots_dev = torch.full((batch,), -1, dtype=torch.int64, device=DEV)  # the warm-up step appends nothing
+    tables_dev = torch.from_numpy(tables).to(DEV)
+    out = torch.empty_like(q)
+    ws = ops.decode_workspace(q, kc)
+
+    def step():
+        ops.kv_scatter(kc, vc, k_new, v_new, slots_dev)
+        ops.decode(q, kc, vc, tables_dev, lens_dev, bs, d ** -0.5, ws, out=out)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()  # warm-up outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        step()
+    k_ref, v_ref = kp.clone(), vp.clone()
+    for it in range(4):
+        lens += 1  # every sequence appends one token, then attends it
+        qh = torch.from_numpy(rng.standard_normal((batch, hq, d)).astype(np.float32)).to(torch.bfloat16)
+        kh = torch.from_numpy(rng.standard_normal((batch, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+        vh = torch.from_numpy(rng.standard_normal((batch, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+        slots = np.array([tables[b, (lens[b] - 1) // bs] * bs + (lens[b] - 1) % bs for b in range(batch)])
+        q.copy_(qh.to(DEV)); k_new.copy_(kh.to(DEV)); v_new.copy_(vh.to(DEV))
+        lens_dev.copy_(torch.from_numpy(lens).to(DEV)); slots_dev.copy_(torch.from_numpy(slots).to(DEV))
+        graph.replay()
+        torch.cuda.synchronize()
+        k_ref[slots] = kh
+        v_ref[slots] = vh
+        want = po.paged_decode(qh, k_ref, v_ref, [t[t >= 0].tolist() for t in tables], lens.tolist(), bs, d ** -0.5)
+        assert_close(out, want, 2e-2, f"replay {it}")
+        assert torch.equal(kc.cpu(), k_ref)
+        (torch.ones(1000, device=DEV) * 2).sum().item()  # eager work between replays

@@ -187,3 +187,30 @@ def test_rope_append_at_full_size():
         untouched = torch.ones(nb * bs, dtype=torch.bool)
         untouched[slots] = False
         assert not kc.cpu()[untouched].any() and not vc.cpu()[untouched].any()
+
+
+def test_forward_rope_dense_prefill_into_an_fp8_pool():
+    """Dense prefill attends the step's own rotated K/V (bf16) while the rows are appended to the fp8 pool."""
+    from research_amd.inference import PagedKVCache, allocate_and_build_context
+
+    announce("backend forward_rope, dense prefill, fp8 pool")
+    g = torch.Generator().manual_seed(62)
+    hq, hkv, d, bs = 8, 2, 64, 16
+    config = CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=8, block_size=bs, device="cuda",
+                         kv_format="fp8_e4m3")
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(hq)
+    n = 37
+    q, k, v = (torch.randn(1, n, h, d, generator=g).to(torch.bfloat16) for h in (hq, hkv, hkv))
+    cos, sin = (t[0] for t in po.rope_tables(torch.arange(n)[None], d, 10000.0, torch.bfloat16))
+    ctx, _ = allocate_and_build_context(PagedKVCache(8, bs), seq_id=0, token_ids=list(range(n)))
+    out = backend.forward_rope(q.cuda(), k.cuda(), v.cuda(), cos[None].cuda(), sin[None].cuda(), 0, ctx)
+    q_r, k_r = po.rope_literal(q[0], cos, sin)[None], po.rope_literal(k[0], cos, sin)[None]
+    assert_close(out, po.dense_prefill(q_r, k_r, v, backend.scale), 2e-2, "dense prefill")
+    bits_k = torch.zeros(8 * bs, hkv, d, dtype=torch.uint8)
+    bits_v = torch.zeros_like(bits_k)
+    sc_k, sc_v = torch.ones(8, hkv), torch.ones(8, hkv)
+    po.append_kv_e4m3(bits_k, sc_k, k_r[0], ctx.slot_mapping, bs)
+    po.append_kv_e4m3(bits_v, sc_v, v[0], ctx.slot_mapping, bs)
+    assert torch.equal(backend.k_cache[0].cpu().view(torch.uint8), bits_k) and torch.equal(backend.k_scale[0].cpu(), sc_k)
+    assert torch.equal(backend.v_cache[0].cpu().view(torch.uint8), bits_v) and torch.equal(backend.v_scale[0].cpu(), sc_v)
