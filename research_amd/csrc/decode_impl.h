@@ -281,7 +281,14 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
             st.init();
             const int lane_voff =
                 role.tok_local * (p.hkv * D * (int)sizeof(KV)) + kvh * (D * (int)sizeof(KV)) + role.lir * 16;
-            if (p.tpw * U > p.bs)  // uniform: few kv heads per wave load and short blocks
+            // uniform choices: few kv heads per wave load and short blocks
+            if (U % 4 == 0 && p.bs == 4 * p.tpw && U > 4)  // 4 steps per block: U/4 blocks per iteration
+                attend_blocks_pk_multi<KV, QT, D, NREP, U, (U % 4 == 0 ? 4 : 2)>(
+                    st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step, lane, lane_voff, kvh, role.tok_local == 0);
+            else if (p.bs == 2 * p.tpw)  // 2 steps per block
+                attend_blocks_pk_multi<KV, QT, D, NREP, U, 2>(st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step,
+                                                              lane, lane_voff, kvh, role.tok_local == 0);
+            else if (p.tpw * U > p.bs)
                 attend_blocks_pk<KV, QT, D, NREP, U, true>(st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step,
                                                            lane, lane_voff, kvh, role.tok_local == 0);
             else

@@ -326,4 +326,155 @@ __device__ __forceinline__ void attend_blocks_pk(
     }
 }
 
+// The same loop for layouts where a token step of the wave covers several tokens and a block holds only SPB
+// steps (one kv head per load, 16-token blocks): the U steps in flight are taken from G = U / SPB consecutive
+// blocks of the wave, each through its own descriptor, so the number of loads in flight and the work per loop
+// entry stay what they are for wide layouts.  Requires p.bs == SPB * p.tpw.
+template <typename KV, typename AT, int D, int NREP, int U, int SPB>
+__device__ __forceinline__ void attend_blocks_pk_multi(
+    PkState<NREP, HeadScatter<NREP, D * (int)sizeof(KV) / 16>::VPL, 2 * PoolWords<KV, AT>::NW> &st,
+    const uint32_t (&qpk)[NREP][PoolWords<KV, AT>::NW], const PoolArgs &p, const int32_t *bt_row, int k_lo, int L,
+    int blk_begin, int blk_end, int blk_step, int lane, int lane_voff, int lane_kvh, bool count_zero_keys) {
+    static_assert(U % SPB == 0 && SPB % 2 == 0, "whole blocks per iteration, token pairs inside one block");
+    constexpr int G = U / SPB;  // blocks per iteration
+    constexpr int LPR = D * (int)sizeof(KV) / 16;
+    constexpr bool kFp8 = sizeof(KV) == 1;
+    using HS = HeadScatter<NREP, LPR>;
+    using PK = Pk16<AT>;
+    using PW = PoolWords<KV, AT>;
+    constexpr int NW = PW::NW;
+    constexpr int VPL = HS::VPL;
+    const int tok_stride = p.hkv * D * (int)sizeof(KV);  // bytes between tokens
+    const int tok_local = (lane / LPR) / p.hpw;
+
+    for (int blk0 = blk_begin; blk0 < blk_end; blk0 += G * blk_step) {
+        int ntok[G], tlo[G];
+        float k_sc[G], v_sc[G];
+        __amdgpu_buffer_rsrc_t rk[G], rv[G];
+        bool partial = false;
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const int blk = blk0 + g * blk_step;
+            const bool in_range = blk < blk_end;
+            ntok[g] = in_range ? min(p.bs, L - blk * p.bs) : 0;
+            tlo[g] = in_range ? max(0, k_lo - blk * p.bs) : 0;
+            const int64_t bid = in_range && blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
+            const bool ok = bid >= 0 && bid < p.num_blocks;
+            if (!ok) {
+                if (in_range && count_zero_keys) st.zero_keys += max(0, ntok[g] - tlo[g]);
+                ntok[g] = 0;
+            }
+            // descriptor of the valid part of this block (empty for a missing block): reads past it return 0
+            const int64_t block_off = (ok ? bid : 0) * p.bs * (int64_t)tok_stride;
+            rk[g] = __builtin_amdgcn_make_buffer_rsrc((void *)(reinterpret_cast<const char *>(p.k) + block_off), 0,
+                                                      ntok[g] * tok_stride, 0x00020000);
+            rv[g] = __builtin_amdgcn_make_buffer_rsrc((void *)(reinterpret_cast<const char *>(p.v) + block_off), 0,
+                                                      ntok[g] * tok_stride, 0x00020000);
+            k_sc[g] = p.scale_log2;
+            v_sc[g] = 1.f;
+            if (kFp8 && ok) {
+                k_sc[g] *= p.k_scale[bid * p.hkv + lane_kvh];
+                v_sc[g] = p.v_scale[bid * p.hkv + lane_kvh];
+            }
+            partial |= ntok[g] < p.bs || tlo[g] > 0;
+        }
+
+        pa_u4 kraw[U], vraw[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            kraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rk[u / SPB], lane_voff + (u % SPB) * p.tpw * tok_stride, 0,
+                                                            kStreamPolicy);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            vraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rv[u / SPB], lane_voff + (u % SPB) * p.tpw * tok_stride, 0,
+                                                            kStreamPolicy);
+
+        // ---- logits: one (token, head) per lane -----------------------
+        float sv[U][VPL];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int g = u / SPB, s0 = (u % SPB) * p.tpw;  // block of the step, its first token in the block
+            if (partial && s0 >= ntok[g]) {  // uniform: the whole step lies past the block's end
+#pragma unroll
+                for (int j = 0; j < VPL; ++j) sv[u][j] = -INFINITY;
+                continue;
+            }
+            uint32_t kw[NW];
+            PW::unpack(kraw[u], kw);
+            float s[NREP];
+#pragma unroll
+            for (int r = 0; r < NREP; ++r) {
+                float d = PK::dot2(kw[0], qpk[r][0], 0.f);
+#pragma unroll
+                for (int i = 1; i < NW; ++i) d = PK::dot2(kw[i], qpk[r][i], d);
+                s[r] = d;
+            }
+            HS::reduce(s, sv[u], lane);
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) sv[u][j] *= k_sc[g];
+            if (partial) {
+                const int tt = s0 + tok_local;
+                const bool ok = tt < ntok[g] && tt >= tlo[g];
+#pragma unroll
+                for (int j = 0; j < VPL; ++j) sv[u][j] = ok ? sv[u][j] : -INFINITY;
+            }
+        }
+        // ---- running maximum; rescale only when some lane's maximum grew ----
+        float mx[VPL];
+        bool grew = false;
+#pragma unroll
+        for (int j = 0; j < VPL; ++j) {
+            mx[j] = st.m[j];
+#pragma unroll
+            for (int u = 0; u < U; ++u) mx[j] = fmaxf(mx[j], sv[u][j]);
+            grew |= mx[j] > st.m[j];
+        }
+        if (__builtin_amdgcn_ballot_w64(grew) != 0) {
+            float alpha[VPL];
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) {
+                alpha[j] = __builtin_amdgcn_exp2f(st.m[j] - mx[j]);
+                st.m[j] = mx[j];
+                st.l[j] *= alpha[j];
+            }
+            StaticFor<NREP>::run([&](auto h) {
+                const float a = HS::template bcast<h.value>(alpha);
+#pragma unroll
+                for (int e = 0; e < 2 * NW; ++e) st.acc[h.value][e] *= a;
+            });
+        }
+        // ---- p.v, two tokens per step ----------------------------------
+#pragma unroll
+        for (int u = 0; u < U; u += 2) {
+            const int g = u / SPB;
+            if (partial && (u % SPB) * p.tpw >= ntok[g]) continue;  // uniform: both steps lie past the block's end
+            uint32_t ppk[VPL];
+#pragma unroll
+            for (int j = 0; j < VPL; ++j) {
+                const float p0 = __builtin_amdgcn_exp2f(sv[u][j] - st.m[j]);  // 0 for masked tokens
+                const float p1 = __builtin_amdgcn_exp2f(sv[u + 1][j] - st.m[j]);
+                st.l[j] += p0 + p1;
+                ppk[j] = kFp8 ? PK::pack(p0 * v_sc[g], p1 * v_sc[g]) : PK::pack(p0, p1);
+            }
+            uint32_t v0[NW], v1[NW];
+            PW::unpack(vraw[u], v0);
+            PW::unpack(vraw[u + 1], v1);
+            uint32_t lo[NW], hi[NW];  // (v_t0[2i], v_t1[2i]) and (v_t0[2i+1], v_t1[2i+1])
+#pragma unroll
+            for (int i = 0; i < NW; ++i) {
+                lo[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x05040100u);
+                hi[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x07060302u);
+            }
+            StaticFor<NREP>::run([&](auto h) {
+                const uint32_t pb = HS::template bcast_u<h.value>(ppk);
+#pragma unroll
+                for (int i = 0; i < NW; ++i) {
+                    st.acc[h.value][2 * i] = PK::dot2(lo[i], pb, st.acc[h.value][2 * i]);
+                    st.acc[h.value][2 * i + 1] = PK::dot2(hi[i], pb, st.acc[h.value][2 * i + 1]);
+                }
+            });
+        }
+    }
+}
+
 }  // namespace pa_decode_detail

@@ -307,3 +307,75 @@ def test_decode_step_in_a_hip_graph():
         assert_close(out, want, 2e-2, f"replay {it}")
         assert torch.equal(kc.cpu(), k_ref)
         (torch.ones(1000, device=DEV) * 2).sum().item()  # eager work between replays
+
+
+@pytest.mark.parametrize("hq,hkv,d,kv", [
+    (8, 1, 128, "bf16"),   # one kv head: a wave load covers 4 tokens, two 16-token blocks per loop iteration
+    (4, 1, 128, "f16"),
+    (4, 1, 64, "bf16"),    # 8 tokens per wave load: four blocks per iteration
+    (6, 2, 64, "bf16"),    # two kv heads of D=64: 4 tokens per load
+    (8, 1, 128, "fp8"),    # fp8 rows of 8 lanes, 8 tokens per load, two blocks per iteration
+    (4, 1, 256, "fp8"),
+])
+def test_few_kv_heads_with_blocks_of_16(hq, hkv, d, kv):
+    """Layouts whose loop takes several blocks per iteration: ragged lengths around block and iteration
+    boundaries, poisoned tails, a short table, a bad block id, an empty sequence, sliding windows and extra
+    zero keys."""
+    announce(f"decode few kv heads hq={hq} hkv={hkv} d={d} {kv}")
+    rng = np.random.default_rng(400 + hq + d)
+    bs, nb = 16, 160
+    dtype = torch.float16 if kv == "f16" else torch.bfloat16
+    lens = [1, 15, 16, 17, 31, 32, 33, 47, 48, 49, 64, 65, 127, 128, 129, 500, 0, 40, 90]
+    perm = rng.permutation(nb).tolist()
+    tables, at = [], 0
+    for n in lens:
+        c = -(-n // bs)
+        tables.append(perm[at : at + c])
+        at += c
+    tables[-2] = tables[-2][:1]          # covers 16 of the 40 keys: the rest are zero keys
+    tables[-1][-1] = 100000              # a block id outside the pool acts as a missing block
+    q = torch.from_numpy(rng.standard_normal((len(lens), hq, d)).astype(np.float32)).to(dtype)
+    kp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
+    vp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
+    for b, n in enumerate(lens):  # poison every slot past a sequence's end inside its last block
+        if n % bs and len(tables[b]) == -(-n // bs) and tables[b][-1] < nb:
+            lo = tables[b][-1] * bs + n % bs
+            kp[lo : (tables[b][-1] + 1) * bs] = float("nan")
+            vp[lo : (tables[b][-1] + 1) * bs] = float("inf")
+    want_tables = [list(t) for t in tables]
+    want_tables[-1][-1] = -1
+    scale = d ** -0.5
+    if kv == "fp8":
+        kp, vp = torch.nan_to_num(kp, nan=0.0), torch.nan_to_num(vp, posinf=0.0)  # a quantised tile holds no NaN
+        kb, ks = ops.quantize_kv_e4m3(kp.to(DEV), bs)
+        vb, vs = ops.quantize_kv_e4m3(vp.to(DEV), bs)
+        kd = po.dequantize_kv_e4m3(kb.cpu().view(torch.uint8), ks.cpu(), bs)
+        vd = po.dequantize_kv_e4m3(vb.cpu().view(torch.uint8), vs.cpu(), bs)
+        pools, ref, extra, tol = (kb, vb), (kd, vd), dict(k_scale=ks, v_scale=vs), 2e-2
+    else:
+        pools, ref, extra, tol = (kp.to(DEV), vp.to(DEV)), (kp, vp), {}, 2e-2
+
+    def checked(window=0, pad=False):
+        kref, vref = ref
+        # blocks the table does not hold are zero keys: give the checker tables cut at the first bad entry
+        cut = []
+        for t in want_tables:
+            good = []
+            for b in t:
+                if b < 0:
+                    break
+                good.append(b)
+            cut.append(good)
+        return po.paged_decode(q, kref, vref, cut, lens, bs, scale, pad_zero_keys=pad, window=window)
+
+    got = run_decode(q.to(DEV), *pools, tables, lens, bs, scale, **extra)
+    assert_close(got, checked(), tol, "plain")
+    assert not got[lens.index(0)].any()
+    ez = [max(lens) - n for n in lens]
+    got = run_decode(q.to(DEV), *pools, tables, lens, bs, scale, extra_zero=ez, **extra)
+    assert_close(got, checked(pad=True), tol, "extra zero keys")
+    ws = ops.decode_workspace(q.to(DEV), pools[0])
+    for window in (1, 5, 16, 33, 100):
+        got = ops.decode(q.to(DEV), *pools, tables_to_device(tables), torch.tensor(lens, dtype=torch.int32, device=DEV),
+                         bs, scale, ws, None, extra.get("k_scale"), extra.get("v_scale"), window=window)
+        assert_close(got, checked(window=window), tol, f"window {window}")
