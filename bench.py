@@ -89,6 +89,23 @@ def cpu_baseline(w, budget_s: float):
     }
 
 
+def cpu_literal(w):
+    """One pass of the literal restatement of the reference's decode (token-by-token gather loop into a
+    zero-padded batch, repeat_interleave, unmasked SDPA) over the whole workload; only for the workloads small
+    enough to run it as written (c1, c2)."""
+    from oracle import paged_oracle as po
+
+    tables = [t.tolist() for t in w.block_tables]
+    t0 = time.perf_counter()
+    po.decode_literal(w.q[:, None], w.k_pool, w.v_pool, tables, w.seq_lens, w.block_size, w.scale)
+    dt = time.perf_counter() - t0
+    padded = 2 * w.batch * int(w.seq_lens.max()) * w.num_q_heads * w.head_dim * w.q.element_size()
+    return {"value": w.algorithmic_bytes() / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(),
+            "kind": "port", "seconds": dt, "tokens_per_s": w.batch / dt,
+            "sample": f"the whole of {w.name} once: {2 * int(w.seq_lens.sum())} row copies issued from Python, "
+                      f"{padded / 1e9:.2f} GB of padded and head-expanded K/V, one SDPA call"}
+
+
 def preheat(fn, seconds):
     """Untimed calls of `fn` for about `seconds`, so that the timed region does not start on idle clocks."""
     t0 = time.perf_counter()
@@ -334,6 +351,8 @@ def main() -> int:
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
+        if args.workload in ("c1", "c2") and args.cpu_seconds > 0:
+            result["cpu_baseline_literal"] = cpu_literal(w)
     print(json.dumps(result))
     return 0
 
