@@ -208,10 +208,16 @@ __device__ __forceinline__ void attend_blocks_pk(
     const int tok_stride = p.hkv * D * (int)sizeof(KV);  // bytes between tokens
     const int tok_local = (lane / LPR) / p.hpw;
 
+    // the table entry of a block is requested one iteration ahead, so its latency is off the wave's critical path
+    int64_t bid_next = blk_begin < blk_end && blk_begin < p.bt_stride ? (int64_t)bt_row[blk_begin] : -1;
     for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
         const int ntok = min(p.bs, L - blk * p.bs);
         const int tlo = max(0, k_lo - blk * p.bs);  // tokens below it lie before the window (first block only)
-        const int64_t bid = blk < p.bt_stride ? (int64_t)bt_row[blk] : -1;
+        const int64_t bid = bid_next;
+        {
+            const int nb = blk + blk_step;
+            bid_next = nb < blk_end && nb < p.bt_stride ? (int64_t)bt_row[nb] : -1;
+        }
         if (bid < 0 || bid >= p.num_blocks) {
             if (count_zero_keys) st.zero_keys += max(0, ntok - tlo);
             continue;
