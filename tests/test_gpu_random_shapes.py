@@ -1,0 +1,107 @@
+"""Seeded random configurations of decode and chunked prefill against the checker: head layouts, head dims,
+block sizes, ragged lengths, windows, fp8 pools, short tables.  Each case is small; together they walk the
+dispatch space (packed / generic loops, single- and multi-block iterations, matrix-core / vector prefill)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import paged_oracle as po
+from research_amd import ops
+from tests.gpu_helpers import DEV, announce, assert_close, tables_to_device
+
+pytestmark = pytest.mark.gpu
+
+
+def _draw(rng):
+    d = int(rng.choice([32, 64, 128, 256]))
+    hkv = int(rng.choice([1, 2, 3, 4, 8]))
+    n_rep = int(rng.choice([1, 2, 3, 4, 7, 8, 12]))
+    bs = int(rng.choice([1, 4, 8, 16, 16, 16, 32, 48]))
+    kind = str(rng.choice(["bf16", "bf16", "f16", "f32", "fp8"]))
+    batch = int(rng.integers(1, 7))
+    return d, hkv, n_rep, bs, kind, batch
+
+
+def _pool(rng, nb, bs, hkv, d, dtype):
+    k = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
+    v = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype)
+    return k, v
+
+
+def _tables(rng, lens, bs, spare=2):
+    need = [-(-int(n) // bs) for n in lens]
+    nb = sum(need) + spare
+    perm = rng.permutation(nb)
+    tables, at = [], 0
+    for n in need:
+        tables.append(perm[at : at + n].tolist())
+        at += n
+    return tables, nb
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_decode(seed):
+    rng = np.random.default_rng(7000 + seed)
+    d, hkv, n_rep, bs, kind, batch = _draw(rng)
+    hq = hkv * n_rep
+    announce(f"random decode seed={seed} hq={hq} hkv={hkv} d={d} bs={bs} {kind} batch={batch}")
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32, "fp8": torch.bfloat16}[kind]
+    lens = rng.integers(0, 6 * max(bs, 16) + 1, batch).tolist()
+    if seed % 3 == 0:
+        lens[0] = int(rng.integers(300, 700))
+    tables, nb = _tables(rng, lens, bs)
+    short = seed % 4 == 1 and len(tables[-1]) > 1
+    if short:
+        tables[-1] = tables[-1][:-1]  # the last block of the last sequence is missing: zero keys
+    k, v = _pool(rng, nb, bs, hkv, d, dtype)
+    q = torch.from_numpy(rng.standard_normal((batch, hq, d)).astype(np.float32)).to(dtype)
+    scale = d ** -0.5
+    window = int(rng.choice([0, 0, 1, 5, 40]))
+    if short:
+        window = 0  # zero keys and windows are separate features
+    if kind == "fp8":
+        if bs > 256 or d % 16:
+            pytest.skip("fp8 tile limits")
+        kb, ks = ops.quantize_kv_e4m3(k.to(DEV), bs)
+        vb, vs = ops.quantize_kv_e4m3(v.to(DEV), bs)
+        kref = po.dequantize_kv_e4m3(kb.cpu().view(torch.uint8), ks.cpu(), bs)
+        vref = po.dequantize_kv_e4m3(vb.cpu().view(torch.uint8), vs.cpu(), bs)
+        pools, extra, tol = (kb, vb), (ks, vs), 2e-2
+    else:
+        kref, vref, pools, extra = k, v, (k.to(DEV), v.to(DEV)), (None, None)
+        tol = 1e-5 if kind == "f32" else 2e-2
+    ws = ops.decode_workspace(q.to(DEV), pools[0])
+    got = ops.decode(q.to(DEV), *pools, tables_to_device(tables), torch.tensor(lens, dtype=torch.int32, device=DEV), bs,
+                     scale, ws, None, *extra, window=window)
+    want = po.paged_decode(q, kref, vref, tables, lens, bs, scale, window=window)
+    assert_close(got, want, tol, f"decode window={window}")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_chunked_prefill(seed):
+    rng = np.random.default_rng(9000 + seed)
+    d, hkv, n_rep, bs, kind, batch = _draw(rng)
+    if kind == "fp8":
+        kind = "bf16"
+    n_rep = min(n_rep, 8)
+    hq = hkv * n_rep
+    announce(f"random prefill seed={seed} hq={hq} hkv={hkv} d={d} bs={bs} {kind} batch={batch}")
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32}[kind]
+    prefix = rng.integers(0, 200, batch).tolist()
+    chunk = rng.integers(1, 100, batch).tolist()
+    if seed % 5 == 0:
+        prefix[0] = 0
+    cmax = max(chunk)
+    tables, nb = _tables(rng, [p + c for p, c in zip(prefix, chunk)], bs)
+    k, v = _pool(rng, nb, bs, hkv, d, dtype)
+    q = torch.from_numpy(rng.standard_normal((batch, cmax, hq, d)).astype(np.float32)).to(dtype)
+    scale = d ** -0.5
+    window = int(rng.choice([0, 0, 7, 64]))
+    out = torch.zeros(batch * cmax, hq, d, dtype=dtype, device=DEV)
+    i32 = lambda x: torch.tensor(list(x), dtype=torch.int32, device=DEV)
+    ops.prefill_paged(q.reshape(-1, hq, d).to(DEV), k.to(DEV), v.to(DEV), tables_to_device(tables),
+                      i32(p + c for p, c in zip(prefix, chunk)), i32(chunk), i32(np.arange(batch) * cmax), cmax, bs, scale,
+                      out=out, window=window)
+    want = po.paged_prefill_chunk(q, k, v, tables, prefix, chunk, bs, scale, window=window)
+    assert_close(out.reshape(batch, cmax, hq, d), want, 1e-5 if kind == "f32" else 2e-2, f"prefill window={window}")
