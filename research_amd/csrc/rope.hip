@@ -14,7 +14,8 @@ constexpr int kRopeThreads = 256;
 // One rounding step to the element type T, value kept as float.
 template <typename T> __device__ __forceinline__ float rope_round(float x);
 template <> __device__ __forceinline__ float rope_round<float>(float x) { return x; }
-template <> __device__ __forceinline__ float rope_round<pa_bf16>(float x) { return pa_bf16_to_f32(pa_f32_to_bf16(x)); }
+// (gfx950 rounds float -> bf16 to nearest even in hardware: v_cvt_pk_bf16_f32)
+template <> __device__ __forceinline__ float rope_round<pa_bf16>(float x) { return (float)(__bf16)x; }
 template <> __device__ __forceinline__ float rope_round<pa_f16>(float x) { return (float)(_Float16)x; }
 
 template <typename T> __device__ __forceinline__ uint4 rope_pack(const float *f);
@@ -25,7 +26,11 @@ template <> __device__ __forceinline__ uint4 rope_pack<float>(const float *f) {
 template <> __device__ __forceinline__ uint4 rope_pack<pa_bf16>(const float *f) {
     uint32_t w[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) w[i] = (uint32_t)pa_f32_to_bf16(f[2 * i]) | ((uint32_t)pa_f32_to_bf16(f[2 * i + 1]) << 16);
+    for (int i = 0; i < 4; ++i) {
+        typedef __bf16 bf2 __attribute__((ext_vector_type(2)));
+        const bf2 pair = {(__bf16)f[2 * i], (__bf16)f[2 * i + 1]};
+        w[i] = __builtin_bit_cast(uint32_t, pair);
+    }
     return make_uint4(w[0], w[1], w[2], w[3]);
 }
 template <> __device__ __forceinline__ uint4 rope_pack<pa_f16>(const float *f) {
@@ -80,18 +85,22 @@ struct RopeArgs {
     int half_vecs;  // 16-byte vectors in half a head
 };
 
-// One thread per (token, head, vector of the first half) for the rotated heads (it also handles the matching
-// vector of the second half), one thread per (token, vector) for V.
-template <typename T> __global__ __launch_bounds__(kRopeThreads) void rope_kv_append_kernel(const RopeArgs a) {
+// One thread per (token, group of HG heads, vector of the first half) for the rotated heads: it loads its four
+// cos/sin vectors once and rotates that vector (and its partner in the second half) of HG heads, so the table
+// rows are fetched HG times less often than the data they multiply.  The heads of a group are hq/HG apart
+// (group g holds heads g, g + hq/HG, ...), so that consecutive lanes touch consecutive heads in every load and
+// store.  One thread per (token, vector) for V.
+template <typename T, int HG> __global__ __launch_bounds__(kRopeThreads) void rope_kv_append_kernel(const RopeArgs a) {
     const int hv = a.half_vecs;
-    const int units = (a.hq + 3 * a.hkv) * hv;  // per token: hv per q head and per k head, 2*hv per v head
+    const int qg = a.hq / HG, kg = a.hkv / HG;  // head groups (hq and hkv are multiples of HG)
+    const int units = (qg + kg + 2 * a.hkv) * hv;  // per token: hv per head group, 2*hv per v head
     const int64_t gid = (int64_t)blockIdx.x * kRopeThreads + threadIdx.x;
     const int64_t tok = gid / units;
     if (tok >= a.n_tokens) return;
     const int u = (int)(gid - tok * units);
     const int64_t slot = a.slots ? a.slots[tok] : -1;
     const bool cached = slot >= 0 && slot < a.total_slots;
-    const int rot_units = (a.hq + a.hkv) * hv;
+    const int rot_units = (qg + kg) * hv;
     if (u >= rot_units) {  // V: plain copy, one vector per thread (a V row holds 2*hkv*hv vectors)
         if (!cached) return;
         const int j = u - rot_units;
@@ -101,43 +110,73 @@ template <typename T> __global__ __launch_bounds__(kRopeThreads) void rope_kv_ap
     }
     int64_t r = a.positions ? (int64_t)a.positions[tok] : tok;
     r = r < 0 ? 0 : (r >= a.rope_rows ? a.rope_rows - 1 : r);  // never read outside the tables
-    const int head = u / hv, j = u - head * hv;
+    const int group = u / hv, j = u - group * hv;
     const uint4 c1 = a.cos[r * 2 * hv + j], c2 = a.cos[r * 2 * hv + hv + j];
     const uint4 s1 = a.sin[r * 2 * hv + j], s2 = a.sin[r * 2 * hv + hv + j];
-    if (head < a.hq) {
-        const int64_t at = (tok * a.hq + head) * 2 * hv + j;
-        uint4 v1 = a.q[at], v2 = a.q[at + hv];
-        rope_rotate<T>(v1, v2, c1, c2, s1, s2);
-        a.q_out[at] = v1;
-        a.q_out[at + hv] = v2;
-    } else {
-        const int kh = head - a.hq;
-        const int64_t at = (tok * a.hkv + kh) * 2 * hv + j;
-        uint4 v1 = a.k_src[at], v2 = a.k_src[at + hv];
-        rope_rotate<T>(v1, v2, c1, c2, s1, s2);
-        if (a.k_out) {
-            a.k_out[at] = v1;
-            a.k_out[at + hv] = v2;
+    if (group < qg) {
+        uint4 v1[HG], v2[HG];
+#pragma unroll
+        for (int h = 0; h < HG; ++h) {
+            const int64_t at = (tok * a.hq + h * qg + group) * 2 * hv + j;
+            v1[h] = a.q[at];
+            v2[h] = a.q[at + hv];
         }
-        if (cached) {
-            const int64_t dst = (slot * a.hkv + kh) * 2 * hv + j;
-            a.k_cache[dst] = v1;
-            a.k_cache[dst + hv] = v2;
+#pragma unroll
+        for (int h = 0; h < HG; ++h) {
+            const int64_t at = (tok * a.hq + h * qg + group) * 2 * hv + j;
+            rope_rotate<T>(v1[h], v2[h], c1, c2, s1, s2);
+            a.q_out[at] = v1[h];
+            a.q_out[at + hv] = v2[h];
+        }
+    } else {
+        const int kgi = group - qg;  // this thread's kv heads: kgi, kgi + kg, kgi + 2 kg, ...
+        uint4 v1[HG], v2[HG];
+#pragma unroll
+        for (int h = 0; h < HG; ++h) {
+            const int64_t at = (tok * a.hkv + h * kg + kgi) * 2 * hv + j;
+            v1[h] = a.k_src[at];
+            v2[h] = a.k_src[at + hv];
+        }
+#pragma unroll
+        for (int h = 0; h < HG; ++h) {
+            const int64_t at = (tok * a.hkv + h * kg + kgi) * 2 * hv + j;
+            rope_rotate<T>(v1[h], v2[h], c1, c2, s1, s2);
+            if (a.k_out) {
+                a.k_out[at] = v1[h];
+                a.k_out[at + hv] = v2[h];
+            }
+            if (cached) {
+                const int64_t dst = (slot * a.hkv + h * kg + kgi) * 2 * hv + j;
+                a.k_cache[dst] = v1[h];
+                a.k_cache[dst + hv] = v2[h];
+            }
         }
     }
 }
 
+template <typename T> void launch_rope_typed(const RopeArgs &a, int hg, int64_t grid, hipStream_t s) {
+    if (hg == 4)
+        rope_kv_append_kernel<T, 4><<<dim3((unsigned)grid), dim3(kRopeThreads), 0, s>>>(a);
+    else if (hg == 2)
+        rope_kv_append_kernel<T, 2><<<dim3((unsigned)grid), dim3(kRopeThreads), 0, s>>>(a);
+    else
+        rope_kv_append_kernel<T, 1><<<dim3((unsigned)grid), dim3(kRopeThreads), 0, s>>>(a);
+}
+
 int launch_rope(const RopeArgs &a, int dtype, hipStream_t s, const char *what) {
-    const int64_t units = (int64_t)(a.hq + 3 * a.hkv) * a.half_vecs;
+    // heads per thread: the largest of 4, 2, 1 that divides both head counts (hkv = 0: q only)
+    int hg = 4;
+    while (hg > 1 && (a.hq % hg != 0 || a.hkv % hg != 0)) hg >>= 1;
+    const int64_t units = (int64_t)(a.hq / hg + a.hkv / hg + 2 * a.hkv) * a.half_vecs;
     PA_REQUIRE(units <= 0x7fffffff, "row of %lld vectors is too large", (long long)units);
     const int64_t grid = (a.n_tokens * units + kRopeThreads - 1) / kRopeThreads;
     PA_REQUIRE(grid <= 0x7fffffff, "n_tokens=%lld is too large for one launch", (long long)a.n_tokens);
     if (dtype == PA_F32)
-        rope_kv_append_kernel<float><<<dim3((unsigned)grid), dim3(kRopeThreads), 0, s>>>(a);
+        launch_rope_typed<float>(a, hg, grid, s);
     else if (dtype == PA_BF16)
-        rope_kv_append_kernel<pa_bf16><<<dim3((unsigned)grid), dim3(kRopeThreads), 0, s>>>(a);
+        launch_rope_typed<pa_bf16>(a, hg, grid, s);
     else
-        rope_kv_append_kernel<pa_f16><<<dim3((unsigned)grid), dim3(kRopeThreads), 0, s>>>(a);
+        launch_rope_typed<pa_f16>(a, hg, grid, s);
     PA_CHECK_LAUNCH(what);
     return PA_OK;
 }
