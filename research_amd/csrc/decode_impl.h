@@ -358,6 +358,16 @@ __device__ __forceinline__ int owner_of(int64_t u, int64_t total, int64_t grid) 
     return (int)(((u + 1) * grid - 1) / total);
 }
 
+// Workgroups of the split pass that take part: with little work (one short sequence, say) a workgroup per
+// pool block would leave hundreds of one-block partials for the reduction pass to chain through, so a
+// workgroup gets at least kMinUnitsPerWorkgroup units and the rest of the grid leaves at once.  Both passes
+// derive the number from the same total.
+constexpr int kMinUnitsPerWorkgroup = 4;
+__device__ __forceinline__ int effective_grid(int64_t total, int grid) {
+    const int64_t g = total / kMinUnitsPerWorkgroup;
+    return g < 1 ? 1 : (g < grid ? (int)g : grid);
+}
+
 // Finish one (sequence, query head): fold `ez` extra all-zero keys into the
 // merged (num, M, den) and normalise.
 __device__ __forceinline__ float finish_row(float num, float M, float den, int ez) {
@@ -425,9 +435,11 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
     const int64_t total = per_plane * planes;
     const LaneRole role = lane_role<KV, D>(lane, p);
     if (total == 0) return;
+    const int grid = effective_grid(total, (int)gridDim.x);
+    if ((int)blockIdx.x >= grid) return;  // uniform
 
-    int64_t cur = unit_begin(blockIdx.x, total, gridDim.x);
-    const int64_t end = unit_begin((int64_t)blockIdx.x + 1, total, gridDim.x);
+    int64_t cur = unit_begin(blockIdx.x, total, grid);
+    const int64_t end = unit_begin((int64_t)blockIdx.x + 1, total, grid);
     while (cur < end) {
         const int plane = (int)(cur / per_plane);
         const int off = (int)(cur - plane * per_plane);
@@ -509,30 +521,48 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_kernel(const DecodeArg
         return;
     }
     const int64_t u0 = plane * per_plane + a.block_prefix[b];
-    const int w0 = owner_of(u0, total, a.split_grid), w1 = owner_of(u0 + nblk - 1, total, a.split_grid);
+    const int grid = effective_grid(total, a.split_grid);
+    const int w0 = owner_of(u0, total, grid), w1 = owner_of(u0 + nblk - 1, total, grid);
     if (w0 == w1) return;  // finished by the split pass
     const int64_t key = (int64_t)plane * a.batch + b;
     const int stride_acc = p.hpw * NREP * D, stride_ml = p.hpw * NREP * 2;
-    // a workgroup whose range is empty (more workgroups than blocks) left no partial
-    auto has_piece = [&](int w) {
-        return unit_begin(w, total, a.split_grid) < unit_begin((int64_t)w + 1, total, a.split_grid) &&
-               w + key < a.slot_cap;
-    };
+    // every taking-part workgroup has units (effective_grid never exceeds the number of units), so every index
+    // in [w0, w1] left a partial unless its slot fell outside the workspace
+    auto has_piece = [&](int w) { return w + key < a.slot_cap; };
     float M = kNegBig, den = 0.f, num[DPL];
 #pragma unroll
     for (int k = 0; k < DPL; ++k) num[k] = 0.f;
-    for (int w = w0 + wave; w <= w1; w += kWaves) {
-        if (!has_piece(w)) continue;
-        const int64_t slot = w + key;
-        const float m = a.part_ml[slot * stride_ml + idx * 2], l = a.part_ml[slot * stride_ml + idx * 2 + 1];
-        const float mn = fmaxf(M, m);
-        const float so = __builtin_amdgcn_exp2f(M - mn), sn = __builtin_amdgcn_exp2f(m - mn);
-        den = den * so + l * sn;
+    // the pieces of a long sequence in a small batch number in the hundreds: each wave keeps the loads of
+    // kPipe of its pieces in flight, then folds them in
+    constexpr int kPipe = 8;
+    for (int w = w0 + wave; w <= w1; w += kWaves * kPipe) {
+        float m[kPipe], l[kPipe], x[kPipe][DPL];
 #pragma unroll
-        for (int k = 0; k < DPL; ++k) {
-            const int d = lane + PA_WAVE * k;
-            const float x = d < D ? a.part_acc[slot * stride_acc + idx * D + d] : 0.f;
-            num[k] = num[k] * so + x * sn;
+        for (int j = 0; j < kPipe; ++j) {
+            const int wj = w + j * kWaves;
+            const bool have = wj <= w1 && has_piece(wj);
+            const int64_t slot = (have ? wj : w0) + key;
+            m[j] = have ? a.part_ml[slot * stride_ml + idx * 2] : kNegBig;
+            l[j] = have ? a.part_ml[slot * stride_ml + idx * 2 + 1] : 0.f;
+#pragma unroll
+            for (int k = 0; k < DPL; ++k) {
+                const int d = lane + PA_WAVE * k;
+                x[j][k] = have && d < D ? a.part_acc[slot * stride_acc + idx * D + d] : 0.f;
+            }
+        }
+        float mn = M;
+#pragma unroll
+        for (int j = 0; j < kPipe; ++j) mn = fmaxf(mn, m[j]);
+        const float so = __builtin_amdgcn_exp2f(M - mn);
+        den *= so;
+#pragma unroll
+        for (int k = 0; k < DPL; ++k) num[k] *= so;
+#pragma unroll
+        for (int j = 0; j < kPipe; ++j) {
+            const float sn = __builtin_amdgcn_exp2f(m[j] - mn);
+            den = fmaf(l[j], sn, den);
+#pragma unroll
+            for (int k = 0; k < DPL; ++k) num[k] = fmaf(x[j][k], sn, num[k]);
         }
         M = mn;
     }
@@ -587,14 +617,12 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_wave_kernel(const Deco
         return;
     }
     const int64_t u0 = plane * per_plane + a.block_prefix[b];
-    const int w0 = owner_of(u0, total, a.split_grid), w1 = owner_of(u0 + nblk - 1, total, a.split_grid);
+    const int grid = effective_grid(total, a.split_grid);
+    const int w0 = owner_of(u0, total, grid), w1 = owner_of(u0 + nblk - 1, total, grid);
     if (w0 == w1) return;  // finished by the split pass
     const int64_t key = (int64_t)plane * a.batch + b;
     const int stride_acc = p.hpw * NREP * D, stride_ml = p.hpw * NREP * 2;
-    auto has_piece = [&](int w) {
-        return w <= w1 && unit_begin(w, total, a.split_grid) < unit_begin((int64_t)w + 1, total, a.split_grid) &&
-               w + key < a.slot_cap;
-    };
+    auto has_piece = [&](int w) { return w <= w1 && w + key < a.slot_cap; };  // every workgroup in range has units
     float M = kNegBig, den = 0.f, num[DPL];
 #pragma unroll
     for (int k = 0; k < DPL; ++k) num[k] = 0.f;
