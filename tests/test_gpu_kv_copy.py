@@ -183,3 +183,35 @@ def test_fp8_append_v_pool_and_edge_cases():
     assert torch.equal(bits2[bs : 3 * bs], want_bits) and torch.equal(scale2[1:3], want_scale)
     # nothing to do
     ops.kv_append_e4m3(kb, vb, ks, vs, src[:0].to(DEV), src[:0].to(DEV), torch.zeros(0, dtype=torch.int64, device=DEV), bs)
+
+
+@pytest.mark.parametrize("hkv,d,bs,dtype", [
+    (12, 64, 16, torch.bfloat16),   # more kv heads than a workgroup's eight groups of lanes: two passes
+    (3, 256, 32, torch.float16),    # tiles larger than a lane keeps in registers
+    (1, 128, 16, torch.float32),    # one kv head: a single group of lanes works
+    (5, 20, 8, torch.bfloat16),     # head_dim not a multiple of 8: the element-wise kernel
+])
+def test_fp8_append_shapes(hkv, d, bs, dtype):
+    """The append kernels over head counts, head dims and block sizes: bytes and scales against the checker's
+    statement of the policy, for a prompt written in one call and growth over the following calls."""
+    announce(f"fp8 append shapes hkv={hkv} d={d} bs={bs} {dtype}")
+    g = torch.Generator().manual_seed(23 + hkv)
+    nb = 7
+    bits, scale = _fp8_pool(nb, bs, hkv, d)
+    kc = bits.clone().view(torch.float8_e4m3fn).to(DEV)
+    vc = bits.clone().view(torch.float8_e4m3fn).to(DEV)
+    ks, vs = scale.clone().to(DEV), scale.clone().to(DEV)
+    vbits, vscale = bits.clone(), scale.clone()
+    table = [4, 1, 6, 0, 3]
+    at = 0
+    for n_new, gain in ((2 * bs + 3, 1.0), (1, 4.0), (bs - 5, 0.5), (bs + 2, 9.0)):
+        pos = list(range(at, at + n_new))
+        at += n_new
+        slots = torch.tensor([table[p // bs] * bs + p % bs for p in pos])
+        k = (torch.randn(n_new, hkv, d, generator=g) * gain).to(dtype)
+        v = (torch.randn(n_new, hkv, d, generator=g) * gain).to(dtype)
+        po.append_kv_e4m3(bits, scale, k, slots.tolist(), bs)
+        po.append_kv_e4m3(vbits, vscale, v, slots.tolist(), bs)
+        ops.kv_append_e4m3(kc, vc, ks, vs, k.to(DEV), v.to(DEV), slots.to(DEV), bs)
+        assert torch.equal(kc.cpu().view(torch.uint8), bits) and torch.equal(ks.cpu(), scale)
+        assert torch.equal(vc.cpu().view(torch.uint8), vbits) and torch.equal(vs.cpu(), vscale)
