@@ -219,17 +219,38 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     for (int c = 0; c < NC; ++c) lo_row[c] = bounded ? row_first(row0[c] + col) : 0;
 
     // ---- Q^T operands: row = row0 + col, d = 16*ks + 8*half .. +8 ----
+    // A lane's operands are 16-byte pieces of 32 different rows, hq*D elements apart: loaded directly, every
+    // instruction touches 32 cache lines.  The rows are staged through LDS instead (the ring is still empty):
+    // wave-wide direct loads of whole rows into the wave's own area, 16-byte chunks swizzled by row so that the
+    // operand reads are free of bank conflicts.  Rows past the chunk's end repeat its last row; they are never
+    // written out.
     X8 qreg[NC][KS];
+    {
+        constexpr int QRB = D * 2;       // bytes of a Q row of one head
+        constexpr int QCPR = QRB / 16;   // 16-byte chunks per row
+        constexpr int QRPI = 64 / QCPR;  // rows per wave-wide load
+        const uint32_t q_stage = (uint32_t)wave * (NC * 32 * QRB);  // this wave's staging area, bytes into s_kv
+        const int lrow = lane / QCPR, lslot = lane % QCPR;
 #pragma unroll
-    for (int c = 0; c < NC; ++c) {
-        const T *qbase = reinterpret_cast<const T *>(a.q) + ((int64_t)a.q_starts[b] * p.hq + qh[c]) * D;
-        const int row = row0[c] + col;
-        const bool ok = live[c] && row < q_len;
+        for (int c = 0; c < NC; ++c) {
+            const char *qb = reinterpret_cast<const char *>(a.q) + ((int64_t)a.q_starts[b] * p.hq + qh[c]) * (D * 2);
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            uint4 raw = ok ? ld16(qbase + (int64_t)row * p.hq * D + 16 * ks + 8 * half) : uint4{0, 0, 0, 0};
-            qreg[c][ks] = __builtin_bit_cast(X8, raw);
+            for (int i = 0; i < 32 / QRPI; ++i) {
+                const int r = i * QRPI + lrow;  // row of the column tile this lane fills
+                const int64_t grow = min(row0[c] + r, q_len - 1);
+                pf_dma16(lds_base + q_stage + (uint32_t)((c * 32 + i * QRPI) * QRB),
+                         qb + grow * p.hq * (D * 2) + ((lslot ^ (r & (QCPR - 1))) * 16));
+            }
         }
+        pf_wait_loads<0>();
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                const int slot = (2 * ks + half) ^ (col & (QCPR - 1));
+                const uint4 raw = *reinterpret_cast<const uint4 *>(s_kv + q_stage + (c * 32 + col) * QRB + slot * 16);
+                qreg[c][ks] = __builtin_bit_cast(X8, raw);
+            }
     }
 
     // (used here, so that the compiler waits for them here and knows inside the loop that they have arrived)
@@ -237,6 +258,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     for (int c = 0; c < NC; ++c)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qreg[c][ks]));  // (product operands live in AGPRs)
+    __syncthreads();  // every wave has read its staged rows: the ring may overwrite them
 
     f32x16 o[NC][DT];
 #pragma unroll
