@@ -313,6 +313,31 @@ def main() -> int:
     ms_split = timed("pa_decode_split", args.steps)  # the dominant kernel alone
     ms_reduce = timed("pa_decode_reduce", args.steps)
 
+    gather = None
+    if args.workload in ("c1", "c2"):
+        # the reference's own decode materialises this copy first (_gather_kv_from_cache): the block-table
+        # gather into zero-padded [B, max_len, Hkv, D] tensors, bit-exact, bound by HBM
+        max_len = int(w.seq_lens.max())
+        gk = torch.empty((w.batch, max_len, w.num_kv_heads, w.head_dim), dtype=k_pool.dtype, device=dev)
+        gv = torch.empty_like(gk)
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        for _ in range(3):
+            ops.kv_gather(k_pool, v_pool, tables, lens, max_len, w.block_size, out=(gk, gv))
+        torch.cuda.synchronize()
+        ev0.record()
+        for _ in range(args.steps):
+            ops.kv_gather(k_pool, v_pool, tables, lens, max_len, w.block_size, out=(gk, gv))
+        ev1.record()
+        torch.cuda.synchronize()
+        ms_gather = ev0.elapsed_time(ev1) / args.steps
+        row = w.num_kv_heads * w.head_dim * k_pool.element_size()
+        g_bytes = 2 * w.batch * max_len * row + 2 * w.total_tokens * row + 4 * int(sum(len(t) for t in w.block_tables)) + 4 * w.batch
+        gather = {"kernel": "kv_gather_kernel", "kernel_ms": ms_gather, "bytes": g_bytes,
+                  "achieved": g_bytes / (ms_gather * 1e-3) / 1e9, "unit": "GB/s",
+                  "frac": g_bytes / (ms_gather * 1e-3) / 1e9 / HBM_PEAK_GBPS,
+                  "note": "written 2*B*max_len rows + read 2*sum(L) rows + tables"}
+        del gk, gv
+
     alg_bytes = w.algorithmic_bytes()
     achieved = alg_bytes / (ms_split * 1e-3) / 1e9
     traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
@@ -349,6 +374,8 @@ def main() -> int:
             "kernel_ms": ms_split, "reduce_kernel_ms": ms_reduce,
         },
     }
+    if gather is not None:
+        result["gather"] = gather
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
         if args.workload in ("c1", "c2") and args.cpu_seconds > 0:

@@ -41,12 +41,19 @@ def kv_scatter(k_cache: Tensor, v_cache: Tensor, k_src: Tensor, v_src: Tensor, s
 
 
 def kv_gather(k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, seq_lens: Tensor, max_len: int,
-              block_size: int) -> Tuple[Tensor, Tensor]:
-    """Zero-padded ``[B, max_len, Hkv, D]`` copies; block_tables int32 ``[B, W]`` (-1 padded), seq_lens int32."""
+              block_size: int, out: Optional[Tuple[Tensor, Tensor]] = None) -> Tuple[Tensor, Tensor]:
+    """Zero-padded ``[B, max_len, Hkv, D]`` copies; block_tables int32 ``[B, W]`` (-1 padded), seq_lens int32.
+    ``out``: a pair of contiguous tensors of that shape and the pool's type to write into."""
     total_slots, hkv, d = k_cache.shape
     batch = block_tables.shape[0]
-    k_out = torch.empty((batch, max_len, hkv, d), dtype=k_cache.dtype, device=k_cache.device)
-    v_out = torch.empty_like(k_out)
+    if out is None:
+        k_out = torch.empty((batch, max_len, hkv, d), dtype=k_cache.dtype, device=k_cache.device)
+        v_out = torch.empty_like(k_out)
+    else:
+        k_out, v_out = out
+        for t in (k_out, v_out):
+            if tuple(t.shape) != (batch, max_len, hkv, d) or t.dtype != k_cache.dtype or not t.is_contiguous():
+                raise ValueError("kv_gather: out tensors must be contiguous [B, max_len, Hkv, D] of the pool's type")
     _run("pa_kv_gather", _ptr(k_cache), _ptr(v_cache), _ptr(k_out), _ptr(v_out), _ptr(block_tables),
          block_tables.shape[1], _ptr(seq_lens), batch, max_len, total_slots // block_size, block_size, hkv, d,
          k_cache.element_size(), _stream(k_cache))
