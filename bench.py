@@ -38,7 +38,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5", "engine"])
     ap.add_argument("--preheat-s", type=float, default=0.5,
                     help="seconds of untimed steps before the warmup steps: an idle GPU sits at its lowest clocks "
                          "and takes a few hundred milliseconds of work to leave them")
@@ -242,6 +242,65 @@ def bench_prefill_c3(args, dev) -> int:
     return 0
 
 
+def bench_engine(args, dev) -> int:
+    """The engine loop on a Qwen2.5-0.5B-shaped model with random weights (24 layers, 14 query / 2 kv heads of
+    64, vocabulary 151 936, bf16): 8 prompts of 512 tokens, 16 rollouts each, 64 new tokens per rollout at
+    temperature 1.  One step = one whole ``generate`` call.  Timed for the paged path (radix allocator: the
+    rollouts of a prompt share its prefix blocks) and, beside it, for the reference engine's own design, the
+    cache-less loop that recomputes every sequence each step (engine.py:218-250), through the same model."""
+    from research_amd.inference import (CacheConfig, EngineConfig, HipPagedAttentionBackend, InferenceEngine,
+                                        ModelConfig, PagedLlama, SamplingParams)
+
+    cfg = ModelConfig(vocab_size=151936, hidden_size=896, intermediate_size=4864, num_layers=24, num_heads=14,
+                      num_kv_heads=2, head_dim=64, rope_theta=1e6, rms_norm_eps=1e-6, max_position_embeddings=2048,
+                      tie_word_embeddings=True, attention_bias=True)
+    n_prompts, n_rollouts, prompt_len, new_tokens = 8, 16, 512, 64
+    g = torch.Generator().manual_seed(7)
+    prompts = [torch.randint(0, cfg.vocab_size, (prompt_len,), generator=g).tolist() for _ in range(n_prompts)]
+    batch = [p for p in prompts for _ in range(n_rollouts)]
+    params = SamplingParams(temperature=1.0, max_tokens=new_tokens)
+    backend = HipPagedAttentionBackend(CacheConfig(
+        num_layers=cfg.num_layers, num_kv_heads=cfg.num_kv_heads, head_dim=cfg.head_dim, num_blocks=8192,
+        block_size=16, device="cuda", dtype=torch.bfloat16))
+    torch.manual_seed(0)
+    model = PagedLlama(cfg, backend).to(torch.bfloat16).to(dev).eval()
+
+    def run(cache_type, reps):
+        engine = InferenceEngine(EngineConfig(model_path="", cache_type=cache_type, block_size=16,
+                                              max_batch_size=len(batch), max_model_len=2048, num_kv_blocks=8192),
+                                 model=model)
+        times = []
+        for _ in range(reps):
+            engine.flush_cache()
+            torch.manual_seed(1)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            samples = engine.generate(batch, params)
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t0)
+            assert len(samples) == len(batch) and all(len(s.completion_tokens) == new_tokens for s in samples)
+        return times
+
+    run("radix", max(1, args.warmup // 5))  # untimed
+    paged = run("radix", max(1, args.steps // 10))
+    recompute = run("none", 1)
+    n_new = len(batch) * new_tokens
+    best = min(paged)
+    result = {
+        "metric": "engine generated tokens/s", "value": n_new / best, "unit": "tokens/s", "n_gpus": 1,
+        "steps": len(paged), "warmup": max(1, args.warmup // 5), "ms_per_step": 1e3 * best,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "engine: Qwen2.5-0.5B-shaped model, 8 prompts x 16 rollouts, 512 + 64 tokens",
+                   "cache_type": "radix", "block_size": 16, "sequences": len(batch), "prompt_len": prompt_len,
+                   "new_tokens": new_tokens, "all_ms": [round(1e3 * t, 1) for t in paged]},
+        "recompute_loop": {"tokens_per_s": n_new / recompute[0], "ms": 1e3 * recompute[0],
+                           "note": "cache_type none: the reference engine's cache-less loop through the same model"},
+        "speedup_over_recompute": recompute[0] / best,
+    }
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     args = parse_args()
     if args.gpus != 1:
@@ -258,6 +317,8 @@ def main() -> int:
     torch.cuda.set_device(dev)
     if args.workload == "c3":
         return bench_prefill_c3(args, dev)
+    if args.workload == "engine":
+        return bench_engine(args, dev)
 
     t_gen = time.perf_counter()
     w = make_decode(args.workload)

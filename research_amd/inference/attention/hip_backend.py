@@ -38,7 +38,7 @@ Differences from the reference, all deliberate:
 from __future__ import annotations
 
 from collections import OrderedDict
-from typing import Optional, Sequence, Tuple
+from typing import List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -91,6 +91,7 @@ class HipPagedAttentionBackend:
         self._mask_cache: dict = {}
         self._step_cache: "OrderedDict[int, _StepTensors]" = OrderedDict()
         self._workspace: Optional[Tensor] = None
+        self._retired_workspaces: List[Tensor] = []
 
         if config.kv_format not in (None, "fp8_e4m3"):
             raise ValueError(f"unknown kv_format {config.kv_format!r}")
@@ -284,8 +285,16 @@ class HipPagedAttentionBackend:
         return np.asarray(values, dtype=np.int64)[:batch]
 
     def _workspace_for(self, nbytes: int) -> Tensor:
+        """The decode workspace, grown on demand.  A buffer that has been handed out is never released while the
+        backend lives: a captured graph of a decode step keeps replaying with the address it was recorded with,
+        so an outgrown buffer is retired, not freed (growth at least doubles, which bounds what is retained)."""
         if self._workspace is None or self._workspace.numel() < nbytes:
-            self._workspace = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=self.k_cache.device)
+            have = 0
+            if self._workspace is not None:
+                have = self._workspace.numel()
+                self._retired_workspaces.append(self._workspace)
+            self._workspace = torch.empty(max(nbytes, 2 * have, 1 << 20), dtype=torch.uint8,
+                                          device=self.k_cache.device)
         return self._workspace
 
     def _layer(self, layer_idx: int) -> Tuple[Tensor, Tensor]:
@@ -382,11 +391,16 @@ class HipPagedAttentionBackend:
         self._require_device(q, self.k_cache)
         step = self._step(ctx)
         if step.seq_lens is None:
-            lens = self._lens(ctx.seq_lens, batch)
             self._tables(step, ctx.block_tables[:batch])
-            step.seq_lens = self._to_device(lens.astype(np.int32))
-            if self.pad_zero_keys and batch > 0:
-                step.extra_zero = self._to_device((lens.max() - lens).astype(np.int32))
+            if isinstance(ctx.seq_lens, Tensor) and ctx.seq_lens.device.type == "cuda" and not self.pad_zero_keys:
+                # already on the device: used as it is, with no host copy (a caller replaying a captured graph
+                # updates the tensor in place between replays)
+                step.seq_lens = ctx.seq_lens[:batch].to(torch.int32).contiguous()
+            else:
+                lens = self._lens(ctx.seq_lens, batch)
+                step.seq_lens = self._to_device(lens.astype(np.int32))
+                if self.pad_zero_keys and batch > 0:
+                    step.extra_zero = self._to_device((lens.max() - lens).astype(np.int32))
         q3 = q.contiguous().view(batch, num_heads, head_dim)
         ws = self._workspace_for(
             ops.decode_workspace_bytes(batch, num_heads, cfg.num_kv_heads, head_dim, self.k_cache.dtype))

@@ -23,7 +23,7 @@ scheduler a made-up block count (engine.py:147) and ``flush_cache`` is empty
 
 from __future__ import annotations
 
-from typing import List, Optional, Tuple
+from typing import Dict, List, Optional, Tuple
 
 import numpy as np
 import torch
@@ -36,6 +36,62 @@ from .sampling import sample_with_logprobs
 from .scheduler import schedule
 from .types import (EngineConfig, InferenceContext, SamplingParams, SchedulerConfig, Sequence, SequenceStatus,
                     TrainingSample)
+
+
+class _DecodeGraph:
+    """One captured forward pass of the decode step for a fixed (padded) batch size.
+
+    Every kernel of the step reads its per-step integers (token ids, positions, slots, block tables, lengths)
+    from device memory and none allocates or synchronises, so the launch sequence does not depend on their
+    values: it is recorded once and replayed with the buffers rewritten in place.  Sampling stays outside."""
+
+    def __init__(self, model: PagedLlama, batch: int, table_width: int, device: torch.device) -> None:
+        self.batch, self.width = batch, table_width
+        self.ids = torch.zeros((batch, 1), dtype=torch.int64, device=device)
+        self.pos = torch.zeros((batch, 1), dtype=torch.int64, device=device)
+        self.slots = torch.full((batch,), -1, dtype=torch.int64, device=device)
+        self.tables = torch.full((batch, table_width), -1, dtype=torch.int32, device=device)
+        self.lens = torch.zeros((batch,), dtype=torch.int32, device=device)
+        self.ctx = InferenceContext(is_prefill=False, slot_mapping=self.slots, block_tables=self.tables,
+                                    seq_lens=self.lens, max_seq_len=table_width)
+        # host staging, one copy per field and step
+        self._h_ids = np.zeros((batch, 1), dtype=np.int64)
+        self._h_pos = np.zeros((batch, 1), dtype=np.int64)
+        self._h_slots = np.full((batch,), -1, dtype=np.int64)
+        self._h_tables = np.full((batch, table_width), -1, dtype=np.int32)
+        self._h_lens = np.zeros((batch,), dtype=np.int32)
+        # one eager pass on a side stream first (workspaces, rotary tables and library handles come into being
+        # outside the capture); all rows are padding, so it writes nothing to the pool
+        side = torch.cuda.Stream(device=device)
+        side.wait_stream(torch.cuda.current_stream(device))
+        with torch.cuda.stream(side), torch.no_grad():
+            model(self.ids, self.pos, self.ctx)
+        torch.cuda.current_stream(device).wait_stream(side)
+        torch.cuda.synchronize(device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.no_grad(), torch.cuda.graph(self.graph):
+            self.hidden = model(self.ids, self.pos, self.ctx)
+
+    def run(self, ids: np.ndarray, last_pos: np.ndarray, slots: np.ndarray, tables: np.ndarray,
+            lens: np.ndarray) -> torch.Tensor:
+        n = len(ids)
+        if tables.shape[1] > self.width:
+            raise ValueError(f"a block table of {tables.shape[1]} entries exceeds max_model_len / block_size = {self.width}")
+        self._h_ids[:n] = ids
+        self._h_ids[n:] = 0
+        self._h_pos[:n, 0] = last_pos
+        self._h_pos[n:] = 0
+        self._h_slots[:n] = slots
+        self._h_slots[n:] = -1
+        self._h_tables.fill(-1)
+        self._h_tables[:n, : tables.shape[1]] = tables
+        self._h_lens[:n] = lens
+        self._h_lens[n:] = 0
+        for dst, src in ((self.ids, self._h_ids), (self.pos, self._h_pos), (self.slots, self._h_slots),
+                         (self.tables, self._h_tables), (self.lens, self._h_lens)):
+            dst.copy_(torch.from_numpy(src))
+        self.graph.replay()
+        return self.hidden
 
 
 class InferenceEngine:
@@ -64,6 +120,7 @@ class InferenceEngine:
         self.seq_counter = 0
         self.weight_version = 0
         self.num_preemptions = 0
+        self._decode_graphs: Dict[int, "_DecodeGraph"] = {}
 
     # ------------------------------------------------------------------ construction
     def _load_model(self, model_path: str) -> nn.Module:
@@ -255,9 +312,28 @@ class InferenceEngine:
         slots = np.asarray([s.block_ids[p // bs] * bs + p % bs for s, p in zip(seqs, last_pos)], dtype=np.int64)
         ctx = InferenceContext(is_prefill=False, slot_mapping=slots, block_tables=self._tables(seqs), seq_lens=lens,
                                max_seq_len=int(lens.max()))
-        hidden = self.model(torch.from_numpy(ids).to(self.device),
-                            torch.from_numpy(last_pos[:, None].copy()).to(self.device), ctx)
+        if self.config.use_graphs:
+            hidden = self._decode_replay(ids, last_pos, slots, ctx.block_tables, lens)
+        else:
+            hidden = self.model(torch.from_numpy(ids).to(self.device),
+                                torch.from_numpy(last_pos[:, None].copy()).to(self.device), ctx)
         return self._sample(seqs, hidden[:, 0])
+
+    def _decode_replay(self, ids: np.ndarray, last_pos: np.ndarray, slots: np.ndarray, tables: np.ndarray,
+                       lens: np.ndarray) -> torch.Tensor:
+        """The decode step's forward pass from a captured graph.  Batches are padded to a bucket size with
+        sequences of length 0 and slot -1 (nothing is written, their rows are ignored); the graph reads token
+        ids, positions, slots, block tables and lengths from buffers that are rewritten before every replay."""
+        n = len(ids)
+        bucket = 8
+        while bucket < n:
+            bucket *= 2
+        bucket = min(bucket, max(self.config.max_batch_size, n))
+        g = self._decode_graphs.get(bucket)
+        if g is None:
+            width = -(-self.config.max_model_len // self.config.block_size)
+            g = self._decode_graphs[bucket] = _DecodeGraph(self.model, bucket, width, self.device)
+        return g.run(ids, last_pos, slots, tables, lens)[:n]
 
     def _recompute(self, seqs: List[Sequence]) -> List[Sequence]:
         """The reference's cache-less step: every sequence's whole token list, one at a time (engine.py:218-250)."""

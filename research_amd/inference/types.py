@@ -54,7 +54,9 @@ class EngineConfig:
     """Engine configuration (types.py:14-24).  ``model_path`` names a local directory with ``config.json`` and
     safetensors weights, or is ignored when the engine is handed a model object.  Added, optional:
     ``num_kv_blocks`` (pool size; default: enough for ``max_batch_size`` sequences of ``max_model_len`` tokens,
-    capped at 65 536 blocks), ``eos_token_id`` (used when there is no tokenizer)."""
+    capped at 65 536 blocks), ``eos_token_id`` (used when there is no tokenizer), ``use_graphs`` (replay the
+    decode step's forward pass from a captured HIP graph per batch-size bucket instead of launching it kernel by
+    kernel)."""
 
     model_path: str
     cache_type: str = "none"  # "paged" | "radix" | "none"
@@ -65,6 +67,7 @@ class EngineConfig:
     tensor_parallel_size: int = 1
     num_kv_blocks: Optional[int] = None
     eos_token_id: Optional[int] = None
+    use_graphs: bool = False
 
 
 @dataclass(frozen=True)

@@ -16,14 +16,14 @@ CFG = ModelConfig(vocab_size=211, hidden_size=128, intermediate_size=256, num_la
                   head_dim=32, max_position_embeddings=512)
 
 
-def _engine(dtype, cache_type, num_blocks, block_size=16, seed=0, max_batch_size=8, eos=None):
+def _engine(dtype, cache_type, num_blocks, block_size=16, seed=0, max_batch_size=8, eos=None, use_graphs=False):
     backend = HipPagedAttentionBackend(CacheConfig(
         num_layers=CFG.num_layers, num_kv_heads=CFG.num_kv_heads, head_dim=CFG.head_dim, num_blocks=num_blocks,
         block_size=block_size, device="cuda", dtype=dtype))
     torch.manual_seed(seed)
     model = PagedLlama(CFG, backend).to(dtype).cuda().eval()
     config = EngineConfig(model_path="", cache_type=cache_type, block_size=block_size, max_batch_size=max_batch_size,
-                          max_model_len=512, eos_token_id=eos)
+                          max_model_len=512, eos_token_id=eos, use_graphs=use_graphs)
     engine = InferenceEngine(config, model=model)
     weights = {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
     return engine, weights
@@ -97,6 +97,51 @@ def test_preemption_is_transparent():
     with pytest.raises(RuntimeError, match="cannot hold"):
         engine.generate([list(range(100))], SamplingParams(temperature=0.0, max_tokens=2))
     engine.shutdown()
+
+
+def test_decode_from_captured_graphs():
+    """use_graphs: every decode step replays one captured forward pass (per batch-size bucket) with its integer
+    inputs rewritten in place; prefills, sampling and allocator work run eagerly between the replays.  Tokens
+    must equal the full-recompute loop on every step, for batches of different sizes and paddings, through
+    preemption, and after a weight update (the graph reads the parameters in place)."""
+    announce("engine graphs")
+    engine, weights = _engine(torch.float32, "radix", num_blocks=64, use_graphs=True, max_batch_size=16)
+    prompts = _prompts()
+    g = torch.Generator().manual_seed(21)
+    more = prompts + [torch.randint(0, 211, (n,), generator=g).tolist() for n in (3, 17, 33, 40, 9)]
+    for batch, max_tokens in ((prompts, 20), (prompts[:3], 9), (more, 12)):  # buckets of 8, 8 and 16 rows
+        with torch.no_grad():
+            want = mo.generate_recompute(weights, CFG, batch, max_tokens=max_tokens)
+        got = _by_prompt(engine.generate(batch, SamplingParams(temperature=0.0, max_tokens=max_tokens)))
+        for prompt, (tokens, logprobs, _) in zip(batch, want):
+            for sample in got[tuple(prompt)]:
+                assert list(sample.completion_tokens) == tokens
+                assert sample.logprobs == pytest.approx(logprobs, abs=2e-4)
+    assert sorted(engine._decode_graphs) == [8, 16]
+    # new weights are read by the same graphs
+    torch.manual_seed(3)
+    fresh = PagedLlama(CFG, engine.backend).float()
+    state = {k: v.cuda() for k, v in fresh.state_dict().items()}
+    engine.update_weights(state)
+    engine.flush_cache()
+    new_weights = {k: v.float().cpu() for k, v in state.items()}
+    with torch.no_grad():
+        want = mo.generate_recompute(new_weights, CFG, prompts[:4], max_tokens=10)
+    got = _by_prompt(engine.generate(prompts[:4], SamplingParams(temperature=0.0, max_tokens=10)))
+    for prompt, (tokens, _, _) in zip(prompts[:4], want):
+        for sample in got[tuple(prompt)]:
+            assert list(sample.completion_tokens) == tokens
+    # a pool too small for all sequences at once: preemption between replays
+    engine2, weights2 = _engine(torch.float32, "radix", num_blocks=11, block_size=8, use_graphs=True)
+    g = torch.Generator().manual_seed(12)
+    small = [torch.randint(0, 211, (15,), generator=g).tolist() for _ in range(4)]
+    with torch.no_grad():
+        want = mo.generate_recompute(weights2, CFG, small, max_tokens=30)
+    got = _by_prompt(engine2.generate(small, SamplingParams(temperature=0.0, max_tokens=30)))
+    assert engine2.num_preemptions > 0
+    for prompt, (tokens, _, _) in zip(small, want):
+        (sample,) = got[tuple(prompt)]
+        assert list(sample.completion_tokens) == tokens
 
 
 def test_bf16_generation_and_weight_update():
