@@ -314,38 +314,85 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
 // Merge the kWaves*TPW row-group partials of every (kv head of the group,
 // query head r) through LDS and hand (qh, d, num, M, den) of the merged
 // partial to `emit`; out = num/den, M is the base-2 running maximum.
+//
+// The waves' lanes hold ROWS = kWaves*RPW partial rows per query head; rows
+// with the same row % hpw belong to the same kv head and are merged.  HR query
+// heads go through LDS per round (as many as the LDS budget allows): every
+// lane writes its accumulators, then one thread per (head, row) computes the
+// row's weight exp2(m_row - M) (and, for the first row of each kv head, M and
+// the merged denominator), then one thread per (head, kv head, d) sums
+// weight * accumulator over the rows.  The row loops are unrolled by 4 (the
+// row count per kv head is kWaves*tpw, a multiple of 4) so that their LDS
+// reads overlap.
+template <typename KV, int D, int NREP> struct MergeShape {
+    static constexpr int ROWS = kWaves * RowShape<KV, D>::RPW;
+    static constexpr int ROWF = D + 2;  // floats of a partial row: D accumulators, m, l
+    static constexpr int kBudget = 28 * 1024;
+    static constexpr int per_head = ROWS * (ROWF + 3) * 4;  // bytes: rows + (weight, M, den) per row
+    static constexpr int HR = NREP >= 8 && 8 * per_head <= kBudget   ? 8
+                              : NREP >= 4 && 4 * per_head <= kBudget ? 4
+                              : NREP >= 2 && 2 * per_head <= kBudget ? 2
+                                                                     : 1;
+    static constexpr int AUX = HR * ROWS * ROWF;   // float offset of the weights
+    static constexpr int FLOATS = HR * ROWS * (ROWF + 3);
+};
+
 template <typename KV, int D, int NREP, typename Emit>
-__device__ __forceinline__ void merge_rows(RowState<NREP, RowShape<KV, D>::EPL> &st,
-                                           float (*s_part)[D + 2], const PoolArgs &p, const LaneRole &role,
-                                           int wave, int tid, int hg, int rep0, Emit emit) {
+__device__ __forceinline__ void merge_rows(RowState<NREP, RowShape<KV, D>::EPL> &st, float *s_part,
+                                           const PoolArgs &p, const LaneRole &role, int wave, int tid, int hg,
+                                           int rep0, Emit emit) {
     using S = RowShape<KV, D>;
+    using MS = MergeShape<KV, D, NREP>;
+    constexpr int ROWS = MS::ROWS, ROWF = MS::ROWF, HR = MS::HR;
     st.fold_zero_keys();
     const int prow = wave * S::RPW + role.row;  // = wave*RPW + tok_local*hpw + head_local
+    float *s_wgt = s_part + MS::AUX, *s_M = s_wgt + HR * ROWS, *s_den = s_M + HR * ROWS;
+    const int hpw = p.hpw;  // a power of two dividing RPW
+    const int lg_hpw = __builtin_ctz(hpw);
 #pragma unroll
-    for (int r = 0; r < NREP; ++r) {
-        if (rep0 + r >= p.n_rep) break;  // uniform over the workgroup
-        __syncthreads();
+    for (int round = 0; round < NREP / HR; ++round) {
+        if (rep0 + round * HR >= p.n_rep) break;  // uniform over the workgroup
+        __syncthreads();  // the readers of the previous round (or of the previous call) are done
 #pragma unroll
-        for (int e = 0; e < S::EPL; ++e) s_part[prow][role.d0 + e] = st.acc[r][e];
-        if (role.lir == 0) {
-            s_part[prow][D] = st.m[r];
-            s_part[prow][D + 1] = st.l[r];
+        for (int h = 0; h < HR; ++h) {
+            float *row = s_part + (h * ROWS + prow) * ROWF;
+#pragma unroll
+            for (int e = 0; e < S::EPL; ++e) row[role.d0 + e] = st.acc[round * HR + h][e];
+            if (role.lir == 0) {
+                row[D] = st.m[round * HR + h];
+                row[D + 1] = st.l[round * HR + h];
+            }
         }
         __syncthreads();
-        for (int o = tid; o < p.hpw * D; o += kThreads) {
-            const int hl = o / D, d = o - hl * D;
+        for (int idx = tid; idx < HR * ROWS; idx += kThreads) {
+            const int h = idx / ROWS, row = idx - h * ROWS;
+            const int hl = row & (hpw - 1);
+            const float *base = s_part + h * ROWS * ROWF;
             float M = kNegBig;
-            for (int w = 0; w < kWaves; ++w)
-                for (int t = 0; t < p.tpw; ++t) M = fmaxf(M, s_part[w * S::RPW + t * p.hpw + hl][D]);
-            float num = 0.f, den = 0.f;
-            for (int w = 0; w < kWaves; ++w)
-                for (int t = 0; t < p.tpw; ++t) {
-                    const float *pr = s_part[w * S::RPW + t * p.hpw + hl];
-                    const float wgt = __builtin_amdgcn_exp2f(pr[D] - M);
-                    num = fmaf(wgt, pr[d], num);
-                    den = fmaf(wgt, pr[D + 1], den);
-                }
-            emit((hg * p.hpw + hl) * p.n_rep + rep0 + r, d, num, M, den);
+#pragma unroll 4
+            for (int r2 = hl; r2 < ROWS; r2 += hpw) M = fmaxf(M, base[r2 * ROWF + D]);
+            s_wgt[idx] = __builtin_amdgcn_exp2f(base[row * ROWF + D] - M);
+            if (row < hpw) {  // first row of its kv head: the merged maximum and denominator
+                float den = 0.f;
+#pragma unroll 4
+                for (int r2 = hl; r2 < ROWS; r2 += hpw)
+                    den = fmaf(__builtin_amdgcn_exp2f(base[r2 * ROWF + D] - M), base[r2 * ROWF + D + 1], den);
+                s_M[idx] = M;
+                s_den[idx] = den;
+            }
+        }
+        __syncthreads();
+        for (int o = tid; o < HR * hpw * D; o += kThreads) {
+            const int d = o & (D - 1), hd = o / D;
+            const int hl = hd & (hpw - 1), h = hd >> lg_hpw;
+            const int r = round * HR + h;
+            if (rep0 + r >= p.n_rep) continue;
+            const float *base = s_part + h * ROWS * ROWF + d;
+            const float *wgt = s_wgt + h * ROWS;
+            float num = 0.f;
+#pragma unroll 4
+            for (int r2 = hl; r2 < ROWS; r2 += hpw) num = fmaf(wgt[r2], base[r2 * ROWF], num);
+            emit((hg * hpw + hl) * p.n_rep + rep0 + r, d, num, s_M[h * ROWS + hl], s_den[h * ROWS + hl]);
         }
     }
     __syncthreads();
@@ -393,7 +440,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
     using S = RowShape<KV, D>;
     extern __shared__ int s_prefix[];  // batch + 1 entries: blocks before each sequence
     __shared__ int s_scan[kThreads];
-    __shared__ float s_part[kWaves * S::RPW][D + 2];
+    __shared__ float s_part[MergeShape<KV, D, NREP>::FLOATS];
 
     const PoolArgs &p = a.p;
     const int tid = threadIdx.x;
@@ -668,7 +715,7 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_wave_kernel(const Deco
 template <typename KV, typename QT, int D, int NREP, int U>
 __global__ __launch_bounds__(kThreads) void prefill_rowwise_kernel(const RowwiseArgs a) {
     using S = RowShape<KV, D>;
-    __shared__ float s_part[kWaves * S::RPW][D + 2];
+    __shared__ float s_part[MergeShape<KV, D, NREP>::FLOATS];
     const PoolArgs &p = a.p;
     const int tid = threadIdx.x;
     const int lane = tid & (PA_WAVE - 1);
