@@ -108,6 +108,9 @@ class InferenceEngine:
             config.max_batch_size, config.max_model_len, config.block_size)
         self.model = model if model is not None else self._load_model(config.model_path)
         self.backend = self.model.backend
+        if config.use_graphs and getattr(self.backend.config, "kv_format", None) == "fp8_e4m3":
+            # the fp8 append works per touched block, and the set of touched blocks has a data-dependent size
+            raise ValueError("use_graphs needs a bf16 / fp16 / fp32 KV pool: the fp8 append is not capturable")
         self.tokenizer = tokenizer if tokenizer is not None else self._load_tokenizer(config.model_path)
         self.scheduler_config = SchedulerConfig(
             max_batch_size=config.max_batch_size,

@@ -160,3 +160,24 @@ def test_attention_layer_delegates():
     x = torch.zeros(1)
     assert layer(x, x, x, ctx) is x and calls == [(3, ctx)]
     assert list(layer.parameters()) == []
+
+
+def test_gather_output_arguments_are_checked_before_any_launch():
+    """kv_gather(out=...) validates shape, type and layout on the host; nothing is launched for a bad pair."""
+    from research_amd import ops
+
+    pool = torch.zeros((32, 2, 8), dtype=torch.float32)
+    tables = torch.zeros((2, 2), dtype=torch.int32)
+    lens = torch.tensor([5, 7], dtype=torch.int32)
+    good = torch.empty((2, 7, 2, 8), dtype=torch.float32)
+    for bad in (torch.empty((2, 6, 2, 8)), torch.empty((2, 7, 2, 8), dtype=torch.float16),
+                torch.empty((2, 7, 8, 2)).transpose(2, 3)):
+        with pytest.raises(ValueError, match="out tensors"):
+            ops.kv_gather(pool, pool, tables, lens, 7, 16, out=(good, bad))
+
+
+def test_engine_config_defaults():
+    from research_amd.inference import EngineConfig
+
+    cfg = EngineConfig(model_path="x")
+    assert cfg.cache_type == "none" and cfg.block_size == 16 and cfg.use_graphs is False  # types.py:14-24 + added

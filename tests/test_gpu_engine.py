@@ -144,6 +144,15 @@ def test_decode_from_captured_graphs():
         assert list(sample.completion_tokens) == tokens
 
 
+def test_graphs_refuse_an_fp8_pool():
+    backend = HipPagedAttentionBackend(CacheConfig(
+        num_layers=CFG.num_layers, num_kv_heads=CFG.num_kv_heads, head_dim=CFG.head_dim, num_blocks=16,
+        block_size=16, device="cuda", dtype=torch.bfloat16, kv_format="fp8_e4m3"))
+    model = PagedLlama(CFG, backend).to(torch.bfloat16).cuda().eval()
+    with pytest.raises(ValueError, match="use_graphs"):
+        InferenceEngine(EngineConfig(model_path="", cache_type="radix", use_graphs=True, max_model_len=512), model=model)
+
+
 def test_bf16_generation_and_weight_update():
     announce("engine bf16, update_weights, flush_cache")
     engine, weights = _engine(torch.bfloat16, "radix", num_blocks=64, seed=1)
