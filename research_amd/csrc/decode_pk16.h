@@ -37,6 +37,13 @@ template <> struct Pk16<pa_bf16> {
     static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
         return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
     }
+    // a.b with no addend: the three-operand encoding with the constant 0 (the compiler's choice for dot2 with a
+    // zero addend is the accumulating encoding behind a v_mov of 0: one more instruction per chain)
+    static __device__ __forceinline__ float dot2_first(uint32_t a, uint32_t b) {
+        float d;
+        asm("v_dot2_f32_bf16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+        return d;
+    }
     static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
         v2 r = {(__bf16)lo, (__bf16)hi};
         return __builtin_bit_cast(uint32_t, r);
@@ -46,6 +53,11 @@ template <> struct Pk16<pa_f16> {
     typedef _Float16 v2 __attribute__((ext_vector_type(2)));
     static __device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
         return __builtin_amdgcn_fdot2(__builtin_bit_cast(v2, a), __builtin_bit_cast(v2, b), c, false);
+    }
+    static __device__ __forceinline__ float dot2_first(uint32_t a, uint32_t b) {
+        float d;
+        asm("v_dot2_f32_f16 %0, %1, %2, 0" : "=v"(d) : "v"(a), "v"(b));
+        return d;
     }
     static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
         v2 r = {(_Float16)lo, (_Float16)hi};
@@ -259,7 +271,7 @@ __device__ __forceinline__ void attend_blocks_pk(
                 float s[NREP];
 #pragma unroll
                 for (int r = 0; r < NREP; ++r) {
-                    float d = PK::dot2(kw[0], qpk[r][0], 0.f);
+                    float d = PK::dot2_first(kw[0], qpk[r][0]);
 #pragma unroll
                     for (int i = 1; i < NW; ++i) d = PK::dot2(kw[i], qpk[r][i], d);
                     s[r] = d;
@@ -267,7 +279,13 @@ __device__ __forceinline__ void attend_blocks_pk(
                 HS::reduce(s, sv[u], lane);
 #pragma unroll
                 for (int j = 0; j < VPL; ++j) sv[u][j] *= k_sc;
-                if (partial) {
+            }
+            if (partial) {
+                // kept a branch (the empty statement stops the compiler from turning it into selects that every
+                // step would execute): only the first and last block of a sequence have tokens to mask
+                asm volatile("");
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
                     const int tt = t0 + u * p.tpw + tok_local;
                     const bool ok = tt < ntok && tt >= tlo;
 #pragma unroll
@@ -410,7 +428,7 @@ __device__ __forceinline__ void attend_blocks_pk_multi(
             float s[NREP];
 #pragma unroll
             for (int r = 0; r < NREP; ++r) {
-                float d = PK::dot2(kw[0], qpk[r][0], 0.f);
+                float d = PK::dot2_first(kw[0], qpk[r][0]);
 #pragma unroll
                 for (int i = 1; i < NW; ++i) d = PK::dot2(kw[i], qpk[r][i], d);
                 s[r] = d;
