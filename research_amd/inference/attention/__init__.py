@@ -7,24 +7,11 @@ that ``from ...attention import CacheConfig, FlexAttentionBackend`` keeps workin
 from .config import CacheConfig
 from .hip_backend import FlexAttentionBackend, HipPagedAttentionBackend
 from .layer import Attention
-from .mask import (
-    PagedMask,
-    create_attention_mask,
-    create_causal_block_mask,
-    create_document_mask,
-    create_sliding_window_causal_mask,
-)
+from .mask import (PagedMask, create_attention_mask, create_causal_block_mask, create_document_mask,
+                   create_sliding_window_causal_mask)
 from .protocol import AttentionBackend
 
-__all__ = [
-    "CacheConfig",
-    "AttentionBackend",
-    "HipPagedAttentionBackend",
-    "FlexAttentionBackend",
-    "Attention",
-    "PagedMask",
-    "create_attention_mask",
-    "create_causal_block_mask",
-    "create_sliding_window_causal_mask",
-    "create_document_mask",
-]
+_BACKEND = ("Attention", "AttentionBackend", "CacheConfig", "FlexAttentionBackend", "HipPagedAttentionBackend")
+_MASKS = ("PagedMask", "create_attention_mask", "create_causal_block_mask", "create_document_mask",
+          "create_sliding_window_causal_mask")
+__all__ = [*_BACKEND, *_MASKS]
