@@ -276,7 +276,6 @@ class InferenceEngine:
         return tables
 
     def _prefill(self, seqs: List[Sequence]) -> List[Sequence]:
-        bs = self.config.block_size
         cached, chunks = [], []
         for s in seqs:
             s.block_ids = list(self.cache.allocate(s.seq_id, s.token_ids))
@@ -284,6 +283,27 @@ class InferenceEngine:
             c = min(self.cache.get_cached_tokens(s.seq_id), n - 1)  # the last token is always computed: its
             cached.append(c)                                         # hidden state gives the next token
             chunks.append(n - c)
+        # One batched forward pads every row to the longest chunk.  N rollouts of one prompt arrive as one row
+        # with the whole prompt and N-1 rows with a single uncached token, so the rows are split in two passes
+        # when that removes most of the padding: first the rows with no cached prefix (they depend on nothing
+        # and write the blocks that later rows share), then the rows with one (their prefix blocks were written
+        # in an earlier step, by the first pass, or by an earlier row of their own pass, whose append precedes
+        # the attention inside every layer).
+        cold = [i for i, c in enumerate(cached) if c == 0]
+        warm = [i for i, c in enumerate(cached) if c > 0]
+        groups = [list(range(len(seqs)))]
+        if cold and warm:
+            padded = lambda idx: len(idx) * max(chunks[i] for i in idx)
+            if padded(cold) + padded(warm) <= 0.7 * padded(groups[0]):
+                groups = [cold, warm]
+        finished: List[Sequence] = []
+        for idx in groups:
+            finished += self._prefill_rows([seqs[i] for i in idx], [cached[i] for i in idx],
+                                           [chunks[i] for i in idx])
+        return finished
+
+    def _prefill_rows(self, seqs: List[Sequence], cached: List[int], chunks: List[int]) -> List[Sequence]:
+        bs = self.config.block_size
         t_max = max(chunks)
         ids = np.zeros((len(seqs), t_max), dtype=np.int64)
         pos = np.zeros((len(seqs), t_max), dtype=np.int64)

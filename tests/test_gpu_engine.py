@@ -144,6 +144,30 @@ def test_decode_from_captured_graphs():
         assert list(sample.completion_tokens) == tokens
 
 
+def test_rollouts_of_one_prompt_prefill_in_two_passes():
+    """Rows with no cached prefix and rows with one are prefilled in separate passes when that removes most of
+    the padding (N rollouts of a prompt = one full row + N-1 one-token rows); results are those of the
+    full-recompute loop either way."""
+    announce("engine two-pass prefill")
+    engine, weights = _engine(torch.float32, "radix", num_blocks=64)
+    g = torch.Generator().manual_seed(31)
+    a = torch.randint(0, 211, (64,), generator=g).tolist()
+    b = torch.randint(0, 211, (48,), generator=g).tolist()
+    prompts = [a, a, a, a, b, b, b]
+    calls = []
+    rows = engine._prefill_rows
+    engine._prefill_rows = lambda seqs, cached, chunks: (calls.append((len(seqs), max(chunks))), rows(seqs, cached, chunks))[1]
+    with torch.no_grad():
+        want = mo.generate_recompute(weights, CFG, [a, b], max_tokens=10)
+    got = _by_prompt(engine.generate(prompts, SamplingParams(temperature=0.0, max_tokens=10)))
+    assert calls == [(2, 64), (5, 1)]  # the two first occurrences, then the five rollouts that found their prompt cached
+    for prompt, (tokens, logprobs, _) in zip([a, b], want):
+        assert len(got[tuple(prompt)]) == (4 if prompt is a else 3)
+        for sample in got[tuple(prompt)]:
+            assert list(sample.completion_tokens) == tokens
+            assert sample.logprobs == pytest.approx(logprobs, abs=2e-4)
+
+
 def test_graphs_refuse_an_fp8_pool():
     backend = HipPagedAttentionBackend(CacheConfig(
         num_layers=CFG.num_layers, num_kv_heads=CFG.num_kv_heads, head_dim=CFG.head_dim, num_blocks=16,
