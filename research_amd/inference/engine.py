@@ -244,6 +244,7 @@ class InferenceEngine:
         self.cache = self._new_cache()
 
     def shutdown(self) -> None:
+        self._decode_graphs.clear()
         self.waiting.clear()
         self.running.clear()
         self.cache = self._new_cache()
