@@ -38,6 +38,19 @@ from .types import (EngineConfig, InferenceContext, SamplingParams, SchedulerCon
                     TrainingSample)
 
 
+def prefill_passes(cached: List[int], chunks: List[int]) -> List[List[int]]:
+    """Row indices of a step's prefill, as one pass or two.  Two passes - rows with no cached prefix, then rows
+    with one - when the rows padded to each pass's longest chunk come to at most 70 % of one batch padded to the
+    longest chunk of all; the order inside a pass is the order of admission."""
+    everything = list(range(len(chunks)))
+    cold = [i for i in everything if cached[i] == 0]
+    warm = [i for i in everything if cached[i] > 0]
+    if not cold or not warm:
+        return [everything]
+    padded = lambda idx: len(idx) * max(chunks[i] for i in idx)
+    return [cold, warm] if padded(cold) + padded(warm) <= 0.7 * padded(everything) else [everything]
+
+
 class _DecodeGraph:
     """One captured forward pass of the decode step for a fixed (padded) batch size.
 
@@ -290,15 +303,8 @@ class InferenceEngine:
         # and write the blocks that later rows share), then the rows with one (their prefix blocks were written
         # in an earlier step, by the first pass, or by an earlier row of their own pass, whose append precedes
         # the attention inside every layer).
-        cold = [i for i, c in enumerate(cached) if c == 0]
-        warm = [i for i, c in enumerate(cached) if c > 0]
-        groups = [list(range(len(seqs)))]
-        if cold and warm:
-            padded = lambda idx: len(idx) * max(chunks[i] for i in idx)
-            if padded(cold) + padded(warm) <= 0.7 * padded(groups[0]):
-                groups = [cold, warm]
         finished: List[Sequence] = []
-        for idx in groups:
+        for idx in prefill_passes(cached, chunks):
             finished += self._prefill_rows([seqs[i] for i in idx], [cached[i] for i in idx],
                                            [chunks[i] for i in idx])
         return finished

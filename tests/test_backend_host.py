@@ -181,3 +181,19 @@ def test_engine_config_defaults():
 
     cfg = EngineConfig(model_path="x")
     assert cfg.cache_type == "none" and cfg.block_size == 16 and cfg.use_graphs is False  # types.py:14-24 + added
+
+
+def test_prefill_passes():
+    """Host logic of the engine's prefill: one pass, or uncached rows first and cached rows second."""
+    from research_amd.inference.engine import prefill_passes
+
+    # 2 prompts x 4 rollouts: one full row and three one-token rows each
+    cached = [0, 63, 63, 63, 0, 47, 47, 47]
+    chunks = [64, 1, 1, 1, 48, 1, 1, 1]
+    assert prefill_passes(cached, chunks) == [[0, 4], [1, 2, 3, 5, 6, 7]]
+    # nothing cached, or everything cached: one pass in admission order
+    assert prefill_passes([0, 0, 0], [5, 9, 2]) == [[0, 1, 2]]
+    assert prefill_passes([16, 32], [3, 1]) == [[0, 1]]
+    # splitting would not remove enough padding (chunks of similar length): one pass
+    assert prefill_passes([0, 16, 0, 16], [40, 30, 38, 35]) == [[0, 1, 2, 3]]
+    assert prefill_passes([], []) == [[]]
