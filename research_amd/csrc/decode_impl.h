@@ -312,8 +312,9 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
 };
 
 // Merge the kWaves*TPW row-group partials of every (kv head of the group,
-// query head r) through LDS and hand (qh, d, num, M, den) of the merged
-// partial to `emit`; out = num/den, M is the base-2 running maximum.
+// query head r) through LDS and hand (qh, d, num[4], M, den) of the merged
+// partial - four consecutive d at a time - to `emit`; out = num/den, M is the
+// base-2 running maximum.
 //
 // The waves' lanes hold ROWS = kWaves*RPW partial rows per query head; rows
 // with the same row % hpw belong to the same kv head and are merged.  HR query
@@ -382,16 +383,22 @@ __device__ __forceinline__ void merge_rows(RowState<NREP, RowShape<KV, D>::EPL> 
             }
         }
         __syncthreads();
-        for (int o = tid; o < HR * hpw * D; o += kThreads) {
-            const int d = o & (D - 1), hd = o / D;
+        // four consecutive d per thread: the results leave as one 16-byte store (a part's partial is 8 KB and
+        // more; as single floats its stores were a measurable share of the pass)
+        for (int o = tid; o < HR * hpw * (D / 4); o += kThreads) {
+            const int d = (o & (D / 4 - 1)) * 4, hd = o / (D / 4);
             const int hl = hd & (hpw - 1), h = hd >> lg_hpw;
             const int r = round * HR + h;
             if (rep0 + r >= p.n_rep) continue;
             const float *base = s_part + h * ROWS * ROWF + d;
             const float *wgt = s_wgt + h * ROWS;
-            float num = 0.f;
+            float num[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll 4
-            for (int r2 = hl; r2 < ROWS; r2 += hpw) num = fmaf(wgt[r2], base[r2 * ROWF], num);
+            for (int r2 = hl; r2 < ROWS; r2 += hpw) {
+                const float w = wgt[r2];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) num[j] = fmaf(w, base[r2 * ROWF + j], num[j]);
+            }
             emit((hg * hpw + hl) * p.n_rep + rep0 + r, d, num, s_M[h * ROWS + hl], s_den[h * ROWS + hl]);
         }
     }
@@ -515,8 +522,11 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
             const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
             QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * D;
             merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
-                                    [&](int qh, int d, float num, float M, float den) {
-                                        pa_scalar<QT>::store(orow + (int64_t)qh * D + d, finish_row(num, M, den, ez));
+                                    [&](int qh, int d, const float (&num)[4], float M, float den) {
+#pragma unroll
+                                        for (int j = 0; j < 4; ++j)
+                                            pa_scalar<QT>::store(orow + (int64_t)qh * D + d + j,
+                                                                 finish_row(num[j], M, den, ez));
                                     });
         } else {
             const int64_t slot = (int64_t)blockIdx.x + (int64_t)plane * B + b;
@@ -524,10 +534,11 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
                 float *acc = a.part_acc + slot * (p.hpw * NREP * D);
                 float *ml = a.part_ml + slot * (p.hpw * NREP * 2);
                 merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
-                                        [&](int qh, int d, float num, float M, float den) {
+                                        [&](int qh, int d, const float (&num)[4], float M, float den) {
                                             const int kv = qh / p.n_rep;
                                             const int idx = (kv - hg * p.hpw) * NREP + (qh - kv * p.n_rep - rep0);
-                                            acc[idx * D + d] = num;
+                                            *reinterpret_cast<float4 *>(acc + idx * D + d) =
+                                                float4{num[0], num[1], num[2], num[3]};
                                             if (d == 0) {
                                                 ml[idx * 2] = M;
                                                 ml[idx * 2 + 1] = den;
@@ -741,8 +752,10 @@ __global__ __launch_bounds__(kThreads) void prefill_rowwise_kernel(const Rowwise
         k_lo / p.bs + wave, nblk, kWaves, role, lane, kvh, rep0);
     QT *orow = reinterpret_cast<QT *>(a.out) + qrow * p.hq * D;
     merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
-                            [&](int qh, int d, float num, float M, float den) {
-                                pa_scalar<QT>::store(orow + (int64_t)qh * D + d, den > 0.f ? num / den : 0.f);
+                            [&](int qh, int d, const float (&num)[4], float M, float den) {
+#pragma unroll
+                                for (int j = 0; j < 4; ++j)
+                                    pa_scalar<QT>::store(orow + (int64_t)qh * D + d + j, den > 0.f ? num[j] / den : 0.f);
                             });
 }
 
