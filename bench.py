@@ -30,7 +30,7 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, vendor figure
 # HBM traffic of one launch of the dominant kernel (c4: decode_split_kernel, c3: prefill_mfma_kernel), from
 # rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/); None until measured.
 # c4: fetch 3 447 663 616 + write 7 592 755; c3: fetch 131 099 238 + write 67 108 864 (the output)
-MEASURED_TRAFFIC_BYTES = {"c4": 3455266816, "c3": 197967872}
+MEASURED_TRAFFIC_BYTES = {"c4": 3455306650, "c3": 197967872}
 
 
 def parse_args():
