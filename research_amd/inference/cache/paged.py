@@ -191,7 +191,32 @@ class CountingPagedKVCache(PagedKVCache):
         super().__init__(num_blocks, block_size)
         self.seq_num_tokens: Dict[int, int] = {}
 
+    def blocks_needed(self, token_ids: List[int]) -> int:
+        """Blocks ``allocate(token_ids)`` would take from the free queue: every block of the prompt except the
+        leading ones found cached in blocks that some sequence still holds (a cached block nobody holds sits in
+        the free queue and is taken from there)."""
+        bs = self.block_size
+        n_blocks = self._blocks_for(len(token_ids))
+        chain = _NO_HASH
+        shared = 0
+        for i in range(len(token_ids) // bs):
+            toks = token_ids[i * bs : (i + 1) * bs]
+            chain = compute_block_hash(toks, chain)
+            candidate = self.hash_to_block_id.get(chain, -1)
+            if candidate == -1 or self.blocks[candidate].token_ids != toks:
+                break
+            if candidate in self.used_block_ids:
+                shared += 1
+        return n_blocks - shared
+
     def allocate(self, seq_id: int, token_ids: List[int]) -> Tuple[int, ...]:
+        """All or nothing: the reference's ``allocate`` runs out of blocks half-way (``IndexError`` from the
+        empty free queue, paged.py:150) and leaves the blocks it had taken owned by nobody; here the need is
+        checked first and a call that cannot be served raises before anything changes."""
+        need = self.blocks_needed(token_ids)
+        if need > len(self.free_block_ids):
+            raise RuntimeError(f"No free blocks for sequence {seq_id}: needs {need}, "
+                               f"{len(self.free_block_ids)} free")
         blocks = super().allocate(seq_id, token_ids)
         self.seq_num_tokens[seq_id] = len(token_ids)
         return blocks

@@ -121,6 +121,11 @@ class InferenceEngine:
             config.max_batch_size, config.max_model_len, config.block_size)
         self.model = model if model is not None else self._load_model(config.model_path)
         self.backend = self.model.backend
+        limit = getattr(getattr(self.model, "cfg", None), "max_position_embeddings", None)
+        if limit is not None and config.max_model_len > limit:
+            # the rotary tables end at max_position_embeddings; later positions would all take the last row
+            raise ValueError(f"max_model_len={config.max_model_len} exceeds the model's "
+                             f"max_position_embeddings={limit}")
         if config.use_graphs and getattr(self.backend.config, "kv_format", None) == "fp8_e4m3":
             # the fp8 append works per touched block, and the set of touched blocks has a data-dependent size
             raise ValueError("use_graphs needs a bf16 / fp16 / fp32 KV pool: the fp8 append is not capturable")
@@ -206,7 +211,14 @@ class InferenceEngine:
         """One scheduling decision and the forward passes it asks for; returns the sequences that finished."""
         if not self.has_pending():
             return []
-        free = self.cache.num_free_blocks() if self.cache is not None else 1000000
+        free = 1000000
+        if self.cache is not None:
+            # Decodes run before the prefills of the same step and take a block for every sequence whose new
+            # token starts one: those blocks are not there for the prompts admitted below.
+            bs = self.config.block_size
+            growth = sum(1 for s in self.running[: self.scheduler_config.max_batch_size]
+                         if (len(s.token_ids) - 1) % bs == 0)
+            free = max(0, self.cache.num_free_blocks() - growth)
         out = schedule(self.waiting, self.running, free, self.scheduler_config)
         if self.cache is not None and not out.prefill_seqs and not out.decode_seqs and self.waiting:
             need = -(-len(self.waiting[0].token_ids) // self.config.block_size)
@@ -274,6 +286,16 @@ class InferenceEngine:
             self._preempt(keep.pop())
         return keep
 
+    def _defer(self, seqs: List[Sequence]) -> None:
+        """Sequences admitted for prefill whose blocks could not be had: back to the head of the waiting queue,
+        in their order, untouched."""
+        ids = {s.seq_id for s in seqs}
+        self.running = [s for s in self.running if s.seq_id not in ids]
+        for s in reversed(seqs):
+            s.status = SequenceStatus.WAITING
+            s.block_ids = []
+            self.waiting.insert(0, s)
+
     def _preempt(self, seq: Sequence) -> None:
         self.cache.deallocate(seq.seq_id)
         seq.status = SequenceStatus.WAITING
@@ -291,8 +313,15 @@ class InferenceEngine:
 
     def _prefill(self, seqs: List[Sequence]) -> List[Sequence]:
         cached, chunks = [], []
-        for s in seqs:
-            s.block_ids = list(self.cache.allocate(s.seq_id, s.token_ids))
+        for i, s in enumerate(seqs):
+            try:
+                s.block_ids = list(self.cache.allocate(s.seq_id, s.token_ids))
+            except RuntimeError:
+                # The pool ran short after all (the schedule counts free blocks, not which of them hold a
+                # prefix this prompt will revive): this prompt and the ones admitted after it wait a step.
+                self._defer(seqs[i:])
+                seqs = seqs[:i]
+                break
             n = len(s.token_ids)
             c = min(self.cache.get_cached_tokens(s.seq_id), n - 1)  # the last token is always computed: its
             cached.append(c)                                         # hidden state gives the next token
@@ -304,6 +333,8 @@ class InferenceEngine:
         # in an earlier step, by the first pass, or by an earlier row of their own pass, whose append precedes
         # the attention inside every layer).
         finished: List[Sequence] = []
+        if not seqs:
+            return finished
         for idx in prefill_passes(cached, chunks):
             finished += self._prefill_rows([seqs[i] for i in idx], [cached[i] for i in idx],
                                            [chunks[i] for i in idx])
@@ -332,10 +363,13 @@ class InferenceEngine:
     def _decode(self, seqs: List[Sequence]) -> List[Sequence]:
         if not seqs:
             return []
-        bs = self.config.block_size
         for s in seqs:
             self.cache.append_token(s.seq_id, s.token_ids[-1])  # hands out a block when the token starts one
             s.block_ids = list(self.cache.get_block_ids(s.seq_id))
+        return self._decode_rows(seqs)
+
+    def _decode_rows(self, seqs: List[Sequence]) -> List[Sequence]:
+        bs = self.config.block_size
         lens = np.asarray([len(s.token_ids) for s in seqs], dtype=np.int64)
         last_pos = lens - 1
         ids = np.asarray([[s.token_ids[-1]] for s in seqs], dtype=np.int64)

@@ -177,6 +177,16 @@ def test_graphs_refuse_an_fp8_pool():
         InferenceEngine(EngineConfig(model_path="", cache_type="radix", use_graphs=True, max_model_len=512), model=model)
 
 
+def test_max_model_len_beyond_the_rotary_table_is_refused():
+    backend = HipPagedAttentionBackend(CacheConfig(
+        num_layers=CFG.num_layers, num_kv_heads=CFG.num_kv_heads, head_dim=CFG.head_dim, num_blocks=16,
+        block_size=16, device="cuda", dtype=torch.bfloat16))
+    model = PagedLlama(CFG, backend).to(torch.bfloat16).cuda().eval()
+    with pytest.raises(ValueError, match="max_position_embeddings"):
+        InferenceEngine(EngineConfig(model_path="", cache_type="radix", max_model_len=CFG.max_position_embeddings + 1),
+                        model=model)
+
+
 def test_bf16_generation_and_weight_update():
     announce("engine bf16, update_weights, flush_cache")
     engine, weights = _engine(torch.bfloat16, "radix", num_blocks=64, seed=1)
