@@ -156,6 +156,28 @@ int pa_decode_reduce(const void *q, const void *k_cache, const void *v_cache, vo
                      size_t workspace_bytes, void *stream);
 
 /*
+ * pa_decode without a workspace argument and without any allocation, for callers that cannot allocate device
+ * memory: code under HIP graph capture, serving loops with a fixed memory plan, harnesses that forbid
+ * hipMalloc.  (No counterpart in the reference, which allocates freely inside its decode,
+ * attention/flex_backend.py:253-264.)  The partial results of the split pass go to a scratch array of
+ * PA_DECODE_STATIC_SCRATCH_BYTES that the library's code object holds on every GPU it is loaded on, from load
+ * until the process ends.  Arguments and results are those of pa_decode, bit for bit.
+ *   - Shapes whose partials do not fit return PA_ERR_WORKSPACE (the message gives the bytes needed); the
+ *     need is (workgroups of the split pass + planes * batch) * heads * (head_dim + 2) * 4 bytes, e.g.
+ *     8.5 MB for batch 256, 32 query / 8 kv heads of 128 on a 256-CU device.
+ *   - Every call on one GPU shares that GPU's array, which keeps the previous call's partials: calls whose
+ *     kernels may overlap on one GPU (different streams, different threads) race; order them.
+ *   - The first call on a device asks the runtime for the array's address (hipGetSymbolAddress); make that
+ *     call outside a stream capture.  No call allocates or frees.
+ */
+#define PA_DECODE_STATIC_SCRATCH_BYTES (16u << 20)
+int pa_decode_static(const void *q, const void *k_cache, const void *v_cache, void *out,
+                     const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
+                     const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale, int batch,
+                     int num_q_heads, int num_kv_heads, int head_dim, int block_size, int64_t num_blocks,
+                     float scale, int window, int q_dtype, int kv_dtype, void *stream);
+
+/*
  * Causal prefill attention over a paged context.  Covers both
  * FlexAttentionBackend._prefill_attention (attention/flex_backend.py:144-185,
  * the is_causal SDPA over the step's own K/V) and chunked prefill over cached

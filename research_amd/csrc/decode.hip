@@ -4,7 +4,16 @@
 // decode_inst_*.hip.
 #include <stdlib.h>
 
+#include <mutex>
+
 #include "decode_impl.h"
+
+// Scratch of pa_decode_static: device memory the library itself holds (one copy per GPU, for the life of the
+// process) so that callers which cannot allocate - code under HIP graph capture, serving loops with a fixed
+// memory plan - still get the split pass's partial results somewhere.  In host code this name is only a handle
+// for hipGetSymbolAddress; kernels receive the address that call returns.
+constexpr size_t kStaticScratchBytes = (size_t)PA_DECODE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 
 namespace pa_decode_detail {
 
@@ -53,10 +62,10 @@ struct WsLayout {
     size_t prefix_off, ml_off, acc_off, total;
     int64_t slots;
 };
-WsLayout ws_layout(int batch, const PoolArgs &p, int nrep_t, int d) {
+WsLayout ws_layout(int batch, const PoolArgs &p, int nrep_t, int d, int grid_cap = kMaxSplitGrid) {
     WsLayout w;
     const size_t heads = (size_t)p.hpw * nrep_t;
-    w.slots = (int64_t)kMaxSplitGrid + (int64_t)p.n_hgroups * p.n_rgroups * batch;
+    w.slots = (int64_t)grid_cap + (int64_t)p.n_hgroups * p.n_rgroups * batch;
     w.prefix_off = 0;
     w.ml_off = align_up((size_t)(batch + 1) * 4, 256);
     w.acc_off = w.ml_off + align_up((size_t)w.slots * heads * 2 * 4, 256);
@@ -64,28 +73,50 @@ WsLayout ws_layout(int batch, const PoolArgs &p, int nrep_t, int d) {
     return w;
 }
 
+constexpr int kMaxDevices = 64;
+
+// Compute units of the current device (asked once per device).
 int num_cus() {
-    static int cached = 0;
-    if (cached == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) != hipSuccess ||
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
-            n = 256;
-        cached = n;
+    static int cached[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
     }
-    return cached;
+    return n;
 }
 
-// Workgroups of the split pass per CU.  PA_DECODE_WGS_PER_CU overrides the
-// default (a tuning aid; read once).
-int wgs_per_cu() {
-    static int cached = 0;
-    if (cached == 0) {
-        const char *e = getenv("PA_DECODE_WGS_PER_CU");
-        const int v = e ? atoi(e) : 0;
-        cached = v >= 1 && v <= 16 ? v : 2;
+// Workgroups of the split pass per compute unit: two workgroups of four waves keep two waves on every SIMD,
+// each with the loads of eight token steps in flight.
+constexpr int kSplitWgsPerCu = 2;
+
+int split_grid() {
+    const int grid = num_cus() * kSplitWgsPerCu;
+    return grid > kMaxSplitGrid ? kMaxSplitGrid : grid;
+}
+
+// Address of `scratch` on the current device.  Every GPU holds its own copy of the array at its own address,
+// so the address is asked for once per device, with that device current, and kept.
+int static_scratch(void **ptr) {
+    static void *addr[kMaxDevices];
+    static std::mutex mu;
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return pa_fail(PA_ERR_HIP, "pa_decode_static: hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= kMaxDevices)
+        return pa_fail(PA_ERR_UNSUPPORTED, "pa_decode_static: device index %d above %d", dev, kMaxDevices - 1);
+    std::lock_guard<std::mutex> lock(mu);
+    if (!addr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p)
+            return pa_fail(PA_ERR_HIP, "pa_decode_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+        addr[dev] = p;
     }
-    return cached;
+    *ptr = addr[dev];
+    return PA_OK;
 }
 
 enum { kPhaseSplit = 1, kPhaseReduce = 2 };
@@ -94,7 +125,8 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
                   const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
                   const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale, int batch,
                   int num_q_heads, int num_kv_heads, int head_dim, int block_size, int64_t num_blocks, float scale,
-                  int window, int q_dtype, int kv_dtype, void *workspace, size_t workspace_bytes, void *stream) {
+                  int window, int q_dtype, int kv_dtype, void *workspace, size_t workspace_bytes, void *stream,
+                  bool use_static = false) {
     pa_clear_error();
     PA_REQUIRE(batch >= 0, "batch=%d is negative", batch);
     PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, "head counts / head_dim must be positive");
@@ -121,10 +153,23 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     PA_REQUIRE(kv_dtype != PA_FP8_E4M3 || (k_scale && v_scale), "fp8 KV needs k_scale and v_scale");
     PA_REQUIRE(pa_aligned16(k_cache) && pa_aligned16(v_cache) && pa_aligned16(q),
                "q and cache pointers must be 16-byte aligned");
-    const WsLayout w = ws_layout(batch, a.p, nrep_t, head_dim);
-    if (!workspace || workspace_bytes < w.total)
-        return pa_fail(PA_ERR_WORKSPACE, "pa_decode: workspace of %zu bytes, need %zu", workspace_bytes, w.total);
-    PA_REQUIRE(((uintptr_t)workspace & 255u) == 0, "workspace must be 256-byte aligned");
+    const int grid = split_grid();
+    // A caller's workspace is sized without asking the device (kMaxSplitGrid workgroups); the library's own
+    // scratch is laid out for the grid this device really gets, which is what makes its fixed size go far.
+    const WsLayout w = ws_layout(batch, a.p, nrep_t, head_dim, use_static ? grid : kMaxSplitGrid);
+    if (use_static) {
+        if (w.total > kStaticScratchBytes)
+            return pa_fail(PA_ERR_WORKSPACE,
+                           "pa_decode_static: these shapes need %zu bytes of scratch, the library holds %zu: use "
+                           "pa_decode with a workspace of pa_decode_workspace_bytes()",
+                           w.total, kStaticScratchBytes);
+        const int rc = static_scratch(&workspace);
+        if (rc != PA_OK) return rc;
+    } else {
+        if (!workspace || workspace_bytes < w.total)
+            return pa_fail(PA_ERR_WORKSPACE, "pa_decode: workspace of %zu bytes, need %zu", workspace_bytes, w.total);
+        PA_REQUIRE(((uintptr_t)workspace & 255u) == 0, "workspace must be 256-byte aligned");
+    }
 
     a.p.k = k_cache; a.p.v = v_cache; a.p.bt = block_tables; a.p.bt_stride = bt_stride;
     a.p.k_scale = k_scale; a.p.v_scale = v_scale;
@@ -140,8 +185,6 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     a.part_acc = (float *)(ws + w.acc_off);
 
     hipStream_t s = (hipStream_t)stream;
-    int grid = num_cus() * wgs_per_cu();
-    if (grid > kMaxSplitGrid) grid = kMaxSplitGrid;
     a.split_grid = grid;
     if (phases & kPhaseSplit) {
         ks.split<<<dim3((unsigned)grid), dim3(kThreads), (size_t)(batch + 1) * sizeof(int), s>>>(a);
@@ -192,3 +235,13 @@ extern "C" size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_
 extern "C" int pa_decode(PA_DECODE_PARAMS) { return decode_launch(kPhaseSplit | kPhaseReduce, PA_DECODE_ARGS); }
 extern "C" int pa_decode_split(PA_DECODE_PARAMS) { return decode_launch(kPhaseSplit, PA_DECODE_ARGS); }
 extern "C" int pa_decode_reduce(PA_DECODE_PARAMS) { return decode_launch(kPhaseReduce, PA_DECODE_ARGS); }
+
+extern "C" int pa_decode_static(const void *q, const void *k_cache, const void *v_cache, void *out,
+                                const int32_t *block_tables, int64_t bt_stride, const int32_t *seq_lens,
+                                const int32_t *extra_zero_keys, const float *k_scale, const float *v_scale, int batch,
+                                int num_q_heads, int num_kv_heads, int head_dim, int block_size, int64_t num_blocks,
+                                float scale, int window, int q_dtype, int kv_dtype, void *stream) {
+    return decode_launch(kPhaseSplit | kPhaseReduce, q, k_cache, v_cache, out, block_tables, bt_stride, seq_lens,
+                         extra_zero_keys, k_scale, v_scale, batch, num_q_heads, num_kv_heads, head_dim, block_size,
+                         num_blocks, scale, window, q_dtype, kv_dtype, nullptr, 0, stream, true);
+}

@@ -97,6 +97,23 @@ def decode(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, se
     return out
 
 
+def decode_static(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, seq_lens: Tensor,
+                  block_size: int, scale: float, extra_zero_keys: Optional[Tensor] = None,
+                  k_scale: Optional[Tensor] = None, v_scale: Optional[Tensor] = None, out: Optional[Tensor] = None,
+                  window: int = 0) -> Tensor:
+    """``decode`` through ``pa_decode_static``: the partials go to the library's own fixed scratch array, the
+    call allocates nothing (pass ``out``); shapes beyond the scratch raise ``PagedAttnError``."""
+    batch, hq, d = q.shape
+    total_slots, hkv, _ = k_cache.shape
+    if out is None:
+        out = torch.empty_like(q)
+    _run("pa_decode_static", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_tables),
+         block_tables.shape[1], _ptr(seq_lens), _ptr(extra_zero_keys), _ptr(k_scale), _ptr(v_scale), batch, hq, hkv,
+         d, block_size, total_slots // block_size, float(scale), int(window), PA_DTYPE[q.dtype],
+         PA_DTYPE[k_cache.dtype], _stream(q))
+    return out
+
+
 def prefill_paged(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, ctx_lens: Tensor,
                   q_lens: Tensor, q_starts: Tensor, max_q_len: int, block_size: int, scale: float,
                   out: Optional[Tensor] = None, window: int = 0, row_first_key: Optional[Tensor] = None) -> Tensor:

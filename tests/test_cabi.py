@@ -106,6 +106,19 @@ def test_decode_argument_errors():
     assert _status("pa_decode", *_decode_args(batch=0, q=None, ws=None, ws_bytes=0))[0] == _lib.PA_OK
 
 
+def test_decode_static_argument_errors():
+    """The entry point without a workspace rejects bad arguments, and shapes whose partials exceed the library's
+    fixed scratch array, before it touches a device."""
+    static = lambda **kw: _decode_args(**kw)[:-3] + [None]
+    rc, msg = _status("pa_decode_static", *static(hq=30))
+    assert rc == _lib.PA_ERR_INVALID_ARG and "multiple of num_kv_heads" in msg
+    rc, msg = _status("pa_decode_static", *static(d=96))
+    assert rc == _lib.PA_ERR_UNSUPPORTED
+    rc, msg = _status("pa_decode_static", *static(batch=8192))
+    assert rc == _lib.PA_ERR_WORKSPACE and "scratch" in msg and "pa_decode_workspace_bytes" in msg
+    assert _status("pa_decode_static", *static(batch=0, q=None))[0] == _lib.PA_OK
+
+
 def test_decode_workspace_arithmetic():
     lib = _lib.load()
     small = lib.pa_decode_workspace_bytes(1, 1, 1, 32, _lib.PA_F32)
