@@ -45,7 +45,7 @@ extern "C" {
 #define PA_F16 2
 #define PA_FP8_E4M3 3 /* OCP e4m3fn, KV pool only; q/out stay 16- or 32-bit */
 
-/* Library ABI version (bumped when a signature changes). */
+/* Library ABI version (bumped when an entry point is added or a signature changes; now 2). */
 int pa_version(void);
 
 /* Text of the calling thread's most recent error; "" if none. */
@@ -207,6 +207,18 @@ int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, vo
                      const int32_t *q_lens, const int32_t *q_starts, const int32_t *row_first_key,
                      int batch, int max_q_len, int num_q_heads, int num_kv_heads, int head_dim,
                      int block_size, int64_t num_blocks, float scale, int window, int dtype, void *stream);
+
+/*
+ * pa_prefill_paged evaluated by the vector kernel (one workgroup per query row, the decode inner loop) whatever
+ * the element type: the path fp32, fp8-pool and head_dim 256 calls take anyway, selectable for the 16-bit shapes
+ * too so that the two kernels can be checked against each other.  Same arguments, same results to rounding.
+ * (No separate counterpart in the reference: both are attention/flex_backend.py:144-185.)
+ */
+int pa_prefill_paged_rowwise(const void *q, const void *k_cache, const void *v_cache, void *out,
+                             const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
+                             const int32_t *q_lens, const int32_t *q_starts, const int32_t *row_first_key,
+                             int batch, int max_q_len, int num_q_heads, int num_kv_heads, int head_dim,
+                             int block_size, int64_t num_blocks, float scale, int window, int dtype, void *stream);
 
 /*
  * fp8-e4m3 pool construction (no counterpart in the reference; its oracle is

@@ -75,6 +75,7 @@ SIGNATURES = {
     ),
 }
 SIGNATURES["pa_decode_split"] = SIGNATURES["pa_decode_reduce"] = SIGNATURES["pa_decode"]
+SIGNATURES["pa_prefill_paged_rowwise"] = SIGNATURES["pa_prefill_paged"]
 # pa_decode without the workspace pointer and size
 SIGNATURES["pa_decode_static"] = (c_int, SIGNATURES["pa_decode"][1][:-3] + [c_void_p])
 

@@ -17,8 +17,7 @@ CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 def build(force: bool = False, jobs: int = 8) -> str:
     if force:
         subprocess.run(["make", "-C", CSRC, "clean"], check=True, stdout=subprocess.DEVNULL)
-    # the library and the stand-alone read-bandwidth measurement (every HIP source of the package)
-    proc = subprocess.run(["make", "-C", CSRC, f"-j{jobs}", "all", "read_ceiling"], stdout=subprocess.PIPE,
+    proc = subprocess.run(["make", "-C", CSRC, f"-j{jobs}", "all"], stdout=subprocess.PIPE,
                           stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
         sys.stderr.write(proc.stdout)

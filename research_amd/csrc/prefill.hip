@@ -1,16 +1,15 @@
 // Host entry point of causal prefill attention over a paged context.
-#include <stdlib.h>
-
 #include "prefill_mfma.h"
 
 using namespace pa_decode_detail;
 
-extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, void *out,
-                                const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
-                                const int32_t *q_lens, const int32_t *q_starts, const int32_t *row_first_key,
-                                int batch, int max_q_len, int num_q_heads, int num_kv_heads, int head_dim,
-                                int block_size, int64_t num_blocks, float scale, int window, int dtype,
-                                void *stream) {
+namespace {
+
+int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const void *v_cache, void *out,
+                   const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens, const int32_t *q_lens,
+                   const int32_t *q_starts, const int32_t *row_first_key, int batch, int max_q_len, int num_q_heads,
+                   int num_kv_heads, int head_dim, int block_size, int64_t num_blocks, float scale, int window,
+                   int dtype, void *stream) {
     pa_clear_error();
     PA_REQUIRE(batch >= 0 && max_q_len >= 0, "batch=%d max_q_len=%d must be non-negative", batch, max_q_len);
     PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, "head counts / head_dim must be positive");
@@ -42,11 +41,8 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     a.row_lo = row_first_key;
     a.batch = batch; a.max_q_len = max_q_len;
     hipStream_t s = (hipStream_t)stream;
-    // bf16 / fp16 with head_dim 32, 64, 128 run on the matrix cores; PA_PREFILL_ROWWISE=1 forces the
-    // vector kernel (used to cross-check the two paths; read on every call so a test can switch it).
-    const char *env_rowwise = getenv("PA_PREFILL_ROWWISE");
-    const bool force_rowwise = env_rowwise && env_rowwise[0] == '1';
-    // (its softmax takes the running maximum of the unscaled logits, which needs scale > 0)
+    // bf16 / fp16 with head_dim 32, 64, 128 run on the matrix cores unless the caller asked for the vector kernel
+    // (the matrix-core softmax takes the running maximum of the unscaled logits, which needs scale > 0)
     const prefill_mfma_fn mfma =
         force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
     if (mfma) {
@@ -63,3 +59,17 @@ extern "C" int pa_prefill_paged(const void *q, const void *k_cache, const void *
     PA_CHECK_LAUNCH("pa_prefill_paged");
     return PA_OK;
 }
+
+}  // namespace
+
+#define PA_PREFILL_PARAMS                                                                                      \
+    const void *q, const void *k_cache, const void *v_cache, void *out, const int32_t *block_tables,          \
+        int64_t bt_stride, const int32_t *ctx_lens, const int32_t *q_lens, const int32_t *q_starts,            \
+        const int32_t *row_first_key, int batch, int max_q_len, int num_q_heads, int num_kv_heads,             \
+        int head_dim, int block_size, int64_t num_blocks, float scale, int window, int dtype, void *stream
+#define PA_PREFILL_ARGS                                                                                        \
+    q, k_cache, v_cache, out, block_tables, bt_stride, ctx_lens, q_lens, q_starts, row_first_key, batch,       \
+        max_q_len, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, window, dtype, stream
+
+extern "C" int pa_prefill_paged(PA_PREFILL_PARAMS) { return prefill_launch(false, PA_PREFILL_ARGS); }
+extern "C" int pa_prefill_paged_rowwise(PA_PREFILL_PARAMS) { return prefill_launch(true, PA_PREFILL_ARGS); }

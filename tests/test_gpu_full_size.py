@@ -138,13 +138,8 @@ def test_c3_full_size_two_kernels_and_sample():
     tables = tables_to_device(w.block_tables)
     i32 = lambda x: torch.tensor(list(x), dtype=torch.int32, device=DEV)
     args = (q, kc, vc, tables, i32([P + C] * S), i32([C] * S), i32(np.arange(S) * C), C, w.block_size, w.scale)
-    assert os.environ.get("PA_PREFILL_ROWWISE", "0") != "1"
     mfma = ops.prefill_paged(*args).float().cpu()
-    os.environ["PA_PREFILL_ROWWISE"] = "1"
-    try:
-        rowwise = ops.prefill_paged(*args).float().cpu()
-    finally:
-        del os.environ["PA_PREFILL_ROWWISE"]
+    rowwise = ops.prefill_paged(*args, rowwise=True).float().cpu()
     assert_close(mfma, rowwise, 2e-2, "matrix-core kernel against the vector kernel, all 32 x 256 x 32 rows")
     seqs = [0, 17, 31]
     want = po.paged_prefill_chunk(w.q[seqs], kc.cpu(), vc.cpu(), [w.block_tables[s] for s in seqs], [P] * 3, [C] * 3,
