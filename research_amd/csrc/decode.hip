@@ -4,6 +4,7 @@
 // decode_inst_*.hip.
 #include <stdlib.h>
 
+#include <atomic>
 #include <mutex>
 
 #include "decode_impl.h"
@@ -27,23 +28,16 @@ KernelSet pa_pick_kernels(int q_dtype, int kv_dtype, int d, int nrep_t) {
 }
 
 int pa_fill_head_mapping(PoolArgs &p, int num_q_heads, int num_kv_heads, int head_dim, int kv_dtype) {
-    const int kv_bytes = pa_dtype_bytes(kv_dtype);
-    if (kv_bytes == 0 || (head_dim != 32 && head_dim != 64 && head_dim != 128 && head_dim != 256)) return 0;
-    const int lpr = head_dim * kv_bytes / 16;  // lanes per K/V row
-    const int rpw = 64 / lpr;                  // rows per wave load
-    int hpw = 1;                               // kv heads per wave load: power of two dividing num_kv_heads
-    while (hpw * 2 <= rpw && num_kv_heads % (hpw * 2) == 0) hpw *= 2;
-    const int n_rep = num_q_heads / num_kv_heads;
-    int nrep_t = 1;
-    while (nrep_t < n_rep && nrep_t < 8) nrep_t *= 2;
-    p.hq = num_q_heads;
-    p.hkv = num_kv_heads;
-    p.n_rep = n_rep;
-    p.hpw = hpw;
-    p.tpw = rpw / hpw;
-    p.n_hgroups = num_kv_heads / hpw;
-    p.n_rgroups = (n_rep + nrep_t - 1) / nrep_t;
-    return nrep_t;
+    const HeadPlan h = plan_heads(num_q_heads, num_kv_heads, head_dim, pa_dtype_bytes(kv_dtype));
+    if (!h.nrep_t) return 0;
+    p.hq = h.hq;
+    p.hkv = h.hkv;
+    p.n_rep = h.n_rep;
+    p.hpw = h.hpw;
+    p.tpw = h.tpw;
+    p.n_hgroups = h.n_hgroups;
+    p.n_rgroups = h.n_rgroups;
+    return h.nrep_t;
 }
 
 }  // namespace pa_decode_detail
@@ -52,26 +46,7 @@ using namespace pa_decode_detail;
 
 namespace {
 
-size_t align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
-
-constexpr int kMaxSplitGrid = 4096;  // upper bound of the split pass's grid, fixes the workspace size
-
-// workspace = [block_prefix int32[batch+1]] [part_ml float[slots][heads][2]] [part_acc float[slots][heads][D]]
-// with heads = hpw * NREP query heads of one plane and slots = kMaxSplitGrid + planes * batch.
-struct WsLayout {
-    size_t prefix_off, ml_off, acc_off, total;
-    int64_t slots;
-};
-WsLayout ws_layout(int batch, const PoolArgs &p, int nrep_t, int d, int grid_cap = kMaxSplitGrid) {
-    WsLayout w;
-    const size_t heads = (size_t)p.hpw * nrep_t;
-    w.slots = (int64_t)grid_cap + (int64_t)p.n_hgroups * p.n_rgroups * batch;
-    w.prefix_off = 0;
-    w.ml_off = align_up((size_t)(batch + 1) * 4, 256);
-    w.acc_off = w.ml_off + align_up((size_t)w.slots * heads * 2 * 4, 256);
-    w.total = w.acc_off + align_up((size_t)w.slots * heads * d * 4, 256);
-    return w;
-}
+constexpr int kMaxSplitGrid = kPlanMaxSplitGrid;  // upper bound of the split pass's grid, fixes the workspace size
 
 constexpr int kMaxDevices = 64;
 
@@ -156,7 +131,8 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     const int grid = split_grid();
     // A caller's workspace is sized without asking the device (kMaxSplitGrid workgroups); the library's own
     // scratch is laid out for the grid this device really gets, which is what makes its fixed size go far.
-    const WsLayout w = ws_layout(batch, a.p, nrep_t, head_dim, use_static ? grid : kMaxSplitGrid);
+    const HeadPlan plan = plan_heads(num_q_heads, num_kv_heads, head_dim, pa_dtype_bytes(kv_dtype));
+    const WsPlan w = plan_workspace(batch, plan, head_dim, use_static ? grid : kMaxSplitGrid);
     if (use_static) {
         if (w.total > kStaticScratchBytes)
             return pa_fail(PA_ERR_WORKSPACE,
@@ -181,8 +157,14 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     a.slot_cap = w.slots;
     char *ws = (char *)workspace;
     a.block_prefix = (int32_t *)(ws + w.prefix_off);
+    a.tickets = (unsigned long long *)(ws + w.ticket_off);
     a.part_ml = (float *)(ws + w.ml_off);
     a.part_acc = (float *)(ws + w.acc_off);
+    // Batches that leave a sequence few pieces are finished by the split pass alone; the tag tells this launch's
+    // tickets from whatever the workspace held before.
+    static std::atomic<unsigned long long> launches{0};
+    a.merge_in_split = phases == (kPhaseSplit | kPhaseReduce) && plan_merge_in_split(batch, plan, grid) ? 1 : 0;
+    a.ticket_tag = ((launches.fetch_add(1, std::memory_order_relaxed) + 1) * 0x9E3779B97F4A7C15ull) >> 24;
 
     hipStream_t s = (hipStream_t)stream;
     a.split_grid = grid;
@@ -190,7 +172,7 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
         ks.split<<<dim3((unsigned)grid), dim3(kThreads), (size_t)(batch + 1) * sizeof(int), s>>>(a);
         PA_CHECK_LAUNCH("pa_decode split pass");
     }
-    if (phases & kPhaseReduce) {
+    if ((phases & kPhaseReduce) && !a.merge_in_split) {
         // Many rows and therefore few pieces per sequence: one wave per row.
         const int64_t rows = (int64_t)batch * num_q_heads;
         if (rows >= 4 * (int64_t)grid)
@@ -218,7 +200,8 @@ extern "C" size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_
                 head_dim);
         return 0;
     }
-    return ws_layout(batch, p, nrep_t, head_dim).total;
+    const HeadPlan plan = plan_heads(num_q_heads, num_kv_heads, head_dim, pa_dtype_bytes(kv_dtype));
+    return plan_workspace(batch, plan, head_dim, kMaxSplitGrid).total;
 }
 
 #define PA_DECODE_PARAMS                                                                                       \

@@ -31,13 +31,14 @@
 #include <type_traits>
 #include <utility>
 
+#include "decode_plan.h"
 #include "pa_common.h"
 
 namespace pa_decode_detail {
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / PA_WAVE;
-constexpr int kMaxBatch = 8192;      // sequences per call (their chunk prefix sum lives in LDS)
+constexpr int kMaxBatch = kPlanMaxBatch;  // sequences per call (their block prefix sum lives in LDS)
 constexpr float kNegBig = -1.0e30f;  // finite stand-in for -inf in running maxima
 
 // What every kernel of this file needs to know about the pool and the heads.
@@ -65,6 +66,9 @@ struct DecodeArgs {
     float *part_acc;        // [slot_cap][hpw*NREP][D]
     float *part_ml;         // [slot_cap][hpw*NREP][2]
     int32_t *block_prefix;  // [batch+1], written by the split pass for the reduction pass
+    unsigned long long *tickets;  // [planes*batch]: (launch tag << 24) | pieces of the (plane, sequence) that have arrived
+    unsigned long long ticket_tag;  // 40-bit tag of this launch: a ticket with another tag counts as zero
+    int merge_in_split;     // the workgroup that delivers a sequence's last piece merges the pieces (no second pass)
 };
 
 struct RowwiseArgs {
@@ -81,7 +85,7 @@ __device__ __forceinline__ uint4 ld16(const void *p) { return *reinterpret_cast<
 
 // First key a query at position n_keys-1 sees under the sliding window (0 without one).
 __device__ __forceinline__ int window_first_key(const PoolArgs &p, int n_keys) {
-    return p.window > 0 ? max(0, n_keys - p.window) : 0;
+    return plan_first_key(n_keys, p.window);
 }
 
 // 16-byte load of pool data: used once, so it carries the non-temporal hint.
@@ -405,22 +409,10 @@ __device__ __forceinline__ void merge_rows(RowState<NREP, RowShape<KV, D>::EPL> 
     __syncthreads();
 }
 
-// Which workgroup of a grid of G owns flattened block unit u of total T:
-// workgroup w owns [floor(w*T/G), floor((w+1)*T/G)).
-__device__ __forceinline__ int64_t unit_begin(int64_t w, int64_t total, int64_t grid) { return w * total / grid; }
-__device__ __forceinline__ int owner_of(int64_t u, int64_t total, int64_t grid) {
-    return (int)(((u + 1) * grid - 1) / total);
-}
-
-// Workgroups of the split pass that take part: with little work (one short sequence, say) a workgroup per
-// pool block would leave hundreds of one-block partials for the reduction pass to chain through, so a
-// workgroup gets at least kMinUnitsPerWorkgroup units and the rest of the grid leaves at once.  Both passes
-// derive the number from the same total.
-constexpr int kMinUnitsPerWorkgroup = 4;
-__device__ __forceinline__ int effective_grid(int64_t total, int grid) {
-    const int64_t g = total / kMinUnitsPerWorkgroup;
-    return g < 1 ? 1 : (g < grid ? (int)g : grid);
-}
+// The partition arithmetic (which workgroup owns which blocks, where its partial goes) is in decode_plan.h.
+__device__ __forceinline__ int64_t unit_begin(int64_t w, int64_t total, int64_t grid) { return plan_unit_begin(w, total, grid); }
+__device__ __forceinline__ int owner_of(int64_t u, int64_t total, int64_t grid) { return plan_owner_of(u, total, grid); }
+__device__ __forceinline__ int effective_grid(int64_t total, int grid) { return plan_effective_grid(total, grid); }
 
 // Finish one (sequence, query head): fold `ez` extra all-zero keys into the
 // merged (num, M, den) and normalise.
@@ -432,6 +424,94 @@ __device__ __forceinline__ float finish_row(float num, float M, float den, int e
         den = den * alpha + (float)ez * __builtin_amdgcn_exp2f(-mn);
     }
     return den > 0.f ? num / den : 0.f;
+}
+
+// Partials that another workgroup merges inside the same launch travel between compute dies (each XCD has its own
+// L2): they are written and read as device-scope 8-byte accesses, which go through to the memory side.  Ordinary
+// stores would need a write-back of the whole L2 before the ticket is counted (what a device-scope release fence
+// does), which costs far more than the merge saves.
+__device__ __forceinline__ void st_coherent(float *p, float a, float b) {
+    const unsigned long long v = (unsigned long long)__builtin_bit_cast(uint32_t, a) |
+                                 ((unsigned long long)__builtin_bit_cast(uint32_t, b) << 32);
+    __hip_atomic_store(reinterpret_cast<unsigned long long *>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float2 ld_coherent(const float *p) {
+    const unsigned long long v = __hip_atomic_load(reinterpret_cast<const unsigned long long *>(p), __ATOMIC_RELAXED,
+                                                   __HIP_MEMORY_SCOPE_AGENT);
+    return float2{__builtin_bit_cast(float, (uint32_t)v), __builtin_bit_cast(float, (uint32_t)(v >> 32))};
+}
+
+// One piece of a (plane, sequence) has been written to the workspace: count it; true for the arrival that completes
+// the sequence.  A ticket is (tag of the launch << 24 | arrivals so far); a ticket carrying another tag is left
+// over from an earlier launch (or was never written) and counts as zero, so the workspace needs no initialisation,
+// and the completing arrival stores zero arrivals, so a replay of the same launch (a captured graph replays with
+// the same tag) starts clean as well.  Called by one thread, after the workgroup's stores were fenced.
+__device__ __forceinline__ bool piece_arrived_last(unsigned long long *ticket, unsigned long long tag, int n_pieces) {
+    unsigned long long old = __hip_atomic_load(ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    for (;;) {  // ends after at most n_pieces rounds: a failed exchange means another piece was counted
+        const unsigned long long cnt = (old >> 24) == tag ? (old & 0xffffffull) : 0ull;
+        const bool last = cnt + 1 == (unsigned long long)n_pieces;
+        const unsigned long long neu = (tag << 24) | (last ? 0ull : cnt + 1);
+        if (__hip_atomic_compare_exchange_strong(ticket, &old, neu, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT))
+            return last;
+    }
+}
+
+// The workgroup that delivered the last piece of (plane, sequence b) merges the pieces of workgroups w0..w1 and
+// writes the plane's output rows: one thread per (query head, four consecutive d), the loads of four pieces in
+// flight at a time.
+template <typename QT, int D, int NREP>
+__device__ __forceinline__ void merge_pieces(const DecodeArgs &a, int plane, int b, int hg, int rep0, int w0, int w1,
+                                             int tid) {
+    constexpr int PIPE = 4;
+    const PoolArgs &p = a.p;
+    const int stride_acc = p.hpw * NREP * D, stride_ml = p.hpw * NREP * 2;
+    const int64_t key = (int64_t)plane * a.batch + b;
+    const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
+    QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * D;
+    for (int item = tid; item < p.hpw * NREP * (D / 4); item += kThreads) {
+        const int idx = item / (D / 4), d = (item - idx * (D / 4)) * 4;
+        const int kv_local = idx / NREP, r = idx - kv_local * NREP;
+        if (rep0 + r >= p.n_rep) continue;
+        const int qh = (hg * p.hpw + kv_local) * p.n_rep + rep0 + r;
+        float M = kNegBig, den = 0.f, num[4] = {0.f, 0.f, 0.f, 0.f};
+        for (int w = w0; w <= w1; w += PIPE) {
+            float m[PIPE], l[PIPE];
+            float4 x[PIPE];
+#pragma unroll
+            for (int j = 0; j < PIPE; ++j) {
+                const bool have = w + j <= w1 && w + j + key < a.slot_cap;
+                const int64_t slot = (have ? w + j : w0) + key;
+                const float2 ml = ld_coherent(a.part_ml + slot * stride_ml + idx * 2);
+                const float2 lo = ld_coherent(a.part_acc + slot * stride_acc + idx * D + d);
+                const float2 hi = ld_coherent(a.part_acc + slot * stride_acc + idx * D + d + 2);
+                x[j] = float4{lo.x, lo.y, hi.x, hi.y};
+                m[j] = have ? ml.x : kNegBig;
+                l[j] = have ? ml.y : 0.f;
+                if (!have) x[j] = float4{0.f, 0.f, 0.f, 0.f};
+            }
+            float mn = M;
+#pragma unroll
+            for (int j = 0; j < PIPE; ++j) mn = fmaxf(mn, m[j]);
+            const float so = __builtin_amdgcn_exp2f(M - mn);
+            den *= so;
+#pragma unroll
+            for (int k = 0; k < 4; ++k) num[k] *= so;
+#pragma unroll
+            for (int j = 0; j < PIPE; ++j) {
+                const float sn = __builtin_amdgcn_exp2f(m[j] - mn);
+                den = fmaf(l[j], sn, den);
+                num[0] = fmaf(x[j].x, sn, num[0]);
+                num[1] = fmaf(x[j].y, sn, num[1]);
+                num[2] = fmaf(x[j].z, sn, num[2]);
+                num[3] = fmaf(x[j].w, sn, num[3]);
+            }
+            M = mn;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) pa_scalar<QT>::store(orow + (int64_t)qh * D + d + j, finish_row(num[j], M, den, ez));
+    }
 }
 
 // Split pass.  The (plane, sequence, block) space - plane = (rep group, head
@@ -448,6 +528,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
     extern __shared__ int s_prefix[];  // batch + 1 entries: blocks before each sequence
     __shared__ int s_scan[kThreads];
     __shared__ float s_part[MergeShape<KV, D, NREP>::FLOATS];
+    __shared__ int s_last;  // this workgroup delivered the last piece of the sequence it just finished a part of
 
     const PoolArgs &p = a.p;
     const int tid = threadIdx.x;
@@ -460,10 +541,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
         const int per = (B + kThreads - 1) / kThreads;
         const int lo = min(B, tid * per), hi = min(B, lo + per);
         // blocks of sequence b that hold visible keys: [first_key(b) / bs, ceil(L / bs))
-        auto blocks_of = [&](int b) {
-            const int len = max(0, a.seq_lens[b]);
-            return (len + p.bs - 1) / p.bs - window_first_key(p, len) / p.bs;
-        };
+        auto blocks_of = [&](int b) { return plan_blocks_of(a.seq_lens[b], p.bs, p.window); };
         int sum = 0;
         for (int b = lo; b < hi; ++b) sum += blocks_of(b);
         s_scan[tid] = sum;
@@ -488,6 +566,14 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
     const int planes = p.n_hgroups * p.n_rgroups;
     const int64_t total = per_plane * planes;
     const LaneRole role = lane_role<KV, D>(lane, p);
+    if (a.merge_in_split) {
+        // no second pass: sequences without a visible key get their zero rows here, dealt out over the grid
+        for (int b = blockIdx.x; b < B; b += gridDim.x) {
+            if (s_prefix[b + 1] != s_prefix[b]) continue;
+            QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * D;
+            for (int i = tid; i < p.hq * D; i += kThreads) pa_scalar<QT>::store(orow + i, 0.f);
+        }
+    }
     if (total == 0) return;
     const int grid = effective_grid(total, (int)gridDim.x);
     if ((int)blockIdx.x >= grid) return;  // uniform
@@ -529,7 +615,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
                                                                  finish_row(num[j], M, den, ez));
                                     });
         } else {
-            const int64_t slot = (int64_t)blockIdx.x + (int64_t)plane * B + b;
+            const int64_t slot = plan_slot((int)blockIdx.x, plane, B, b);
             if (slot < a.slot_cap) {  // never write outside the workspace
                 float *acc = a.part_acc + slot * (p.hpw * NREP * D);
                 float *ml = a.part_ml + slot * (p.hpw * NREP * 2);
@@ -537,13 +623,31 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
                                         [&](int qh, int d, const float (&num)[4], float M, float den) {
                                             const int kv = qh / p.n_rep;
                                             const int idx = (kv - hg * p.hpw) * NREP + (qh - kv * p.n_rep - rep0);
-                                            *reinterpret_cast<float4 *>(acc + idx * D + d) =
-                                                float4{num[0], num[1], num[2], num[3]};
-                                            if (d == 0) {
-                                                ml[idx * 2] = M;
-                                                ml[idx * 2 + 1] = den;
+                                            if (a.merge_in_split) {  // uniform: read by another workgroup of this launch
+                                                st_coherent(acc + idx * D + d, num[0], num[1]);
+                                                st_coherent(acc + idx * D + d + 2, num[2], num[3]);
+                                                if (d == 0) st_coherent(ml + idx * 2, M, den);
+                                            } else {
+                                                *reinterpret_cast<float4 *>(acc + idx * D + d) =
+                                                    float4{num[0], num[1], num[2], num[3]};
+                                                if (d == 0) {
+                                                    ml[idx * 2] = M;
+                                                    ml[idx * 2 + 1] = den;
+                                                }
                                             }
                                         });
+            }
+            if (a.merge_in_split) {
+                // Every thread's part of the partial is made visible to the whole device, then one thread counts
+                // the piece; the workgroup whose piece completes the sequence reads all of them back and merges.
+                const int64_t u0 = plane * per_plane + s_prefix[b];
+                const int w0 = owner_of(u0, total, grid), w1 = owner_of(u0 + nblk - 1, total, grid);
+                __builtin_amdgcn_s_waitcnt(0);  // this thread's stores have reached the memory side
+                __syncthreads();
+                if (tid == 0)
+                    s_last = piece_arrived_last(a.tickets + ((int64_t)plane * B + b), a.ticket_tag, w1 - w0 + 1);
+                __syncthreads();
+                if (s_last) merge_pieces<QT, D, NREP>(a, plane, b, hg, rep0, w0, w1, tid);  // uniform
             }
         }
         cur += blk1 - blk0;

@@ -1,0 +1,108 @@
+// Bookkeeping of the split pass of paged decode attention: how the (plane, sequence, block) space is cut into
+// workgroup ranges, which workgroup owns a block, where a range's partial result goes in the workspace and how
+// the workspace is laid out.  Integer arithmetic only; shared by the kernels (decode_impl.h), the host entry
+// point (decode.hip) and a plain C++ replay of both passes that the CPU tests compile with g++ (no HIP needed).
+#pragma once
+#include <stddef.h>
+#include <stdint.h>
+
+#if defined(__HIPCC__)
+#define PA_PLAN_FN __host__ __device__ inline __attribute__((always_inline))
+#else
+#define PA_PLAN_FN inline
+#endif
+
+namespace pa_decode_detail {
+
+constexpr int kPlanMaxBatch = 8192;      // sequences per call (their block prefix sum lives in LDS)
+constexpr int kPlanMaxSplitGrid = 4096;  // upper bound of the split pass's grid, fixes the caller's workspace size
+constexpr int kPlanMinUnitsPerWorkgroup = 4;
+
+// How the heads are spread over wave loads and planes (a plane = one group of hpw kv heads x one group of <= nrep_t
+// query heads per kv head).  lpr lanes of 16 bytes hold one K/V row; a wave load covers rpw = 64/lpr rows, mapped
+// to hpw neighbouring kv heads of tpw consecutive tokens.
+struct HeadPlan {
+    int hq, hkv, n_rep;
+    int hpw, tpw, n_hgroups, n_rgroups;
+    int nrep_t;  // padded group size (kernel template parameter); 0 = no kernel for this head_dim / element size
+    PA_PLAN_FN int planes() const { return n_hgroups * n_rgroups; }
+    PA_PLAN_FN int heads_per_slot() const { return hpw * nrep_t; }
+};
+
+PA_PLAN_FN HeadPlan plan_heads(int num_q_heads, int num_kv_heads, int head_dim, int kv_elem_bytes) {
+    HeadPlan h = {};
+    if (kv_elem_bytes <= 0 || (head_dim != 32 && head_dim != 64 && head_dim != 128 && head_dim != 256)) return h;
+    if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) return h;
+    const int lpr = head_dim * kv_elem_bytes / 16;  // lanes per K/V row
+    const int rpw = 64 / lpr;                        // rows per wave load
+    int hpw = 1;                                     // kv heads per wave load: power of two dividing num_kv_heads
+    while (hpw * 2 <= rpw && num_kv_heads % (hpw * 2) == 0) hpw *= 2;
+    const int n_rep = num_q_heads / num_kv_heads;
+    int nrep_t = 1;
+    while (nrep_t < n_rep && nrep_t < 8) nrep_t *= 2;
+    h.hq = num_q_heads;
+    h.hkv = num_kv_heads;
+    h.n_rep = n_rep;
+    h.hpw = hpw;
+    h.tpw = rpw / hpw;
+    h.n_hgroups = num_kv_heads / hpw;
+    h.n_rgroups = (n_rep + nrep_t - 1) / nrep_t;
+    h.nrep_t = nrep_t;
+    return h;
+}
+
+// Blocks of a sequence of `len` keys that hold visible keys under a sliding window (0 = none): the query sits at
+// position len-1 and sees keys j >= len - window, so blocks [first_key / bs, ceil(len / bs)) take part.
+PA_PLAN_FN int plan_first_key(int len, int window) { return window > 0 && len > window ? len - window : 0; }
+PA_PLAN_FN int plan_blocks_of(int len, int block_size, int window) {
+    if (len <= 0) return 0;
+    return (len + block_size - 1) / block_size - plan_first_key(len, window) / block_size;
+}
+
+// Workgroup w of a grid of G owns the flattened units [floor(w*T/G), floor((w+1)*T/G)) of T.
+PA_PLAN_FN int64_t plan_unit_begin(int64_t w, int64_t total, int64_t grid) { return w * total / grid; }
+PA_PLAN_FN int plan_owner_of(int64_t u, int64_t total, int64_t grid) { return (int)(((u + 1) * grid - 1) / total); }
+
+// Workgroups that take part: with little work a workgroup per pool block would leave hundreds of one-block
+// partials, so a workgroup gets at least kPlanMinUnitsPerWorkgroup units and the rest of the grid leaves at once.
+PA_PLAN_FN int plan_effective_grid(int64_t total, int grid) {
+    const int64_t g = total / kPlanMinUnitsPerWorkgroup;
+    return g < 1 ? 1 : (g < grid ? (int)g : grid);
+}
+
+// Partial slot of the piece of (plane, sequence) that workgroup w computed: unique, because along the flattened
+// order both w and plane*batch + sequence only grow.
+PA_PLAN_FN int64_t plan_slot(int w, int plane, int batch, int b) { return (int64_t)w + (int64_t)plane * batch + b; }
+
+// workspace = [block_prefix int32[batch+1]] [tickets uint64[planes*batch]] [part_ml float[slots][heads][2]]
+//             [part_acc float[slots][heads][D]], heads = hpw*nrep_t query heads of one plane,
+// slots = grid_cap + planes*batch (slot indices stay below grid + planes*batch - 1).
+struct WsPlan {
+    size_t prefix_off, ticket_off, ml_off, acc_off, total;
+    int64_t slots;
+};
+PA_PLAN_FN size_t plan_align_up(size_t x, size_t a) { return (x + a - 1) / a * a; }
+PA_PLAN_FN WsPlan plan_workspace(int batch, const HeadPlan &h, int head_dim, int grid_cap) {
+    WsPlan w;
+    const size_t heads = (size_t)h.heads_per_slot();
+    const size_t keys = (size_t)h.planes() * (size_t)batch;
+    w.slots = (int64_t)grid_cap + (int64_t)keys;
+    w.prefix_off = 0;
+    w.ticket_off = plan_align_up((size_t)(batch + 1) * 4, 256);
+    w.ml_off = w.ticket_off + plan_align_up(keys * 8, 256);
+    w.acc_off = w.ml_off + plan_align_up((size_t)w.slots * heads * 2 * 4, 256);
+    w.total = w.acc_off + plan_align_up((size_t)w.slots * heads * (size_t)head_dim * 4, 256);
+    return w;
+}
+
+// Whether the split pass merges the pieces of a sequence itself (the workgroup that delivers a sequence's last
+// outstanding piece merges them all) instead of leaving them to a second launch: when the batch is so large that a
+// (plane, sequence) has two pieces on average at most.  Measured on MI355X: 256 sequences (two pieces each) gain
+// 1 % over the two launches, 64 sequences (four pieces each) lose 2 % - delivering a piece costs the workgroup a
+// round trip to the memory side before its next part - and a few long sequences spread over the whole grid are
+// merged much faster by the second launch, whose workgroups take one output row each.
+PA_PLAN_FN bool plan_merge_in_split(int batch, const HeadPlan &h, int grid) {
+    return (int64_t)grid <= 2 * (int64_t)h.planes() * batch;
+}
+
+}  // namespace pa_decode_detail
