@@ -121,6 +121,8 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
         return pa_fail(PA_ERR_UNSUPPORTED, "pa_decode: no kernel for q_dtype=%d kv_dtype=%d head_dim=%d", q_dtype,
                        kv_dtype, head_dim);
     PA_REQUIRE(batch <= kMaxBatch, "batch=%d above the %d sequences one call handles", batch, kMaxBatch);
+    PA_REQUIRE(plan_split_lds_bytes(batch, head_dim, pa_dtype_bytes(kv_dtype), nrep_t) <= 65536,
+               "batch=%d needs more than 64 KB of LDS per workgroup", batch);
     if (batch == 0) return PA_OK;
     PA_REQUIRE(q && out && seq_lens, "NULL q / out / seq_lens");
     PA_REQUIRE(k_cache && v_cache, "NULL cache pointer");

@@ -340,6 +340,10 @@ template <typename KV, int D, int NREP> struct MergeShape {
                                                                      : 1;
     static constexpr int AUX = HR * ROWS * ROWF;   // float offset of the weights
     static constexpr int FLOATS = HR * ROWS * (ROWF + 3);
+    // the host-visible statement of the same arithmetic (the launch checks the workgroup's LDS against it)
+    static_assert(ROWS == plan_merge_rows(D, (int)sizeof(KV)) && HR == plan_merge_heads_per_round(D, (int)sizeof(KV), NREP) &&
+                      FLOATS == plan_merge_floats(D, (int)sizeof(KV), NREP),
+                  "decode_plan.h and MergeShape disagree");
 };
 
 template <typename KV, int D, int NREP, typename Emit>

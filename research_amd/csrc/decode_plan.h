@@ -95,6 +95,28 @@ PA_PLAN_FN WsPlan plan_workspace(int batch, const HeadPlan &h, int head_dim, int
     return w;
 }
 
+// LDS of the merge of a workgroup's row-group partials (decode_impl.h: merge_rows): rows = 4 waves x rows per wave
+// load, each D + 2 floats plus 3 floats of weights; as many query heads per round (8, 4, 2 or 1 of the nrep_t) as
+// 28 KB hold.
+constexpr int kPlanThreads = 256;
+constexpr int kPlanMergeBudget = 28 * 1024;
+PA_PLAN_FN constexpr int plan_merge_rows(int head_dim, int kv_elem_bytes) { return 4 * (64 / (head_dim * kv_elem_bytes / 16)); }
+PA_PLAN_FN constexpr int plan_merge_heads_per_round(int head_dim, int kv_elem_bytes, int nrep_t) {
+    const int per_head = plan_merge_rows(head_dim, kv_elem_bytes) * (head_dim + 2 + 3) * 4;
+    return nrep_t >= 8 && 8 * per_head <= kPlanMergeBudget   ? 8
+           : nrep_t >= 4 && 4 * per_head <= kPlanMergeBudget ? 4
+           : nrep_t >= 2 && 2 * per_head <= kPlanMergeBudget ? 2
+                                                             : 1;
+}
+PA_PLAN_FN constexpr int plan_merge_floats(int head_dim, int kv_elem_bytes, int nrep_t) {
+    return plan_merge_heads_per_round(head_dim, kv_elem_bytes, nrep_t) * plan_merge_rows(head_dim, kv_elem_bytes) *
+           (head_dim + 2 + 3);
+}
+// LDS of one workgroup of the split pass: the block prefix sums (dynamic), the scan scratch, the merge area, a flag.
+PA_PLAN_FN constexpr size_t plan_split_lds_bytes(int batch, int head_dim, int kv_elem_bytes, int nrep_t) {
+    return (size_t)(batch + 1) * 4 + kPlanThreads * 4 + (size_t)plan_merge_floats(head_dim, kv_elem_bytes, nrep_t) * 4 + 4;
+}
+
 // Whether the split pass merges the pieces of a sequence itself (the workgroup that delivers a sequence's last
 // outstanding piece merges them all) instead of leaving them to a second launch: when the batch is so large that a
 // (plane, sequence) has two pieces on average at most.  Measured on MI355X: 256 sequences (two pieces each) gain
