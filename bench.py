@@ -1,12 +1,15 @@
 #!/usr/bin/env python3
 """Benchmark of the paged decode-attention hot path on one MI355X.
 
-One step = one ``pa_decode`` call (split-K pass + reduction pass) over one
-batch of the synthetic workload, inputs resident in HBM.  The headline
-workload is workload c4 (Llama-3-8B shape, B=256, bf16 pool,
-lognormal context lengths, seed 1004).  Prints one JSON line.
+One step = one ``pa_decode`` call over one batch of the synthetic workload,
+inputs resident in HBM.  The headline workload is workload c4 (Llama-3-8B
+shape, B=256, bf16 pool, lognormal context lengths, seed 1004).  Prints one
+JSON line; with the default workload the line also carries short runs of the
+other configurations (c2, c5 decode, c3 append + chunked prefill) under
+``secondary``.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1|c3|engine] [--no-secondary]
+    python bench.py --traffic-from-pmc NAME KERNEL FETCH.csv WRITE.csv   # refresh profiles/traffic.json
 """
 
 from __future__ import annotations
@@ -27,10 +30,58 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0  # MI355X HBM3E, vendor figure
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, vendor figure
 
-# HBM traffic of one launch of the dominant kernel (c4: decode_split_kernel, c3: prefill_mfma_kernel), from
-# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (summaries under profiles/); None until measured.
-# c4: fetch 3 447 663 616 + write 7 592 755; c3: fetch 131 099 238 + write 67 108 864 (the output)
-MEASURED_TRAFFIC_BYTES = {"c4": 3455306650, "c3": 197967872}
+# HBM traffic of one launch of each workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# scaled by a device copy of known size in the same run: written by `--traffic-from-pmc` from the counter files,
+# never typed in; a workload without an entry reports null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def measured_traffic(name):
+    try:
+        with open(TRAFFIC_FILE) as f:
+            entry = json.load(f).get(name)
+    except (OSError, ValueError):
+        return None
+    return None if entry is None else entry["bytes"]
+
+
+def traffic_from_pmc(name, kernel, fetch_csv, write_csv) -> int:
+    """Average FETCH_SIZE / WRITE_SIZE (KiB per dispatch) of `kernel` in two rocprofv3 counter_collection CSVs,
+    each scaled by what the same counter reads for the 1 GiB device copy of `--copy-calibration` in the same file;
+    stores the sum as workload `name` in profiles/traffic.json."""
+    import csv
+
+    def one(path, counter, copied_kib):
+        mine, copy = [], []
+        with open(path) as f:
+            for r in csv.DictReader(f):
+                if r["Counter_Name"] != counter:
+                    continue
+                if kernel in r["Kernel_Name"]:
+                    mine.append(float(r["Counter_Value"]))
+                elif "copyBuffer" in r["Kernel_Name"]:
+                    copy.append(float(r["Counter_Value"]))
+        if not mine or not copy:
+            raise SystemExit(f"{path}: no {counter} rows for {kernel!r} or for the calibration copy")
+        # the calibration copy (1 GiB, in one dispatch or split in two) is the largest device copy of the run
+        big = [c for c in copy if c >= 0.9 * max(copy)]
+        factor = copied_kib / sum(big)
+        return sum(mine) / len(mine) * factor * 1024.0, factor
+
+    fetch, f_scale = one(fetch_csv, "FETCH_SIZE", 1024 * 1024)
+    write, w_scale = one(write_csv, "WRITE_SIZE", 1024 * 1024)
+    try:
+        with open(TRAFFIC_FILE) as f:
+            table = json.load(f)
+    except (OSError, ValueError):
+        table = {}
+    table[name] = {"bytes": int(round(fetch + write)), "kernel": kernel, "fetch_bytes": int(round(fetch)),
+                   "write_bytes": int(round(write)), "fetch_scale": round(f_scale, 4), "write_scale": round(w_scale, 4)}
+    with open(TRAFFIC_FILE, "w") as f:
+        json.dump(table, f, indent=1, sort_keys=True)
+        f.write("\n")
+    print(json.dumps({name: table[name]}))
+    return 0
 
 
 def parse_args():
@@ -46,6 +97,10 @@ def parse_args():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="rough budget of the CPU baseline sample")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy, as the known-size kernel HBM counters are scaled by")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="with the default workload: leave out the short runs of c2, c5 and c3")
+    ap.add_argument("--traffic-from-pmc", nargs=4, metavar=("NAME", "KERNEL", "FETCH_CSV", "WRITE_CSV"),
+                    help="no benchmark: compute a workload's HBM traffic from two rocprofv3 counter files")
     return ap.parse_args()
 
 
@@ -127,7 +182,24 @@ def timed_ms(fn, steps):
     return start.elapsed_time(stop) / steps
 
 
-def bench_prefill_c3(args, dev) -> int:
+def timed_steps(fn, steps):
+    """(mean, median) milliseconds per call over exactly `steps` calls: one HIP event on the launch stream before
+    the first call and one behind every call; the mean is the whole bracket, the median is over the steps."""
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    torch.cuda.synchronize()
+    marks[0].record()
+    for i in range(steps):
+        fn()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    each = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    return marks[0].elapsed_time(marks[steps]) / steps, each[steps // 2]
+
+
+KERNEL_LAUNCHES = 50  # launches the dominant kernel's average duration is taken over
+
+
+def bench_prefill_c3(args, dev) -> dict:
     """Workload c3: append 32 x 256 new K/V rows, then chunked causal prefill over 2048 shared prefix keys.
 
     One step = pa_kv_scatter + pa_prefill_paged.  The value is the step's attention FLOP rate; the roofline
@@ -172,9 +244,9 @@ def bench_prefill_c3(args, dev) -> int:
     preheat(step, args.preheat_s)
     for _ in range(args.warmup):
         step()
-    ms_step = timed_ms(step, args.steps)
-    ms_prefill = timed_ms(prefill, args.steps)
-    ms_append = timed_ms(append, args.steps)
+    ms_step, ms_step_median = timed_steps(step, args.steps)
+    ms_prefill = timed_ms(prefill, max(args.steps, KERNEL_LAUNCHES))
+    ms_append = timed_ms(append, max(args.steps, KERNEL_LAUNCHES))
     # The same append with the rotary embedding of q and k fused in (the step a model runs right before this
     # path), beside the two-pass form: rotation into dense buffers, then the scatter.
     pos = (torch.arange(C, dtype=torch.int32, device=dev) + P).repeat(S)
@@ -202,7 +274,8 @@ def bench_prefill_c3(args, dev) -> int:
     result = {
         "metric": "prefill-attn TFLOP/s", "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
         "tokens_per_s": S * C / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_median": ms_step_median,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "c3 shared-prefix chunked prefill + KV append, 32 x (2048 + 256), bf16",
                    "num_seqs": S, "prefix_len": P, "chunk_len": C, "num_q_heads": w.num_q_heads,
@@ -210,7 +283,8 @@ def bench_prefill_c3(args, dev) -> int:
                    "attention_flops": flops, "append_bytes": w.append_bytes(), "seed": 1003},
         "roofline": {"bound": "mfma", "kernel": "prefill_mfma_kernel", "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": MEASURED_TRAFFIC_BYTES.get("c3"), "kernel_ms": ms_prefill},
+                     "traffic": measured_traffic("c3"), "kernel_ms": ms_prefill,
+                     "kernel_launches": max(args.steps, KERNEL_LAUNCHES)},
         "append": {"kernel": "kv_scatter_kernel", "kernel_ms": ms_append,
                    "achieved_gbps": w.append_bytes() / (ms_append * 1e-3) / 1e9, "peak_gbps": HBM_PEAK_GBPS},
         "rope_append": {"kernel": "rope_kv_append_kernel", "kernel_ms": ms_rope, "bytes": rope_bytes,
@@ -238,8 +312,7 @@ def bench_prefill_c3(args, dev) -> int:
                       f"SDPA over {P + C} tokens (rows {P}..{P + C - 1} are the chunk), {threads} threads, {dt:.1f} s; "
                       "FLOPs counted for the chunk rows only",
         }
-    print(json.dumps(result))
-    return 0
+    return result
 
 
 def bench_engine(args, dev) -> int:
@@ -304,27 +377,13 @@ def bench_engine(args, dev) -> int:
     return 0
 
 
-def main() -> int:
-    args = parse_args()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1", file=sys.stderr)
-        return 2
+def bench_decode(name, args, dev) -> dict:
+    """One decode workload: the pa_decode step, its dominant kernel alone, the CPU restatement beside it."""
     from research_amd import _lib, ops
     from research_amd.workloads import make_decode
 
-    _lib.load()  # no fallback: raises if the HIP library is missing
-    if not torch.cuda.is_available():
-        print("bench.py needs a HIP device", file=sys.stderr)
-        return 2
-    dev = torch.device("cuda:0")
-    torch.cuda.set_device(dev)
-    if args.workload == "c3":
-        return bench_prefill_c3(args, dev)
-    if args.workload == "engine":
-        return bench_engine(args, dev)
-
     t_gen = time.perf_counter()
-    w = make_decode(args.workload)
+    w = make_decode(name)
     t_gen = time.perf_counter() - t_gen
 
     q = w.q.to(dev)
@@ -343,23 +402,15 @@ def main() -> int:
     n_pools = 4 if kv_bytes < (1 << 30) else 1
     pools = [(k_pool, v_pool)] + [(k_pool.clone(), v_pool.clone()) for _ in range(n_pools - 1)]
     turn = [0]
+    # one launch (the split pass merges the pieces itself) or two (split pass, reduction pass)
+    passes = int(_lib.load().pa_decode_passes(w.batch, w.num_q_heads, w.num_kv_heads, w.head_dim,
+                                              ops.PA_DTYPE[k_pool.dtype]))
 
     def step(entry="pa_decode"):
         kp, vp = pools[turn[0] % n_pools]
         turn[0] += 1
         ops.decode(q, kp, vp, tables, lens, w.block_size, w.scale, ws, k_scale=k_scale, v_scale=v_scale,
                    out=out, entry=entry)
-
-    def timed(entry, steps):
-        """Average milliseconds per launch: HIP events on the launch stream around `steps` calls."""
-        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        torch.cuda.synchronize()
-        start.record()
-        for _ in range(steps):
-            step(entry)
-        stop.record()
-        torch.cuda.synchronize()
-        return start.elapsed_time(stop) / steps
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -372,28 +423,24 @@ def main() -> int:
         step()
     torch.cuda.synchronize()
     wall = time.perf_counter()
-    ms_step = timed("pa_decode", args.steps)
+    ms_step, ms_step_median = timed_steps(step, args.steps)
     wall = time.perf_counter() - wall
-    ms_split = timed("pa_decode_split", args.steps)  # the dominant kernel alone
-    ms_reduce = timed("pa_decode_reduce", args.steps)
+    n_kernel = max(args.steps, KERNEL_LAUNCHES)
+    # the dominant kernel alone: the split pass (with one launch per step it IS the step)
+    ms_split = timed_ms(lambda: step("pa_decode" if passes == 1 else "pa_decode_split"), n_kernel)
+    ms_reduce = None if passes == 1 else timed_ms(lambda: step("pa_decode_reduce"), n_kernel)
 
     gather = None
-    if args.workload in ("c1", "c2"):
+    if name in ("c1", "c2") and not getattr(args, "secondary_run", False):
         # the reference's own decode materialises this copy first (_gather_kv_from_cache): the block-table
         # gather into zero-padded [B, max_len, Hkv, D] tensors, bit-exact, bound by HBM
         max_len = int(w.seq_lens.max())
         gk = torch.empty((w.batch, max_len, w.num_kv_heads, w.head_dim), dtype=k_pool.dtype, device=dev)
         gv = torch.empty_like(gk)
-        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        run_gather = lambda: ops.kv_gather(k_pool, v_pool, tables, lens, max_len, w.block_size, out=(gk, gv))
         for _ in range(3):
-            ops.kv_gather(k_pool, v_pool, tables, lens, max_len, w.block_size, out=(gk, gv))
-        torch.cuda.synchronize()
-        ev0.record()
-        for _ in range(args.steps):
-            ops.kv_gather(k_pool, v_pool, tables, lens, max_len, w.block_size, out=(gk, gv))
-        ev1.record()
-        torch.cuda.synchronize()
-        ms_gather = ev0.elapsed_time(ev1) / args.steps
+            run_gather()
+        ms_gather = timed_ms(run_gather, args.steps)
         row = w.num_kv_heads * w.head_dim * k_pool.element_size()
         g_bytes = 2 * w.batch * max_len * row + 2 * w.total_tokens * row + 4 * int(sum(len(t) for t in w.block_tables)) + 4 * w.batch
         gather = {"kernel": "kv_gather_kernel", "kernel_ms": ms_gather, "bytes": g_bytes,
@@ -404,7 +451,6 @@ def main() -> int:
 
     alg_bytes = w.algorithmic_bytes()
     achieved = alg_bytes / (ms_split * 1e-3) / 1e9
-    traffic = MEASURED_TRAFFIC_BYTES.get(args.workload)
     result = {
         "metric": "decode-attn HBM GB/s",
         "value": alg_bytes / (ms_step * 1e-3) / 1e9,
@@ -416,6 +462,8 @@ def main() -> int:
         "warmup": args.warmup,
         "preheat_s": args.preheat_s,
         "ms_per_step": ms_step,
+        "ms_per_step_median": ms_step_median,
+        "value_at_median": alg_bytes / (ms_step_median * 1e-3) / 1e9,
         "wall_ms_per_step": wall * 1e3 / args.steps,
         "higher_is_better": True,
         "scaling": "weak",
@@ -425,25 +473,71 @@ def main() -> int:
         "config": {
             "workload": {"c1": "c1 fp32 decode B=4", "c2": "c2 Qwen3-0.6B-shaped decode B=64 bf16",
                          "c4": "c4 Llama-3-8B-shaped decode B=256 bf16 paged KV",
-                         "c5": "c5 long-context fp8-e4m3 KV decode B=8"}[args.workload],
+                         "c5": "c5 long-context fp8-e4m3 KV decode B=8"}[name],
             "batch": w.batch, "num_q_heads": w.num_q_heads, "num_kv_heads": w.num_kv_heads,
             "head_dim": w.head_dim, "block_size": w.block_size, "total_keys": w.total_tokens,
             "max_len": int(w.seq_lens.max()), "kv_format": w.kv_format or str(w.dtype).replace("torch.", ""),
-            "algorithmic_bytes": alg_bytes, "pool_copies_rotated": n_pools,
-            "seed": 1000 + int(args.workload[1]), "generate_s": round(t_gen, 1),
+            "algorithmic_bytes": alg_bytes, "pool_copies_rotated": n_pools, "launches_per_step": passes,
+            "seed": 1000 + int(name[1]), "generate_s": round(t_gen, 1),
         },
         "roofline": {
             "bound": "hbm", "kernel": "decode_split_kernel", "achieved": achieved, "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
-            "kernel_ms": ms_split, "reduce_kernel_ms": ms_reduce,
+            "unit": "GB/s", "frac": achieved / HBM_PEAK_GBPS, "traffic": measured_traffic(name),
+            "kernel_ms": ms_split, "kernel_launches": n_kernel, "reduce_kernel_ms": ms_reduce,
         },
     }
     if gather is not None:
         result["gather"] = gather
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
-        if args.workload in ("c1", "c2") and args.cpu_seconds > 0:
+        if name in ("c1", "c2") and args.cpu_seconds > 0 and not getattr(args, "secondary_run", False):
             result["cpu_baseline_literal"] = cpu_literal(w)
+    return result
+
+
+def secondary(args, dev) -> dict:
+    """Short runs of the configurations that are not the headline: what the step costs, the dominant kernel
+    against its roofline and a few seconds of the CPU restatement, per workload."""
+    import copy
+
+    short = copy.copy(args)
+    short.steps, short.warmup, short.preheat_s = 30, 5, 0.3
+    short.cpu_seconds = min(args.cpu_seconds, 4.0)
+    short.copy_calibration = False
+    short.secondary_run = True
+    out = {}
+    for name in ("c2", "c5", "c3"):
+        r = bench_prefill_c3(short, dev) if name == "c3" else bench_decode(name, short, dev)
+        keep = ("metric", "value", "unit", "ms_per_step", "ms_per_step_median", "steps", "warmup", "tokens_per_s",
+                "dtype", "roofline", "cpu_baseline", "append", "pct_of_hbm_peak")
+        entry = {k: r[k] for k in keep if k in r}
+        entry["workload"] = r["config"]["workload"]
+        out[name] = entry
+        torch.cuda.empty_cache()
+    return out
+
+
+def main() -> int:
+    args = parse_args()
+    if args.traffic_from_pmc:
+        return traffic_from_pmc(*args.traffic_from_pmc)
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path, run with --gpus 1", file=sys.stderr)
+        return 2
+    from research_amd import _lib
+
+    _lib.load()  # no fallback: raises if the HIP library is missing
+    if not torch.cuda.is_available():
+        print("bench.py needs a HIP device", file=sys.stderr)
+        return 2
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    if args.workload == "engine":
+        return bench_engine(args, dev)
+    result = bench_prefill_c3(args, dev) if args.workload == "c3" else bench_decode(args.workload, args, dev)
+    if args.workload == "c4" and not args.no_secondary:
+        torch.cuda.empty_cache()
+        result["secondary"] = secondary(args, dev)
     print(json.dumps(result))
     return 0
 

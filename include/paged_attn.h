@@ -95,10 +95,18 @@ int pa_kv_gather(const void *k_cache, const void *v_cache, void *k_out, void *v_
  * leaves one partial result per piece in the workspace.  The size depends on
  * the shapes only, never on the sequence lengths, so one allocation serves
  * every step of a model.  Alignment: 256 bytes.  Contents need not be
- * initialised and are not kept between calls.
+ * initialised (a call recognises what an earlier call or nobody left there);
+ * calls that share a workspace must not overlap in time.
  */
 size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads, int head_dim,
                                  int kv_dtype);
+
+/*
+ * Kernel launches one pa_decode call of these shapes makes on the current device: 1 when the batch is large
+ * enough that the split pass merges a sequence's pieces itself, else 2 (split pass, reduction pass); negative on
+ * error.  For callers that time or profile the passes.  (No counterpart in the reference.)
+ */
+int pa_decode_passes(int batch, int num_q_heads, int num_kv_heads, int head_dim, int kv_dtype);
 
 /*
  * Paged decode attention.  Replaces FlexAttentionBackend._decode_attention
@@ -136,9 +144,11 @@ int pa_decode(const void *q, const void *k_cache, const void *v_cache, void *out
               size_t workspace_bytes, void *stream);
 
 /*
- * The two passes of pa_decode as separate calls, same arguments: pa_decode ==
+ * The two passes of pa_decode as separate calls, same arguments:
  * pa_decode_split followed by pa_decode_reduce on the same stream and
- * workspace.  For callers that time or schedule the passes separately.  (The
+ * workspace give pa_decode's result (to rounding: for large batches pa_decode
+ * merges inside its one launch, in another order; see pa_decode_passes).  For
+ * callers that time or schedule the passes separately.  (The
  * reference has one fused call site, attention/flex_backend.py:227-229; these
  * have no separate counterpart there.)
  */

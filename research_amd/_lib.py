@@ -38,6 +38,7 @@ SIGNATURES = {
          c_int, c_int, c_int, c_void_p],
     ),
     "pa_decode_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "pa_decode_passes": (c_int, [c_int, c_int, c_int, c_int, c_int]),
     "pa_decode": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p,

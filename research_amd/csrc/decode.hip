@@ -206,6 +206,13 @@ extern "C" size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_
     return plan_workspace(batch, plan, head_dim, kMaxSplitGrid).total;
 }
 
+extern "C" int pa_decode_passes(int batch, int num_q_heads, int num_kv_heads, int head_dim, int kv_dtype) {
+    pa_clear_error();
+    const HeadPlan plan = plan_heads(num_q_heads, num_kv_heads, head_dim, pa_dtype_bytes(kv_dtype));
+    if (batch < 0 || !plan.nrep_t) return pa_fail(PA_ERR_UNSUPPORTED, "pa_decode_passes: no kernel for these shapes");
+    return plan_merge_in_split(batch, plan, split_grid()) ? 1 : 2;
+}
+
 #define PA_DECODE_PARAMS                                                                                       \
     const void *q, const void *k_cache, const void *v_cache, void *out, const int32_t *block_tables,          \
         int64_t bt_stride, const int32_t *seq_lens, const int32_t *extra_zero_keys, const float *k_scale,      \
