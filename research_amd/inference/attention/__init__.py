@@ -1,7 +1,8 @@
 """Attention over a paged KV pool (reference: rollouts/rollouts/inference/attention/__init__.py).
 
-``FlexAttentionBackend`` is kept as an alias of ``HipPagedAttentionBackend`` so
-that ``from ...attention import CacheConfig, FlexAttentionBackend`` keeps working.
+``FlexAttentionBackend`` is ``HipPagedAttentionBackend`` with the reference's decode numerics as
+defaults, so that ``from ...attention import CacheConfig, FlexAttentionBackend`` keeps working and
+keeps its results.
 """
 
 from .config import CacheConfig

@@ -9,7 +9,13 @@ pointers of the same tensors to the C ABI of ``libpaged_attn.so``; torch is used
 for device memory and the current stream only.  There is no eager fallback: a
 missing library, or tensors that are not on a HIP device, raise.
 
-Differences from the reference, all deliberate:
+Two classes: ``HipPagedAttentionBackend`` defaults to exact-length, windowed
+decode (the first and third points below); ``FlexAttentionBackend``, the
+reference's name, is the same class with the reference's decode numerics as
+defaults (``pad_zero_keys=True, window_in_decode=False``), so code that imports
+it by that name gets the reference's results on ragged batches too.
+
+Differences of ``HipPagedAttentionBackend`` from the reference, all deliberate:
 
 * Decode attends exactly ``seq_lens[b]`` keys per sequence.  The reference
   zero-pads a ragged batch to its longest sequence and attends without a mask
@@ -169,7 +175,7 @@ class HipPagedAttentionBackend:
         The append runs first, so a decode step sees its own token.
         """
         if ctx.slot_mapping is not None:
-            self._store_kv(k, v, layer_idx, ctx.slot_mapping, _step=self._step(ctx))
+            self._store_kv(k, v, layer_idx, ctx.slot_mapping, _step=self._step(ctx), _ctx=ctx)
         return self._attend(q, k, v, layer_idx, ctx)
 
     __call__ = forward
@@ -217,8 +223,8 @@ class HipPagedAttentionBackend:
             slots = self._device_slots(ctx.slot_mapping, n, step)
         dense = ctx.is_prefill and getattr(ctx, "prefix_lens", None) is None  # attends the step's own K/V
         kc, vc = self._layer(layer_idx)
-        if self._fp8 and slots is not None and step.touched is None:
-            step.touched = ops.touched_blocks(slots, cfg.block_size, cfg.num_blocks)
+        if self._fp8 and slots is not None:
+            self._touched(step, slots, ctx, layer_idx)
         if self._fp8 and slots is not None and not dense:
             ops.rope_kv_append_e4m3(q3, k3, v3, cos2, sin2, kc, vc, self.k_scale[layer_idx], self.v_scale[layer_idx],
                                     slots, cfg.block_size, positions=pos, q_out=q_rot, touched=step.touched)
@@ -269,7 +275,13 @@ class HipPagedAttentionBackend:
             if isinstance(block_tables, Tensor):
                 if block_tables.dim() != 2:
                     raise ValueError("block_tables tensor must be [num_seqs, width], padded with -1")
-                step.tables = block_tables.to(device=self.k_cache.device, dtype=torch.int32).contiguous()
+                if block_tables.device.type == "cuda":
+                    # used as it is: a caller that rewrites it in place between graph replays must be read live
+                    if block_tables.dtype != torch.int32 or not block_tables.is_contiguous():
+                        raise TypeError("a device-resident block_tables must be a contiguous int32 tensor")
+                    step.tables = block_tables
+                else:
+                    step.tables = block_tables.to(device=self.k_cache.device, dtype=torch.int32).contiguous()
             elif isinstance(block_tables, np.ndarray):
                 if block_tables.ndim != 2:
                     raise ValueError("block_tables array must be [num_seqs, width], padded with -1")
@@ -313,7 +325,9 @@ class HipPagedAttentionBackend:
         if isinstance(slot_mapping, Tensor) and slot_mapping.device.type == "cuda":
             # already on the device: used as it is (out-of-range slots are dropped by the kernel, not reported)
             self._require_device(*tensors, self.k_cache)
-            slots = slot_mapping.to(torch.int64).contiguous()
+            if slot_mapping.dtype != torch.int64 or not slot_mapping.is_contiguous():
+                raise TypeError("a device-resident slot_mapping must be a contiguous int64 tensor")
+            slots = slot_mapping
         else:
             if isinstance(slot_mapping, Tensor):
                 slot_mapping = slot_mapping.numpy()
@@ -328,8 +342,35 @@ class HipPagedAttentionBackend:
         return slots
 
     # ------------------------------------------------------------------ KV append
+    def _touched(self, step: Optional[_StepTensors], slots: Tensor, ctx: Optional[InferenceContext],
+                 layer_idx: int) -> Tensor:
+        """int32 device list of the blocks an fp8 append works on (one workgroup each; entries outside the pool
+        are skipped by the kernel).
+
+        A decode step whose slot mapping lives on the device writes one row per sequence, and every sequence
+        writes into a block of its own, so the list is simply each slot's block (-1 for a padding row's slot
+        -1): two device operations with no data-dependent shape and no host round trip, which a graph capture
+        can record.  It is rebuilt at the first layer of every pass, so a pass recorded after an eager warm-up
+        on the same context object contains it.  Everything else (prefill, host slot mappings) takes the distinct
+        blocks, once per step."""
+        cfg = self.config
+        on_device = (ctx is not None and not ctx.is_prefill and isinstance(ctx.slot_mapping, Tensor)
+                     and ctx.slot_mapping.device.type == "cuda")
+        if on_device:
+            if step is None or step.touched is None or layer_idx == 0:
+                touched = torch.div(slots, cfg.block_size, rounding_mode="floor").to(torch.int32)
+                if step is None:
+                    return touched
+                step.touched = touched
+            return step.touched
+        if step is None:
+            return ops.touched_blocks(slots, cfg.block_size, cfg.num_blocks)
+        if step.touched is None:
+            step.touched = ops.touched_blocks(slots, cfg.block_size, cfg.num_blocks)
+        return step.touched
+
     def _store_kv(self, k: Tensor, v: Tensor, layer_idx: int, slot_mapping: Tuple[int, ...],
-                  _step: Optional[_StepTensors] = None) -> None:
+                  _step: Optional[_StepTensors] = None, _ctx: Optional[InferenceContext] = None) -> None:
         """``cache[layer, slot] = row`` for every non-negative slot (flex_backend.py:116-142)."""
         cfg = self.config
         k_flat = k.reshape(-1, cfg.num_kv_heads, cfg.head_dim)
@@ -353,12 +394,7 @@ class HipPagedAttentionBackend:
         kc, vc = self._layer(layer_idx)
         if self._fp8:
             # rows are encoded with the tile's scale; a row that raises a tile's absmax re-rounds the tile
-            if _step is not None and _step.touched is not None:
-                touched = _step.touched
-            else:
-                touched = ops.touched_blocks(slots, cfg.block_size, cfg.num_blocks)
-                if _step is not None:
-                    _step.touched = touched
+            touched = self._touched(_step, slots, _ctx, layer_idx)
             ops.kv_append_e4m3(kc, vc, self.k_scale[layer_idx], self.v_scale[layer_idx], k_flat, v_flat, slots,
                                cfg.block_size, touched)
             return
@@ -392,10 +428,14 @@ class HipPagedAttentionBackend:
         step = self._step(ctx)
         if step.seq_lens is None:
             self._tables(step, ctx.block_tables[:batch])
-            if isinstance(ctx.seq_lens, Tensor) and ctx.seq_lens.device.type == "cuda" and not self.pad_zero_keys:
+            if isinstance(ctx.seq_lens, Tensor) and ctx.seq_lens.device.type == "cuda":
                 # already on the device: used as it is, with no host copy (a caller replaying a captured graph
-                # updates the tensor in place between replays)
-                step.seq_lens = ctx.seq_lens[:batch].to(torch.int32).contiguous()
+                # updates the tensor in place between replays, so a converted copy would go stale)
+                if ctx.seq_lens.dtype != torch.int32 or not ctx.seq_lens.is_contiguous():
+                    raise TypeError("a device-resident seq_lens must be a contiguous int32 tensor")
+                step.seq_lens = ctx.seq_lens[:batch]
+                if self.pad_zero_keys and batch > 0:
+                    step.extra_zero = (step.seq_lens.max() - step.seq_lens).to(torch.int32)
             else:
                 lens = self._lens(ctx.seq_lens, batch)
                 step.seq_lens = self._to_device(lens.astype(np.int32))
@@ -506,4 +546,12 @@ class HipPagedAttentionBackend:
 
 
 # name under which code written for the reference finds its backend
-FlexAttentionBackend = HipPagedAttentionBackend
+class FlexAttentionBackend(HipPagedAttentionBackend):
+    """The reference's class name with the reference's numerics as defaults: a ragged decode batch attends
+    the zero-padded keys the reference's unmasked SDPA sees (flex_backend.py:253-264, :227-229;
+    ``pad_zero_keys=True``) and a configured sliding window is not applied in decode unless the context carries
+    a mask (:220-225; ``window_in_decode=False``).  ``HipPagedAttentionBackend`` itself defaults to
+    exact-length, windowed decode."""
+
+    def __init__(self, config: CacheConfig, pad_zero_keys: bool = True, window_in_decode: bool = False) -> None:
+        super().__init__(config, pad_zero_keys=pad_zero_keys, window_in_decode=window_in_decode)

@@ -126,9 +126,6 @@ class InferenceEngine:
             # the rotary tables end at max_position_embeddings; later positions would all take the last row
             raise ValueError(f"max_model_len={config.max_model_len} exceeds the model's "
                              f"max_position_embeddings={limit}")
-        if config.use_graphs and getattr(self.backend.config, "kv_format", None) == "fp8_e4m3":
-            # the fp8 append works per touched block, and the set of touched blocks has a data-dependent size
-            raise ValueError("use_graphs needs a bf16 / fp16 / fp32 KV pool: the fp8 append is not capturable")
         self.tokenizer = tokenizer if tokenizer is not None else self._load_tokenizer(config.model_path)
         self.scheduler_config = SchedulerConfig(
             max_batch_size=config.max_batch_size,

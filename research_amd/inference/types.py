@@ -27,7 +27,7 @@ class InferenceContext:
                       its tokens, in order.
     ``seq_lens``      decode: context length of each sequence *including* the
                       token appended in this step.
-    ``block_mask``    opaque mask object; this backend accepts ``None`` only.
+    ``block_mask``    ``None`` (the configured mask) or a ``PagedMask`` of attention/mask.py that replaces it.
 
     Extension (not in the reference, keyword-only in spirit, defaulted so the
     reference's positional construction still works):

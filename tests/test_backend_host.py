@@ -29,7 +29,11 @@ def test_cache_config_surface():
 
 def test_backend_attributes_match_reference_surface():
     be = HipPagedAttentionBackend(_cfg())
-    assert FlexAttentionBackend is HipPagedAttentionBackend
+    # the reference's name: the same class with the reference's decode numerics as defaults
+    assert issubclass(FlexAttentionBackend, HipPagedAttentionBackend)
+    ref = FlexAttentionBackend(_cfg())
+    assert ref.pad_zero_keys and not ref.window_in_decode
+    assert not be.pad_zero_keys and be.window_in_decode
     assert be.num_heads_per_kv == 1 and be.scale == 32**-0.5
     assert be.k_cache.shape == (2, 64, 4, 32) and be.k_cache.dtype == torch.bfloat16
     assert not be.k_cache.any() and not be.v_cache.any()

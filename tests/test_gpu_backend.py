@@ -11,6 +11,7 @@ from research_amd.inference import (
     Attention,
     CacheConfig,
     FlexAttentionBackend,
+    HipPagedAttentionBackend,
     InferenceContext,
     PagedKVCache,
     allocate_and_build_context,
@@ -27,7 +28,7 @@ pytestmark = pytest.mark.gpu
 def test_store_kv_like_the_reference_script():
     announce("backend store_kv")
     config = CacheConfig(num_layers=2, num_kv_heads=4, head_dim=32, num_blocks=16, block_size=4, device="cuda")
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(8)
     k = torch.randn(1, 4, 4, 32, device="cuda", dtype=torch.bfloat16)
     v = torch.randn(1, 4, 4, 32, device="cuda", dtype=torch.bfloat16)
@@ -40,7 +41,7 @@ def test_store_kv_like_the_reference_script():
 def test_attention_correctness_like_the_reference_script():
     announce("backend prefill correctness")
     config = CacheConfig(num_layers=1, num_kv_heads=2, head_dim=32, num_blocks=16, block_size=16, device="cuda")
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(4)
     torch.manual_seed(42)
     q = torch.randn(2, 8, 4, 32, device="cuda", dtype=torch.bfloat16)
@@ -58,7 +59,7 @@ def test_end_to_end_like_the_reference_script_with_values():
     announce("backend end to end")
     cache = PagedKVCache(num_blocks=16, block_size=4)
     config = CacheConfig(num_layers=2, num_kv_heads=4, head_dim=32, num_blocks=16, block_size=4, device="cuda")
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(8)
     layer = Attention(layer_idx=1, backend=backend)
     torch.manual_seed(1)
@@ -98,7 +99,7 @@ def test_dropped_token_when_the_table_cannot_grow():
     cache = PagedKVCache(num_blocks=4, block_size=2)
     config = CacheConfig(num_layers=1, num_kv_heads=1, head_dim=32, num_blocks=4, block_size=2, device="cuda",
                          dtype=torch.float32)
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(2)
     ctx, _ = allocate_and_build_context(cache, 0, [7])
     torch.manual_seed(2)
@@ -128,7 +129,7 @@ def test_ragged_decode_both_semantics_on_c1():
     for pad in (False, True):
         config = CacheConfig(num_layers=1, num_kv_heads=2, head_dim=64, num_blocks=128, block_size=16,
                              dtype=torch.float32, device="cuda")
-        backend = FlexAttentionBackend(config, pad_zero_keys=pad)
+        backend = HipPagedAttentionBackend(config, pad_zero_keys=pad)
         backend.set_num_heads(8)
         backend.k_cache[0].copy_(w.k_pool)
         backend.v_cache[0].copy_(w.v_pool)
@@ -141,6 +142,64 @@ def test_ragged_decode_both_semantics_on_c1():
             assert_close(out, lit, 1e-5, "literal reference restatement")
 
 
+def test_reference_name_keeps_reference_decode_numerics():
+    """``FlexAttentionBackend`` with its defaults on a ragged batch, with a sliding window configured: the
+    statement of flex_backend.py:227-229 evaluated with torch itself on the gathered batch of :253-264 (rows
+    past a sequence's length are zero keys, no mask, no window in decode), for fp32 and bf16, with tuple and
+    with device-resident context fields."""
+    announce("backend reference-name defaults against torch SDPA")
+    w = make_decode("c1")
+    tables = tuple(tuple(int(b) for b in t) for t in w.block_tables)
+    lens = tuple(int(n) for n in w.seq_lens)
+    assert len(set(lens)) > 1
+    n_rep = w.num_q_heads // w.num_kv_heads
+    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 2e-2)):
+        config = CacheConfig(num_layers=1, num_kv_heads=2, head_dim=64, num_blocks=128, block_size=16,
+                             sliding_window=24, dtype=dtype, device="cuda")
+        backend = FlexAttentionBackend(config)
+        backend.set_num_heads(8)
+        backend.k_cache[0].copy_(w.k_pool)
+        backend.v_cache[0].copy_(w.v_pool)
+        q = w.q[:, None].to(dtype).cuda()
+        # the gathered, zero-padded batch, by plain indexing of the pool
+        k_g = torch.zeros(len(lens), max(lens), 2, 64, dtype=dtype, device="cuda")
+        v_g = torch.zeros_like(k_g)
+        for b, (blocks, n) in enumerate(zip(tables, lens)):
+            pos = torch.arange(n)
+            slots = (torch.tensor(blocks)[pos // 16] * 16 + pos % 16).cuda()
+            k_g[b, :n], v_g[b, :n] = backend.k_cache[0, slots], backend.v_cache[0, slots]
+        want = torch.nn.functional.scaled_dot_product_attention(
+            q.float().transpose(1, 2), k_g.float().transpose(1, 2).repeat_interleave(n_rep, dim=1),
+            v_g.float().transpose(1, 2).repeat_interleave(n_rep, dim=1), is_causal=False,
+            scale=backend.scale).transpose(1, 2)
+        ctx = InferenceContext(is_prefill=False, block_tables=tables, seq_lens=lens, max_seq_len=max(lens))
+        assert_close(backend.forward(q, None, None, 0, ctx), want, tol, f"{dtype} tuples")
+        width = max(len(t) for t in tables)
+        dev_tables = torch.tensor([list(t) + [-1] * (width - len(t)) for t in tables], dtype=torch.int32, device="cuda")
+        dev_lens = torch.tensor(lens, dtype=torch.int32, device="cuda")
+        ctx = InferenceContext(is_prefill=False, block_tables=dev_tables, seq_lens=dev_lens, max_seq_len=max(lens))
+        assert_close(backend.forward(q, None, None, 0, ctx), want, tol, f"{dtype} device-resident fields")
+        # the native class on the same context masks instead: a different result on the shorter sequences
+        native = HipPagedAttentionBackend(CacheConfig(num_layers=1, num_kv_heads=2, head_dim=64, num_blocks=128,
+                                                      block_size=16, dtype=dtype, device="cuda"))
+        native.set_num_heads(8)
+        native.k_cache[0].copy_(w.k_pool)
+        native.v_cache[0].copy_(w.v_pool)
+        masked = native.forward(q, None, None, 0, ctx).float()
+        short = [b for b, n in enumerate(lens) if n < max(lens)]
+        assert (masked[short] - want[short]).abs().max() > 10 * tol
+    # device-resident fields of another integer type are refused, not converted
+    with pytest.raises(TypeError, match="int32"):
+        backend.forward(q, None, None, 0, InferenceContext(
+            is_prefill=False, block_tables=dev_tables, seq_lens=dev_lens.long(), max_seq_len=max(lens)))
+    with pytest.raises(TypeError, match="int32"):
+        backend.forward(q, None, None, 0, InferenceContext(
+            is_prefill=False, block_tables=dev_tables.long(), seq_lens=dev_lens, max_seq_len=max(lens)))
+    with pytest.raises(TypeError, match="int64"):
+        backend._store_kv(torch.zeros(2, 2, 64, device="cuda", dtype=dtype), torch.zeros(2, 2, 64, device="cuda", dtype=dtype),
+                          0, torch.tensor([0, 1], dtype=torch.int32, device="cuda"))
+
+
 def test_chunked_prefill_through_the_backend_with_allocator_shared_prefix():
     """Two prompts with a common 32-token prefix: the allocator hands out the same
     leading block ids, the second prompt is prefilled as a chunk over the cached prefix."""
@@ -148,7 +207,7 @@ def test_chunked_prefill_through_the_backend_with_allocator_shared_prefix():
     bs = 16
     cache = PagedKVCache(num_blocks=32, block_size=bs)
     config = CacheConfig(num_layers=1, num_kv_heads=2, head_dim=64, num_blocks=32, block_size=bs, device="cuda")
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(4)
     rng = np.random.default_rng(3)
     prefix = rng.integers(0, 100, 32).tolist()
@@ -178,7 +237,7 @@ def test_fp8_backend_decode():
     w = make_decode("c5", batch=2, len_range=(500, 2000))
     config = CacheConfig(num_layers=1, num_kv_heads=8, head_dim=128, num_blocks=w.num_blocks, block_size=16,
                          device="cuda", kv_format="fp8_e4m3")
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(32)
     backend.quantize_from(w.k_pool.cuda(), w.v_pool.cuda(), 0)
     tables = tuple(tuple(int(b) for b in t) for t in w.block_tables)
@@ -199,7 +258,7 @@ def test_fp8_backend_prefill_then_decode_appends():
     hq, hkv, d, bs = 8, 2, 64, 16
     config = CacheConfig(num_layers=2, num_kv_heads=hkv, head_dim=d, num_blocks=16, block_size=bs, device="cuda",
                          kv_format="fp8_e4m3")
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(hq)
     cache = PagedKVCache(config.num_blocks, bs)
     layer = 1
@@ -244,7 +303,7 @@ def test_sliding_window_through_the_backend():
                          sliding_window=window)
     outs = {}
     for in_decode in (True, False):
-        backend = FlexAttentionBackend(config, window_in_decode=in_decode)
+        backend = HipPagedAttentionBackend(config, window_in_decode=in_decode)
         backend.set_num_heads(hq)
         cache = PagedKVCache(8, bs)
         n = 21
@@ -271,7 +330,7 @@ def test_context_fields_as_arrays_and_tensors():
     w = make_decode("c2", batch=6, len_range=(20, 300), seed=8)
     config = CacheConfig(num_layers=1, num_kv_heads=8, head_dim=128, num_blocks=w.num_blocks, block_size=16,
                          device="cuda", dtype=torch.bfloat16)
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(16)
     backend.k_cache[0].copy_(w.k_pool.cuda())
     backend.v_cache[0].copy_(w.v_pool.cuda())
@@ -307,7 +366,7 @@ def test_block_mask_objects_through_the_backend():
     hq, hkv, d, bs = 8, 2, 64, 16
     config = CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=16, block_size=bs, device="cuda",
                          sliding_window=9)
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(hq)
     b, t = 2, 100
     q = torch.randn(b, t, hq, d, generator=g).to(torch.bfloat16)
@@ -349,7 +408,7 @@ def test_prefix_reuse_through_the_radix_cache():
     g = torch.Generator().manual_seed(71)
     hq, hkv, d, bs = 8, 2, 64, 16
     config = CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=32, block_size=bs, device="cuda")
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(hq)
     cache = RadixKVCache(32, bs)
     prompt_len, n_rollouts = 70, 4  # 4 full blocks + 6 tokens
@@ -398,7 +457,7 @@ def test_fp8_blocks_dequantise_bit_exact_and_chunked_prefill_over_an_fp8_pool():
     hq, hkv, d, bs, nb = 8, 2, 128, 16, 24
     config = CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=nb, block_size=bs, device="cuda",
                          kv_format="fp8_e4m3")
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(hq)
     pool_k = torch.randn(nb * bs, hkv, d, generator=g).to(torch.bfloat16)
     pool_v = (torch.randn(nb * bs, hkv, d, generator=g) * 3).to(torch.bfloat16)

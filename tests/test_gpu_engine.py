@@ -168,13 +168,42 @@ def test_rollouts_of_one_prompt_prefill_in_two_passes():
             assert sample.logprobs == pytest.approx(logprobs, abs=2e-4)
 
 
-def test_graphs_refuse_an_fp8_pool():
+def _fp8_engine(use_graphs):
     backend = HipPagedAttentionBackend(CacheConfig(
-        num_layers=CFG.num_layers, num_kv_heads=CFG.num_kv_heads, head_dim=CFG.head_dim, num_blocks=16,
+        num_layers=CFG.num_layers, num_kv_heads=CFG.num_kv_heads, head_dim=CFG.head_dim, num_blocks=64,
         block_size=16, device="cuda", dtype=torch.bfloat16, kv_format="fp8_e4m3"))
+    torch.manual_seed(1)
     model = PagedLlama(CFG, backend).to(torch.bfloat16).cuda().eval()
-    with pytest.raises(ValueError, match="use_graphs"):
-        InferenceEngine(EngineConfig(model_path="", cache_type="radix", use_graphs=True, max_model_len=512), model=model)
+    engine = InferenceEngine(EngineConfig(model_path="", cache_type="radix", max_batch_size=8, max_model_len=512,
+                                          use_graphs=use_graphs), model=model)
+    return engine, {k: v.detach().float().cpu() for k, v in model.state_dict().items()}
+
+
+def test_decode_graphs_on_an_fp8_pool():
+    """use_graphs with an fp8-e4m3 pool: the append's block list is computed on the device inside the captured
+    pass.  A full bucket (8 unrelated prompts, all finishing together) replays exactly the launches of the eager
+    engine, so tokens and log probabilities are those of the eager engine; a padded bucket (6 prompts, some
+    sharing a prefix) is held to the full-precision checker like the eager fp8 engine."""
+    announce("engine fp8 pool with graphs")
+    g = torch.Generator().manual_seed(44)
+    full = [torch.randint(0, 211, (n,), generator=g).tolist() for n in (5, 16, 17, 31, 40, 9, 23, 12)]
+    eager, _ = _fp8_engine(False)
+    want = _by_prompt(eager.generate(full, SamplingParams(temperature=0.0, max_tokens=14)))
+    engine, weights = _fp8_engine(True)
+    got = _by_prompt(engine.generate(full, SamplingParams(temperature=0.0, max_tokens=14)))
+    assert sorted(engine._decode_graphs) == [8]
+    for prompt in full:
+        (a,), (b,) = got[tuple(prompt)], want[tuple(prompt)]
+        assert a.completion_tokens == b.completion_tokens
+        assert a.logprobs == pytest.approx(b.logprobs, abs=1e-6)
+    assert torch.equal(engine.backend.k_cache.view(torch.uint8), eager.backend.k_cache.view(torch.uint8))
+    assert torch.equal(engine.backend.v_scale, eager.backend.v_scale)
+    samples = engine.generate(_prompts(), SamplingParams(temperature=0.0, max_tokens=12))
+    assert len(samples) == 6
+    for s in samples:
+        with torch.no_grad():
+            ref = mo.logprobs_of(weights, CFG, list(s.prompt_tokens + s.completion_tokens), len(s.prompt_tokens))
+        assert s.logprobs == pytest.approx(ref, abs=0.25)
 
 
 def test_max_model_len_beyond_the_rotary_table_is_refused():

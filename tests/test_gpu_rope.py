@@ -8,7 +8,7 @@ import torch
 
 from oracle import paged_oracle as po
 from research_amd import ops
-from research_amd.inference import CacheConfig, FlexAttentionBackend, InferenceContext
+from research_amd.inference import CacheConfig, HipPagedAttentionBackend, InferenceContext
 from tests.gpu_helpers import DEV, announce, assert_close
 
 pytestmark = pytest.mark.gpu
@@ -129,7 +129,7 @@ def test_forward_rope_through_the_backend():
     g = torch.Generator().manual_seed(61)
     hq, hkv, d, bs = 8, 2, 64, 16
     config = CacheConfig(num_layers=2, num_kv_heads=hkv, head_dim=d, num_blocks=8, block_size=bs, device="cuda")
-    fused, plain = FlexAttentionBackend(config), FlexAttentionBackend(config)
+    fused, plain = HipPagedAttentionBackend(config), HipPagedAttentionBackend(config)
     for be in (fused, plain):
         be.set_num_heads(hq)
     caches = [PagedKVCache(8, bs), PagedKVCache(8, bs)]
@@ -198,7 +198,7 @@ def test_forward_rope_dense_prefill_into_an_fp8_pool():
     hq, hkv, d, bs = 8, 2, 64, 16
     config = CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=8, block_size=bs, device="cuda",
                          kv_format="fp8_e4m3")
-    backend = FlexAttentionBackend(config)
+    backend = HipPagedAttentionBackend(config)
     backend.set_num_heads(hq)
     n = 37
     q, k, v = (torch.randn(1, n, h, d, generator=g).to(torch.bfloat16) for h in (hq, hkv, hkv))
