@@ -1,6 +1,11 @@
 // Host entry point of causal prefill attention over a paged context.
 #include "prefill_mfma.h"
 
+namespace pa_decode_detail {
+constexpr int kPaCapTiles = 1600;  // (prefill_asm.h)
+prefill_mfma_fn pa_prefill_asm_kernel(int dtype);
+}
+
 using namespace pa_decode_detail;
 
 namespace {
@@ -43,8 +48,13 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     hipStream_t s = (hipStream_t)stream;
     // bf16 / fp16 with head_dim 32, 64, 128 run on the matrix cores unless the caller asked for the vector kernel
     // (the matrix-core softmax takes the running maximum of the unscaled logits, which needs scale > 0)
-    const prefill_mfma_fn mfma =
+    prefill_mfma_fn mfma =
         force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
+    // head_dim 128 without a window or per-row first keys, blocks of a multiple of 16 tokens and a table the
+    // kernel's LDS copy can hold: the kernel whose whole tile loop is scheduled assembly
+    if (mfma && head_dim == 128 && window == 0 && !row_first_key && block_size % 16 == 0 && num_blocks > 0 &&
+        num_blocks * (int64_t)block_size < (1ll << 31) && bt_stride * (int64_t)block_size <= (int64_t)kPaCapTiles * kPfKeys)
+        mfma = pa_prefill_asm_kernel(dtype);
     if (mfma) {
         PA_REQUIRE(pa_aligned16(q) && pa_aligned16(out), "q and out must be 16-byte aligned");
         const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;

@@ -1,0 +1,333 @@
+// Causal prefill attention over a paged context for head_dim 128 (bf16 / fp16) with the whole tile loop in
+// scheduled assembly (prefill_mfma_loop.inc, written by gen_prefill_loop.py).
+//
+// Same computation, work split, LDS ring and operand layouts as prefill_mfma_kernel (prefill_mfma.h); what
+// differs is what surrounds the loop:
+//   * the pool slots of the context's 16-key groups are looked up once per workgroup and kept in LDS behind the
+//     ring (table A: slot of the group's first key; table B: first row of the group that does not exist, 16 =
+//     none), so a tile's loads are a table read, four scalar multiplies and eight direct loads, for any block
+//     size that is a multiple of 16;
+//   * rows past the context end and absent blocks are loaded from a slot that exists (the group's own block,
+//     or slot 0) and cleared in LDS before the tile is published; a zero key takes part with logit 0 and a
+//     zero value row, which is what the other kernels do for absent blocks;
+//   * every wave runs every tile of the workgroup with the causal / context-end mask applied where needed, so
+//     there is no per-wave tail code: a wave past its last key multiplies exact zeros;
+//   * sliding windows and per-row first keys are not handled here: the host launches prefill_mfma_kernel for
+//     those (and for other head sizes, block sizes that are not multiples of 16 and tables past kPaCapTiles).
+// Only the set-up, the first subtile's S^T and the write-out are compiled code, so the register allocator sees
+// one asm statement with pinned operands and little else.
+#pragma once
+#include "prefill_mfma.h"
+#include "prefill_mfma_loop.inc"
+
+namespace pa_decode_detail {
+
+constexpr int kPaCapTiles = 1600;  // tiles of 64 keys the slot tables hold: contexts of up to 102400 keys
+
+template <typename T>
+__global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseArgs a) {
+    using M = Mfma16<T>;
+    using X8 = typename M::x8;
+    constexpr int D = 128;
+    using G = PfTile<D>;
+    constexpr int KS = D / 16, DT = D / 32, NC = kPfCols;
+    constexpr int GPT = kPfKeys / 16;  // 16-key groups per tile
+    typedef __attribute__((address_space(3))) char lds_char;
+    constexpr int kRingBytes = kPfStages * 2 * G::BYTES;
+    constexpr int kTabABytes = kPaCapTiles * GPT * 4, kTabBBytes = (kPaCapTiles + 1) * GPT;
+    static_assert(kPfStages == 4 && kPfKeys == 64 && kPfWaves == 4 && NC == 2, "the assembly loop is written for this shape");
+    __shared__ __attribute__((aligned(1024))) char s_mem[kRingBytes + kTabABytes + kTabBBytes];
+    __shared__ int s_special;  // first tile with a row that does not exist
+    const uint32_t lds_base = (uint32_t)(size_t)(lds_char *)s_mem;
+    int32_t *tab_a = reinterpret_cast<int32_t *>(s_mem + kRingBytes);
+    uint8_t *tab_b = reinterpret_cast<uint8_t *>(s_mem + kRingBytes + kTabABytes);
+
+    const PoolArgs &p = a.p;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5, col = lane & 31;
+
+    // workgroup -> (kv head, group of 8 tasks, sequence), heaviest groups first when the prefix is short
+    // (the launch order of prefill_mfma_kernel)
+    const int kvh = blockIdx.x;
+    const int n_groups = gridDim.y, n_seqs = gridDim.z;
+    const int lin = blockIdx.y + n_groups * blockIdx.z;
+    const bool group_major = a.ctx_lens[0] - a.q_lens[0] < a.q_lens[0];
+    const int group = group_major ? n_groups - 1 - lin / n_seqs : (int)blockIdx.y;
+    const int b = group_major ? lin % n_seqs : (int)blockIdx.z;
+    const int q_len = a.q_lens[b];
+    const int ctx_len = a.ctx_lens[b];
+    const int prefix = ctx_len - q_len;
+    const int n_rowblocks = (q_len + kPfRows - 1) / kPfRows;
+    const int n_tasks = n_rowblocks * p.n_rep;
+    const int task0 = group * kPfTasks;
+    if (task0 >= n_tasks || q_len <= 0) return;  // uniform over the workgroup
+
+    bool live[NC];
+    int row0[NC], qh[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const int task = task0 + wave * NC + c;
+        live[c] = task < n_tasks;
+        const int rb = live[c] ? task / p.n_rep : 0;
+        const int rep = live[c] ? task - rb * p.n_rep : 0;
+        row0[c] = rb * kPfRows;
+        qh[c] = kvh * p.n_rep + rep;
+    }
+    const int last_task = min(n_tasks, task0 + kPfTasks) - 1;
+    const int wg_keys = min(ctx_len, prefix + min(q_len, (last_task / p.n_rep) * kPfRows + kPfRows));
+    const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys;  // >= 1
+    const int n_real = min(n_tiles, kPaCapTiles);           // tiles with table entries
+    // subtiles that reach past this key hold keys some row of the wave must not see
+    const int mask_from = min(prefix + min(row0[0], row0[1]) + 1, ctx_len);
+    // a lane's last visible key per column tile, less the 4 keys its half of the wave is ahead by
+    int lim[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) lim[c] = min(ctx_len - 1, prefix + row0[c] + col) - 4 * half;
+
+    if (tid == 0) s_special = n_tiles;
+    __syncthreads();
+
+    // ---- Q^T operands, staged through the (still empty) ring as whole rows: see prefill_mfma_kernel ----
+    constexpr int QRB = D * 2, QCPR = QRB / 16, QRPI = 64 / QCPR;
+    const uint32_t q_stage = (uint32_t)wave * (NC * 32 * QRB);
+    {
+        const int lrow = lane / QCPR, lslot = lane % QCPR;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const char *qb = reinterpret_cast<const char *>(a.q) + ((int64_t)a.q_starts[b] * p.hq + qh[c]) * (D * 2);
+#pragma unroll
+            for (int i = 0; i < 32 / QRPI; ++i) {
+                const int r = i * QRPI + lrow;
+                const int64_t grow = min(row0[c] + r, q_len - 1);
+                pf_dma16(lds_base + q_stage + (uint32_t)((c * 32 + i * QRPI) * QRB),
+                         qb + grow * p.hq * (D * 2) + ((lslot ^ (r & (QCPR - 1))) * 16));
+            }
+        }
+    }
+    // ---- slot tables (in flight together with the Q rows) ----
+    {
+        const int32_t *bt_seq = p.bt + (int64_t)b * p.bt_stride;
+        const int n_entries = n_real * GPT;
+        int first_special = n_tiles;
+        for (int i = tid; i < n_entries; i += kPfThreads) {
+            const int key = 16 * i, blk = key / p.bs;
+            int64_t bid = -1;
+            if (blk < p.bt_stride) bid = bt_seq[blk];
+            const bool present = bid >= 0 && bid < p.num_blocks;
+            const int rows = present ? min(max(ctx_len - key, 0), 16) : 0;  // rows of the group that exist
+            tab_a[i] = present ? (int32_t)(bid * p.bs + key % p.bs) : 0;
+            tab_b[i] = (uint8_t)rows;
+            if (rows < 16) first_special = min(first_special, i / GPT);
+        }
+        if (tid < GPT) tab_b[kPaCapTiles * GPT + tid] = 0;  // tiles past the tables: nothing exists
+        if (n_tiles > n_real) first_special = min(first_special, n_real);
+        if (first_special < n_tiles) atomicMin(&s_special, first_special);
+    }
+    pf_wait_loads<0>();
+    X8 qreg[NC][KS];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const int slot = (2 * ks + half) ^ (col & (QCPR - 1));
+            const uint4 raw = *reinterpret_cast<const uint4 *>(s_mem + q_stage + (c * 32 + col) * QRB + slot * 16);
+            qreg[c][ks] = __builtin_bit_cast(X8, raw);
+        }
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qreg[c][ks]));
+    __syncthreads();  // the tables are complete and the staged rows have been read: the ring may overwrite them
+    const int first_special = __builtin_amdgcn_readfirstlane(s_special);
+
+    // ---- loads of a tile: wave w fetches rows 4w .. 4w+3 of each of the tile's four 16-key groups ----
+    const int64_t tok_stride = (int64_t)p.hkv * D * 2;
+    const char *pool_k = reinterpret_cast<const char *>(p.k) + (int64_t)kvh * D * 2;
+    const char *pool_v = reinterpret_cast<const char *>(p.v) + (int64_t)kvh * D * 2;
+    const int ld_row = lane / G::CPR, ld_slot = lane % G::CPR;
+    const int arow = wave * G::RPL + ld_row;  // this lane's row inside a 16-key group
+    const uint32_t lane_k = (uint32_t)(arow * tok_stride) + (uint32_t)((ld_slot ^ G::swz_k(arow)) * 16);
+    const uint32_t lane_v = (uint32_t)(arow * tok_stride) + (uint32_t)((ld_slot ^ G::swz_v(arow)) * 16);
+    const uint32_t m0w = lds_base + (uint32_t)wave * (G::RPL * G::RB);
+    auto issue = [&](int tile) PF_INLINE {
+        const int src = tile < n_real ? tile : 0;
+        const uint32_t dst0 = m0w + (uint32_t)(tile % kPfStages) * 2 * G::BYTES;
+#pragma unroll
+        for (int n = 0; n < GPT; ++n) {
+            const uint32_t slot = (uint32_t)__builtin_amdgcn_readfirstlane(tab_a[src * GPT + n]);
+            const uint64_t ofs = (uint64_t)slot * (uint32_t)tok_stride;
+            pf_dma16(dst0 + n * 16 * G::RB, pf_scalar_ptr(pool_k + ofs), lane_k);
+            pf_dma16(dst0 + G::BYTES + n * 16 * G::RB, pf_scalar_ptr(pool_v + ofs), lane_v);
+        }
+    };
+    issue(0);
+    issue(1);
+    issue(2);
+    pf_wait_loads<4 * GPT>();  // tile 0 has landed
+    if (first_special == 0) {  // clear the rows of tile 0 that do not exist (the loop does it for later tiles)
+#pragma unroll
+        for (int n = 0; n < GPT; ++n)
+            if (arow >= tab_b[n]) {
+                const uint32_t at = (m0w - lds_base) + n * 16 * G::RB + lane * 16;
+                *reinterpret_cast<uint4 *>(s_mem + at) = uint4{0, 0, 0, 0};
+                *reinterpret_cast<uint4 *>(s_mem + at + G::BYTES) = uint4{0, 0, 0, 0};
+            }
+    }
+    __syncthreads();  // tile 0 is visible
+
+    // ---- operand read addresses (stage 0), as in prefill_mfma_kernel ----
+    uint32_t kad[KS], vad[DT];
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kad[ks] = lds_base + col * G::RB + (((2 * ks + half) ^ G::swz_k(col)) * 16);
+    {
+        const int g16 = lane >> 4, s16 = lane & 15;
+        const int v_key = 4 * (g16 >> 1) + (s16 >> 2);
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+            vad[dt] = lds_base + G::BYTES + v_key * G::RB +
+                      ((((4 * dt) ^ G::swz_v(v_key)) + 2 * (g16 & 1) + ((s16 & 3) >> 1)) * 16) + 8 * (s16 & 1);
+    }
+
+    // ---- first subtile: S^T, mask, row maxima; K operands of the second subtile ----
+    const float sc = p.scale_log2;
+    const float slack_raw = kPfSlack / sc;
+    f32x16 s0[NC];
+    X8 ka[KS];
+    float mx[NC];
+    {
+        auto read_k = [&](int kt) PF_INLINE {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+                ka[ks] = __builtin_bit_cast(X8, *reinterpret_cast<const __attribute__((address_space(3))) uint4 *>(
+                                                    (const lds_char *)(size_t)kad[ks] + kt * 32 * G::RB));
+        };
+        read_k(0);
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s0[c][i] = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int c = 0; c < NC; ++c) s0[c] = M::mma(ka[ks], qreg[c][ks], s0[c]);
+        read_k(1);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            float m = kNegBig;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                if (8 * (i >> 2) + (i & 3) > lim[c]) s0[c][i] = -INFINITY;
+                m = fmaxf(m, s0[c][i]);
+            }
+            const uint32_t u = __builtin_bit_cast(uint32_t, m);
+            const auto sw = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+            mx[c] = fmaxf(__builtin_bit_cast(float, (uint32_t)sw[0]), __builtin_bit_cast(float, (uint32_t)sw[1]));
+        }
+    }
+
+    f32x16 o[NC][DT];
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[c][dt][i] = 0.f;
+    // running maximum of the raw logits, its threshold and scaled copy, running sum (lazy rescale: see
+    // prefill_mfma_kernel)
+    float m_raw[NC], m_sc[NC], m_thr[NC], l_run[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) { m_raw[c] = kNegBig; m_thr[c] = kNegBig; m_sc[c] = kNegBig * sc; l_run[c] = 0.f; }
+
+    {
+        int n_left = n_tiles;
+        uint32_t s_t = 3, s_p = 1, s_kb = 0;
+        const uint32_t tab_a_base = lds_base + kRingBytes, tab_b_base = tab_a_base + kTabABytes;
+        const uint32_t sp_lo = (uint32_t)first_special, sp_span = (uint32_t)(n_tiles - first_special);
+        const uint32_t n_real_u = (uint32_t)n_real, cap_tiles = kPaCapTiles, mask_from_u = (uint32_t)mask_from;
+        const uint32_t lane16 = (uint32_t)lane * 16, arow_u = (uint32_t)arow;
+        const uint64_t pk = reinterpret_cast<uint64_t>(pool_k), pv = reinterpret_cast<uint64_t>(pool_v);
+        const uint32_t pklo = __builtin_amdgcn_readfirstlane((uint32_t)pk), pkhi = __builtin_amdgcn_readfirstlane((uint32_t)(pk >> 32));
+        const uint32_t pvlo = __builtin_amdgcn_readfirstlane((uint32_t)pv), pvhi = __builtin_amdgcn_readfirstlane((uint32_t)(pv >> 32));
+        const uint32_t stride = (uint32_t)tok_stride;
+#define PA_LOOP_OPERANDS                                                                                              \
+    : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[0][2]), "+{a[48:63]}"(o[0][3]),                    \
+      "+{a[64:79]}"(o[1][0]), "+{a[80:95]}"(o[1][1]), "+{a[96:111]}"(o[1][2]), "+{a[112:127]}"(o[1][3]),                \
+      "+{v[0:15]}"(s0[0]), "+{v[16:31]}"(s0[1]),                                                                      \
+      "+{a[192:195]}"(ka[0]), "+{a[196:199]}"(ka[1]), "+{a[200:203]}"(ka[2]), "+{a[204:207]}"(ka[3]),                   \
+      "+{a[208:211]}"(ka[4]), "+{a[212:215]}"(ka[5]), "+{a[216:219]}"(ka[6]), "+{a[220:223]}"(ka[7]),                   \
+      [mx0] "+v"(mx[0]), [mx1] "+v"(mx[1]), [msc0] "+v"(m_sc[0]), [msc1] "+v"(m_sc[1]), [thr0] "+v"(m_thr[0]),          \
+      [thr1] "+v"(m_thr[1]), [mraw0] "+v"(m_raw[0]), [mraw1] "+v"(m_raw[1]), [l0] "+v"(l_run[0]), [l1] "+v"(l_run[1]),  \
+      [ntiles] "+s"(n_left), [sT] "+s"(s_t), [sP] "+s"(s_p), [skb] "+s"(s_kb)                                         \
+    : "{a[128:131]}"(qreg[0][0]), "{a[132:135]}"(qreg[0][1]), "{a[136:139]}"(qreg[0][2]), "{a[140:143]}"(qreg[0][3]),   \
+      "{a[144:147]}"(qreg[0][4]), "{a[148:151]}"(qreg[0][5]), "{a[152:155]}"(qreg[0][6]), "{a[156:159]}"(qreg[0][7]),   \
+      "{a[160:163]}"(qreg[1][0]), "{a[164:167]}"(qreg[1][1]), "{a[168:171]}"(qreg[1][2]), "{a[172:175]}"(qreg[1][3]),   \
+      "{a[176:179]}"(qreg[1][4]), "{a[180:183]}"(qreg[1][5]), "{a[184:187]}"(qreg[1][6]), "{a[188:191]}"(qreg[1][7]),   \
+      [kad0] "v"(kad[0]), [kad1] "v"(kad[1]), [kad2] "v"(kad[2]), [kad3] "v"(kad[3]), [kad4] "v"(kad[4]),               \
+      [kad5] "v"(kad[5]), [kad6] "v"(kad[6]), [kad7] "v"(kad[7]), [vad0] "v"(vad[0]), [vad1] "v"(vad[1]),               \
+      [vad2] "v"(vad[2]), [vad3] "v"(vad[3]), [lanek] "v"(lane_k), [lanev] "v"(lane_v), [lane16] "v"(lane16),           \
+      [arow] "v"(arow_u), [lim0] "v"(lim[0]), [lim1] "v"(lim[1]), [sc] "s"(sc), [slack] "s"(slack_raw),                 \
+      [pklo] "s"(pklo), [pkhi] "s"(pkhi), [pvlo] "s"(pvlo), [pvhi] "s"(pvhi), [stride] "s"(stride), [m0w] "s"(m0w),     \
+      [nreal] "s"(n_real_u), [tabA] "s"(tab_a_base), [tabB] "s"(tab_b_base), [splo] "s"(sp_lo),                       \
+      [spspan] "s"(sp_span), [captiles] "s"(cap_tiles), [maskfrom] "s"(mask_from_u)                                   \
+    : "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47",  \
+      "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63",  \
+      "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79",  \
+      "v80", "v81", "v82", "v83", "v84", "v85", "v86", "v87", "v88", "v89", "v90", "v91", "v92", "v93", "v94", "v95",  \
+      "v96", "v97", "v98", "v99", "v100", "v101", "v102", "v103", "v104", "v105", "v106", "v107", "v108", "v109",      \
+      "v110", "v111", "v112", "v113", "v114", "v115", "v116", "a224", "a225", "a226", "a227", "a228", "a229", "a230",  \
+      "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244",  \
+      "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255", "s40", "s41", "s42",     \
+      "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58",  \
+      "s59", "vcc", "scc", "memory"
+        if constexpr (std::is_same<T, pa_bf16>::value) {
+            asm volatile(PF_LOOP_ASM_BF16 PA_LOOP_OPERANDS);
+        } else {
+            asm volatile(PF_LOOP_ASM_F16 PA_LOOP_OPERANDS);
+        }
+#undef PA_LOOP_OPERANDS
+    }
+
+    // ---- normalise; rows go through LDS so that every store instruction writes whole 256-byte rows ----
+    __syncthreads();  // every wave is done with the ring
+    const uint32_t out_stage = (uint32_t)wave * (NC * 32 * QRB);  // this wave's 64 rows of 256 bytes
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const float l_tot = l_run[c] + __shfl_xor(l_run[c], 32, 64);
+        const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+        // lane owns row col, d = 32*dt + 8*g + 4*half + j: the 8 bytes are half `half` of 16-byte chunk 4*dt + g,
+        // chunks swizzled by row so that the 32 rows of a store spread over the banks
+        char *rowp = s_mem + out_stage + (c * 32 + col) * QRB;
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                uint2 w;
+                w.x = M::pack(o[c][dt][4 * g] * inv, o[c][dt][4 * g + 1] * inv);
+                w.y = M::pack(o[c][dt][4 * g + 2] * inv, o[c][dt][4 * g + 3] * inv);
+                *reinterpret_cast<uint2 *>(rowp + (((4 * dt + g) ^ (col & 15)) * 16) + 8 * half) = w;
+            }
+    }
+    // (a wave reads only what it wrote itself: no barrier, the compiler waits for the LDS writes)
+    {
+        const int r_in = lane / QCPR, chunk = lane % QCPR;  // 4 rows per instruction, 16 bytes per lane
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            if (!live[c]) continue;
+            T *obase = reinterpret_cast<T *>(a.out) + (((int64_t)a.q_starts[b] + row0[c]) * p.hq + qh[c]) * D;
+#pragma unroll
+            for (int i = 0; i < 32 / QRPI; ++i) {
+                const int r = i * QRPI + r_in;
+                const uint4 v = *reinterpret_cast<const uint4 *>(s_mem + out_stage + (c * 32 + r) * QRB + ((chunk ^ (r & 15)) * 16));
+                if (row0[c] + r < q_len)
+                    *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(obase + (int64_t)r * p.hq * D) + chunk * 16) = v;
+            }
+        }
+    }
+}
+
+// nullptr unless the element type has this kernel
+prefill_mfma_fn pa_prefill_asm_kernel(int dtype);
+
+}  // namespace pa_decode_detail

@@ -197,3 +197,16 @@ def test_error_text_is_cleared_by_a_good_call():
     assert _lib.last_error() != ""
     assert _status("pa_kv_scatter", None, None, None, None, None, 0, 64, 8, 128, 2, None)[0] == 0
     assert _lib.last_error() == ""
+
+
+def test_generated_prefill_loop_is_current(tmp_path):
+    """research_amd/csrc/prefill_mfma_loop.inc is what gen_prefill_loop.py writes (the generator also checks the
+    instruction distances the hardware does not interlock, so a schedule that violates one cannot be committed)."""
+    import os
+    import subprocess
+    import sys
+    csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "research_amd", "csrc")
+    out = tmp_path / "loop.inc"
+    subprocess.run([sys.executable, os.path.join(csrc, "gen_prefill_loop.py"), str(out)], check=True,
+                   stdout=subprocess.DEVNULL)
+    assert out.read_text() == open(os.path.join(csrc, "prefill_mfma_loop.inc")).read()
