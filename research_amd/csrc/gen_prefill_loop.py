@@ -31,7 +31,7 @@ Register map (per lane; the kernel pins its variables to the same registers):
               (v95 also a row's last visible key relative to the subtile), v[97:98] pair sums, v99 scratch
   v[100:111]  LDS addresses of stages 2 and 3 (the operands hold those of stages 0 and 1)
   v[112:115]  zeros, v116 -inf
-  s[40:59]    scalars of the tile loads, the calls and the masks
+  s[40:63]    scalars of the tile loads, the calls, the masks and the rescale checks
 
 Usage: python3 gen_prefill_loop.py [output file]   (default: prefill_mfma_loop.inc beside this script)
 """
@@ -77,6 +77,9 @@ def S(buf, c):
 
 def PP(c, j):
     return 64 + 8 * c + j
+
+
+STUBS = []  # out-of-line code of the loop being generated: the common path of every check falls through
 
 
 class Ins:
@@ -147,11 +150,11 @@ def subtile_ops(ty, j, kt):
     streams = {}
 
     # ---- rescale check (start of the subtile) ----
-    chk = [Ins("v_cmp_gt_f32_e32 vcc, %[mx0], %[thr0]"), Ins("v_cmp_gt_f32_e64 s[52:53], %[mx1], %[thr1]"),
-           Ins("s_add_u32 %[skb], %[skb], 32", kind="salu"),  # first key of the subtile whose S^T is formed next
-           Ins("s_nop 0", kind="salu"), Ins("s_or_b64 vcc, vcc, s[52:53]", kind="salu"),
-           Ins(f"s_cbranch_vccz .Lpf_norescale_{j}{kt}_%=\n\ts_call_b64 s[50:51], .Lpf_rescale_%=\n.Lpf_norescale_{j}{kt}_%=:",
-               kind="salu", units=2, n=1)]
+    # (the two compares sit behind the maxima of the previous subtile, so their results are long there)
+    chk = [Ins("s_add_u32 %[skb], %[skb], 32", kind="salu"),  # first key of the subtile whose S^T is formed next
+           Ins("s_or_b64 vcc, s[60:61], s[62:63]", kind="salu"),
+           Ins(f"s_cbranch_vccnz .Lpf_rescale_{j}{kt}_%=\n.Lpf_rescaled_{j}{kt}_%=:", kind="salu", n=1)]
+    STUBS.append([f".Lpf_rescale_{j}{kt}_%=:", "s_call_b64 s[50:51], .Lpf_rescale_%=", f"s_branch .Lpf_rescaled_{j}{kt}_%="])
     streams["chk"] = [Op(chk, 0, 0)]
 
     # ---- LDS operand reads ----
@@ -173,8 +176,10 @@ def subtile_ops(ty, j, kt):
         # (a tile in [splo, splo + spspan) has rows past the context end or in absent blocks: the wave clears the
         # rows it loaded itself; unsigned compare of the distance covers both ends)
         lds.append(Op(Ins("s_waitcnt vmcnt(8)\n\ts_sub_u32 s56, %[sP], %[splo]\n\ts_cmp_lt_u32 s56, %[spspan]\n"
-                          f"\ts_cbranch_scc0 .Lpf_nofix_{j}_%=\n\ts_call_b64 s[50:51], .Lpf_fixup_%=\n.Lpf_nofix_{j}_%=:\n"
-                          "\ts_add_u32 %[sP], %[sP], 1\n\ts_barrier", kind="sync", units=6, n=6), 16, 16))
+                          f"\ts_cbranch_scc1 .Lpf_fix_{j}_%=\n.Lpf_fixed_{j}_%=:\n"
+                          "\ts_add_u32 %[sP], %[sP], 1\n\t" + ("s_nop 0" if "nobarrier" in X else "s_barrier"),
+                          kind="sync", units=6, n=6), 16, 16))
+        STUBS.append([f".Lpf_fix_{j}_%=:", "s_call_b64 s[50:51], .Lpf_fixup_%=", f"s_branch .Lpf_fixed_{j}_%="])
     # K operands of subtile g+2 = subtile kt of the next tile (stage j+1)
     nstage = (j + 1) % NSTAGE
     for ks in range(KS):
@@ -192,8 +197,8 @@ def subtile_ops(ty, j, kt):
         ta, tb = 80 + 2 * (n % 4), 81 + 2 * (n % 4)
         return [Ins(f"v_fma_f32 v{ta}, v{s0}, %[sc], -%[msc{c}]", reads=(f"v{s0}",), writes=(f"v{ta}",)),
                 Ins(f"v_fma_f32 v{tb}, v{s0 + 1}, %[sc], -%[msc{c}]", reads=(f"v{s0 + 1}",), writes=(f"v{tb}",)),
-                Ins(f"v_exp_f32_e32 v{ta}, v{ta}", units=2, kind="trans", reads=(f"v{ta}",), writes=(f"v{ta}",)),
-                Ins(f"v_exp_f32_e32 v{tb}, v{tb}", units=2, kind="trans", reads=(f"v{tb}",), writes=(f"v{tb}",))]
+                Ins(f"{'v_mov_b32_e32' if 'noexp' in X else 'v_exp_f32_e32'} v{ta}, v{ta}", units=2, kind="trans", reads=(f"v{ta}",), writes=(f"v{ta}",)),
+                Ins(f"{'v_mov_b32_e32' if 'noexp' in X else 'v_exp_f32_e32'} v{tb}, v{tb}", units=2, kind="trans", reads=(f"v{tb}",), writes=(f"v{tb}",))]
 
     # The row sums are plain fp32 additions: v_dot2 on the packed words would be one instruction instead of
     # two, but it does not run beside the matrix unit (measured: a product followed by two of them takes 58
@@ -228,14 +233,16 @@ def subtile_ops(ty, j, kt):
     m = [93, 94]   # running maxima
     w = [95, 96]   # copies for the half-wave exchange
     # keys a row must not see: value i of a lane is key skb + 8*(i/4) + i%4 (+ 4*half, folded into lim)
-    blk = [f"s_add_u32 s56, %[skb], 32", f"s_cmp_le_u32 s56, %[maskfrom]", f"s_cbranch_scc1 .Lpf_nomask_{j}{kt}_%="]
+    blk = [f".Lpf_mask_{j}{kt}_%=:"]
     for c in range(NC):
         s = S(nb, c)
         blk.append(f"v_subrev_u32_e32 v95, %[skb], %[lim{c}]")
         for i in range(16):
             blk += [f"v_cmp_gt_i32_e32 vcc, {8 * (i >> 2) + (i & 3)}, v95", f"v_cndmask_b32_e32 v{s + i}, v{s + i}, v116, vcc"]
-    blk.append(f".Lpf_nomask_{j}{kt}_%=:")
-    mx.append(Op(Ins("\n\t".join(blk[:-1]) + "\n" + blk[-1], kind="salu", units=3, n=3,
+    blk.append(f"s_branch .Lpf_masked_{j}{kt}_%=")
+    STUBS.append(blk)
+    mx.append(Op(Ins(f"s_add_u32 s56, %[skb], 32\n\ts_cmp_gt_u32 s56, %[maskfrom]\n\ts_cbranch_scc1 .Lpf_mask_{j}{kt}_%=\n"
+                     f".Lpf_masked_{j}{kt}_%=:", kind="salu", units=3, n=3,
                      reads=[f"v{S(nb, c) + i}" for c in range(NC) for i in range(16)]), 21))
     for c in range(NC):
         s = S(nb, c)
@@ -252,6 +259,9 @@ def subtile_ops(ty, j, kt):
         mx.append(Op(Ins(f"v_permlane32_swap_b32_e32 v{m[c]}, v{w[c]}", kind="swap", reads=(f"v{m[c]}", f"v{w[c]}"),
                          writes=(f"v{m[c]}", f"v{w[c]}")), 21))
         mx.append(Op(Ins(f"v_max_f32_e32 %[mx{c}], v{m[c]}, v{w[c]}", reads=(f"v{m[c]}", f"v{w[c]}")), 21))
+    # does a row's maximum exceed its reference by more than the slack?  (read at the start of the next subtile)
+    mx.append(Op(Ins("v_cmp_gt_f32_e64 s[60:61], %[mx0], %[thr0]"), 21))
+    mx.append(Op(Ins("v_cmp_gt_f32_e64 s[62:63], %[mx1], %[thr1]"), 21))
     # (order: chain 0, copy 0, chain 1, copy 1, swap 0, max 0, swap 1, max 1: two instructions between a copy and its swap)
     streams["max"] = mx
 
@@ -271,19 +281,18 @@ def subtile_ops(ty, j, kt):
     groups = (0, 1) if kt == 0 else (2, 3)
     for n in groups:
         e = 24 if kt == 0 else 0
+        # slot * row stride (64 bits), then per tensor: LDS destination into m0, pool base + offset, load.  The
+        # two additions between the write of m0 and the load are the wait state that write needs.
         ldr.append(Op([Ins(f"s_mul_i32 s44, s{40 + n}, %[stride]", kind="salu"),
                        Ins(f"s_mul_hi_u32 s45, s{40 + n}, %[stride]", kind="salu")], e))
-        ldr.append(Op(Ins("s_add_u32 s46, %[pklo], s44\n\ts_addc_u32 s47, %[pkhi], s45", kind="salu", units=2, n=2), e))
-        ldr.append(Op(Ins("s_add_u32 s48, %[pvlo], s44\n\ts_addc_u32 s49, %[pvhi], s45", kind="salu", units=2, n=2), e))
         dst = dst_stage * STAGE + n * 4096
-        ldk = f"global_load_lds_dwordx4 %[lanek], s[46:47]"
-        ldv = f"global_load_lds_dwordx4 %[lanev], s[48:49]"
-        if "noloads" in X:
-            ldk = ldv = "s_nop 0"
-        ldr.append(Op(Ins(f"s_add_u32 m0, %[m0w], {dst}\n\ts_nop 0\n\t{ldk}",
-                          kind="vmem", units=4, n=3), e))
-        ldr.append(Op(Ins(f"s_add_u32 m0, %[m0w], {dst + TENSOR}\n\ts_nop 0\n\t{ldv}",
-                          kind="vmem", units=4, n=3), e))
+        ld = "s_nop 0" if "noloads" in X else "global_load_lds_dwordx4"
+        ldr.append(Op(Ins(f"s_add_u32 m0, %[m0w], {dst}\n\ts_add_u32 s46, %[pklo], s44\n\ts_addc_u32 s47, %[pkhi], s45\n"
+                          f"\t{ld} %[lanek], s[46:47]".replace("s_nop 0 %[lanek], s[46:47]", "s_nop 0"),
+                          kind="vmem", units=5, n=4), e))
+        ldr.append(Op(Ins(f"s_add_u32 m0, %[m0w], {dst + TENSOR}\n\ts_add_u32 s48, %[pvlo], s44\n\ts_addc_u32 s49, %[pvhi], s45\n"
+                          f"\t{ld} %[lanev], s[48:49]".replace("s_nop 0 %[lanev], s[48:49]", "s_nop 0"),
+                          kind="vmem", units=5, n=4), e))
     streams["ldr"] = ldr
     for k in list(streams):
         if f"drop_{k}" in X:  # (timing experiments only: results are garbage)
@@ -379,7 +388,10 @@ def add_waits(bodies):
         for body in bodies:
             cur = []
             for ins in body:
-                need = [pos[g] for g in ins.need if g in pos]
+                # (one wait per batch of reads: the first consumer of a batch waits for all of it, which has
+                # long been issued by then, instead of one wait instruction per operand)
+                fam = {g.rstrip("0123456789").rstrip("_") for g in ins.need}
+                need = [q for g, q in pos.items() if g.rstrip("0123456789").rstrip("_") in fam]
                 if need and max(need) > done:
                     n_after = issued - 1 - max(need)
                     n = min(15, n_after)
@@ -453,6 +465,7 @@ def rescale(ty):
 
 
 def loop_text(ty):
+    del STUBS[:]
     bodies = [tile_body(ty, j) for j in range(NSTAGE)]
     bodies = add_waits(bodies)
     if not (X - {""}):
@@ -464,12 +477,15 @@ def loop_text(ty):
     for dt in range(DT):
         lines.append(f"v_add_u32_e32 v{108 + dt}, {2 * STAGE}, %[vad{dt}]")
     lines += [f"v_mov_b32_e32 v{r}, 0" for r in range(112, 116)]
-    lines += ["v_mov_b32_e32 v116, 0xff800000", "s_waitcnt lgkmcnt(0)"]
+    lines += ["v_mov_b32_e32 v116, 0xff800000", "v_cmp_gt_f32_e64 s[60:61], %[mx0], %[thr0]",
+              "v_cmp_gt_f32_e64 s[62:63], %[mx1], %[thr1]", "s_waitcnt lgkmcnt(0)", "s_nop 3"]
     for j in range(NSTAGE):
         lines.append(f".Lpf_tile{j}_%=:")
         lines += [ins.text for ins in bodies[j]]
         lines += ["s_sub_u32 %[ntiles], %[ntiles], 1", "s_cmp_eq_u32 %[ntiles], 0", "s_cbranch_scc1 .Lpf_done_%="]
     lines.append("s_branch .Lpf_tile0_%=")
+    for stub in STUBS:
+        lines += stub
     lines.append(".Lpf_rescale_%=:")
     lines += rescale(ty)
     lines.append(".Lpf_fixup_%=:")

@@ -37,7 +37,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     constexpr int kTabABytes = kPaCapTiles * GPT * 4, kTabBBytes = (kPaCapTiles + 1) * GPT;
     static_assert(kPfStages == 4 && kPfKeys == 64 && kPfWaves == 4 && NC == 2, "the assembly loop is written for this shape");
     __shared__ __attribute__((aligned(1024))) char s_mem[kRingBytes + kTabABytes + kTabBBytes];
-    __shared__ int s_special;  // first tile with a row that does not exist
+    __shared__ int s_special[kPfWaves];  // per wave: first tile with a row that does not exist
     const uint32_t lds_base = (uint32_t)(size_t)(lds_char *)s_mem;
     int32_t *tab_a = reinterpret_cast<int32_t *>(s_mem + kRingBytes);
     uint8_t *tab_b = reinterpret_cast<uint8_t *>(s_mem + kRingBytes + kTabABytes);
@@ -86,9 +86,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 #pragma unroll
     for (int c = 0; c < NC; ++c) lim[c] = min(ctx_len - 1, prefix + row0[c] + col) - 4 * half;
 
-    if (tid == 0) s_special = n_tiles;
-    __syncthreads();
-
     // ---- Q^T operands, staged through the (still empty) ring as whole rows: see prefill_mfma_kernel ----
     constexpr int QRB = D * 2, QCPR = QRB / 16, QRPI = 64 / QCPR;
     const uint32_t q_stage = (uint32_t)wave * (NC * 32 * QRB);
@@ -123,7 +120,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         }
         if (tid < GPT) tab_b[kPaCapTiles * GPT + tid] = 0;  // tiles past the tables: nothing exists
         if (n_tiles > n_real) first_special = min(first_special, n_real);
-        if (first_special < n_tiles) atomicMin(&s_special, first_special);
+        // minimum over the wave here, over the waves behind the barrier below
+#pragma unroll
+        for (int d = 32; d >= 1; d >>= 1) first_special = min(first_special, __shfl_xor(first_special, d, 64));
+        if (lane == 0) s_special[wave] = first_special;
     }
     pf_wait_loads<0>();
     X8 qreg[NC][KS];
@@ -140,7 +140,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qreg[c][ks]));
     __syncthreads();  // the tables are complete and the staged rows have been read: the ring may overwrite them
-    const int first_special = __builtin_amdgcn_readfirstlane(s_special);
+    const int first_special =
+        __builtin_amdgcn_readfirstlane(min(min(s_special[0], s_special[1]), min(s_special[2], s_special[3])));
 
     // ---- loads of a tile: wave w fetches rows 4w .. 4w+3 of each of the tile's four 16-key groups ----
     const int64_t tok_stride = (int64_t)p.hkv * D * 2;
@@ -280,7 +281,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
       "a231", "a232", "a233", "a234", "a235", "a236", "a237", "a238", "a239", "a240", "a241", "a242", "a243", "a244",  \
       "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255", "s40", "s41", "s42",     \
       "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58",  \
-      "s59", "vcc", "scc", "memory"
+      "s59", "s60", "s61", "s62", "s63", "vcc", "scc", "memory"
         if constexpr (std::is_same<T, pa_bf16>::value) {
             asm volatile(PF_LOOP_ASM_BF16 PA_LOOP_OPERANDS);
         } else {
