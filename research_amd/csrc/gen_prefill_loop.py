@@ -151,8 +151,7 @@ def subtile_ops(ty, j, kt):
 
     # ---- rescale check (start of the subtile) ----
     # (the two compares sit behind the maxima of the previous subtile, so their results are long there)
-    chk = [Ins("s_add_u32 %[skb], %[skb], 32", kind="salu"),  # first key of the subtile whose S^T is formed next
-           Ins("s_or_b64 vcc, s[60:61], s[62:63]", kind="salu"),
+    chk = [Ins("s_or_b64 vcc, s[60:61], s[62:63]", kind="salu"),
            Ins(f"s_cbranch_vccnz .Lpf_rescale_{j}{kt}_%=\n.Lpf_rescaled_{j}{kt}_%=:", kind="salu", n=1)]
     STUBS.append([f".Lpf_rescale_{j}{kt}_%=:", "s_call_b64 s[50:51], .Lpf_rescale_%=", f"s_branch .Lpf_rescaled_{j}{kt}_%="])
     streams["chk"] = [Op(chk, 0, 0)]
@@ -232,17 +231,20 @@ def subtile_ops(ty, j, kt):
     mx = []
     m = [93, 94]   # running maxima
     w = [95, 96]   # copies for the half-wave exchange
-    # keys a row must not see: value i of a lane is key skb + 8*(i/4) + i%4 (+ 4*half, folded into lim)
+    # keys a row must not see.  srem = maskfrom - 64*t in tile t; the S^T formed in subtile kt starts at key
+    # 64*t + 32*(kt+1) and needs the mask if it reaches past maskfrom: srem < 32*(kt+2).  Value i of a lane is key
+    # 8*(i/4) + i%4 of the subtile (+ 4*half, folded into lim), visible up to lim - first key of the subtile.
     blk = [f".Lpf_mask_{j}{kt}_%=:"]
     for c in range(NC):
         s = S(nb, c)
-        blk.append(f"v_subrev_u32_e32 v95, %[skb], %[lim{c}]")
+        blk += [f"v_subrev_u32_e32 v95, %[maskfrom], %[lim{c}]", "v_add_u32_e32 v95, %[srem], v95",
+                f"v_subrev_u32_e32 v95, {32 * (kt + 1)}, v95"]
         for i in range(16):
             blk += [f"v_cmp_gt_i32_e32 vcc, {8 * (i >> 2) + (i & 3)}, v95", f"v_cndmask_b32_e32 v{s + i}, v{s + i}, v116, vcc"]
     blk.append(f"s_branch .Lpf_masked_{j}{kt}_%=")
     STUBS.append(blk)
-    mx.append(Op(Ins(f"s_add_u32 s56, %[skb], 32\n\ts_cmp_gt_u32 s56, %[maskfrom]\n\ts_cbranch_scc1 .Lpf_mask_{j}{kt}_%=\n"
-                     f".Lpf_masked_{j}{kt}_%=:", kind="salu", units=3, n=3,
+    mx.append(Op(Ins(f"s_cmp_lt_i32 %[srem], {32 * (kt + 2)}\n\ts_cbranch_scc1 .Lpf_mask_{j}{kt}_%=\n"
+                     f".Lpf_masked_{j}{kt}_%=:", kind="salu", units=2, n=2,
                      reads=[f"v{S(nb, c) + i}" for c in range(NC) for i in range(16)]), 21))
     for c in range(NC):
         s = S(nb, c)
@@ -482,7 +484,8 @@ def loop_text(ty):
     for j in range(NSTAGE):
         lines.append(f".Lpf_tile{j}_%=:")
         lines += [ins.text for ins in bodies[j]]
-        lines += ["s_sub_u32 %[ntiles], %[ntiles], 1", "s_cmp_eq_u32 %[ntiles], 0", "s_cbranch_scc1 .Lpf_done_%="]
+        # (ntiles counts the tiles after this one: the subtraction borrows behind the last)
+        lines += ["s_sub_u32 %[srem], %[srem], 64", "s_sub_u32 %[ntiles], %[ntiles], 1", "s_cbranch_scc1 .Lpf_done_%="]
     lines.append("s_branch .Lpf_tile0_%=")
     for stub in STUBS:
         lines += stub

@@ -242,8 +242,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     for (int c = 0; c < NC; ++c) { m_raw[c] = kNegBig; m_thr[c] = kNegBig; m_sc[c] = kNegBig * sc; l_run[c] = 0.f; }
 
     {
-        int n_left = n_tiles;
-        uint32_t s_t = 3, s_p = 1, s_kb = 0;
+        int n_left = n_tiles - 1;  // tiles after the current one
+        uint32_t s_t = 3, s_p = 1;
+        int s_rem = mask_from;  // mask_from - 64 * tile
         const uint32_t tab_a_base = lds_base + kRingBytes, tab_b_base = tab_a_base + kTabABytes;
         const uint32_t sp_lo = (uint32_t)first_special, sp_span = (uint32_t)(n_tiles - first_special);
         const uint32_t n_real_u = (uint32_t)n_real, cap_tiles = kPaCapTiles, mask_from_u = (uint32_t)mask_from;
@@ -258,9 +259,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
       "+{v[0:15]}"(s0[0]), "+{v[16:31]}"(s0[1]),                                                                      \
       "+{a[192:195]}"(ka[0]), "+{a[196:199]}"(ka[1]), "+{a[200:203]}"(ka[2]), "+{a[204:207]}"(ka[3]),                   \
       "+{a[208:211]}"(ka[4]), "+{a[212:215]}"(ka[5]), "+{a[216:219]}"(ka[6]), "+{a[220:223]}"(ka[7]),                   \
-      [mx0] "+v"(mx[0]), [mx1] "+v"(mx[1]), [msc0] "+v"(m_sc[0]), [msc1] "+v"(m_sc[1]), [thr0] "+v"(m_thr[0]),          \
-      [thr1] "+v"(m_thr[1]), [mraw0] "+v"(m_raw[0]), [mraw1] "+v"(m_raw[1]), [l0] "+v"(l_run[0]), [l1] "+v"(l_run[1]),  \
-      [ntiles] "+s"(n_left), [sT] "+s"(s_t), [sP] "+s"(s_p), [skb] "+s"(s_kb)                                         \
+      [mx0] "+&v"(mx[0]), [mx1] "+&v"(mx[1]), [msc0] "+&v"(m_sc[0]), [msc1] "+&v"(m_sc[1]), [thr0] "+&v"(m_thr[0]),          \
+      [thr1] "+&v"(m_thr[1]), [mraw0] "+&v"(m_raw[0]), [mraw1] "+&v"(m_raw[1]), [l0] "+&v"(l_run[0]), [l1] "+&v"(l_run[1]),  \
+      [ntiles] "+&s"(n_left), [sT] "+&s"(s_t), [sP] "+&s"(s_p), [srem] "+&s"(s_rem)                                         \
     : "{a[128:131]}"(qreg[0][0]), "{a[132:135]}"(qreg[0][1]), "{a[136:139]}"(qreg[0][2]), "{a[140:143]}"(qreg[0][3]),   \
       "{a[144:147]}"(qreg[0][4]), "{a[148:151]}"(qreg[0][5]), "{a[152:155]}"(qreg[0][6]), "{a[156:159]}"(qreg[0][7]),   \
       "{a[160:163]}"(qreg[1][0]), "{a[164:167]}"(qreg[1][1]), "{a[168:171]}"(qreg[1][2]), "{a[172:175]}"(qreg[1][3]),   \
