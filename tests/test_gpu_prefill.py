@@ -238,3 +238,61 @@ def test_packed_documents_chunked_prefill_over_a_prefix():
                       _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk), _i32(np.arange(2) * cmax), cmax, bs,
                       d ** -0.5, out=out, row_first_key=torch.from_numpy(first.reshape(-1)).to(DEV))
     assert_close(out.reshape(2, cmax, hq, d), want, 2e-2, "chunked documents")
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype):
+    """head_dim 128 takes the kernel whose tile loop is scheduled assembly.  Block ids of -1 or past the pool, and
+    contexts longer than the table, stand for zero key / value rows there as in the vector kernel (which is the
+    statement of that rule: flex_backend.py:272-277 leaves rows of absent blocks zero); the two kernels must
+    agree on every row, for 16-token and 64-token blocks, with the bad entries in the first tile, in the middle
+    and at the end."""
+    announce(f"prefill assembly loop, absent blocks {dtype}")
+    rng = np.random.default_rng(77)
+    hq, hkv, d = 8, 2, 128
+    for bs in (16, 64):
+        prefix = [200, 0, 333, 64]
+        chunk = [100, 190, 31, 64]
+        cmax = max(chunk)
+        need = [-(-(p + c) // bs) for p, c in zip(prefix, chunk)]
+        nb = sum(need) + 2
+        perm = rng.permutation(nb)
+        tables, at = [], 0
+        for n in need:
+            tables.append(perm[at : at + n].tolist())
+            at += n
+        tables[0][0] = -1               # first tile
+        tables[0][need[0] // 2] = nb + 5  # past the pool
+        tables[1][-1] = -1              # last block
+        tables[2] = tables[2][: need[2] - 2]  # table shorter than the context
+        width = max(len(t) for t in tables)
+        dev_tables = torch.tensor([t + [-1] * (width - len(t)) for t in tables], dtype=torch.int32, device=DEV)
+        kc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype).to(DEV)
+        vc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(dtype).to(DEV)
+        q = torch.from_numpy(rng.standard_normal((len(chunk) * cmax, hq, d)).astype(np.float32)).to(dtype).to(DEV)
+        args = (q, kc, vc, dev_tables, _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk),
+                _i32(np.arange(len(chunk)) * cmax), cmax, bs, d ** -0.5)
+        got = ops.prefill_paged(*args).float().cpu().reshape(len(chunk), cmax, hq, d)
+        want = ops.prefill_paged(*args, rowwise=True).float().cpu().reshape(len(chunk), cmax, hq, d)
+        for b, c in enumerate(chunk):
+            assert_close(got[b, :c], want[b, :c], 2e-2, f"block_size {bs} sequence {b}")
+
+
+def test_assembly_loop_kernel_long_context_and_table_limit():
+    """A 70 000-key context (more than a thousand tiles of slot-table entries) through the assembly-loop kernel,
+    and a table just past what that kernel's LDS tables hold (the host then launches the other matrix-core
+    kernel): both against the vector kernel on the chunk's rows."""
+    announce("prefill assembly loop, long context")
+    rng = np.random.default_rng(78)
+    hq, hkv, d, bs = 4, 1, 128, 16
+    for ctx in (70000, 1600 * 64 + 40):
+        chunk = 48
+        nblk = -(-ctx // bs)
+        kc = torch.from_numpy(rng.standard_normal((nblk * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+        vc = torch.from_numpy(rng.standard_normal((nblk * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+        q = (0.3 * torch.from_numpy(rng.standard_normal((chunk, hq, d)).astype(np.float32))).to(torch.bfloat16).to(DEV)
+        table = torch.from_numpy(rng.permutation(nblk).astype(np.int32)).reshape(1, -1).to(DEV)
+        args = (q, kc, vc, table, _i32([ctx]), _i32([chunk]), _i32([0]), chunk, bs, d ** -0.5)
+        got = ops.prefill_paged(*args).float().cpu()
+        want = ops.prefill_paged(*args, rowwise=True).float().cpu()
+        assert_close(got, want, 2e-2, f"context of {ctx} keys")
