@@ -281,7 +281,7 @@ def bench_prefill_c3(args, dev) -> dict:
                    "num_seqs": S, "prefix_len": P, "chunk_len": C, "num_q_heads": w.num_q_heads,
                    "num_kv_heads": w.num_kv_heads, "head_dim": w.head_dim, "block_size": w.block_size,
                    "attention_flops": flops, "append_bytes": w.append_bytes(), "seed": 1003},
-        "roofline": {"bound": "mfma", "kernel": "prefill_mfma_kernel", "achieved": achieved,
+        "roofline": {"bound": "mfma", "kernel": "prefill_asm_kernel", "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": measured_traffic("c3"), "kernel_ms": ms_prefill,
                      "kernel_launches": max(args.steps, KERNEL_LAUNCHES)},

@@ -45,7 +45,7 @@ extern "C" {
 #define PA_F16 2
 #define PA_FP8_E4M3 3 /* OCP e4m3fn, KV pool only; q/out stay 16- or 32-bit */
 
-/* Library ABI version (bumped when an entry point is added or a signature changes; now 2). */
+/* Library ABI version (bumped when an entry point is added or a signature changes; now 3). */
 int pa_version(void);
 
 /* Text of the calling thread's most recent error; "" if none. */
@@ -217,6 +217,26 @@ int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, vo
                      const int32_t *q_lens, const int32_t *q_starts, const int32_t *row_first_key,
                      int batch, int max_q_len, int num_q_heads, int num_kv_heads, int head_dim,
                      int block_size, int64_t num_blocks, float scale, int window, int dtype, void *stream);
+
+/*
+ * Attention under an arbitrary mask: what FlexAttentionBackend does with a ctx.block_mask built from any
+ * mask_mod(b, h, q_idx, kv_idx) predicate (attention/flex_backend.py:170-178 in prefill, :220-225 in decode;
+ * predicates such as attention/mask.py:42, :84, :171).  The caller evaluates the predicate into bits; row r of
+ * sequence b (packed row q_starts[b] + r), query head h attends key j < n_keys iff bit j of its mask row is
+ * set - nothing else is implied, a causal bound included.  Keys j >= ctx_lens[b] and keys in absent blocks are
+ * zero rows (logit 0, zero value), which is what the reference's zero-padded decode gather hands to
+ * flex_attention (:253-264); a row with no bit set gives zeros.
+ *   q, out  : [total_q][num_q_heads][head_dim], dtype F32 / BF16 / F16 = the pool's dtype
+ *   mask    : uint32 [total_q][mask_heads][mask_words], bit j of word j/32; mask_heads is 1 (all heads share
+ *             the row) or num_q_heads
+ * The general path, not a fast one: one workgroup per (head, row), a wave-wide reduction per visible key.  The
+ * structured masks (causal, sliding window, packed documents) go through pa_prefill_paged / pa_decode.
+ */
+int pa_attend_masked(const void *q, const void *k_cache, const void *v_cache, void *out,
+                     const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
+                     const int32_t *q_lens, const int32_t *q_starts, const uint32_t *mask, int mask_heads,
+                     int mask_words, int n_keys, int batch, int max_q_len, int num_q_heads, int num_kv_heads,
+                     int head_dim, int block_size, int64_t num_blocks, float scale, int dtype, void *stream);
 
 /*
  * pa_prefill_paged evaluated by the vector kernel (one workgroup per query row, the decode inner loop) whatever

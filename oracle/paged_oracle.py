@@ -285,6 +285,44 @@ def paged_prefill_chunk(q, k_cache, v_cache, block_tables, prefix_lens, chunk_le
     return out
 
 
+def paged_attend_masked(q, k_cache, v_cache, block_tables, ctx_lens, q_lens, keep, block_size: int,
+                        scale: float) -> np.ndarray:
+    """Attention under an arbitrary boolean mask: what the reference gets from ``flex_attention(q, k, v,
+    block_mask=..., scale=...)`` (flex_backend.py:175-178 in prefill, :220-225 in decode) for the mask_mod the
+    block mask was built from, stated densely.  q ``[B, Tmax, Hq, D]``; ``keep`` bool ``[B, Tmax, Hq or 1,
+    n_keys]`` = mask_mod(b, h, q_idx, kv_idx) evaluated on every entry; keys are gathered through the block
+    table with zero rows past ``ctx_lens[b]`` and for absent blocks (the zero-initialised gather of
+    flex_backend.py:253-277); kv heads are repeated to the query heads (:213-216).  softmax over the kept keys
+    only (a masked score is -inf); a row that keeps no key gives zeros, as flex_attention does; rows past
+    ``q_lens[b]`` give zeros."""
+    q, kc, vc = to_f64(q), to_f64(k_cache), to_f64(v_cache)
+    keep = np.asarray(keep, dtype=bool)
+    batch, tmax, hq, d = q.shape
+    hkv = kc.shape[1]
+    n_rep = hq // hkv
+    n_keys = keep.shape[-1]
+    num_blocks = kc.shape[0] // block_size
+    out = np.zeros_like(q)
+    for b in range(batch):
+        blocks = np.asarray(block_tables[b], dtype=np.int64)
+        k = np.zeros((n_keys, hkv, d))
+        v = np.zeros((n_keys, hkv, d))
+        for j in range(min(n_keys, int(ctx_lens[b]))):
+            blk = j // block_size
+            if blk < len(blocks) and 0 <= blocks[blk] < num_blocks:
+                slot = blocks[blk] * block_size + j % block_size
+                k[j], v[j] = kc[slot], vc[slot]
+        for t in range(int(q_lens[b])):
+            for h in range(hq):
+                m = keep[b, t, h if keep.shape[2] > 1 else 0]
+                if not m.any():
+                    continue
+                s = (k[m, h // n_rep] @ q[b, t, h]) * scale
+                w = np.exp(s - s.max())
+                out[b, t, h] = (w / w.sum()) @ v[m, h // n_rep]
+    return out
+
+
 # --------------------------------------------------------------------------- rotary embedding
 # (rollouts/tools/functional_extractor/llama_functional.py; the step a model runs right before attention)
 

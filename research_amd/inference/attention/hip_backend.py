@@ -62,13 +62,15 @@ class _StepTensors:
     """Device copies of one context's integer fields, built once per step."""
 
     __slots__ = ("ctx", "slots", "touched", "tables", "bt_stride", "seq_lens", "extra_zero", "ctx_lens", "q_lens",
-                 "q_starts", "max_q_len", "row_first_key", "fp8_blocks", "fp8_tables")
+                 "q_starts", "max_q_len", "row_first_key", "fp8_blocks", "fp8_tables", "mask_words", "mask_keys")
 
     def __init__(self, ctx: InferenceContext) -> None:
         self.ctx = ctx  # keeps id(ctx) alive while the entry is cached
         self.slots = self.touched = self.tables = self.seq_lens = self.extra_zero = None
         self.ctx_lens = self.q_lens = self.q_starts = self.row_first_key = None
         self.fp8_blocks = self.fp8_tables = None  # distinct blocks of the tables and the tables renumbered to them
+        self.mask_words = None  # bits of an arbitrary mask predicate evaluated for this step, and their key count
+        self.mask_keys = 0
         self.bt_stride = self.max_q_len = 0
 
 
@@ -141,8 +143,40 @@ class HipPagedAttentionBackend:
         if not isinstance(mask, PagedMask):
             raise NotImplementedError(
                 f"block_mask of type {type(mask).__name__}: the HIP backend takes the PagedMask objects of "
-                "attention/mask.py (causal, sliding window, documents), not arbitrary mask objects")
+                "attention/mask.py (causal, sliding window, documents), a mask_mod(b, h, q_idx, kv_idx) callable "
+                "or an object that carries one (a FlexAttention BlockMask)")
         return int(mask.window or 0)
+
+    @staticmethod
+    def _mask_predicate(mask: object):
+        """The ``mask_mod(b, h, q_idx, kv_idx)`` predicate of a mask that is not a ``PagedMask``: the object
+        itself when callable, or its ``mask_mod`` attribute (what a FlexAttention ``BlockMask`` built by
+        ``create_block_mask`` carries; the reference passes such objects to ``flex_attention``,
+        flex_backend.py:170-178, :220-225).  None for ``None`` and for ``PagedMask`` objects, which the kernels
+        apply themselves."""
+        if mask is None or isinstance(mask, PagedMask):
+            return None
+        mod = getattr(mask, "mask_mod", None)
+        if callable(mod):
+            return mod
+        return mask if callable(mask) else None
+
+    def _mask_bits(self, step: _StepTensors, mod, batch: int, heads: int, q_pos: Tensor, n_keys: int) -> Tensor:
+        """The predicate evaluated on every (sequence, head, row, key) of the step, packed into the words
+        ``pa_attend_masked`` takes; computed once per context (all layers share it).  ``q_pos`` int ``[B, T]``:
+        the q_idx of every row.  A predicate that does not look at ``h`` gives one row of bits for all heads."""
+        if step.mask_words is None:
+            dev = self.k_cache.device
+            b = torch.arange(batch, device=dev)[:, None, None, None]
+            h = torch.arange(heads, device=dev)[None, :, None, None]
+            kv = torch.arange(n_keys, device=dev)[None, None, None, :]
+            keep = torch.as_tensor(mod(b, h, q_pos.to(dev)[:, None, :, None], kv), device=dev).to(torch.bool)
+            while keep.dim() < 4:
+                keep = keep[None]
+            keep = keep.expand(batch, keep.shape[1], q_pos.shape[1], n_keys)
+            rows = keep.permute(0, 2, 1, 3).reshape(batch * q_pos.shape[1], keep.shape[1], n_keys)
+            step.mask_words, step.mask_keys = ops.pack_mask(rows), n_keys
+        return step.mask_words
 
     def _mask_first_keys(self, mask: object, step: _StepTensors, batch: int, seq_len: int,
                          prefix: Optional[np.ndarray]) -> Optional[Tensor]:
@@ -418,6 +452,9 @@ class HipPagedAttentionBackend:
         assert seq_len == 1, "Decode should have seq_len=1"
         if ctx.block_tables is None or ctx.seq_lens is None:
             raise ValueError("Decode requires block_tables and seq_lens in context")
+        mod = self._mask_predicate(ctx.block_mask)
+        if mod is not None:
+            return self._decode_masked(q, layer_idx, ctx, mod)
         window = self._mask_window(ctx.block_mask, self._window if self.window_in_decode else 0)
         if isinstance(ctx.block_mask, PagedMask) and ctx.block_mask.boundaries is not None:
             raise NotImplementedError("a document mask describes packed prefill rows, not a decode step")
@@ -451,6 +488,29 @@ class HipPagedAttentionBackend:
                          ksc, vsc, window=window)
         return out.view(batch, 1, num_heads, head_dim)
 
+    def _decode_masked(self, q: Tensor, layer_idx: int, ctx: InferenceContext, mod) -> Tensor:
+        """Decode under an arbitrary predicate, literally as the reference evaluates it (flex_backend.py:203-225):
+        the one query row has q_idx 0, kv_idx runs over the batch's longest sequence, and the positions past a
+        shorter sequence's end are zero rows that take part wherever the predicate keeps them."""
+        if self._fp8:
+            raise NotImplementedError("arbitrary mask predicates are not evaluated over an fp8 pool")
+        cfg = self.config
+        batch, _, num_heads, head_dim = q.shape
+        self._require_device(q, self.k_cache)
+        step = self._step(ctx)
+        if step.ctx_lens is None:
+            lens = self._lens(ctx.seq_lens, batch)
+            self._tables(step, ctx.block_tables[:batch])
+            step.ctx_lens = self._to_device(lens.astype(np.int32))
+            step.q_lens = torch.ones(batch, dtype=torch.int32, device=q.device)
+            step.q_starts = torch.arange(batch, dtype=torch.int32, device=q.device)
+            step.max_q_len = int(lens.max()) if batch else 0  # (here: the key count of the mask)
+        words = self._mask_bits(step, mod, batch, num_heads, torch.zeros((batch, 1), dtype=torch.int64), step.max_q_len)
+        kc, vc = self._layer(layer_idx)
+        out = ops.attend_masked(q.contiguous().view(batch, num_heads, head_dim), kc, vc, step.tables, step.ctx_lens,
+                                step.q_lens, step.q_starts, 1, cfg.block_size, self.scale, words, step.mask_keys)
+        return out.view(batch, 1, num_heads, head_dim)
+
     # ------------------------------------------------------------------ prefill
     def _prefill_attention(self, q: Tensor, k: Tensor, v: Tensor, ctx: InferenceContext) -> Tensor:
         """Causal attention over the step's own K/V, cache not read (flex_backend.py:144-185).
@@ -458,12 +518,27 @@ class HipPagedAttentionBackend:
         The dense ``[B, T, Hkv, D]`` inputs are handed to the paged kernel as a
         pool of ``B`` blocks of ``T`` tokens with the identity block table.
         """
-        window = self._mask_window(ctx.block_mask, self._window)
+        mod = self._mask_predicate(ctx.block_mask)
+        window = 0 if mod is not None else self._mask_window(ctx.block_mask, self._window)
         batch, seq_len, num_heads, head_dim = q.shape
         out = torch.empty(q.shape, dtype=q.dtype, device=q.device)
         if out.numel() == 0:
             return out
         dev = self._require_device(q, k, v)
+        if mod is not None:
+            # an arbitrary predicate over the step's own K/V (flex_backend.py:170-178): q_idx = kv_idx = position
+            # in the step; the dense K/V are a pool of `batch` blocks of `seq_len` tokens, as below
+            pos = torch.arange(seq_len, dtype=torch.int64)[None].expand(batch, seq_len)
+            words = self._mask_bits(self._step(ctx), mod, batch, num_heads, pos, seq_len)
+            ar = torch.arange(batch, dtype=torch.int32, device=dev)
+            lens = torch.full((batch,), seq_len, dtype=torch.int32, device=dev)
+            num_kv = k.shape[2]
+            ops.attend_masked(q.contiguous().view(batch * seq_len, num_heads, head_dim),
+                              k.contiguous().view(batch * seq_len, num_kv, head_dim),
+                              v.contiguous().view(batch * seq_len, num_kv, head_dim),
+                              ar.reshape(batch, 1).contiguous(), lens, lens, ar * seq_len, seq_len, seq_len, self.scale,
+                              words, seq_len, out=out.view(batch * seq_len, num_heads, head_dim))
+            return out
         first = self._mask_first_keys(ctx.block_mask, self._step(ctx), batch, seq_len, None)
         num_kv = k.shape[2]
         if num_heads != num_kv * self.num_heads_per_kv:
@@ -481,7 +556,8 @@ class HipPagedAttentionBackend:
 
     def _prefill_paged(self, q: Tensor, layer_idx: int, ctx: InferenceContext) -> Tensor:
         """Chunked prefill: ``q[b]`` holds the last ``T`` positions of a context of ``seq_lens[b]`` keys."""
-        window = self._mask_window(ctx.block_mask, self._window)
+        mod = self._mask_predicate(ctx.block_mask)
+        window = 0 if mod is not None else self._mask_window(ctx.block_mask, self._window)
         if ctx.block_tables is None or ctx.seq_lens is None:
             raise ValueError("Chunked prefill requires block_tables and seq_lens in context")
         cfg = self.config
@@ -507,6 +583,17 @@ class HipPagedAttentionBackend:
         out.zero_()  # rows past a sequence's chunk length are padding and stay zero
         kc, vc = self._layer(layer_idx)
         tables = step.tables
+        if mod is not None:
+            # an arbitrary predicate over the cached context: row t of sequence b has q_idx = prefix + t
+            if self._fp8:
+                raise NotImplementedError("arbitrary mask predicates are not evaluated over an fp8 pool")
+            totals = self._lens(ctx.seq_lens, batch)
+            pos = torch.from_numpy(self._lens(ctx.prefix_lens, batch)[:, None] + np.arange(seq_len, dtype=np.int64)[None, :])
+            words = self._mask_bits(step, mod, batch, num_heads, pos, int(totals.max()))
+            ops.attend_masked(q.contiguous().view(batch * seq_len, num_heads, head_dim), kc, vc, tables, step.ctx_lens,
+                              step.q_lens, step.q_starts, step.max_q_len, cfg.block_size, self.scale, words,
+                              step.mask_keys, out=out.view(batch * seq_len, num_heads, head_dim))
+            return out
         if self._fp8:
             # The matrix-core kernel reads 16-bit pools: dequantise the blocks the tables name into a compact
             # pool (each block once, however many sequences share it) and renumber the tables to match.

@@ -136,6 +136,37 @@ def prefill_paged(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Ten
     return out
 
 
+def pack_mask(keep: Tensor) -> Tensor:
+    """Bits of a boolean mask ``[rows, heads (or 1), keys]`` as int32 words ``[rows, heads, ceil(keys / 32)]``
+    (bit j of word j // 32 = keep[..., j]), the layout ``attend_masked`` takes."""
+    rows, heads, keys = keep.shape
+    words = max(1, -(-keys // 32))
+    padded = torch.zeros((rows, heads, words * 32), dtype=torch.int64, device=keep.device)
+    padded[..., :keys] = keep
+    weights = torch.ones(32, dtype=torch.int64, device=keep.device) << torch.arange(32, device=keep.device)
+    packed = (padded.view(rows, heads, words, 32) * weights).sum(-1)
+    return torch.where(packed >= 2 ** 31, packed - 2 ** 32, packed).to(torch.int32).contiguous()
+
+
+def attend_masked(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, ctx_lens: Tensor, q_lens: Tensor,
+                  q_starts: Tensor, max_q_len: int, block_size: int, scale: float, mask_words: Tensor, n_keys: int,
+                  out: Optional[Tensor] = None) -> Tensor:
+    """Attention of packed q rows ``[total_q, Hq, D]`` over a paged context under an arbitrary mask
+    (``pa_attend_masked``): ``mask_words`` int32 ``[total_q, 1 or Hq, words]`` from ``pack_mask``; row r attends
+    key j < n_keys iff its bit is set; keys at or past ``ctx_lens[b]`` are zero rows."""
+    total_q, hq, d = q.shape
+    total_slots, hkv, _ = k_cache.shape
+    if mask_words.dtype != torch.int32 or mask_words.dim() != 3 or mask_words.shape[0] != total_q:
+        raise ValueError("mask_words must be int32 [total_q, heads, words]")
+    if out is None:
+        out = torch.empty_like(q)
+    _run("pa_attend_masked", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_tables),
+         block_tables.shape[1], _ptr(ctx_lens), _ptr(q_lens), _ptr(q_starts), _ptr(mask_words), mask_words.shape[1],
+         mask_words.shape[2], int(n_keys), block_tables.shape[0], max_q_len, hq, hkv, d, block_size,
+         total_slots // block_size, float(scale), PA_DTYPE[q.dtype], _stream(q))
+    return out
+
+
 def quantize_kv_e4m3(pool: Tensor, block_size: int) -> Tuple[Tensor, Tensor]:
     """e4m3fn bytes (as ``torch.float8_e4m3fn``) and ``float32 [num_blocks, Hkv]`` scales of a pool."""
     total_slots, hkv, d = pool.shape

@@ -575,3 +575,50 @@ def test_rope_literal_is_a_rotation():
     gb = po.rope_literal(xb, cos.to(torch.bfloat16), sin.to(torch.bfloat16))
     assert gb.dtype == torch.bfloat16
     np.testing.assert_allclose(gb.float().numpy(), po.rope_exact(xb, angle), atol=0.06, rtol=0.02)
+
+
+# ---------------------------------------------------------------- arbitrary masks
+def test_masked_attention_against_sdpa_with_a_boolean_mask_and_the_causal_case():
+    """paged_attend_masked: (1) the library routine with attn_mask on the gathered, head-expanded tensors
+    (rows with at least one kept key); (2) a row that keeps nothing gives zeros; (3) keys past the context end
+    are zero rows that still take softmax mass when kept (the reference's padded decode gather); (4) with the
+    causal predicate it is the chunked prefill of the other checker function; (5) a head-dependent mask uses each
+    head's own row."""
+    rng = np.random.default_rng(41)
+    bs, hq, hkv, d = 4, 4, 2, 8
+    kc, vc = _tiny_pool(rng, num_blocks=8, bs=bs, hkv=hkv, d=d)
+    tables = [[5, 2, 7], [1, 3]]
+    ctx, ql = [10, 7], [3, 2]
+    n_keys = 12
+    q = torch.from_numpy(rng.standard_normal((2, 3, hq, d)).astype(np.float32))
+    keep = rng.random((2, 3, hq, n_keys)) < 0.5
+    keep[0, 1] = False          # a row that keeps nothing
+    keep[1, 0, :, 7:] = True    # keys past the context end (7) kept
+    got = po.paged_attend_masked(q, kc, vc, tables, ctx, ql, keep, bs, 0.3)
+    kg, vg = po.kv_gather_padded(kc, vc, [t + [0] * 3 for t in tables], [n_keys, n_keys], bs)
+    for b in range(2):
+        kb, vb = kg[b].clone(), vg[b].clone()
+        kb[ctx[b]:] = 0
+        vb[ctx[b]:] = 0
+        for t in range(ql[b]):
+            for h in range(hq):
+                if not keep[b, t, h].any():
+                    assert not got[b, t, h].any()
+                    continue
+                want = F.scaled_dot_product_attention(
+                    q[b, t, h][None, None].double(), kb[:, h // 2][None].double(), vb[:, h // 2][None].double(),
+                    attn_mask=torch.from_numpy(keep[b, t, h])[None, None], scale=0.3)
+                np.testing.assert_allclose(got[b, t, h], want[0, 0].numpy(), rtol=1e-9, atol=1e-12)
+    assert not got[1, 2].any()  # past q_lens
+    # (3) zero keys take mass: dropping them from the mask changes the row
+    keep2 = keep.copy()
+    keep2[1, 0, :, 7:] = False
+    assert np.abs(po.paged_attend_masked(q, kc, vc, tables, ctx, ql, keep2, bs, 0.3)[1, 0] - got[1, 0]).max() > 1e-3
+    # (4) the causal predicate over a prefix: chunk row t sits at position P + t
+    prefix = [c - n for c, n in zip(ctx, ql)]
+    causal = np.zeros((2, 3, 1, n_keys), dtype=bool)
+    for b in range(2):
+        for t in range(ql[b]):
+            causal[b, t, 0, : prefix[b] + t + 1] = True
+    np.testing.assert_allclose(po.paged_attend_masked(q, kc, vc, tables, ctx, ql, causal, bs, 0.3),
+                               po.paged_prefill_chunk(q, kc, vc, tables, prefix, ql, bs, 0.3), rtol=1e-10, atol=1e-12)
