@@ -44,6 +44,7 @@ TENSOR = 64 * RB        # one tensor's tile of 64 keys
 STAGE = 2 * TENSOR      # K tile + V tile
 NSTAGE = 4
 GAPS = 33               # places for other instructions around the 32 products of a subtile
+SYNC_GAP = int(os.environ.get("PF_GEN_SYNCGAP", "16"))  # where tile t+1 is published in a tile's first subtile
 X = set(os.environ.get("PF_GEN_X", "").split(","))  # experiment switches
 
 
@@ -177,7 +178,7 @@ def subtile_ops(ty, j, kt):
         lds.append(Op(Ins("s_waitcnt vmcnt(8)\n\ts_sub_u32 s56, %[sP], %[splo]\n\ts_cmp_lt_u32 s56, %[spspan]\n"
                           f"\ts_cbranch_scc1 .Lpf_fix_{j}_%=\n.Lpf_fixed_{j}_%=:\n"
                           "\ts_add_u32 %[sP], %[sP], 1\n\t" + ("s_nop 0" if "nobarrier" in X else "s_barrier"),
-                          kind="sync", units=6, n=6), 16, 16))
+                          kind="sync", units=6, n=6), SYNC_GAP, SYNC_GAP))
         STUBS.append([f".Lpf_fix_{j}_%=:", "s_call_b64 s[50:51], .Lpf_fixup_%=", f"s_branch .Lpf_fixed_{j}_%="])
     # K operands of subtile g+2 = subtile kt of the next tile (stage j+1)
     nstage = (j + 1) % NSTAGE
@@ -270,7 +271,7 @@ def subtile_ops(ty, j, kt):
     # ---- loads of tile j+3 into stage (j+3) % 4: table entries, then per 16-key group one K and one V load ----
     ldr = []
     dst_stage = (j + 3) % NSTAGE
-    first = 17 if kt == 0 else 0
+    first = SYNC_GAP + 1 if kt == 0 else 0
     if kt == 0:
         # tile sT = t+3; past the last tile: tile 0 again (same loads and barriers for every wave, data unused)
         ldr.append(Op([Ins("s_cmp_lt_u32 %[sT], %[nreal]\n\ts_cselect_b32 s55, %[sT], 0", kind="salu", units=2, n=2),
@@ -279,10 +280,10 @@ def subtile_ops(ty, j, kt):
                        Ins("v_mov_b32_e32 v92, s55", writes=("v92",))], first))
         ldr.append(Op(Ins("ds_read_b128 v[88:91], v92", kind="lds", reads=("v92",), issue="tab"), first))
         for n in range(4):
-            ldr.append(Op(Ins(f"v_readfirstlane_b32 s{40 + n}, v{88 + n}", reads=(f"v{88 + n}",), need=("tab",)), 22))
+            ldr.append(Op(Ins(f"v_readfirstlane_b32 s{40 + n}, v{88 + n}", reads=(f"v{88 + n}",), need=("tab",)), max(22, SYNC_GAP + 5)))
     groups = (0, 1) if kt == 0 else (2, 3)
     for n in groups:
-        e = 24 if kt == 0 else 0
+        e = max(24, SYNC_GAP + 7) if kt == 0 else 0
         # slot * row stride (64 bits), then per tensor: LDS destination into m0, pool base + offset, load.  The
         # two additions between the write of m0 and the load are the wait state that write needs.
         ldr.append(Op([Ins(f"s_mul_i32 s44, s{40 + n}, %[stride]", kind="salu"),
@@ -305,7 +306,7 @@ def subtile_ops(ty, j, kt):
     return mf, streams
 
 
-def schedule(mf, streams, spare=0.6):
+def schedule(mf, streams, spare=float(os.environ.get("PF_GEN_SPARE", "0.6"))):
     """Places the other instructions into the 33 gaps around the products: earliest deadline first within the
     capacity of a gap, a stream's instructions in their order, everything due in a gap placed there."""
     total = sum(op.units for ops in streams.values() for op in ops)
