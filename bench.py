@@ -430,6 +430,43 @@ def bench_decode(name, args, dev) -> dict:
     ms_split = timed_ms(lambda: step("pa_decode" if passes == 1 else "pa_decode_split"), n_kernel)
     ms_reduce = None if passes == 1 else timed_ms(lambda: step("pa_decode_reduce"), n_kernel)
 
+    host_path = None
+    if w.kv_format != "fp8_e4m3" and not getattr(args, "secondary_run", False):
+        # What a decode call costs through the backend class, host side included, by the form the context's
+        # integer fields arrive in: the reference's tuples of tuples (converted block id by block id in Python),
+        # padded int32 arrays, or device tensors (used in place).  A new context object per call, as a new step
+        # brings; wall time of one call including the wait for the GPU, best of three.
+        from research_amd.inference import CacheConfig, HipPagedAttentionBackend, InferenceContext
+
+        be = HipPagedAttentionBackend(CacheConfig(num_layers=1, num_kv_heads=w.num_kv_heads, head_dim=w.head_dim,
+                                                  num_blocks=1, block_size=w.block_size, dtype=k_pool.dtype,
+                                                  device=str(dev)))
+        be.set_num_heads(w.num_q_heads)
+        be.config = CacheConfig(num_layers=1, num_kv_heads=w.num_kv_heads, head_dim=w.head_dim,
+                                num_blocks=k_pool.shape[0] // w.block_size, block_size=w.block_size,
+                                dtype=k_pool.dtype, device=str(dev))
+        be.k_cache, be.v_cache = k_pool.unsqueeze(0), v_pool.unsqueeze(0)  # the workload's pools, not a copy
+        q4 = q.unsqueeze(1)
+        forms = {
+            "tuples": lambda: (tuple(tuple(int(x) for x in t) for t in w.block_tables), tuple(int(n) for n in w.seq_lens)),
+            "int32_arrays": lambda: (w.padded_tables(), w.seq_lens.astype(np.int32)),
+            "device_tensors": lambda: (tables, lens),
+        }
+        host_path = {"unit": "ms per backend decode call, host and GPU", "kernel_ms": ms_step}
+        for form, make in forms.items():
+            best = None
+            for _ in range(3):
+                bt, sl = make()  # the caller's own bookkeeping, outside the timed call
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                be._decode_attention(q4, 0, InferenceContext(is_prefill=False, block_tables=bt, seq_lens=sl,
+                                                             max_seq_len=int(w.seq_lens.max())))
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) * 1e3
+                best = dt if best is None else min(best, dt)
+            host_path[form] = best
+        del be
+
     gather = None
     if name in ("c1", "c2") and not getattr(args, "secondary_run", False):
         # the reference's own decode materialises this copy first (_gather_kv_from_cache): the block-table
@@ -488,6 +525,8 @@ def bench_decode(name, args, dev) -> dict:
     }
     if gather is not None:
         result["gather"] = gather
+    if host_path is not None:
+        result["host_path"] = host_path
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, args.cpu_seconds)
         if name in ("c1", "c2") and args.cpu_seconds > 0 and not getattr(args, "secondary_run", False):
