@@ -4,6 +4,8 @@
 namespace pa_decode_detail {
 constexpr int kPaCapTiles = 1600;  // (prefill_asm.h)
 prefill_mfma_fn pa_prefill_asm_kernel(int dtype);
+constexpr int kWdTasks = 4, kWdCapGroups = 6144;  // (prefill_d256.h)
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype);
 }
 
 using namespace pa_decode_detail;
@@ -46,7 +48,8 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     a.row_lo = row_first_key;
     a.batch = batch; a.max_q_len = max_q_len;
     hipStream_t s = (hipStream_t)stream;
-    // bf16 / fp16 with head_dim 32, 64, 128 run on the matrix cores unless the caller asked for the vector kernel
+    // bf16 / fp16 with head_dim 32, 64, 128 (and 256, below) run on the matrix cores unless the caller asked for the
+    // vector kernel
     // (the matrix-core softmax takes the running maximum of the unscaled logits, which needs scale > 0)
     prefill_mfma_fn mfma =
         force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
@@ -55,10 +58,18 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     if (mfma && head_dim == 128 && window == 0 && !row_first_key && block_size % 16 == 0 && num_blocks > 0 &&
         num_blocks * (int64_t)block_size < (1ll << 31) && bt_stride * (int64_t)block_size <= (int64_t)kPaCapTiles * kPfKeys)
         mfma = pa_prefill_asm_kernel(dtype);
+    // head_dim 256: one 32-row task per wave, loads driven by a table of 16-key groups - which must lie inside one
+    // pool block (block sizes that are multiples of 16, or a single block per sequence) - that LDS can hold
+    int tasks_per_wg = kPfTasks;
+    if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) && num_blocks > 0 &&
+        num_blocks * (int64_t)block_size < (1ll << 31) && bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16) {
+        mfma = pa_prefill_d256_kernel(dtype);
+        tasks_per_wg = kWdTasks;
+    }
     if (mfma) {
         PA_REQUIRE(pa_aligned16(q) && pa_aligned16(out), "q and out must be 16-byte aligned");
         const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
-        const int groups = (row_blocks * a.p.n_rep + kPfTasks - 1) / kPfTasks;
+        const int groups = (row_blocks * a.p.n_rep + tasks_per_wg - 1) / tasks_per_wg;
         PA_REQUIRE(groups <= 65535, "max_q_len=%d is too long for one launch", max_q_len);
         mfma<<<dim3((unsigned)num_kv_heads, (unsigned)groups, (unsigned)batch), dim3(kPfThreads), 0, s>>>(a);
         PA_CHECK_LAUNCH("pa_prefill_paged (matrix-core kernel)");

@@ -1,0 +1,12 @@
+// Instantiates the head_dim 256 matrix-core prefill kernels (bf16 / fp16).
+#include "prefill_d256.h"
+
+namespace pa_decode_detail {
+
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype) {
+    if (dtype == PA_BF16) return prefill_d256_kernel<pa_bf16>;
+    if (dtype == PA_F16) return prefill_d256_kernel<pa_f16>;
+    return nullptr;
+}
+
+}  // namespace pa_decode_detail
