@@ -8,7 +8,7 @@ JSON line; with the default workload the line also carries short runs of the
 other configurations (c2, c5 decode, c3 append + chunked prefill) under
 ``secondary``.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1|c3|engine] [--no-secondary]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1|c3|c3-d256|engine] [--no-secondary]
     python bench.py --traffic-from-pmc NAME KERNEL FETCH.csv WRITE.csv   # refresh profiles/traffic.json
 """
 
@@ -89,7 +89,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c4", "c5", "engine"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c3-d256", "c4", "c5", "engine"])
     ap.add_argument("--preheat-s", type=float, default=0.5,
                     help="seconds of untimed steps before the warmup steps: an idle GPU sits at its lowest clocks "
                          "and takes a few hundred milliseconds of work to leave them")
@@ -313,6 +313,52 @@ def bench_prefill_c3(args, dev) -> dict:
                       "FLOPs counted for the chunk rows only",
         }
     return result
+
+
+def bench_prefill_d256(args, dev) -> dict:
+    """The c3 shape with 16 query / 8 kv heads of 256 (32 x (2048 shared + 256 own) tokens, 16-token blocks,
+    bf16): the chunked-prefill kernel for that head size alone, against the bf16 matrix-core peak."""
+    from research_amd import ops
+    from research_amd.workloads import make_prefill_c3
+
+    w = make_prefill_c3(num_q_heads=16, num_kv_heads=8, head_dim=256, seed=1006)
+    S, C, P = w.num_seqs, w.chunk_len, w.prefix_len
+    shape = (w.num_blocks * w.block_size, w.num_kv_heads, w.head_dim)
+    kc = torch.zeros(shape, dtype=w.dtype, device=dev)
+    vc = torch.zeros_like(kc)
+    ops.kv_scatter(kc, vc, w.k_prefix.to(dev), w.v_prefix.to(dev), torch.from_numpy(w.prefix_slots()).to(dev))
+    ops.kv_scatter(kc, vc, w.k_chunk.reshape(S * C, *shape[1:]).to(dev), w.v_chunk.reshape(S * C, *shape[1:]).to(dev),
+                   torch.from_numpy(w.chunk_slots()).to(dev))
+    q = w.q.reshape(S * C, w.num_q_heads, w.head_dim).to(dev)
+    tables = torch.from_numpy(np.stack(w.block_tables).astype(np.int32)).to(dev)
+    ctx = torch.full((S,), P + C, dtype=torch.int32, device=dev)
+    ql = torch.full((S,), C, dtype=torch.int32, device=dev)
+    qs = torch.arange(S, dtype=torch.int32, device=dev) * C
+    out = torch.empty_like(q)
+
+    def prefill():
+        ops.prefill_paged(q, kc, vc, tables, ctx, ql, qs, C, w.block_size, w.scale, out=out)
+
+    preheat(prefill, args.preheat_s)
+    for _ in range(args.warmup):
+        prefill()
+    ms_step, ms_step_median = timed_steps(prefill, args.steps)
+    ms_kernel = timed_ms(prefill, max(args.steps, KERNEL_LAUNCHES))
+    flops = w.attention_flops()
+    achieved = flops / (ms_kernel * 1e-3) / 1e12
+    return {
+        "metric": "prefill-attn TFLOP/s", "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "tokens_per_s": S * C / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_median": ms_step_median,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "c3 shape at head_dim 256: chunked prefill, 32 x (2048 + 256), 16 q / 8 kv heads, bf16",
+                   "num_seqs": S, "prefix_len": P, "chunk_len": C, "num_q_heads": w.num_q_heads,
+                   "num_kv_heads": w.num_kv_heads, "head_dim": w.head_dim, "block_size": w.block_size,
+                   "attention_flops": flops, "seed": 1006},
+        "roofline": {"bound": "mfma", "kernel": "prefill_d256_kernel", "achieved": achieved,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": None, "kernel_ms": ms_kernel, "kernel_launches": max(args.steps, KERNEL_LAUNCHES)},
+    }
 
 
 def bench_engine(args, dev) -> int:
@@ -545,8 +591,9 @@ def secondary(args, dev) -> dict:
     short.copy_calibration = False
     short.secondary_run = True
     out = {}
-    for name in ("c2", "c5", "c3"):
-        r = bench_prefill_c3(short, dev) if name == "c3" else bench_decode(name, short, dev)
+    for name in ("c2", "c5", "c3", "c3-d256"):
+        r = (bench_prefill_c3(short, dev) if name == "c3" else bench_prefill_d256(short, dev) if name == "c3-d256"
+             else bench_decode(name, short, dev))
         keep = ("metric", "value", "unit", "ms_per_step", "ms_per_step_median", "steps", "warmup", "tokens_per_s",
                 "dtype", "roofline", "cpu_baseline", "append", "pct_of_hbm_peak")
         entry = {k: r[k] for k in keep if k in r}
@@ -573,7 +620,10 @@ def main() -> int:
     torch.cuda.set_device(dev)
     if args.workload == "engine":
         return bench_engine(args, dev)
-    result = bench_prefill_c3(args, dev) if args.workload == "c3" else bench_decode(args.workload, args, dev)
+    if args.workload == "c3-d256":
+        result = bench_prefill_d256(args, dev)
+    else:
+        result = bench_prefill_c3(args, dev) if args.workload == "c3" else bench_decode(args.workload, args, dev)
     if args.workload == "c4" and not args.no_secondary:
         torch.cuda.empty_cache()
         result["secondary"] = secondary(args, dev)

@@ -112,14 +112,17 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     }
     // ---- slot tables (in flight together with the Q rows) ----
     const int64_t pool_rows = p.num_blocks * p.bs;  // < 2^31 (the host checks)
-    const int n_entries = min(2 * n_tiles, CAP);
+    // (entries of kLookahead tiles past the workgroup's last one follow as groups of which nothing exists: the
+    // loads run that far ahead and past the end, so that every wave issues the same loads per stage)
+    constexpr int kLookahead = 6;
+    const int n_entries = min(2 * (n_tiles + kLookahead), CAP);
     {
         const int32_t *bt_seq = p.bt + (int64_t)b * p.bt_stride;
         int first_special = n_tiles;
         for (int i = tid; i < n_entries; i += kPfThreads) {
             const int key = 16 * i, blk = key / p.bs;
             int64_t bid = -1;
-            if (blk < p.bt_stride) bid = bt_seq[blk];
+            if (i < 2 * n_tiles && blk < p.bt_stride) bid = bt_seq[blk];
             const bool present = bid >= 0 && bid < p.num_blocks;
             // rows of the group that exist: inside the context and inside the group's block (a block that is not
             // a multiple of 16 keys long is the only block of its sequence: what follows it is absent)
@@ -165,8 +168,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         lane_v[n] = (uint32_t)(r * tok_stride) + (uint32_t)((ld_slot ^ ((r & 3) * 4)) * 16);
     }
     const uint32_t wave_rows = (uint32_t)wave * (8 * RB);  // the wave's rows inside a tensor of a stage
-    // table entry of the wave's group of tile `tile`; tiles the workgroup does not multiply read entry CAP
-    auto entry_of = [&](int tile) PF_INLINE { return tile >= 0 && tile < n_tiles ? min(2 * tile + (wave >> 1), CAP) : CAP; };
+    // table entry of the wave's group of tile `tile` (>= 0, at most kLookahead - 1 past the last tile)
+    const int wave_group = wave >> 1;
+    auto entry_of = [&](int tile) PF_INLINE { return min(2 * tile + wave_group, CAP); };
     // one tensor's rows of one tile into LDS at byte offset `dst` of s_mem (always NL direct loads)
     auto issue_rows = [&](const char *pool, const uint32_t (&lane_ofs)[NL], int chunk_swz_mask, int tile, uint32_t dst) PF_INLINE {
         const int slot = __builtin_amdgcn_readfirstlane(tab_a[entry_of(tile)]);
@@ -190,6 +194,46 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     auto stage_ofs = [&](int s) PF_INLINE { return (uint32_t)(s & (kWdStages - 1)) * STAGE; };
     auto issue_k = [&](int s) PF_INLINE { issue_rows(pool_k, lane_k, 15, s + 1, stage_ofs(s) + wave_rows); };
     auto issue_v = [&](int s) PF_INLINE { issue_rows(pool_v, lane_v, 3, s, stage_ofs(s) + TENSOR + wave_rows); };
+    // The same inside the loop, trimmed: the two table entries are read one subtile ahead (pre_k, pre_v), and the
+    // eight loads of a stage are one block of instructions.  A direct load adds its immediate offset to the LDS
+    // address and to the global address alike, so with the global side compensated in the per-lane offsets the
+    // four loads of a tensor share one LDS base (one write of m0).
+    int pre_k = 0, pre_v = 0;
+    auto prefetch_entries = [&](int s) PF_INLINE { pre_k = tab_a[entry_of(s + 1)]; pre_v = tab_a[entry_of(s)]; };
+    uint32_t lane_kb[NL], lane_vb[NL];
+#pragma unroll
+    for (int n = 0; n < NL; ++n) {
+        lane_kb[n] = lane_k[n] + (NL - 1 - n) * 2 * RB;
+        lane_vb[n] = lane_v[n] + (NL - 1 - n) * 2 * RB;
+    }
+    const char *pool_kb = pool_k - (NL - 1) * 2 * RB, *pool_vb = pool_v - (NL - 1) * 2 * RB;
+    const int slot_max = (int)max(pool_rows - 16, (int64_t)-1);  // last slot a whole group can start at
+    auto issue_stage = [&](int s) PF_INLINE {
+        const int slot_k = __builtin_amdgcn_readfirstlane(pre_k), slot_v = __builtin_amdgcn_readfirstlane(pre_v);
+        if (__builtin_expect(max(slot_k, slot_v) <= slot_max, 1)) {
+            const uint32_t dst_k = lds_base + stage_ofs(s) + wave_rows, dst_v = dst_k + TENSOR;
+            const char *bk = pf_scalar_ptr(pool_kb + (uint64_t)(uint32_t)slot_k * (uint32_t)tok_stride);
+            const char *bv = pf_scalar_ptr(pool_vb + (uint64_t)(uint32_t)slot_v * (uint32_t)tok_stride);
+            static_assert(2 * RB == 1024 && NL == 4, "immediate offsets of the loads below");
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
+                         "global_load_lds_dwordx4 %2, %1 offset:0\n\t"
+                         "global_load_lds_dwordx4 %3, %1 offset:1024\n\t"
+                         "global_load_lds_dwordx4 %4, %1 offset:2048\n\t"
+                         "global_load_lds_dwordx4 %5, %1 offset:3072\n\t"
+                         "s_mov_b32 m0, %6\n\ts_nop 0\n\t"
+                         "global_load_lds_dwordx4 %8, %7 offset:0\n\t"
+                         "global_load_lds_dwordx4 %9, %7 offset:1024\n\t"
+                         "global_load_lds_dwordx4 %10, %7 offset:2048\n\t"
+                         "global_load_lds_dwordx4 %11, %7 offset:3072"
+                         :
+                         : "s"(dst_k), "s"(bk), "v"(lane_kb[0]), "v"(lane_kb[1]), "v"(lane_kb[2]), "v"(lane_kb[3]),
+                           "s"(dst_v), "s"(bv), "v"(lane_vb[0]), "v"(lane_vb[1]), "v"(lane_vb[2]), "v"(lane_vb[3])
+                         : "memory", "m0");
+        } else {
+            issue_k(s);
+            issue_v(s);
+        }
+    };
     // clear the rows this wave loaded that do not exist (after its loads have landed, before the barrier)
     auto clear_rows = [&](int tile, uint32_t dst) PF_INLINE {
         const int rows = tab_b[entry_of(tile)];
@@ -304,6 +348,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     __builtin_amdgcn_s_waitcnt((15) | (7 << 4) | (0 << 8) | (3 << 14));  // lgkmcnt(0)
     __syncthreads();
     issue_k(t0 + 3); issue_v(t0 + 3);
+    prefetch_entries(t0 + 4);
     PF_FENCE();
 
     // One subtile g (= tile g, stage g); PAR = parity of g - t0: which S^T buffer is the current one.
@@ -316,10 +361,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         float sum = 0.f;
         // exponentials of S^T values 2*j, 2*j+1, packed as a P^T operand word
         auto exp_piece = [&](int j) PF_INLINE {
-            float scl = sc;
-            asm volatile("" : "+s"(scl));
-            const float p0 = __builtin_amdgcn_exp2f(fmaf(s[2 * j], scl, -m_sc));
-            const float p1 = __builtin_amdgcn_exp2f(fmaf(s[2 * j + 1], scl, -m_sc));
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(s[2 * j], sc, -m_sc));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(s[2 * j + 1], sc, -m_sc));
             sum += p0 + p1;
             uint32_t w = M::pack(p0, p1);
             asm volatile("" : "+v"(w), "+v"(sum));
@@ -355,7 +398,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         fix_k(g + 1); fix_v(g + 1);
         __builtin_amdgcn_s_waitcnt((15) | (7 << 4) | (0 << 8) | (3 << 14));  // lgkmcnt(0): this wave's reads of stage g
         __syncthreads();
-        issue_k(g + 4); issue_v(g + 4);
+        issue_stage(g + 4);
+        prefetch_entries(g + 5);
         PF_FENCE();
         read_k(g + 1, ka);  // K of subtile g+2: consumed in (a) of g+1
         PF_FENCE();

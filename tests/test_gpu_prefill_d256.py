@@ -152,3 +152,30 @@ def test_long_context_and_table_limit():
         got = ops.prefill_paged(*args).float().cpu()
         want = ops.prefill_paged(*args, rowwise=True).float().cpu()
         assert_close(got, want, 2e-2, f"context of {ctx} keys")
+
+
+def test_c3_shape_at_head_dim_256_full_size():
+    """The chunked-prefill workload's shape (32 x (2048 shared + 256 own) tokens, 16-token blocks) with 16 query /
+    8 kv heads of 256: every output element against the vector kernel, and all 32 sequences against the
+    checker."""
+    from research_amd.workloads import make_prefill_c3
+
+    announce("prefill d256, c3 shape, full size")
+    w = make_prefill_c3(num_q_heads=16, num_kv_heads=8, head_dim=D, seed=905)
+    S, C, P = w.num_seqs, w.chunk_len, w.prefix_len
+    shape = (w.num_blocks * w.block_size, w.num_kv_heads, D)
+    kc = torch.zeros(shape, dtype=w.dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    ops.kv_scatter(kc, vc, w.k_prefix.to(DEV), w.v_prefix.to(DEV), torch.from_numpy(w.prefix_slots()).to(DEV))
+    ops.kv_scatter(kc, vc, w.k_chunk.reshape(S * C, *shape[1:]).to(DEV), w.v_chunk.reshape(S * C, *shape[1:]).to(DEV),
+                   torch.from_numpy(w.chunk_slots()).to(DEV))
+    q = w.q.reshape(S * C, w.num_q_heads, D).to(DEV)
+    args = (q, kc, vc, tables_to_device(w.block_tables), _i32([P + C] * S), _i32([C] * S), _i32(np.arange(S) * C), C,
+            w.block_size, w.scale)
+    mfma = ops.prefill_paged(*args).float().cpu()
+    rowwise = ops.prefill_paged(*args, rowwise=True).float().cpu()
+    assert_close(mfma, rowwise, 2e-2, "matrix-core kernel against the vector kernel, all rows")
+    seqs = list(range(S))
+    want = po.paged_prefill_chunk(w.q[seqs], kc.cpu(), vc.cpu(), [w.block_tables[s] for s in seqs], [P] * S, [C] * S,
+                                  w.block_size, w.scale)
+    assert_close(mfma.reshape(S, C, w.num_q_heads, D), want, 2e-2, "against the checker, all sequences")
