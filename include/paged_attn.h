@@ -240,8 +240,8 @@ int pa_attend_masked(const void *q, const void *k_cache, const void *v_cache, vo
 
 /*
  * pa_prefill_paged evaluated by the vector kernel (one workgroup per query row, the decode inner loop) whatever
- * the element type: the path fp32, fp8-pool and head_dim 256 calls take anyway, selectable for the 16-bit shapes
- * too so that the two kernels can be checked against each other.  Same arguments, same results to rounding.
+ * the element type: the path fp32 and fp8-pool calls take anyway, selectable for the 16-bit shapes too so that
+ * the two kernels can be checked against each other.  Same arguments, same results to rounding.
  * (No separate counterpart in the reference: both are attention/flex_backend.py:144-185.)
  */
 int pa_prefill_paged_rowwise(const void *q, const void *k_cache, const void *v_cache, void *out,
