@@ -339,6 +339,12 @@ def bench_prefill_d256(args, dev) -> dict:
     def prefill():
         ops.prefill_paged(q, kc, vc, tables, ctx, ql, qs, C, w.block_size, w.scale, out=out)
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     preheat(prefill, args.preheat_s)
     for _ in range(args.warmup):
         prefill()
@@ -357,7 +363,8 @@ def bench_prefill_d256(args, dev) -> dict:
                    "attention_flops": flops, "seed": 1006},
         "roofline": {"bound": "mfma", "kernel": "prefill_d256_kernel", "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": None, "kernel_ms": ms_kernel, "kernel_launches": max(args.steps, KERNEL_LAUNCHES)},
+                     "traffic": measured_traffic("c3-d256"), "kernel_ms": ms_kernel,
+                     "kernel_launches": max(args.steps, KERNEL_LAUNCHES)},
     }
 
 

@@ -208,6 +208,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     }
     const char *pool_kb = pool_k - (NL - 1) * 2 * RB, *pool_vb = pool_v - (NL - 1) * 2 * RB;
     const int slot_max = (int)max(pool_rows - 16, (int64_t)-1);  // last slot a whole group can start at
+    auto dma_one = [&](uint32_t dst, const char *base, uint32_t lane_ofs, int n) PF_INLINE {
+        if (n == 0) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:0" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
+        if (n == 1) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:1024" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
+        if (n == 2) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:2048" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
+        if (n == 3) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:3072" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
+    };
     auto issue_stage = [&](int s) PF_INLINE {
         const int slot_k = __builtin_amdgcn_readfirstlane(pre_k), slot_v = __builtin_amdgcn_readfirstlane(pre_v);
         if (__builtin_expect(max(slot_k, slot_v) <= slot_max, 1)) {
@@ -277,6 +283,20 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 #pragma unroll
             for (int e = 0; e < 4; ++e) { va[dt][e] = lo[e]; va[dt][4 + e] = hi[e]; }
         }
+    };
+    // the same reads one operand at a time (the loop spreads them between the products)
+    auto read_k_one = [&](int s, int ks, X8 &dst) PF_INLINE {
+        const uint32_t adr = lds_base + stage_ofs(s) + k_ofs[ks & 7];
+        dst = __builtin_bit_cast(X8, *reinterpret_cast<const __attribute__((address_space(3))) uint4 *>(
+                                         (const lds_char *)(size_t)adr + (ks >> 3) * 256));
+    };
+    auto read_v_one = [&](int s, int step, int dt, X8 &dst) PF_INLINE {
+        const lds_char *at = (const lds_char *)(size_t)(lds_base + stage_ofs(s) + v_ofs[dt & 3]) + (dt >> 2) * 256 + 16 * step * RB;
+        const X4 lo = __builtin_bit_cast(X4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((pa_s16x4 __attribute__((address_space(3))) *)at));
+        const X4 hi = __builtin_bit_cast(
+            X4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((pa_s16x4 __attribute__((address_space(3))) *)(at + 8 * RB)));
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { dst[e] = lo[e]; dst[4 + e] = hi[e]; }
     };
     // mask of S^T of the subtile that starts at key_base: value i of a lane is key 8*(i/4) + i%4 (+ 4*half)
     auto mask_s = [&](f32x16 &s, int key_base) PF_INLINE {
@@ -382,14 +402,14 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             m_sc = m_new * sc;
         }
         PF_FENCE();
-        read_v(g, 1, va1);  // second k-step's V^T: consumed in (c)
-        PF_FENCE();
         // ---- (a) S^T of subtile g+1, with the exponentials of subtile g between the products ----
 #pragma unroll
         for (int i = 0; i < 16; ++i) s_nx[i] = 0.f;
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             s_nx = M::mma(ka[ks], qreg[ks], s_nx);
+            PF_FENCE();
+            if (!(ks & 1)) read_v_one(g, 1, ks >> 1, va1[ks >> 1]);  // second k-step's V^T: consumed in (c)
             if (ks & 1) exp_piece(ks >> 1);
             PF_FENCE();
         }
@@ -398,10 +418,15 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         fix_k(g + 1); fix_v(g + 1);
         __builtin_amdgcn_s_waitcnt((15) | (7 << 4) | (0 << 8) | (3 << 14));  // lgkmcnt(0): this wave's reads of stage g
         __syncthreads();
-        issue_stage(g + 4);
+        // the loads of stage g+4, one behind each product of (b); a group that reaches past the end of the pool
+        // takes the per-lane path here instead
+        const int slot_k = __builtin_amdgcn_readfirstlane(pre_k), slot_v = __builtin_amdgcn_readfirstlane(pre_v);
+        const bool fast = max(slot_k, slot_v) <= slot_max;
+        const uint32_t dst_k = lds_base + stage_ofs(g + 4) + wave_rows, dst_v = dst_k + TENSOR;
+        const char *bk = pf_scalar_ptr(pool_kb + (uint64_t)(uint32_t)slot_k * (uint32_t)tok_stride);
+        const char *bv = pf_scalar_ptr(pool_vb + (uint64_t)(uint32_t)slot_v * (uint32_t)tok_stride);
+        if (__builtin_expect(!fast, 0)) { issue_k(g + 4); issue_v(g + 4); }
         prefetch_entries(g + 5);
-        PF_FENCE();
-        read_k(g + 1, ka);  // K of subtile g+2: consumed in (a) of g+1
         PF_FENCE();
         // ---- (b) O^T += V^T . P^T, first k-step ----
         {
@@ -410,9 +435,11 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             for (int dt = 0; dt < DT; ++dt) {
                 o[dt] = M::mma(va0[dt], pb, o[dt]);
                 PF_FENCE();
+                if (fast) dma_one(dt < 4 ? dst_k : dst_v, dt < 4 ? bk : bv, dt < 4 ? lane_kb[dt & 3] : lane_vb[dt & 3], dt & 3);
+                read_k_one(g + 1, dt, ka[dt]);  // K of subtile g+2 (k-steps 0..7 here, 8..15 in (c)): consumed in (a) of g+1
+                PF_FENCE();
             }
         }
-        read_v(g + 1, 0, va0);  // first k-step's V^T of the next subtile
         if (mask_next) mask_s(s_nx, 32 * (g + 1));
         PF_FENCE();
         // ---- (c) second k-step, with the next subtile's row maximum ----
@@ -421,6 +448,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
                 o[dt] = M::mma(va1[dt], pb, o[dt]);
+                PF_FENCE();
+                read_v_one(g + 1, 0, dt, va0[dt]);  // first k-step's V^T of the next subtile
+                read_k_one(g + 1, 8 + dt, ka[8 + dt]);
                 if (dt == 1) max_piece(s_nx, 0, mx);
                 if (dt == 3) max_piece(s_nx, 1, mx);
                 PF_FENCE();
