@@ -45,7 +45,7 @@ extern "C" {
 #define PA_F16 2
 #define PA_FP8_E4M3 3 /* OCP e4m3fn, KV pool only; q/out stay 16- or 32-bit */
 
-/* Library ABI version (bumped when an entry point is added or a signature changes; now 3). */
+/* Library ABI version (bumped when an entry point is added or a signature changes; now 4). */
 int pa_version(void);
 
 /* Text of the calling thread's most recent error; "" if none. */
@@ -276,13 +276,21 @@ int pa_quantize_kv_e4m3(const void *src, void *dst, float *scale, int64_t num_bl
  *                    of two tokens with the same slot the later one is stored
  *   touched_blocks : int32[n_touched], the distinct blocks the slots fall in (extra entries are harmless,
  *                    a block must not appear twice)
+ *   row_order, block_start : optional index of the rows by touched block (both NULL: every workgroup scans the
+ *                    whole slot list, n_touched * n_tokens slot reads per tensor, fine for a decode step and
+ *                    quadratic in the length of a prefill chunk).  row_order int32[n_tokens]: token indices
+ *                    grouped by touched block; block_start int32[n_touched + 1]: tokens
+ *                    row_order[block_start[i]] .. row_order[block_start[i+1] - 1] are those whose slots fall in
+ *                    touched_blocks[i].  A token the index leaves out is not stored; entries out of range are
+ *                    ignored.
  *   k_src, v_src   : [n_tokens][num_kv_heads][head_dim] in src_dtype (F32/BF16/F16)
  *   k_scale,v_scale: float[num_blocks][num_kv_heads], updated in place
  */
 int pa_kv_append_e4m3(void *k_cache, void *v_cache, float *k_scale, float *v_scale, const void *k_src,
                       const void *v_src, const int64_t *slots, int64_t n_tokens,
-                      const int32_t *touched_blocks, int n_touched, int64_t num_blocks, int block_size,
-                      int num_kv_heads, int head_dim, int src_dtype, void *stream);
+                      const int32_t *touched_blocks, int n_touched, const int32_t *row_order,
+                      const int32_t *block_start, int64_t num_blocks, int block_size, int num_kv_heads,
+                      int head_dim, int src_dtype, void *stream);
 
 /*
  * Rotary position embedding fused with the KV append: the step a model runs immediately before this path
@@ -318,8 +326,9 @@ int pa_rope_kv_append(const void *q, void *q_out, const void *k_src, const void 
 int pa_rope_kv_append_e4m3(const void *q, void *q_out, const void *k_src, const void *v_src, void *k_cache,
                            void *v_cache, float *k_scale, float *v_scale, const void *cos, const void *sin,
                            const int32_t *positions, int64_t rope_rows, const int64_t *slots, int64_t n_tokens,
-                           const int32_t *touched_blocks, int n_touched, int64_t num_blocks, int block_size,
-                           int num_q_heads, int num_kv_heads, int head_dim, int src_dtype, void *stream);
+                           const int32_t *touched_blocks, int n_touched, const int32_t *row_order,
+                           const int32_t *block_start, int64_t num_blocks, int block_size, int num_q_heads,
+                           int num_kv_heads, int head_dim, int src_dtype, void *stream);
 
 /*
  * Dequantise listed blocks of an fp8-e4m3 pool into a compact 16-bit pool (no counterpart in the reference):

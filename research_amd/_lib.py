@@ -62,8 +62,8 @@ SIGNATURES = {
     ),
     "pa_kv_append_e4m3": (
         c_int,
-        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_int64,
-         c_int, c_int, c_int, c_int, c_void_p],
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_int, c_void_p,
+         c_void_p, c_int64, c_int, c_int, c_int, c_int, c_void_p],
     ),
     "pa_dequantize_blocks_e4m3": (
         c_int,
@@ -77,7 +77,8 @@ SIGNATURES = {
     "pa_rope_kv_append_e4m3": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-         c_int64, c_void_p, c_int64, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int, c_int, c_void_p],
+         c_int64, c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int, c_int,
+         c_void_p],
     ),
 }
 SIGNATURES["pa_decode_split"] = SIGNATURES["pa_decode_reduce"] = SIGNATURES["pa_decode"]

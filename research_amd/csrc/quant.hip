@@ -140,20 +140,26 @@ __device__ __forceinline__ void load_src8(const T *src, const RopeTables &rt, in
     }
 }
 
-template <typename T, bool ROPE, bool VEC>
-__global__ __launch_bounds__(kQThreads) void append_e4m3_kernel(const T *__restrict__ src, uint8_t *__restrict__ dst,
-                                                                 float *__restrict__ scale,
-                                                                 const int64_t *__restrict__ slots, int64_t n_tokens,
-                                                                 const int32_t *__restrict__ touched, int64_t num_blocks,
-                                                                 int block_size, int hkv, int d, const RopeTables rt) {
-    __shared__ int s_token[kMaxBlockTokens];  // token of this call that writes offset i (-1: none); highest index wins
-    __shared__ float s_max[2][kQThreads / PA_WAVE];
-    const int64_t blk = touched[blockIdx.x];
-    const int h = blockIdx.y;
-    if (blk < 0 || blk >= num_blocks) return;  // uniform
-    for (int i = threadIdx.x; i < block_size; i += kQThreads) s_token[i] = -1;
-    __syncthreads();
-    const int64_t slot0 = blk * block_size;
+// Optional index of a call's rows by touched block: rows order[start[i]] .. order[start[i+1]-1] are the tokens
+// whose slots fall in touched block i.  Without it (order == nullptr) every workgroup scans the whole slot list.
+struct RowIndex {
+    const int32_t *order, *start;
+};
+
+// s_token[offset] = the token of this call that writes that offset of the block (the highest index wins)
+__device__ __forceinline__ void find_rows(int *s_token, const int64_t *__restrict__ slots, int64_t n_tokens,
+                                          int64_t slot0, int block_size, const RowIndex rows, int touched_idx) {
+    if (rows.order) {
+        const int64_t lo = max(0, rows.start[touched_idx]);
+        const int64_t hi = min(n_tokens, (int64_t)rows.start[touched_idx + 1]);
+        for (int64_t i = lo + threadIdx.x; i < hi; i += kQThreads) {
+            const int64_t t = rows.order[i];
+            if (t < 0 || t >= n_tokens) continue;  // (a bad index entry names no row)
+            const int64_t off = slots[t] - slot0;
+            if (off >= 0 && off < block_size) atomicMax(&s_token[off], (int)t);
+        }
+        return;
+    }
     for (int64_t t0 = threadIdx.x; t0 < n_tokens; t0 += 8 * kQThreads) {  // eight loads in flight per thread
         int64_t off[8];
 #pragma unroll
@@ -165,6 +171,24 @@ __global__ __launch_bounds__(kQThreads) void append_e4m3_kernel(const T *__restr
         for (int k = 0; k < 8; ++k)
             if (off[k] >= 0 && off[k] < block_size) atomicMax(&s_token[off[k]], (int)(t0 + (int64_t)k * kQThreads));
     }
+}
+
+template <typename T, bool ROPE, bool VEC>
+__global__ __launch_bounds__(kQThreads) void append_e4m3_kernel(const T *__restrict__ src, uint8_t *__restrict__ dst,
+                                                                 float *__restrict__ scale,
+                                                                 const int64_t *__restrict__ slots, int64_t n_tokens,
+                                                                 const int32_t *__restrict__ touched, const RowIndex rows,
+                                                                 int64_t num_blocks, int block_size, int hkv, int d,
+                                                                 const RopeTables rt) {
+    __shared__ int s_token[kMaxBlockTokens];  // token of this call that writes offset i (-1: none); highest index wins
+    __shared__ float s_max[2][kQThreads / PA_WAVE];
+    const int64_t blk = touched[blockIdx.x];
+    const int h = blockIdx.y;
+    if (blk < 0 || blk >= num_blocks) return;  // uniform
+    for (int i = threadIdx.x; i < block_size; i += kQThreads) s_token[i] = -1;
+    __syncthreads();
+    const int64_t slot0 = blk * block_size;
+    find_rows(s_token, slots, n_tokens, slot0, block_size, rows, blockIdx.x);
     __syncthreads();
     int first = block_size;  // lowest offset written
     for (int i = 0; i < block_size; ++i)
@@ -312,7 +336,7 @@ template <typename T, bool ROPE>
 __global__ __launch_bounds__(kQThreads) void append_e4m3_block_kernel(const T *__restrict__ src, uint8_t *__restrict__ dst,
                                                                        float *__restrict__ scale,
                                                                        const int64_t *__restrict__ slots, int64_t n_tokens,
-                                                                       const int32_t *__restrict__ touched,
+                                                                       const int32_t *__restrict__ touched, const RowIndex rows,
                                                                        int64_t num_blocks, int block_size, int hkv, int d,
                                                                        const RopeTables rt) {
     __shared__ int s_token[kMaxBlockTokens];
@@ -321,17 +345,7 @@ __global__ __launch_bounds__(kQThreads) void append_e4m3_block_kernel(const T *_
     for (int i = threadIdx.x; i < block_size; i += kQThreads) s_token[i] = -1;
     __syncthreads();
     const int64_t slot0 = blk * block_size;
-    for (int64_t t0 = threadIdx.x; t0 < n_tokens; t0 += 8 * kQThreads) {  // eight loads in flight per thread
-        int64_t off[8];
-#pragma unroll
-        for (int k = 0; k < 8; ++k) {
-            const int64_t t = t0 + (int64_t)k * kQThreads;
-            off[k] = t < n_tokens ? slots[t] - slot0 : -1;
-        }
-#pragma unroll
-        for (int k = 0; k < 8; ++k)
-            if (off[k] >= 0 && off[k] < block_size) atomicMax(&s_token[off[k]], (int)(t0 + (int64_t)k * kQThreads));
-    }
+    find_rows(s_token, slots, n_tokens, slot0, block_size, rows, blockIdx.x);
     __syncthreads();
     int first = block_size;  // lowest offset written
     for (int i = 0; i < block_size; ++i)
@@ -426,31 +440,31 @@ __global__ __launch_bounds__(kQThreads) void append_e4m3_block_kernel(const T *_
 
 template <bool ROPE, bool VEC>
 void launch_append_v(const void *src, uint8_t *dst, float *sc, const int64_t *slots, int64_t n_tokens,
-                     const int32_t *touched, int n_touched, int64_t num_blocks, int block_size, int hkv, int d,
+                     const int32_t *touched, int n_touched, const RowIndex rows, int64_t num_blocks, int block_size, int hkv, int d,
                      int src_dtype, const RopeTables &rt, hipStream_t s) {
     const dim3 block(kQThreads);
     if constexpr (VEC) {
         const dim3 grid((unsigned)n_touched);
         if (src_dtype == PA_F32)
             append_e4m3_block_kernel<float, ROPE><<<grid, block, 0, s>>>((const float *)src, dst, sc, slots, n_tokens,
-                                                                         touched, num_blocks, block_size, hkv, d, rt);
+                                                                         touched, rows, num_blocks, block_size, hkv, d, rt);
         else if (src_dtype == PA_BF16)
             append_e4m3_block_kernel<pa_bf16, ROPE><<<grid, block, 0, s>>>((const pa_bf16 *)src, dst, sc, slots, n_tokens,
-                                                                           touched, num_blocks, block_size, hkv, d, rt);
+                                                                           touched, rows, num_blocks, block_size, hkv, d, rt);
         else
             append_e4m3_block_kernel<pa_f16, ROPE><<<grid, block, 0, s>>>((const pa_f16 *)src, dst, sc, slots, n_tokens,
-                                                                          touched, num_blocks, block_size, hkv, d, rt);
+                                                                          touched, rows, num_blocks, block_size, hkv, d, rt);
     } else {
         const dim3 grid((unsigned)n_touched, (unsigned)hkv);
         if (src_dtype == PA_F32)
             append_e4m3_kernel<float, ROPE, false><<<grid, block, 0, s>>>((const float *)src, dst, sc, slots, n_tokens,
-                                                                          touched, num_blocks, block_size, hkv, d, rt);
+                                                                          touched, rows, num_blocks, block_size, hkv, d, rt);
         else if (src_dtype == PA_BF16)
             append_e4m3_kernel<pa_bf16, ROPE, false><<<grid, block, 0, s>>>((const pa_bf16 *)src, dst, sc, slots, n_tokens,
-                                                                            touched, num_blocks, block_size, hkv, d, rt);
+                                                                            touched, rows, num_blocks, block_size, hkv, d, rt);
         else
             append_e4m3_kernel<pa_f16, ROPE, false><<<grid, block, 0, s>>>((const pa_f16 *)src, dst, sc, slots, n_tokens,
-                                                                           touched, num_blocks, block_size, hkv, d, rt);
+                                                                           touched, rows, num_blocks, block_size, hkv, d, rt);
     }
 }
 
@@ -458,15 +472,15 @@ void launch_append_v(const void *src, uint8_t *dst, float *sc, const int64_t *sl
 // thread and step when the rows allow 16-byte loads and 8-byte stores, one element otherwise.
 template <bool ROPE>
 void launch_append(const void *src, uint8_t *dst, float *sc, const int64_t *slots, int64_t n_tokens,
-                   const int32_t *touched, int n_touched, int64_t num_blocks, int block_size, int hkv, int d,
+                   const int32_t *touched, int n_touched, const RowIndex rows, int64_t num_blocks, int block_size, int hkv, int d,
                    int src_dtype, const RopeTables &rt, hipStream_t s) {
     const bool vec = d % (ROPE ? 16 : 8) == 0 && pa_aligned16(src) && ((uintptr_t)dst & 7u) == 0 &&
                      (!ROPE || (pa_aligned16(rt.cos) && pa_aligned16(rt.sin)));
     if (vec)
-        launch_append_v<ROPE, true>(src, dst, sc, slots, n_tokens, touched, n_touched, num_blocks, block_size, hkv, d,
+        launch_append_v<ROPE, true>(src, dst, sc, slots, n_tokens, touched, n_touched, rows, num_blocks, block_size, hkv, d,
                                     src_dtype, rt, s);
     else
-        launch_append_v<ROPE, false>(src, dst, sc, slots, n_tokens, touched, n_touched, num_blocks, block_size, hkv, d,
+        launch_append_v<ROPE, false>(src, dst, sc, slots, n_tokens, touched, n_touched, rows, num_blocks, block_size, hkv, d,
                                      src_dtype, rt, s);
 }
 
@@ -484,18 +498,21 @@ int check_append(int64_t n_tokens, int n_touched, int block_size, int num_kv_hea
 
 extern "C" int pa_kv_append_e4m3(void *k_cache, void *v_cache, float *k_scale, float *v_scale, const void *k_src,
                                  const void *v_src, const int64_t *slots, int64_t n_tokens,
-                                 const int32_t *touched_blocks, int n_touched, int64_t num_blocks, int block_size,
-                                 int num_kv_heads, int head_dim, int src_dtype, void *stream) {
+                                 const int32_t *touched_blocks, int n_touched, const int32_t *row_order,
+                                 const int32_t *block_start, int64_t num_blocks, int block_size, int num_kv_heads,
+                                 int head_dim, int src_dtype, void *stream) {
     pa_clear_error();
     if (int rc = check_append(n_tokens, n_touched, block_size, num_kv_heads, head_dim, src_dtype)) return rc;
     if (n_tokens == 0 || n_touched == 0) return PA_OK;
     PA_REQUIRE(k_cache && v_cache && k_scale && v_scale && k_src && v_src && slots && touched_blocks, "NULL pointer argument");
+    PA_REQUIRE((row_order == nullptr) == (block_start == nullptr), "row_order and block_start go together (both or neither)");
+    const RowIndex rows{row_order, block_start};
     hipStream_t s = (hipStream_t)stream;
     const RopeTables none{};
-    launch_append<false>(k_src, (uint8_t *)k_cache, k_scale, slots, n_tokens, touched_blocks, n_touched, num_blocks,
+    launch_append<false>(k_src, (uint8_t *)k_cache, k_scale, slots, n_tokens, touched_blocks, n_touched, rows, num_blocks,
                          block_size, num_kv_heads, head_dim, src_dtype, none, s);
     PA_CHECK_LAUNCH("pa_kv_append_e4m3");
-    launch_append<false>(v_src, (uint8_t *)v_cache, v_scale, slots, n_tokens, touched_blocks, n_touched, num_blocks,
+    launch_append<false>(v_src, (uint8_t *)v_cache, v_scale, slots, n_tokens, touched_blocks, n_touched, rows, num_blocks,
                          block_size, num_kv_heads, head_dim, src_dtype, none, s);
     PA_CHECK_LAUNCH("pa_kv_append_e4m3");
     return PA_OK;
@@ -505,8 +522,9 @@ extern "C" int pa_rope_kv_append_e4m3(const void *q, void *q_out, const void *k_
                                       void *v_cache, float *k_scale, float *v_scale, const void *cos, const void *sin,
                                       const int32_t *positions, int64_t rope_rows, const int64_t *slots,
                                       int64_t n_tokens, const int32_t *touched_blocks, int n_touched,
-                                      int64_t num_blocks, int block_size, int num_q_heads, int num_kv_heads,
-                                      int head_dim, int src_dtype, void *stream) {
+                                      const int32_t *row_order, const int32_t *block_start, int64_t num_blocks,
+                                      int block_size, int num_q_heads, int num_kv_heads, int head_dim, int src_dtype,
+                                      void *stream) {
     pa_clear_error();
     if (int rc = check_append(n_tokens, n_touched, block_size, num_kv_heads, head_dim, src_dtype)) return rc;
     if (int rc = pa_rope_check("pa_rope_kv_append_e4m3", n_tokens, rope_rows, positions, num_q_heads, num_kv_heads,
@@ -520,12 +538,14 @@ extern "C" int pa_rope_kv_append_e4m3(const void *q, void *q_out, const void *k_
         return rc;
     if (n_touched == 0) return PA_OK;
     PA_REQUIRE(k_cache && v_cache && k_scale && v_scale && k_src && v_src && slots && touched_blocks, "NULL pointer argument");
+    PA_REQUIRE((row_order == nullptr) == (block_start == nullptr), "row_order and block_start go together (both or neither)");
+    const RowIndex rows{row_order, block_start};
     hipStream_t s = (hipStream_t)stream;
     const RopeTables rt{cos, sin, positions, rope_rows};
-    launch_append<true>(k_src, (uint8_t *)k_cache, k_scale, slots, n_tokens, touched_blocks, n_touched, num_blocks,
+    launch_append<true>(k_src, (uint8_t *)k_cache, k_scale, slots, n_tokens, touched_blocks, n_touched, rows, num_blocks,
                         block_size, num_kv_heads, head_dim, src_dtype, rt, s);
     PA_CHECK_LAUNCH("pa_rope_kv_append_e4m3");
-    launch_append<false>(v_src, (uint8_t *)v_cache, v_scale, slots, n_tokens, touched_blocks, n_touched, num_blocks,
+    launch_append<false>(v_src, (uint8_t *)v_cache, v_scale, slots, n_tokens, touched_blocks, n_touched, rows, num_blocks,
                          block_size, num_kv_heads, head_dim, src_dtype, RopeTables{}, s);
     PA_CHECK_LAUNCH("pa_rope_kv_append_e4m3");
     return PA_OK;

@@ -377,16 +377,18 @@ class HipPagedAttentionBackend:
 
     # ------------------------------------------------------------------ KV append
     def _touched(self, step: Optional[_StepTensors], slots: Tensor, ctx: Optional[InferenceContext],
-                 layer_idx: int) -> Tensor:
-        """int32 device list of the blocks an fp8 append works on (one workgroup each; entries outside the pool
-        are skipped by the kernel).
+                 layer_idx: int):
+        """The blocks an fp8 append works on (one workgroup each; entries outside the pool are skipped by the
+        kernel): an ``ops.TouchedBlocks`` (distinct blocks and the index of the step's rows by block), or a bare
+        int32 device list.
 
         A decode step whose slot mapping lives on the device writes one row per sequence, and every sequence
         writes into a block of its own, so the list is simply each slot's block (-1 for a padding row's slot
         -1): two device operations with no data-dependent shape and no host round trip, which a graph capture
         can record.  It is rebuilt at the first layer of every pass, so a pass recorded after an eager warm-up
-        on the same context object contains it.  Everything else (prefill, host slot mappings) takes the distinct
-        blocks, once per step."""
+        on the same context object contains it (no row index: with one row per sequence the kernel's scan of
+        the slot list is short).  Everything else (prefill, host slot mappings) takes the distinct blocks with
+        the index of their rows, once per step."""
         cfg = self.config
         on_device = (ctx is not None and not ctx.is_prefill and isinstance(ctx.slot_mapping, Tensor)
                      and ctx.slot_mapping.device.type == "cuda")

@@ -8,7 +8,7 @@ Python and nothing is routed to torch kernels.
 
 from __future__ import annotations
 
-from typing import Optional, Tuple
+from typing import NamedTuple, Optional, Tuple
 
 import torch
 from torch import Tensor
@@ -178,28 +178,52 @@ def quantize_kv_e4m3(pool: Tensor, block_size: int) -> Tuple[Tensor, Tensor]:
     return dst, scale
 
 
-def touched_blocks(slots: Tensor, block_size: int, num_blocks: int) -> Tensor:
-    """Distinct blocks (int32, on the device) that the non-negative, in-pool slots fall in."""
+class TouchedBlocks(NamedTuple):
+    """The distinct blocks a slot list writes to and the index of its rows by block that ``pa_kv_append_e4m3``
+    takes: rows ``row_order[block_start[i]:block_start[i + 1]]`` are the tokens whose slots fall in ``blocks[i]``."""
+
+    blocks: Tensor       # int32 [n_touched]
+    row_order: Tensor    # int32 [n_rows], token indices grouped by block
+    block_start: Tensor  # int32 [n_touched + 1]
+
+
+def touched_blocks(slots: Tensor, block_size: int, num_blocks: int) -> TouchedBlocks:
+    """Distinct blocks (int32, on the device) that the non-negative, in-pool slots fall in, with the rows of
+    each: an append workgroup then reads the slots of its own block instead of the whole list."""
     blocks = torch.div(slots, block_size, rounding_mode="floor")
-    blocks = blocks[(slots >= 0) & (blocks < num_blocks)]
-    return torch.unique(blocks).to(torch.int32)
+    rows = torch.nonzero((slots >= 0) & (blocks < num_blocks)).reshape(-1)
+    uniq, inverse, counts = torch.unique(blocks[rows], return_inverse=True, return_counts=True)
+    order = rows[torch.argsort(inverse, stable=True)]
+    start = torch.zeros(uniq.numel() + 1, dtype=torch.int32, device=slots.device)
+    start[1:] = torch.cumsum(counts, 0)
+    return TouchedBlocks(uniq.to(torch.int32), order.to(torch.int32).contiguous(), start)
+
+
+def _touched_args(touched, slots: Tensor, block_size: int, num_blocks: int):
+    """(blocks, row_order, block_start) for the append calls: ``touched`` is a TouchedBlocks, a bare int32 tensor
+    of blocks (no index: every workgroup scans the slot list) or None (computed here)."""
+    if touched is None:
+        touched = touched_blocks(slots, block_size, num_blocks)
+    if isinstance(touched, TouchedBlocks):
+        return touched.blocks, touched.row_order, touched.block_start
+    return touched, None, None
 
 
 def kv_append_e4m3(k_cache: Tensor, v_cache: Tensor, k_scale: Tensor, v_scale: Tensor, k_src: Tensor, v_src: Tensor,
-                   slots: Tensor, block_size: int, touched: Optional[Tensor] = None) -> None:
+                   slots: Tensor, block_size: int, touched=None) -> None:
     """Append rows to an fp8-e4m3 pool with the "re-round on growth" policy of ``pa_kv_append_e4m3``.
 
     k_cache/v_cache ``[total_slots, Hkv, D]`` float8_e4m3fn, scales ``float32 [num_blocks, Hkv]`` (updated in
-    place), k_src/v_src ``[N, Hkv, D]`` fp32/bf16/fp16, slots ``int64 [N]``.  ``touched`` (the distinct target
-    blocks) is computed with torch when not given.
+    place), k_src/v_src ``[N, Hkv, D]`` fp32/bf16/fp16, slots ``int64 [N]``.  ``touched`` (a ``TouchedBlocks``
+    from ``touched_blocks``, or a bare int32 tensor of the distinct target blocks without the row index) is
+    computed with torch when not given.
     """
     total_slots, hkv, d = k_cache.shape
     num_blocks = total_slots // block_size
-    if touched is None:
-        touched = touched_blocks(slots, block_size, num_blocks)
+    blocks, order, start = _touched_args(touched, slots, block_size, num_blocks)
     _run("pa_kv_append_e4m3", _ptr(k_cache), _ptr(v_cache), _ptr(k_scale), _ptr(v_scale), _ptr(k_src), _ptr(v_src),
-         _ptr(slots), slots.numel(), _ptr(touched), touched.numel(), num_blocks, block_size, hkv, d,
-         PA_DTYPE[k_src.dtype], _stream(k_cache))
+         _ptr(slots), slots.numel(), _ptr(blocks), blocks.numel(), _ptr(order), _ptr(start), num_blocks, block_size,
+         hkv, d, PA_DTYPE[k_src.dtype], _stream(k_cache))
 
 
 def rope_kv_append(q: Tensor, k_src: Tensor, v_src: Tensor, cos: Tensor, sin: Tensor, k_cache: Optional[Tensor],
@@ -233,7 +257,7 @@ def rope_kv_append(q: Tensor, k_src: Tensor, v_src: Tensor, cos: Tensor, sin: Te
 def rope_kv_append_e4m3(q: Tensor, k_src: Tensor, v_src: Tensor, cos: Tensor, sin: Tensor, k_cache: Tensor,
                         v_cache: Tensor, k_scale: Tensor, v_scale: Tensor, slots: Tensor, block_size: int,
                         positions: Optional[Tensor] = None, q_out: Optional[Tensor] = None,
-                        touched: Optional[Tensor] = None) -> Tensor:
+                        touched=None) -> Tensor:
     """``rope_kv_append`` into an fp8-e4m3 pool (``pa_rope_kv_append_e4m3``): k is rotated while the fp8 append
     reads it; arguments as in ``rope_kv_append`` and ``kv_append_e4m3``."""
     n, hq, d = q.shape
@@ -246,11 +270,11 @@ def rope_kv_append_e4m3(q: Tensor, k_src: Tensor, v_src: Tensor, cos: Tensor, si
             raise RuntimeError("q, k, v, cos and sin must have the same dtype")
     if positions is not None and positions.dtype != torch.int32:
         raise ValueError("positions must be int32")
-    if touched is None:
-        touched = touched_blocks(slots, block_size, num_blocks)
+    blocks, order, start = _touched_args(touched, slots, block_size, num_blocks)
     _run("pa_rope_kv_append_e4m3", _ptr(q), _ptr(q_out), _ptr(k_src), _ptr(v_src), _ptr(k_cache), _ptr(v_cache),
          _ptr(k_scale), _ptr(v_scale), _ptr(cos), _ptr(sin), _ptr(positions), cos.shape[0], _ptr(slots), n,
-         _ptr(touched), touched.numel(), num_blocks, block_size, hq, hkv, d, PA_DTYPE[q.dtype], _stream(q))
+         _ptr(blocks), blocks.numel(), _ptr(order), _ptr(start), num_blocks, block_size, hq, hkv, d,
+         PA_DTYPE[q.dtype], _stream(q))
     return q_out
 
 

@@ -33,7 +33,7 @@ def test_binding_table_matches_header():
 
 def test_version_and_dtype_sizes():
     lib = _lib.load()
-    assert lib.pa_version() == 3
+    assert lib.pa_version() == 4
     assert [lib.pa_dtype_bytes(c) for c in (0, 1, 2, 3, 4, -1)] == [4, 2, 2, 1, 0, 0]
 
 
@@ -146,16 +146,19 @@ def test_prefill_and_quantize_argument_errors():
     assert rc == _lib.PA_ERR_INVALID_ARG and "src_dtype" in msg
     rc, msg = _status("pa_quantize_kv_e4m3", None, FAKE, FAKE, 4, 16, 8, 128, _lib.PA_F32, None)
     assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
-    append = [FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 5, FAKE, 2, 64, 16, 8, 128, _lib.PA_BF16, None]
-    bad = list(append); bad[14] = _lib.PA_FP8_E4M3
+    append = [FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 5, FAKE, 2, None, None, 64, 16, 8, 128, _lib.PA_BF16, None]
+    bad = list(append); bad[16] = _lib.PA_FP8_E4M3
     rc, msg = _status("pa_kv_append_e4m3", *bad)
     assert rc == _lib.PA_ERR_INVALID_ARG and "src_dtype" in msg
-    bad = list(append); bad[11] = 1024
+    bad = list(append); bad[13] = 1024
     rc, msg = _status("pa_kv_append_e4m3", *bad)
     assert rc == _lib.PA_ERR_INVALID_ARG and "block_size" in msg
     bad = list(append); bad[8] = None
     rc, msg = _status("pa_kv_append_e4m3", *bad)
     assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
+    bad = list(append); bad[10] = FAKE  # a row order without the block starts
+    rc, msg = _status("pa_kv_append_e4m3", *bad)
+    assert rc == _lib.PA_ERR_INVALID_ARG and "row_order" in msg
     bad = list(append); bad[7] = 0  # nothing to append: fine even with no device
     rc, msg = _status("pa_kv_append_e4m3", *bad)
     assert rc == _lib.PA_OK
@@ -180,9 +183,9 @@ def test_rope_argument_errors():
     assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
     bad = list(rope); bad[12] = 0
     assert _status("pa_rope_kv_append", *bad)[0] == _lib.PA_OK
-    fp8 = [FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, None, 8, FAKE, 4, FAKE, 1, 64, 16, 32, 8, 128,
-           _lib.PA_BF16, None]
-    bad = list(fp8); bad[17] = 1024
+    fp8 = [FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, None, 8, FAKE, 4, FAKE, 1, None, None, 64, 16, 32,
+           8, 128, _lib.PA_BF16, None]
+    bad = list(fp8); bad[19] = 1024
     rc, msg = _status("pa_rope_kv_append_e4m3", *bad)
     assert rc == _lib.PA_ERR_INVALID_ARG and "block_size" in msg
     bad = list(fp8); bad[11] = 2

@@ -215,3 +215,45 @@ def test_fp8_append_shapes(hkv, d, bs, dtype):
         ops.kv_append_e4m3(kc, vc, ks, vs, k.to(DEV), v.to(DEV), slots.to(DEV), bs)
         assert torch.equal(kc.cpu().view(torch.uint8), bits) and torch.equal(ks.cpu(), scale)
         assert torch.equal(vc.cpu().view(torch.uint8), vbits) and torch.equal(vs.cpu(), vscale)
+
+
+def test_fp8_append_with_and_without_the_row_index():
+    """The append with the index of rows by touched block (what ops.touched_blocks builds), with a bare list of
+    blocks (every workgroup scans the slot list) and with the list in another order than the index's sort: the
+    same bytes and scales, on a shuffled slot list with skipped rows and a slot written twice."""
+    announce("fp8 append row index")
+    g = torch.Generator().manual_seed(31)
+    nb, bs, hkv, d = 40, 16, 4, 128
+    n = 500
+    slots = torch.randperm(nb * bs, generator=g)[:n]
+    slots[7] = -1
+    slots[300] = nb * bs + 3
+    slots[450] = slots[20]  # written twice: the later row is stored
+    k = torch.randn(n, hkv, d, generator=g).to(torch.bfloat16)
+    v = torch.randn(n, hkv, d, generator=g).to(torch.bfloat16)
+    results = []
+    for mode in ("index", "scan", "reordered"):
+        bits, scale = _fp8_pool(nb, bs, hkv, d)
+        kc = bits.clone().view(torch.float8_e4m3fn).to(DEV)
+        vc = bits.clone().view(torch.float8_e4m3fn).to(DEV)
+        ks, vs = scale.clone().to(DEV), scale.clone().to(DEV)
+        touched = ops.touched_blocks(slots.to(DEV), bs, nb)
+        assert int(touched.block_start[-1]) == n - 2 and touched.row_order.numel() == n - 2
+        if mode == "scan":
+            touched = touched.blocks
+        elif mode == "reordered":
+            perm = torch.randperm(touched.blocks.numel(), generator=g).to(DEV)
+            counts = (touched.block_start[1:] - touched.block_start[:-1])[perm]
+            start = torch.zeros_like(touched.block_start)
+            start[1:] = torch.cumsum(counts, 0)
+            order = torch.cat([touched.row_order[int(touched.block_start[i]): int(touched.block_start[i + 1])]
+                               for i in perm.tolist()])
+            touched = ops.TouchedBlocks(touched.blocks[perm].contiguous(), order.contiguous(), start)
+        ops.kv_append_e4m3(kc, vc, ks, vs, k.to(DEV), v.to(DEV), slots.to(DEV), bs, touched)
+        results.append((kc.cpu().view(torch.uint8), vc.cpu().view(torch.uint8), ks.cpu(), vs.cpu()))
+    want_bits, want_scale = _fp8_pool(nb, bs, hkv, d)
+    po.append_kv_e4m3(want_bits, want_scale, k, slots.tolist(), bs)
+    for got in results:
+        assert torch.equal(got[0], want_bits) and torch.equal(got[2], want_scale)
+        for a, b in zip(got, results[0]):
+            assert torch.equal(a, b)
