@@ -31,6 +31,8 @@ Register map (per lane; the kernel pins its variables to the same registers):
               (v95 also a row's last visible key relative to the subtile), v[97:98] pair sums, v99 scratch
   v[100:111]  LDS addresses of stages 2 and 3 (the operands hold those of stages 0 and 1)
   v[112:115]  zeros, v116 -inf
+  v[118:149]  minus the rows' reference maxima, one 16-register tile per column tile (the accumulator input of
+              the first S^T product)
   s[40:63]    scalars of the tile loads, the calls, the masks and the rescale checks
 
 Usage: python3 gen_prefill_loop.py [output file]   (default: prefill_mfma_loop.inc beside this script)
@@ -78,6 +80,10 @@ def S(buf, c):
 
 def PP(c, j):
     return 64 + 8 * c + j
+
+
+def CT(c):
+    return 118 + 16 * c
 
 
 STUBS = []  # out-of-line code of the loop being generated: the common path of every check falls through
@@ -139,8 +145,12 @@ def subtile_ops(ty, j, kt):
     for ks in range(KS):
         for c in range(NC):
             s = S(nb, c)
-            src_c = "0" if ks == 0 else vreg(s, 16)
+            # The first product of a column tile accumulates onto minus the row's reference maximum (the same
+            # value in all 16 registers of a lane), and Q^T arrives scaled by softmax scale * log2(e): S^T comes
+            # out as the argument of the exponential, and no instruction per value is spent on forming it.
+            src_c = vreg(CT(c), 16) if ks == 0 else vreg(s, 16)
             mf.append(Ins(f"{ty.mfma} {vreg(s, 16)}, {areg(KA(ks), 4)}, {Q(c, ks)}, {src_c}", units=2, kind="mfma",
+                          reads=[f"v{CT(c) + i}" for i in range(16)] if ks == 0 else (),
                           writes=[f"v{s + i}" for i in range(16)], need=(f"ka{ks}",)))
     for step in range(2):
         for dt in range(DT):
@@ -198,10 +208,8 @@ def subtile_ops(ty, j, kt):
         c, jj = n & 1, n >> 1
         s0 = S(cb, c) + 2 * jj
         ta, tb = 80 + 2 * (n % 4), 81 + 2 * (n % 4)
-        return [Ins(f"v_fma_f32 v{ta}, v{s0}, %[sc], -%[msc{c}]", reads=(f"v{s0}",), writes=(f"v{ta}",)),
-                Ins(f"v_fma_f32 v{tb}, v{s0 + 1}, %[sc], -%[msc{c}]", reads=(f"v{s0 + 1}",), writes=(f"v{tb}",)),
-                Ins(f"{'v_mov_b32_e32' if 'noexp' in X else 'v_exp_f32_e32'} v{ta}, v{ta}", units=2, kind="trans", reads=(f"v{ta}",), writes=(f"v{ta}",)),
-                Ins(f"{'v_mov_b32_e32' if 'noexp' in X else 'v_exp_f32_e32'} v{tb}, v{tb}", units=2, kind="trans", reads=(f"v{tb}",), writes=(f"v{tb}",))]
+        return [Ins(f"{'v_mov_b32_e32' if 'noexp' in X else 'v_exp_f32_e32'} v{ta}, v{s0}", units=2, kind="trans", reads=(f"v{s0}",), writes=(f"v{ta}",)),
+                Ins(f"{'v_mov_b32_e32' if 'noexp' in X else 'v_exp_f32_e32'} v{tb}, v{s0 + 1}", units=2, kind="trans", reads=(f"v{s0 + 1}",), writes=(f"v{tb}",))]
 
     # The row sums are plain fp32 additions: v_dot2 on the packed words would be one instruction instead of
     # two, but it does not run beside the matrix unit (measured: a product followed by two of them takes 58
@@ -266,8 +274,8 @@ def subtile_ops(ty, j, kt):
                          writes=(f"v{m[c]}", f"v{w[c]}")), 21))
         mx.append(Op(Ins(f"v_max_f32_e32 %[mx{c}], v{m[c]}, v{w[c]}", reads=(f"v{m[c]}", f"v{w[c]}")), 21))
     # does a row's maximum exceed its reference by more than the slack?  (read at the start of the next subtile)
-    mx.append(Op(Ins("v_cmp_gt_f32_e64 s[60:61], %[mx0], %[thr0]"), 21))
-    mx.append(Op(Ins("v_cmp_gt_f32_e64 s[62:63], %[mx1], %[thr1]"), 21))
+    mx.append(Op(Ins("v_cmp_gt_f32_e64 s[60:61], %[mx0], %[slack]"), 21))
+    mx.append(Op(Ins("v_cmp_gt_f32_e64 s[62:63], %[mx1], %[slack]"), 21))
     # (order: chain 0, copy 0, chain 1, copy 1, swap 0, max 0, swap 1, max 1: two instructions between a copy and its swap)
     streams["max"] = mx
 
@@ -448,18 +456,23 @@ def check_hazards(bodies):
 
 
 def rescale(ty):
-    """Called when a row's maximum outgrew its reference by more than the slack: the textbook rescale of sums
-    and accumulators for both column tiles, with the accumulators read from and written back to AGPRs."""
+    """Called when the S^T values of a row (which are relative to the row's reference maximum) exceed the slack:
+    the reference moves up by delta = max(maximum, 0) for both column tiles - the reference tiles, both S^T
+    buffers (the current one was formed against the old reference; the other is dead and about to be
+    overwritten) and the maximum itself shift by -delta, sums and accumulators (read from and written back to
+    AGPRs) shrink by 2^-delta."""
     out = ["s_nop 7", "s_nop 7", "s_nop 7"]  # products still writing the accumulators
     for c in range(NC):
-        out += [f"v_max_f32_e32 v97, %[mraw{c}], %[mx{c}]",
-                f"v_sub_f32_e32 v98, %[mraw{c}], v97",
-                f"v_mul_f32_e32 v98, %[sc], v98",
-                f"v_exp_f32_e32 v98, v98",
-                f"v_mov_b32_e32 %[mraw{c}], v97",
-                f"v_add_f32_e32 %[thr{c}], %[slack], v97",
-                f"v_mul_f32_e32 %[msc{c}], %[sc], v97",
+        out += [f"v_max_f32_e32 v97, 0, %[mx{c}]",
+                "v_exp_f32_e64 v98, -v97",
+                f"v_sub_f32_e32 %[mx{c}], %[mx{c}], v97",
+                "s_nop 0",
                 f"v_mul_f32_e32 %[l{c}], %[l{c}], v98"]
+        for i in range(16):
+            out.append(f"v_sub_f32_e32 v{CT(c) + i}, v{CT(c) + i}, v97")
+        for buf in range(2):
+            for i in range(16):
+                out.append(f"v_sub_f32_e32 v{S(buf, c) + i}, v{S(buf, c) + i}, v97")
         for dt in range(DT):
             base = 16 * (4 * c + dt)
             for i in range(0, 16, 2):
@@ -483,8 +496,8 @@ def loop_text(ty):
     for dt in range(DT):
         lines.append(f"v_add_u32_e32 v{108 + dt}, {2 * STAGE}, %[vad{dt}]")
     lines += [f"v_mov_b32_e32 v{r}, 0" for r in range(112, 116)]
-    lines += ["v_mov_b32_e32 v116, 0xff800000", "v_cmp_gt_f32_e64 s[60:61], %[mx0], %[thr0]",
-              "v_cmp_gt_f32_e64 s[62:63], %[mx1], %[thr1]", "s_waitcnt lgkmcnt(0)", "s_nop 3"]
+    lines += ["v_mov_b32_e32 v116, 0xff800000", "v_cmp_gt_f32_e64 s[60:61], %[mx0], %[slack]",
+              "v_cmp_gt_f32_e64 s[62:63], %[mx1], %[slack]", "s_waitcnt lgkmcnt(0)", "s_nop 3"]
     for j in range(NSTAGE):
         lines.append(f".Lpf_tile{j}_%=:")
         lines += [ins.text for ins in bodies[j]]

@@ -126,6 +126,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         if (lane == 0) s_special[wave] = first_special;
     }
     pf_wait_loads<0>();
+    const float sc = p.scale_log2;
     X8 qreg[NC][KS];
 #pragma unroll
     for (int c = 0; c < NC; ++c)
@@ -133,7 +134,13 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         for (int ks = 0; ks < KS; ++ks) {
             const int slot = (2 * ks + half) ^ (col & (QCPR - 1));
             const uint4 raw = *reinterpret_cast<const uint4 *>(s_mem + q_stage + (c * 32 + col) * QRB + slot * 16);
-            qreg[c][ks] = __builtin_bit_cast(X8, raw);
+            // scaled by softmax scale * log2(e) here, once per workgroup: S^T then comes out of the products in
+            // the units of the exponential's argument (one more rounding of q to its 16-bit type)
+            const X8 q8 = __builtin_bit_cast(X8, raw);
+            uint32_t w[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) w[e] = M::pack((float)q8[2 * e] * sc, (float)q8[2 * e + 1] * sc);
+            qreg[c][ks] = __builtin_bit_cast(X8, uint4{w[0], w[1], w[2], w[3]});
         }
 #pragma unroll
     for (int c = 0; c < NC; ++c)
@@ -192,8 +199,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     }
 
     // ---- first subtile: S^T, mask, row maxima; K operands of the second subtile ----
-    const float sc = p.scale_log2;
-    const float slack_raw = kPfSlack / sc;
     f32x16 s0[NC];
     X8 ka[KS];
     float mx[NC];
@@ -227,6 +232,22 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             mx[c] = fmaxf(__builtin_bit_cast(float, (uint32_t)sw[0]), __builtin_bit_cast(float, (uint32_t)sw[1]));
         }
     }
+    // The reference maximum of a row starts as the maximum of its first subtile (every row sees key 0, so it is
+    // finite).  From here on S^T is kept relative to the reference: the loop's first product of each column
+    // tile accumulates onto ref[c] = minus the reference in all 16 registers, the exponentials take S^T as it
+    // is, and mx is the maximum relative to the reference (0 now).  The reference moves up only when a later
+    // maximum exceeds it by more than kPfSlack (lazy rescale: see prefill_mfma_kernel).
+    f32x16 ref[NC];
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+        const float m0 = mx[c] > kNegBig ? mx[c] : 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            s0[c][i] -= m0;
+            ref[c][i] = -m0;
+        }
+        mx[c] = 0.f;
+    }
 
     f32x16 o[NC][DT];
 #pragma unroll
@@ -235,11 +256,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) o[c][dt][i] = 0.f;
-    // running maximum of the raw logits, its threshold and scaled copy, running sum (lazy rescale: see
-    // prefill_mfma_kernel)
-    float m_raw[NC], m_sc[NC], m_thr[NC], l_run[NC];
-#pragma unroll
-    for (int c = 0; c < NC; ++c) { m_raw[c] = kNegBig; m_thr[c] = kNegBig; m_sc[c] = kNegBig * sc; l_run[c] = 0.f; }
+    float l_run[NC] = {0.f, 0.f};  // running sums
 
     {
         int n_left = n_tiles - 1;  // tiles after the current one
@@ -253,14 +270,14 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         const uint32_t pklo = __builtin_amdgcn_readfirstlane((uint32_t)pk), pkhi = __builtin_amdgcn_readfirstlane((uint32_t)(pk >> 32));
         const uint32_t pvlo = __builtin_amdgcn_readfirstlane((uint32_t)pv), pvhi = __builtin_amdgcn_readfirstlane((uint32_t)(pv >> 32));
         const uint32_t stride = (uint32_t)tok_stride;
+        const float slack = kPfSlack;  // in the units of S^T here: log2 of the factor a row's reference may lag by
 #define PA_LOOP_OPERANDS                                                                                              \
     : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[0][2]), "+{a[48:63]}"(o[0][3]),                    \
       "+{a[64:79]}"(o[1][0]), "+{a[80:95]}"(o[1][1]), "+{a[96:111]}"(o[1][2]), "+{a[112:127]}"(o[1][3]),                \
-      "+{v[0:15]}"(s0[0]), "+{v[16:31]}"(s0[1]),                                                                      \
+      "+{v[0:15]}"(s0[0]), "+{v[16:31]}"(s0[1]), "+{v[118:133]}"(ref[0]), "+{v[134:149]}"(ref[1]),                    \
       "+{a[192:195]}"(ka[0]), "+{a[196:199]}"(ka[1]), "+{a[200:203]}"(ka[2]), "+{a[204:207]}"(ka[3]),                   \
       "+{a[208:211]}"(ka[4]), "+{a[212:215]}"(ka[5]), "+{a[216:219]}"(ka[6]), "+{a[220:223]}"(ka[7]),                   \
-      [mx0] "+&v"(mx[0]), [mx1] "+&v"(mx[1]), [msc0] "+&v"(m_sc[0]), [msc1] "+&v"(m_sc[1]), [thr0] "+&v"(m_thr[0]),          \
-      [thr1] "+&v"(m_thr[1]), [mraw0] "+&v"(m_raw[0]), [mraw1] "+&v"(m_raw[1]), [l0] "+&v"(l_run[0]), [l1] "+&v"(l_run[1]),  \
+      [mx0] "+&v"(mx[0]), [mx1] "+&v"(mx[1]), [l0] "+&v"(l_run[0]), [l1] "+&v"(l_run[1]),                             \
       [ntiles] "+&s"(n_left), [sT] "+&s"(s_t), [sP] "+&s"(s_p), [srem] "+&s"(s_rem)                                         \
     : "{a[128:131]}"(qreg[0][0]), "{a[132:135]}"(qreg[0][1]), "{a[136:139]}"(qreg[0][2]), "{a[140:143]}"(qreg[0][3]),   \
       "{a[144:147]}"(qreg[0][4]), "{a[148:151]}"(qreg[0][5]), "{a[152:155]}"(qreg[0][6]), "{a[156:159]}"(qreg[0][7]),   \
@@ -269,7 +286,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
       [kad0] "v"(kad[0]), [kad1] "v"(kad[1]), [kad2] "v"(kad[2]), [kad3] "v"(kad[3]), [kad4] "v"(kad[4]),               \
       [kad5] "v"(kad[5]), [kad6] "v"(kad[6]), [kad7] "v"(kad[7]), [vad0] "v"(vad[0]), [vad1] "v"(vad[1]),               \
       [vad2] "v"(vad[2]), [vad3] "v"(vad[3]), [lanek] "v"(lane_k), [lanev] "v"(lane_v), [lane16] "v"(lane16),           \
-      [arow] "v"(arow_u), [lim0] "v"(lim[0]), [lim1] "v"(lim[1]), [sc] "s"(sc), [slack] "s"(slack_raw),                 \
+      [arow] "v"(arow_u), [lim0] "v"(lim[0]), [lim1] "v"(lim[1]), [slack] "s"(slack),                                   \
       [pklo] "s"(pklo), [pkhi] "s"(pkhi), [pvlo] "s"(pvlo), [pvhi] "s"(pvhi), [stride] "s"(stride), [m0w] "s"(m0w),     \
       [nreal] "s"(n_real_u), [tabA] "s"(tab_a_base), [tabB] "s"(tab_b_base), [splo] "s"(sp_lo),                       \
       [spspan] "s"(sp_span), [captiles] "s"(cap_tiles), [maskfrom] "s"(mask_from_u)                                   \

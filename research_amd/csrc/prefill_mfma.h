@@ -14,22 +14,20 @@
 // order, so P never moves between lanes.
 //
 // Work split
-//   workgroup = 8 waves (two per SIMD, so one wave's softmax arithmetic runs
-//   under the other's matrix instructions); a wave owns 32 query rows (one MFMA
-//   column tile) of ONE query head and keeps everything in ordinary VGPRs
-//   (64 accumulators + 32 for Q + 16 for S); the 8 waves take 8 consecutive
-//   (row block, query head of the kv head) tasks, so they share every K/V tile
-//   (GQA packing: K/V are fetched once per kv head, not per query head).
-//   grid.x = kv head (fastest): with 8 XCDs a kv head's K/V stays in one XCD's
-//   L2 while all sequences and row blocks that share prefix blocks re-read it.
-//   K/V tiles of 64 keys go global -> LDS directly (global_load_lds, 16 bytes per
-//   lane, no staging registers) into one of two buffers, so the next tile's
-//   loads are in flight while the current tile is multiplied and there is one
-//   barrier per tile.  A direct load puts lane i's 16 bytes at base + 16*i, so
-//   rows cannot be padded; instead each lane fetches the chunk that belongs at
-//   its position under an XOR swizzle of the chunk index by the row, chosen so
-//   that the 128-bit operand reads (16 rows, same chunk) and the transpose
-//   reads (4 rows x 64 bytes) each touch all 64 banks once.
+//   workgroup = 4 waves, one per SIMD; a wave owns two 32-row column tiles (tasks): 64 query rows of one or two
+//   (row block, query head of the kv head) pairs, so every K / V^T operand it reads from LDS feeds two products.
+//   Accumulators (128 registers), Q^T operands (64) and S^T (2 x 32) fill the 512 registers a lane has, which is
+//   why there is one wave per SIMD and why the instruction order below is written out: nothing but the wave's
+//   own order hides latency.  The 8 tasks of a workgroup are consecutive (row block, head) pairs of one kv
+//   head, so they share every K/V tile (GQA packing: K/V are fetched once per kv head, not per query head).
+//   grid.x = kv head (fastest): with 8 XCDs a kv head's K/V stays in one XCD's L2 while all sequences and row
+//   blocks that share prefix blocks re-read it.
+//   K/V tiles of 64 keys go global -> LDS directly (global_load_lds, 16 bytes per lane, no staging registers)
+//   into a ring of four stages: the loads of tile t+3 are in flight while tile t is multiplied, and there is
+//   one barrier per tile.  A direct load puts lane i's 16 bytes at base + 16*i, so rows cannot be padded;
+//   instead each lane fetches the chunk that belongs at its position under an XOR swizzle of the chunk index by
+//   the row, chosen so that the 128-bit operand reads (16 rows, same chunk) and the transpose reads (4 rows x
+//   64 bytes) each touch all 64 banks once.
 #pragma once
 #include "decode_impl.h"
 
