@@ -296,3 +296,42 @@ def test_assembly_loop_kernel_long_context_and_table_limit():
         got = ops.prefill_paged(*args).float().cpu()
         want = ops.prefill_paged(*args, rowwise=True).float().cpu()
         assert_close(got, want, 2e-2, f"context of {ctx} keys")
+
+
+@pytest.mark.parametrize("d", [64, 128, 256])
+def test_logits_that_grow_along_the_context(d):
+    """Keys whose logits rise steeply with the key index (about 9 in base-2 units per 32 keys, from far below
+    zero to far above), so that every row's reference maximum is outgrown by more than the lazy-rescale slack
+    again and again, by some rows of a wave earlier than by others; then the same keys in falling order (the
+    first subtile holds the maximum, nothing is ever rescaled).  All three matrix-core kernels (head_dim 64
+    compiled, 128 assembly loop, 256), chunked over a prefix, against the checker."""
+    announce(f"prefill rescale paths d={d}")
+    rng = np.random.default_rng(500 + d)
+    hq, hkv, bs = 4, 2, 16
+    prefix, chunk = [700, 0, 333], [200, 130, 64]
+    cmax = max(chunk)
+    need = [-(-(p + c) // bs) for p, c in zip(prefix, chunk)]
+    nb = sum(need) + 1
+    perm = rng.permutation(nb)
+    tables, at = [], 0
+    for n in need:
+        tables.append(perm[at : at + n].tolist())
+        at += n
+    q = torch.from_numpy((rng.standard_normal((len(chunk), cmax, hq, d)) + 2.0).astype(np.float32)).to(torch.bfloat16)
+    vc = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+    for direction in (1, -1):
+        kc = torch.zeros(nb * bs, hkv, d)
+        for b, (p, c) in enumerate(zip(prefix, chunk)):
+            n = p + c
+            # natural-unit logit of key j for a row with sum(q) = 2d: about ramp[j]
+            ramp = np.linspace(-40.0, 0.2 * n - 40.0, n)[::direction].copy()
+            rows = ramp[:, None, None] * np.ones((1, hkv, d)) / (2.0 * d ** 0.5) + 0.05 * rng.standard_normal((n, hkv, d))
+            for j in range(n):
+                kc[tables[b][j // bs] * bs + j % bs] = torch.from_numpy(rows[j].astype(np.float32))
+        kc = kc.to(torch.bfloat16)
+        want = po.paged_prefill_chunk(q, kc, vc, tables, prefix, chunk, bs, d ** -0.5)
+        out = torch.zeros(len(chunk) * cmax, hq, d, device=DEV, dtype=torch.bfloat16)
+        ops.prefill_paged(q.reshape(-1, hq, d).to(DEV), kc.to(DEV), vc.to(DEV), tables_to_device(tables),
+                          _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk), _i32(np.arange(len(chunk)) * cmax),
+                          cmax, bs, d ** -0.5, out=out)
+        assert_close(out.reshape(len(chunk), cmax, hq, d), want, 2e-2, f"logits {'rising' if direction > 0 else 'falling'}")
