@@ -143,7 +143,13 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     for (int ks = 0; ks < KS; ++ks) {
         const int slot = (2 * ks + half) ^ (col & (CPR - 1));
         const uint4 raw = *reinterpret_cast<const uint4 *>(s_mem + q_stage + col * RB + slot * 16);
-        qreg[ks] = __builtin_bit_cast(X8, raw);
+        // scaled by softmax scale * log2(e) here, once per workgroup: S^T then comes out of the products in the
+        // units of the exponential's argument (one more rounding of q to its 16-bit type)
+        const X8 q8 = __builtin_bit_cast(X8, raw);
+        uint32_t w[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) w[e] = M::pack((float)q8[2 * e] * p.scale_log2, (float)q8[2 * e + 1] * p.scale_log2);
+        qreg[ks] = __builtin_bit_cast(X8, uint4{w[0], w[1], w[2], w[3]});
     }
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qreg[ks]));  // (product operands live in AGPRs)
@@ -338,14 +344,18 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     fix_k(t0); fix_v(t0);
     __syncthreads();
 
-    const float sc = p.scale_log2;
-    const float slack_raw = kPfSlack / sc;
     f32x16 o[DT];
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
-    float m_raw = kNegBig, m_thr = kNegBig, m_sc = kNegBig * sc, l_run = 0.f, mx = kNegBig;
+    // S^T is kept relative to the row's reference maximum (see prefill_mfma_kernel): the first product of a
+    // subtile accumulates onto ref = minus the reference in all 16 registers, the exponentials take S^T as it
+    // is, mx is relative too; m_thr is what mx must exceed for a rescale (kNegBig until the row has seen a key).
+    f32x16 ref;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) ref[i] = 0.f;
+    float m_thr = kNegBig, l_run = 0.f, mx = kNegBig;
     X8 ka[KS], va0[DT], va1[DT];
     f32x16 sb[2];  // S^T of the current and of the next subtile, swapping roles every subtile
 
@@ -354,9 +364,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     read_v(t0, 0, va0);
     PF_FENCE();
 #pragma unroll
-    for (int i = 0; i < 16; ++i) sb[0][i] = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) sb[0] = M::mma(ka[ks], qreg[ks], sb[0]);
+    for (int ks = 0; ks < KS; ++ks) sb[0] = M::mma(ka[ks], qreg[ks], ks == 0 ? ref : sb[0]);
     PF_FENCE();
     read_k(t0, ka);
     PF_FENCE();
@@ -381,8 +389,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         float sum = 0.f;
         // exponentials of S^T values 2*j, 2*j+1, packed as a P^T operand word
         auto exp_piece = [&](int j) PF_INLINE {
-            const float p0 = __builtin_amdgcn_exp2f(fmaf(s[2 * j], sc, -m_sc));
-            const float p1 = __builtin_amdgcn_exp2f(fmaf(s[2 * j + 1], sc, -m_sc));
+            const float p0 = __builtin_amdgcn_exp2f(s[2 * j]);
+            const float p1 = __builtin_amdgcn_exp2f(s[2 * j + 1]);
             sum += p0 + p1;
             uint32_t w = M::pack(p0, p1);
             asm volatile("" : "+v"(w), "+v"(sum));
@@ -390,24 +398,30 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         };
         // ---- the row maximum outgrew its reference by more than the slack (rare): rescale ----
         if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m_thr) != 0, 0)) {
-            const float m_new = fmaxf(m_raw, mx);
-            const float alpha = __builtin_amdgcn_exp2f((m_raw - m_new) * sc);
+            // the reference moves by delta: up to the new maximum, or - for a row that had seen no key so far
+            // (sum and accumulators still zero) - to its first maximum, whatever its sign
+            const bool unset = m_thr == kNegBig;
+            const bool seen = mx > kNegBig;
+            const float delta = unset ? (seen ? mx : 0.f) : fmaxf(mx, 0.f);
+            const float alpha = unset ? 1.f : __builtin_amdgcn_exp2f(-delta);
             l_run *= alpha;
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
-            m_raw = m_new;
-            m_thr = m_new + slack_raw;
-            m_sc = m_new * sc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                ref[i] -= delta;
+                s[i] -= delta;  // formed against the old reference
+            }
+            mx -= delta;
+            if (seen) m_thr = kPfSlack;
         }
         PF_FENCE();
         // ---- (a) S^T of subtile g+1, with the exponentials of subtile g between the products ----
 #pragma unroll
-        for (int i = 0; i < 16; ++i) s_nx[i] = 0.f;
-#pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            s_nx = M::mma(ka[ks], qreg[ks], s_nx);
+            s_nx = M::mma(ka[ks], qreg[ks], ks == 0 ? ref : s_nx);
             PF_FENCE();
             if (!(ks & 1)) read_v_one(g, 1, ks >> 1, va1[ks >> 1]);  // second k-step's V^T: consumed in (c)
             if (ks & 1) exp_piece(ks >> 1);

@@ -247,7 +247,13 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
             for (int ks = 0; ks < KS; ++ks) {
                 const int slot = (2 * ks + half) ^ (col & (QCPR - 1));
                 const uint4 raw = *reinterpret_cast<const uint4 *>(s_kv + q_stage + (c * 32 + col) * QRB + slot * 16);
-                qreg[c][ks] = __builtin_bit_cast(X8, raw);
+                // scaled by softmax scale * log2(e) here, once per workgroup: S^T then comes out of the products
+                // in the units of the exponential's argument (one more rounding of q to its 16-bit type)
+                const X8 q8 = __builtin_bit_cast(X8, raw);
+                uint32_t w[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) w[e] = M::pack((float)q8[2 * e] * p.scale_log2, (float)q8[2 * e + 1] * p.scale_log2);
+                qreg[c][ks] = __builtin_bit_cast(X8, uint4{w[0], w[1], w[2], w[3]});
             }
     }
 
@@ -265,17 +271,24 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int i = 0; i < 16; ++i) o[c][dt][i] = 0.f;
-    // Running maximum of the raw (unscaled) logits, the same times scale*log2e, and the running sum.
-    // The reference maximum of a row is allowed to lag behind the true running maximum by up to 2^kPfSlack
-    // (as a factor on the probabilities): sums and accumulators are rescaled only when a row's maximum grows
-    // by more than that, which it rarely does, instead of on nearly every subtile.  The result is the same
-    // quotient either way; probabilities stay below 2^kPfSlack, far inside the range of fp32 sums and of the
-    // 16-bit operand types.
-    const float sc = p.scale_log2;
-    const float slack_raw = kPfSlack / sc;
-    float m_raw[NC], m_sc[NC], m_thr[NC], l_run[NC];
+    // S^T is kept relative to a reference maximum per row, in base-2 units (Q^T is scaled): the first product
+    // of a column tile accumulates onto ref[c] = minus the reference in all 16 registers of a lane, so the
+    // exponentials take the S^T values as they are, and a row's maximum mx is relative to its reference too.
+    // The reference is allowed to lag behind the true running maximum by up to 2^kPfSlack (as a factor on the
+    // probabilities): sums and accumulators are rescaled only when a row's maximum grows by more than that,
+    // which it rarely does, instead of on nearly every subtile.  The result is the same quotient either way;
+    // probabilities stay below 2^kPfSlack, far inside the range of fp32 sums and of the 16-bit operand types.
+    // m_thr is what mx must exceed for a rescale: kNegBig while the row has seen no key yet (its reference is
+    // then set by the first maximum, whatever its sign), kPfSlack afterwards.
+    f32x16 ref[NC];
+    float m_thr[NC], l_run[NC];
 #pragma unroll
-    for (int c = 0; c < NC; ++c) { m_raw[c] = kNegBig; m_thr[c] = kNegBig; m_sc[c] = kNegBig * sc; l_run[c] = 0.f; }
+    for (int c = 0; c < NC; ++c) {
+        m_thr[c] = kNegBig;
+        l_run[c] = 0.f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) ref[c][i] = 0.f;
+    }
 
     // ---- tile loader: wave-wide direct load l covers rows l*RPL .. of the tile; wave w issues l = w, w+4, ... ----
     const int32_t *bt_row = p.bt + (int64_t)b * p.bt_stride;
@@ -502,13 +515,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
     };
     auto s_products = [&](const X8 (&ka)[KS], f32x16 (&s)[NC]) PF_INLINE {
 #pragma unroll
-        for (int c = 0; c < NC; ++c)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s[c][i] = 0.f;
-#pragma unroll
         for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-            for (int c = 0; c < NC; ++c) s[c] = M::mma(ka[ks], qreg[c][ks], s[c]);
+            for (int c = 0; c < NC; ++c) s[c] = M::mma(ka[ks], qreg[c][ks], ks == 0 ? ref[c] : s[c]);
     };
 
     // ---- fill the ring: tiles t0 .. t0 + kPfStages-2 ----
@@ -566,10 +575,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
             // exponentials of the pair of S^T values 2*j, 2*j+1 of column tile c, packed as a P^T operand word
             // (pinned like the maxima above: otherwise the compiler gathers all exponentials behind the products)
             auto exp_pair = [&](int c, int j) PF_INLINE {
-                float scl = sc;
-                asm volatile("" : "+s"(scl));  // a scalar copy defined here: the arithmetic cannot start earlier
-                const float p0 = __builtin_amdgcn_exp2f(fmaf(s[c][2 * j], scl, -m_sc[c]));
-                const float p1 = __builtin_amdgcn_exp2f(fmaf(s[c][2 * j + 1], scl, -m_sc[c]));
+                float x0 = s[c][2 * j], x1 = s[c][2 * j + 1];
+                asm volatile("" : "+v"(x0), "+v"(x1));  // copies defined here: the arithmetic cannot start earlier
+                const float p0 = __builtin_amdgcn_exp2f(x0);
+                const float p1 = __builtin_amdgcn_exp2f(x1);
                 sum[c] += p0 + p1;
                 uint32_t w = M::pack(p0, p1);
                 asm volatile("" : "+v"(w), "+v"(sum[c]));
@@ -582,16 +591,24 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
                 if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx[0] > m_thr[0] || mx[1] > m_thr[1]) != 0, 0)) {
 #pragma unroll
                     for (int c = 0; c < NC; ++c) {
-                        const float m_new = fmaxf(m_raw[c], mx[c]);
-                        const float alpha = __builtin_amdgcn_exp2f((m_raw[c] - m_new) * sc);
+                        // the reference moves by delta: up to the new maximum, or - for a row that had seen no
+                        // key so far (sums and accumulators still zero) - to its first maximum, whatever its sign
+                        const bool unset = m_thr[c] == kNegBig;
+                        const bool seen = mx[c] > kNegBig;
+                        const float delta = unset ? (seen ? mx[c] : 0.f) : fmaxf(mx[c], 0.f);
+                        const float alpha = unset ? 1.f : __builtin_amdgcn_exp2f(-delta);
                         l_run[c] *= alpha;
 #pragma unroll
                         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                             for (int i = 0; i < 16; ++i) o[c][dt][i] *= alpha;
-                        m_raw[c] = m_new;
-                        m_thr[c] = m_new + slack_raw;
-                        m_sc[c] = m_new * sc;
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            ref[c][i] -= delta;
+                            s[c][i] -= delta;  // formed against the old reference
+                        }
+                        mx[c] -= delta;
+                        if (seen) m_thr[c] = kPfSlack;
                     }
                 }
                 PF_FENCE();
@@ -601,13 +618,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
                 constexpr int PA = 8 / KS;  // pieces per k-step
                 if (has_next) {
 #pragma unroll
-                    for (int c = 0; c < NC; ++c)
-#pragma unroll
-                        for (int i = 0; i < 16; ++i) s_nx[c][i] = 0.f;
-#pragma unroll
                     for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-                        for (int c = 0; c < NC; ++c) s_nx[c] = M::mma(ka[ks], qreg[c][ks], s_nx[c]);
+                        for (int c = 0; c < NC; ++c) s_nx[c] = M::mma(ka[ks], qreg[c][ks], ks == 0 ? ref[c] : s_nx[c]);
 #pragma unroll
                         for (int n = 0; n < PA; ++n) exp_piece(ks * PA + n);
                         PF_FENCE();
