@@ -86,6 +86,7 @@ def CT(c):
     return 118 + 16 * c
 
 
+LO = False  # the variant being generated also applies lower bounds (sliding window, per-row first keys)
 STUBS = []  # out-of-line code of the loop being generated: the common path of every check falls through
 
 
@@ -246,6 +247,8 @@ def subtile_ops(ty, j, kt):
     # keys a row must not see.  srem = maskfrom - 64*t in tile t; the S^T formed in subtile kt starts at key
     # 64*t + 32*(kt+1) and needs the mask if it reaches past maskfrom: srem < 32*(kt+2).  Value i of a lane is key
     # 8*(i/4) + i%4 of the subtile (+ 4*half, folded into lim), visible up to lim - first key of the subtile.
+    # With lower bounds (LO): slo = (first key the wave's last row sees) - 64*t; the same S^T needs the mask too if
+    # it starts below that key: slo > 32*(kt+1); a value is then also masked below lo - first key of the subtile.
     blk = [f".Lpf_mask_{j}{kt}_%=:"]
     for c in range(NC):
         s = S(nb, c)
@@ -253,10 +256,17 @@ def subtile_ops(ty, j, kt):
                 f"v_subrev_u32_e32 v95, {32 * (kt + 1)}, v95"]
         for i in range(16):
             blk += [f"v_cmp_gt_i32_e32 vcc, {8 * (i >> 2) + (i & 3)}, v95", f"v_cndmask_b32_e32 v{s + i}, v{s + i}, v116, vcc"]
+        if LO:
+            blk += [f"v_subrev_u32_e32 v96, %[maskfrom], %[lo{c}]", "v_add_u32_e32 v96, %[srem], v96",
+                    f"v_subrev_u32_e32 v96, {32 * (kt + 1)}, v96"]
+            for i in range(16):
+                blk += [f"v_cmp_lt_i32_e32 vcc, {8 * (i >> 2) + (i & 3)}, v96", f"v_cndmask_b32_e32 v{s + i}, v{s + i}, v116, vcc"]
     blk.append(f"s_branch .Lpf_masked_{j}{kt}_%=")
     STUBS.append(blk)
-    mx.append(Op(Ins(f"s_cmp_lt_i32 %[srem], {32 * (kt + 2)}\n\ts_cbranch_scc1 .Lpf_mask_{j}{kt}_%=\n"
-                     f".Lpf_masked_{j}{kt}_%=:", kind="salu", units=2, n=2,
+    check = f"s_cmp_lt_i32 %[srem], {32 * (kt + 2)}\n\ts_cbranch_scc1 .Lpf_mask_{j}{kt}_%=\n"
+    if LO:
+        check += f"\ts_cmp_gt_i32 %[slo], {32 * (kt + 1)}\n\ts_cbranch_scc1 .Lpf_mask_{j}{kt}_%=\n"
+    mx.append(Op(Ins(check + f".Lpf_masked_{j}{kt}_%=:", kind="salu", units=4 if LO else 2, n=4 if LO else 2,
                      reads=[f"v{S(nb, c) + i}" for c in range(NC) for i in range(16)]), 21))
     for c in range(NC):
         s = S(nb, c)
@@ -274,8 +284,10 @@ def subtile_ops(ty, j, kt):
                          writes=(f"v{m[c]}", f"v{w[c]}")), 21))
         mx.append(Op(Ins(f"v_max_f32_e32 %[mx{c}], v{m[c]}, v{w[c]}", reads=(f"v{m[c]}", f"v{w[c]}")), 21))
     # does a row's maximum exceed its reference by more than the slack?  (read at the start of the next subtile)
-    mx.append(Op(Ins("v_cmp_gt_f32_e64 s[60:61], %[mx0], %[slack]"), 21))
-    mx.append(Op(Ins("v_cmp_gt_f32_e64 s[62:63], %[mx1], %[slack]"), 21))
+    # (with lower bounds a row may not have seen a key yet: its threshold thr is a large negative number until
+    # it has, so that its first maximum, whatever its sign, becomes its reference)
+    mx.append(Op(Ins(f"v_cmp_gt_f32_e64 s[60:61], %[mx0], {'%[thr0]' if LO else '%[slack]'}"), 21))
+    mx.append(Op(Ins(f"v_cmp_gt_f32_e64 s[62:63], %[mx1], {'%[thr1]' if LO else '%[slack]'}"), 21))
     # (order: chain 0, copy 0, chain 1, copy 1, swap 0, max 0, swap 1, max 1: two instructions between a copy and its swap)
     streams["max"] = mx
 
@@ -463,11 +475,26 @@ def rescale(ty):
     AGPRs) shrink by 2^-delta."""
     out = ["s_nop 7", "s_nop 7", "s_nop 7"]  # products still writing the accumulators
     for c in range(NC):
-        out += [f"v_max_f32_e32 v97, 0, %[mx{c}]",
-                "v_exp_f32_e64 v98, -v97",
-                f"v_sub_f32_e32 %[mx{c}], %[mx{c}], v97",
-                "s_nop 0",
-                f"v_mul_f32_e32 %[l{c}], %[l{c}], v98"]
+        if LO:
+            # a row that had seen no key so far (thr still the large negative number; sum and accumulators zero)
+            # takes its first maximum as reference whatever its sign, and nothing of it is scaled
+            out += [f"v_max_f32_e32 v97, 0, %[mx{c}]",
+                    f"v_cmp_lt_f32_e64 s[54:55], %[negbig], %[mx{c}]",       # this maximum is of visible keys
+                    f"v_cndmask_b32_e64 v99, 0, %[mx{c}], s[54:55]",
+                    f"v_cmp_eq_f32_e64 vcc, %[negbig], %[thr{c}]",            # no reference yet
+                    "v_cndmask_b32_e32 v97, v97, v99, vcc",
+                    "v_exp_f32_e64 v98, -v97",
+                    f"v_sub_f32_e32 %[mx{c}], %[mx{c}], v97",
+                    "v_mov_b32_e32 v99, %[slack]",
+                    f"v_cndmask_b32_e64 %[thr{c}], %[thr{c}], v99, s[54:55]",
+                    "v_cndmask_b32_e64 v98, v98, 1.0, vcc",
+                    f"v_mul_f32_e32 %[l{c}], %[l{c}], v98"]
+        else:
+            out += [f"v_max_f32_e32 v97, 0, %[mx{c}]",
+                    "v_exp_f32_e64 v98, -v97",
+                    f"v_sub_f32_e32 %[mx{c}], %[mx{c}], v97",
+                    "s_nop 0",
+                    f"v_mul_f32_e32 %[l{c}], %[l{c}], v98"]
         for i in range(16):
             out.append(f"v_sub_f32_e32 v{CT(c) + i}, v{CT(c) + i}, v97")
         for buf in range(2):
@@ -496,13 +523,15 @@ def loop_text(ty):
     for dt in range(DT):
         lines.append(f"v_add_u32_e32 v{108 + dt}, {2 * STAGE}, %[vad{dt}]")
     lines += [f"v_mov_b32_e32 v{r}, 0" for r in range(112, 116)]
-    lines += ["v_mov_b32_e32 v116, 0xff800000", "v_cmp_gt_f32_e64 s[60:61], %[mx0], %[slack]",
-              "v_cmp_gt_f32_e64 s[62:63], %[mx1], %[slack]", "s_waitcnt lgkmcnt(0)", "s_nop 3"]
+    lines += ["v_mov_b32_e32 v116, 0xff800000",
+              f"v_cmp_gt_f32_e64 s[60:61], %[mx0], {'%[thr0]' if LO else '%[slack]'}",
+              f"v_cmp_gt_f32_e64 s[62:63], %[mx1], {'%[thr1]' if LO else '%[slack]'}", "s_waitcnt lgkmcnt(0)", "s_nop 3"]
     for j in range(NSTAGE):
         lines.append(f".Lpf_tile{j}_%=:")
         lines += [ins.text for ins in bodies[j]]
         # (ntiles counts the tiles after this one: the subtraction borrows behind the last)
-        lines += ["s_sub_u32 %[srem], %[srem], 64", "s_sub_u32 %[ntiles], %[ntiles], 1", "s_cbranch_scc1 .Lpf_done_%="]
+        lines += ["s_sub_u32 %[srem], %[srem], 64"] + (["s_sub_u32 %[slo], %[slo], 64"] if LO else [])
+        lines += ["s_sub_u32 %[ntiles], %[ntiles], 1", "s_cbranch_scc1 .Lpf_done_%="]
     lines.append("s_branch .Lpf_tile0_%=")
     for stub in STUBS:
         lines += stub
@@ -537,14 +566,17 @@ def main():
     parts = ["// Generated by gen_prefill_loop.py - do not edit.  The tile loop of prefill_asm_kernel (head_dim 128)",
              "// as inline assembly; the register map and the schedule are described in the generator.",
              ""]
-    for name in ("bf16", "f16"):
-        lines, stats = loop_text(Types(name))
-        per_tile = {k: v // NSTAGE for k, v in sorted(stats.items())}
-        parts.append(f"// {name}: instructions per 64-key tile: {per_tile}")
-        parts.append(f"#define PF_LOOP_ASM_{name.upper()} \\")
-        body = c_string(lines).split("\n")
-        parts.append(" \\\n".join(body))
-        parts.append("")
+    global LO
+    for lo in (False, True):
+        LO = lo
+        for name in ("bf16", "f16"):
+            lines, stats = loop_text(Types(name))
+            per_tile = {k: v // NSTAGE for k, v in sorted(stats.items())}
+            parts.append(f"// {name}{', with lower bounds' if lo else ''}: instructions per 64-key tile: {per_tile}")
+            parts.append(f"#define PF_LOOP_ASM_{name.upper()}{'_LO' if lo else ''} \\")
+            body = c_string(lines).split("\n")
+            parts.append(" \\\n".join(body))
+            parts.append("")
     with open(path, "w") as f:
         f.write("\n".join(parts))
     print("wrote", path)

@@ -24,7 +24,9 @@ namespace pa_decode_detail {
 
 constexpr int kPaCapTiles = 1600;  // tiles of 64 keys the slot tables hold: contexts of up to 102400 keys
 
-template <typename T>
+// LO: the instance that also applies lower bounds (sliding window, per-row first keys): the workgroup starts at
+// the tile of the first key its first row sees, everything the loop counts in is relative to that tile.
+template <typename T, bool LO>
 __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
@@ -77,14 +79,35 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     }
     const int last_task = min(n_tasks, task0 + kPfTasks) - 1;
     const int wg_keys = min(ctx_len, prefix + min(q_len, (last_task / p.n_rep) * kPfRows + kPfRows));
-    const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys;  // >= 1
-    const int n_real = min(n_tiles, kPaCapTiles);           // tiles with table entries
     // subtiles that reach past this key hold keys some row of the wave must not see
     const int mask_from = min(prefix + min(row0[0], row0[1]) + 1, ctx_len);
     // a lane's last visible key per column tile, less the 4 keys its half of the wave is ahead by
     int lim[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) lim[c] = min(ctx_len - 1, prefix + row0[c] + col) - 4 * half;
+    // Lower bounds (see prefill_mfma_kernel): a row's first visible key under the window and / or the per-row
+    // first keys, clamped so that the row always sees its own position; non-decreasing along a sequence.
+    int t0 = 0;             // first tile of the workgroup
+    int lo_mask_until = 0;  // subtiles that start below this key hold keys some row of the wave cannot see any more
+    int lo[NC] = {0, 0};    // a lane's first visible key per column tile, less 4 * half like lim
+    if constexpr (LO) {
+        const int win = p.window;
+        const int32_t *rlo = a.row_lo ? a.row_lo + a.q_starts[b] : nullptr;
+        auto row_first = [&](int row) PF_INLINE {
+            const int pos = prefix + row;
+            int first = win > 0 ? pos - win + 1 : 0;
+            if (rlo) first = max(first, rlo[min(row, q_len - 1)]);
+            return min(max(first, 0), min(pos, ctx_len - 1));
+        };
+        t0 = row_first((task0 / p.n_rep) * kPfRows) / kPfKeys;
+        lo_mask_until = row_first(min(q_len, max(row0[0], row0[1]) + kPfRows) - 1);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) lo[c] = row_first(row0[c] + col) - 4 * half;
+    }
+    // tiles the loop runs (>= 1), those of them with table entries, and the table's limit, all relative to t0
+    const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys - t0;
+    const int n_real = max(min(n_tiles + t0, kPaCapTiles) - t0, 0);
+    const int cap_rel = max(kPaCapTiles - t0, 0);
 
     // ---- Q^T operands, staged through the (still empty) ring as whole rows: see prefill_mfma_kernel ----
     constexpr int QRB = D * 2, QCPR = QRB / 16, QRPI = 64 / QCPR;
@@ -106,10 +129,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     // ---- slot tables (in flight together with the Q rows) ----
     {
         const int32_t *bt_seq = p.bt + (int64_t)b * p.bt_stride;
-        const int n_entries = n_real * GPT;
+        const int n_entries = max(n_real, 1) * GPT;  // (the loads of tiles past the last fetch tile 0 again: it has entries)
         int first_special = n_tiles;
         for (int i = tid; i < n_entries; i += kPfThreads) {
-            const int key = 16 * i, blk = key / p.bs;
+            const int key = 16 * (t0 * GPT + i), blk = key / p.bs;
             int64_t bid = -1;
             if (blk < p.bt_stride) bid = bt_seq[blk];
             const bool present = bid >= 0 && bid < p.num_blocks;
@@ -118,7 +141,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             tab_b[i] = (uint8_t)rows;
             if (rows < 16) first_special = min(first_special, i / GPT);
         }
-        if (tid < GPT) tab_b[kPaCapTiles * GPT + tid] = 0;  // tiles past the tables: nothing exists
+        if (tid < GPT) tab_b[cap_rel * GPT + tid] = 0;  // tiles past the tables: nothing exists
         if (n_tiles > n_real) first_special = min(first_special, n_real);
         // minimum over the wave here, over the waves behind the barrier below
 #pragma unroll
@@ -224,7 +247,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             float m = kNegBig;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                if (8 * (i >> 2) + (i & 3) > lim[c]) s0[c][i] = -INFINITY;
+                const int idx = 8 * (i >> 2) + (i & 3) + kPfKeys * t0;  // (+ 4 * half: folded into lim and lo)
+                if (idx > lim[c] || (LO && idx < lo[c])) s0[c][i] = -INFINITY;
                 m = fmaxf(m, s0[c][i]);
             }
             const uint32_t u = __builtin_bit_cast(uint32_t, m);
@@ -232,23 +256,28 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             mx[c] = fmaxf(__builtin_bit_cast(float, (uint32_t)sw[0]), __builtin_bit_cast(float, (uint32_t)sw[1]));
         }
     }
-    // The reference maximum of a row starts as the maximum of its first subtile (every row sees key 0, so it is
-    // finite).  From here on S^T is kept relative to the reference: the loop's first product of each column
-    // tile accumulates onto ref[c] = minus the reference in all 16 registers, the exponentials take S^T as it
-    // is, and mx is the maximum relative to the reference (0 now).  The reference moves up only when a later
-    // maximum exceeds it by more than kPfSlack (lazy rescale: see prefill_mfma_kernel).
+    // The reference maximum of a row starts as the maximum of its first subtile.  From here on S^T is kept
+    // relative to the reference: the loop's first product of each column tile accumulates onto ref[c] = minus
+    // the reference in all 16 registers, the exponentials take S^T as it is, and mx is the maximum relative to
+    // the reference (0 now).  The reference moves up only when a later maximum exceeds it by more than kPfSlack
+    // (lazy rescale: see prefill_mfma_kernel).  Without lower bounds every row sees key 0, so the maximum is
+    // finite; with them a row may see nothing of the first subtile: its reference stays unset (thr = a large
+    // negative number instead of the slack) until a maximum of visible keys arrives, which then becomes the
+    // reference whatever its sign.
     f32x16 ref[NC];
+    float thr[NC];
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
-        const float m0 = mx[c] > kNegBig ? mx[c] : 0.f;
+        const bool seen = mx[c] > kNegBig;
+        const float m0 = seen ? mx[c] : 0.f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             s0[c][i] -= m0;
             ref[c][i] = -m0;
         }
-        mx[c] = 0.f;
+        if (seen) mx[c] = 0.f;
+        thr[c] = seen ? kPfSlack : kNegBig;
     }
-
     f32x16 o[NC][DT];
 #pragma unroll
     for (int c = 0; c < NC; ++c)
@@ -259,26 +288,29 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     float l_run[NC] = {0.f, 0.f};  // running sums
 
     {
-        int n_left = n_tiles - 1;  // tiles after the current one
+        // (wave-uniform values the compiler may hold in vector registers are moved to scalar ones for the "s" operands)
+        auto uni = [](int v) PF_INLINE { return __builtin_amdgcn_readfirstlane(v); };
+        int n_left = uni(n_tiles - 1);  // tiles after the current one
         uint32_t s_t = 3, s_p = 1;
-        int s_rem = mask_from;  // mask_from - 64 * tile
+        int s_rem = uni(mask_from - kPfKeys * t0);  // mask_from - 64 * (absolute) tile
+        int s_lo = uni(lo_mask_until - kPfKeys * t0);  // the same for the lower bound
         const uint32_t tab_a_base = lds_base + kRingBytes, tab_b_base = tab_a_base + kTabABytes;
-        const uint32_t sp_lo = (uint32_t)first_special, sp_span = (uint32_t)(n_tiles - first_special);
-        const uint32_t n_real_u = (uint32_t)n_real, cap_tiles = kPaCapTiles, mask_from_u = (uint32_t)mask_from;
+        const uint32_t sp_lo = (uint32_t)uni(first_special), sp_span = (uint32_t)uni(n_tiles - first_special);
+        const uint32_t n_real_u = (uint32_t)uni(n_real), cap_tiles = (uint32_t)uni(cap_rel), mask_from_u = (uint32_t)uni(mask_from);
         const uint32_t lane16 = (uint32_t)lane * 16, arow_u = (uint32_t)arow;
         const uint64_t pk = reinterpret_cast<uint64_t>(pool_k), pv = reinterpret_cast<uint64_t>(pool_v);
         const uint32_t pklo = __builtin_amdgcn_readfirstlane((uint32_t)pk), pkhi = __builtin_amdgcn_readfirstlane((uint32_t)(pk >> 32));
         const uint32_t pvlo = __builtin_amdgcn_readfirstlane((uint32_t)pv), pvhi = __builtin_amdgcn_readfirstlane((uint32_t)(pv >> 32));
         const uint32_t stride = (uint32_t)tok_stride;
         const float slack = kPfSlack;  // in the units of S^T here: log2 of the factor a row's reference may lag by
-#define PA_LOOP_OPERANDS                                                                                              \
+#define PA_LOOP_OPERANDS(MORE_OUT, MORE_IN)                                                                           \
     : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[0][2]), "+{a[48:63]}"(o[0][3]),                    \
       "+{a[64:79]}"(o[1][0]), "+{a[80:95]}"(o[1][1]), "+{a[96:111]}"(o[1][2]), "+{a[112:127]}"(o[1][3]),                \
       "+{v[0:15]}"(s0[0]), "+{v[16:31]}"(s0[1]), "+{v[118:133]}"(ref[0]), "+{v[134:149]}"(ref[1]),                    \
       "+{a[192:195]}"(ka[0]), "+{a[196:199]}"(ka[1]), "+{a[200:203]}"(ka[2]), "+{a[204:207]}"(ka[3]),                   \
       "+{a[208:211]}"(ka[4]), "+{a[212:215]}"(ka[5]), "+{a[216:219]}"(ka[6]), "+{a[220:223]}"(ka[7]),                   \
       [mx0] "+&v"(mx[0]), [mx1] "+&v"(mx[1]), [l0] "+&v"(l_run[0]), [l1] "+&v"(l_run[1]),                             \
-      [ntiles] "+&s"(n_left), [sT] "+&s"(s_t), [sP] "+&s"(s_p), [srem] "+&s"(s_rem)                                         \
+      [ntiles] "+&s"(n_left), [sT] "+&s"(s_t), [sP] "+&s"(s_p), [srem] "+&s"(s_rem) MORE_OUT                                \
     : "{a[128:131]}"(qreg[0][0]), "{a[132:135]}"(qreg[0][1]), "{a[136:139]}"(qreg[0][2]), "{a[140:143]}"(qreg[0][3]),   \
       "{a[144:147]}"(qreg[0][4]), "{a[148:151]}"(qreg[0][5]), "{a[152:155]}"(qreg[0][6]), "{a[156:159]}"(qreg[0][7]),   \
       "{a[160:163]}"(qreg[1][0]), "{a[164:167]}"(qreg[1][1]), "{a[168:171]}"(qreg[1][2]), "{a[172:175]}"(qreg[1][3]),   \
@@ -289,7 +321,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
       [arow] "v"(arow_u), [lim0] "v"(lim[0]), [lim1] "v"(lim[1]), [slack] "s"(slack),                                   \
       [pklo] "s"(pklo), [pkhi] "s"(pkhi), [pvlo] "s"(pvlo), [pvhi] "s"(pvhi), [stride] "s"(stride), [m0w] "s"(m0w),     \
       [nreal] "s"(n_real_u), [tabA] "s"(tab_a_base), [tabB] "s"(tab_b_base), [splo] "s"(sp_lo),                       \
-      [spspan] "s"(sp_span), [captiles] "s"(cap_tiles), [maskfrom] "s"(mask_from_u)                                   \
+      [spspan] "s"(sp_span), [captiles] "s"(cap_tiles), [maskfrom] "s"(mask_from_u) MORE_IN                           \
     : "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47",  \
       "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63",  \
       "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79",  \
@@ -300,12 +332,28 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
       "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255", "s40", "s41", "s42",     \
       "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58",  \
       "s59", "s60", "s61", "s62", "s63", "vcc", "scc", "memory"
-        if constexpr (std::is_same<T, pa_bf16>::value) {
-            asm volatile(PF_LOOP_ASM_BF16 PA_LOOP_OPERANDS);
+#define PA_NOTHING
+#define PA_LO_OUT , [thr0] "+&v"(thr[0]), [thr1] "+&v"(thr[1]), [slo] "+&s"(s_lo)
+#define PA_LO_IN , [lo0] "v"(lo[0]), [lo1] "v"(lo[1]), [negbig] "s"(neg_big)
+        const float neg_big = kNegBig;
+        if constexpr (LO) {
+            if constexpr (std::is_same<T, pa_bf16>::value) {
+                asm volatile(PF_LOOP_ASM_BF16_LO PA_LOOP_OPERANDS(PA_LO_OUT, PA_LO_IN));
+            } else {
+                asm volatile(PF_LOOP_ASM_F16_LO PA_LOOP_OPERANDS(PA_LO_OUT, PA_LO_IN));
+            }
         } else {
-            asm volatile(PF_LOOP_ASM_F16 PA_LOOP_OPERANDS);
+            (void)s_lo; (void)neg_big;
+            if constexpr (std::is_same<T, pa_bf16>::value) {
+                asm volatile(PF_LOOP_ASM_BF16 PA_LOOP_OPERANDS(PA_NOTHING, PA_NOTHING));
+            } else {
+                asm volatile(PF_LOOP_ASM_F16 PA_LOOP_OPERANDS(PA_NOTHING, PA_NOTHING));
+            }
         }
 #undef PA_LOOP_OPERANDS
+#undef PA_NOTHING
+#undef PA_LO_OUT
+#undef PA_LO_IN
     }
 
     // ---- normalise; rows go through LDS so that every store instruction writes whole 256-byte rows ----
@@ -346,7 +394,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     }
 }
 
-// nullptr unless the element type has this kernel
-prefill_mfma_fn pa_prefill_asm_kernel(int dtype);
+// nullptr unless the element type has this kernel; `lower_bounds`: the instance for sliding windows and per-row
+// first keys
+prefill_mfma_fn pa_prefill_asm_kernel(int dtype, bool lower_bounds);
 
 }  // namespace pa_decode_detail

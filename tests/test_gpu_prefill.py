@@ -272,10 +272,11 @@ def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype):
         q = torch.from_numpy(rng.standard_normal((len(chunk) * cmax, hq, d)).astype(np.float32)).to(dtype).to(DEV)
         args = (q, kc, vc, dev_tables, _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk),
                 _i32(np.arange(len(chunk)) * cmax), cmax, bs, d ** -0.5)
-        got = ops.prefill_paged(*args).float().cpu().reshape(len(chunk), cmax, hq, d)
-        want = ops.prefill_paged(*args, rowwise=True).float().cpu().reshape(len(chunk), cmax, hq, d)
-        for b, c in enumerate(chunk):
-            assert_close(got[b, :c], want[b, :c], 2e-2, f"block_size {bs} sequence {b}")
+        for window in (0, 70):  # (with a window: the instance of the kernel that applies lower bounds)
+            got = ops.prefill_paged(*args, window=window).float().cpu().reshape(len(chunk), cmax, hq, d)
+            want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu().reshape(len(chunk), cmax, hq, d)
+            for b, c in enumerate(chunk):
+                assert_close(got[b, :c], want[b, :c], 2e-2, f"block_size {bs} sequence {b} window {window}")
 
 
 def test_assembly_loop_kernel_long_context_and_table_limit():
@@ -293,9 +294,10 @@ def test_assembly_loop_kernel_long_context_and_table_limit():
         q = (0.3 * torch.from_numpy(rng.standard_normal((chunk, hq, d)).astype(np.float32))).to(torch.bfloat16).to(DEV)
         table = torch.from_numpy(rng.permutation(nblk).astype(np.int32)).reshape(1, -1).to(DEV)
         args = (q, kc, vc, table, _i32([ctx]), _i32([chunk]), _i32([0]), chunk, bs, d ** -0.5)
-        got = ops.prefill_paged(*args).float().cpu()
-        want = ops.prefill_paged(*args, rowwise=True).float().cpu()
-        assert_close(got, want, 2e-2, f"context of {ctx} keys")
+        for window in (0, 3000):  # (with a window the workgroup starts more than a thousand tiles into the tables)
+            got = ops.prefill_paged(*args, window=window).float().cpu()
+            want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu()
+            assert_close(got, want, 2e-2, f"context of {ctx} keys, window {window}")
 
 
 @pytest.mark.parametrize("d", [64, 128, 256])
@@ -329,9 +331,12 @@ def test_logits_that_grow_along_the_context(d):
             for j in range(n):
                 kc[tables[b][j // bs] * bs + j % bs] = torch.from_numpy(rows[j].astype(np.float32))
         kc = kc.to(torch.bfloat16)
-        want = po.paged_prefill_chunk(q, kc, vc, tables, prefix, chunk, bs, d ** -0.5)
-        out = torch.zeros(len(chunk) * cmax, hq, d, device=DEV, dtype=torch.bfloat16)
-        ops.prefill_paged(q.reshape(-1, hq, d).to(DEV), kc.to(DEV), vc.to(DEV), tables_to_device(tables),
-                          _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk), _i32(np.arange(len(chunk)) * cmax),
-                          cmax, bs, d ** -0.5, out=out)
-        assert_close(out.reshape(len(chunk), cmax, hq, d), want, 2e-2, f"logits {'rising' if direction > 0 else 'falling'}")
+        # (with a window the kernels also start rows whose first subtiles hold no visible key, far below zero)
+        for window in (0, 100):
+            want = po.paged_prefill_chunk(q, kc, vc, tables, prefix, chunk, bs, d ** -0.5, window=window)
+            out = torch.zeros(len(chunk) * cmax, hq, d, device=DEV, dtype=torch.bfloat16)
+            ops.prefill_paged(q.reshape(-1, hq, d).to(DEV), kc.to(DEV), vc.to(DEV), tables_to_device(tables),
+                              _i32([p + c for p, c in zip(prefix, chunk)]), _i32(chunk),
+                              _i32(np.arange(len(chunk)) * cmax), cmax, bs, d ** -0.5, out=out, window=window)
+            assert_close(out.reshape(len(chunk), cmax, hq, d), want, 2e-2,
+                         f"logits {'rising' if direction > 0 else 'falling'}, window {window}")
