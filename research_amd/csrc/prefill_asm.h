@@ -12,8 +12,11 @@
 //     zero value row, which is what the other kernels do for absent blocks;
 //   * every wave runs every tile of the workgroup with the causal / context-end mask applied where needed, so
 //     there is no per-wave tail code: a wave past its last key multiplies exact zeros;
-//   * sliding windows and per-row first keys are not handled here: the host launches prefill_mfma_kernel for
-//     those (and for other head sizes, block sizes that are not multiples of 16 and tables past kPaCapTiles).
+//   * sliding windows and per-row first keys have an instance of their own (LO): the out-of-line mask block also
+//     applies the lower bound, a row that has seen no key yet takes its first maximum as reference, and the
+//     workgroup starts at the tile of the first key its first row sees;
+//   * the host launches prefill_mfma_kernel for other head sizes, block sizes that are not multiples of 16 and
+//     tables past kPaCapTiles.
 // Only the set-up, the first subtile's S^T and the write-out are compiled code, so the register allocator sees
 // one asm statement with pinned operands and little else.
 #pragma once
