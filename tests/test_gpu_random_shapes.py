@@ -105,3 +105,60 @@ def test_random_chunked_prefill(seed):
                       out=out, window=window)
     want = po.paged_prefill_chunk(q, k, v, tables, prefix, chunk, bs, scale, window=window)
     assert_close(out.reshape(batch, cmax, hq, d), want, 1e-5 if kind == "f32" else 2e-2, f"prefill window={window}")
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_matrix_core_prefill(seed):
+    """Shapes the table-driven matrix-core prefill kernels take (head_dim 128: the assembly loop with and without
+    lower bounds; head_dim 256), drawn at random: block sizes that are multiples of 16, ragged prefixes and
+    chunks, sliding windows, per-row first keys, absent blocks.  Every case against the vector kernel (which
+    states the zero-row rule of absent blocks), cases without absent blocks and first keys also against the
+    checker."""
+    rng = np.random.default_rng(9500 + seed)
+    d = int(rng.choice([128, 128, 256]))
+    hkv = int(rng.choice([1, 2, 4]))
+    n_rep = int(rng.choice([1, 2, 3, 4, 8]))
+    hq = hkv * n_rep
+    bs = int(rng.choice([16, 16, 32, 48, 64]))
+    dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
+    batch = int(rng.integers(1, 5))
+    prefix = rng.integers(0, 1500, batch).tolist()
+    chunk = rng.integers(1, 300, batch).tolist()
+    if seed % 4 == 0:
+        prefix[0] = 0
+    window = int(rng.choice([0, 0, 20, 64, 300]))
+    with_first = rng.random() < 0.4
+    with_absent = rng.random() < 0.4
+    announce(f"random matrix-core prefill seed={seed} hq={hq} hkv={hkv} d={d} bs={bs} {dtype} batch={batch} "
+             f"window={window} first_keys={with_first} absent={with_absent}")
+    cmax = max(chunk)
+    tables, nb = _tables(rng, [p + c for p, c in zip(prefix, chunk)], bs)
+    k, v = _pool(rng, nb, bs, hkv, d, dtype)
+    if with_absent:
+        for t in tables:
+            for i in range(len(t)):
+                if rng.random() < 0.15:
+                    t[i] = -1 if rng.random() < 0.7 else nb + 3
+    q = torch.from_numpy(rng.standard_normal((batch, cmax, hq, d)).astype(np.float32)).to(dtype)
+    first = None
+    if with_first:  # a row's document starts at a random earlier position, non-decreasing along the sequence
+        rows = []
+        for p, c in zip(prefix, chunk):
+            starts = np.sort(rng.integers(0, p + c, max(1, (p + c) // 150)))
+            pos = p + np.arange(cmax)
+            f = np.zeros(cmax, dtype=np.int32)
+            for st in starts:
+                f = np.where(pos >= st, st, f)
+            rows.append(np.minimum(f, pos).astype(np.int32))
+        first = torch.from_numpy(np.stack(rows).reshape(-1)).to(DEV)
+    i32 = lambda x: torch.tensor(list(x), dtype=torch.int32, device=DEV)
+    args = (q.reshape(-1, hq, d).to(DEV), k.to(DEV), v.to(DEV), tables_to_device(tables),
+            i32(p + c for p, c in zip(prefix, chunk)), i32(chunk), i32(np.arange(batch) * cmax), cmax, bs, d ** -0.5)
+    out = torch.zeros(batch * cmax, hq, d, dtype=dtype, device=DEV)
+    got = ops.prefill_paged(*args, out=out, window=window, row_first_key=first).float().cpu().reshape(batch, cmax, hq, d)
+    ref = ops.prefill_paged(*args, window=window, row_first_key=first, rowwise=True).float().cpu().reshape(batch, cmax, hq, d)
+    for b, c in enumerate(chunk):
+        assert_close(got[b, :c], ref[b, :c], 2e-2, f"against the vector kernel, sequence {b}")
+    if not with_absent and not with_first:
+        want = po.paged_prefill_chunk(q, k, v, tables, prefix, chunk, bs, d ** -0.5, window=window)
+        assert_close(got, want, 2e-2, "against the checker")
