@@ -18,6 +18,9 @@
 // past the context end or in absent blocks are fetched from a slot that exists and cleared in LDS before the
 // stage is published, so every wave issues the same number of loads per stage and the waits are plain counts.
 // A group must lie inside one pool block: block sizes that are multiples of 16, or one block per sequence.
+// CHECKED: the instance for block sizes that are not multiples of 16 (one block per sequence), where a sequence's
+// last group can reach past the end of the pool: such a group is fetched lane by lane with clamped rows.  With
+// blocks of a multiple of 16 keys no group can, and the other instance carries neither the test nor that path.
 // Every wave runs every subtile of the workgroup, with the masks applied where needed: a wave past its last
 // visible key multiplies exact zeros.
 #pragma once
@@ -30,7 +33,7 @@ constexpr int kWdStages = 4;
 constexpr int kWdTasks = kPfWaves;   // tasks (32 query rows of one head) per workgroup: one per wave
 constexpr int kWdCapGroups = 6144;   // 16-key groups the slot tables hold: contexts of up to 98304 keys
 
-template <typename T>
+template <typename T, bool CHECKED>
 __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
@@ -180,7 +183,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     // one tensor's rows of one tile into LDS at byte offset `dst` of s_mem (always NL direct loads)
     auto issue_rows = [&](const char *pool, const uint32_t (&lane_ofs)[NL], int chunk_swz_mask, int tile, uint32_t dst) PF_INLINE {
         const int slot = __builtin_amdgcn_readfirstlane(tab_a[entry_of(tile)]);
-        if (__builtin_expect((int64_t)slot + 16 <= pool_rows, 1)) {
+        if (!CHECKED || __builtin_expect((int64_t)slot + 16 <= pool_rows, 1)) {
             const uint64_t ofs = (uint64_t)(uint32_t)slot * (uint32_t)tok_stride;  // 32 x 32 -> 64 bits, scalar
             const char *base = pf_scalar_ptr(pool + ofs);
 #pragma unroll
@@ -219,32 +222,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         if (n == 1) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:1024" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
         if (n == 2) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:2048" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
         if (n == 3) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:3072" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
-    };
-    auto issue_stage = [&](int s) PF_INLINE {
-        const int slot_k = __builtin_amdgcn_readfirstlane(pre_k), slot_v = __builtin_amdgcn_readfirstlane(pre_v);
-        if (__builtin_expect(max(slot_k, slot_v) <= slot_max, 1)) {
-            const uint32_t dst_k = lds_base + stage_ofs(s) + wave_rows, dst_v = dst_k + TENSOR;
-            const char *bk = pf_scalar_ptr(pool_kb + (uint64_t)(uint32_t)slot_k * (uint32_t)tok_stride);
-            const char *bv = pf_scalar_ptr(pool_vb + (uint64_t)(uint32_t)slot_v * (uint32_t)tok_stride);
-            static_assert(2 * RB == 1024 && NL == 4, "immediate offsets of the loads below");
-            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\t"
-                         "global_load_lds_dwordx4 %2, %1 offset:0\n\t"
-                         "global_load_lds_dwordx4 %3, %1 offset:1024\n\t"
-                         "global_load_lds_dwordx4 %4, %1 offset:2048\n\t"
-                         "global_load_lds_dwordx4 %5, %1 offset:3072\n\t"
-                         "s_mov_b32 m0, %6\n\ts_nop 0\n\t"
-                         "global_load_lds_dwordx4 %8, %7 offset:0\n\t"
-                         "global_load_lds_dwordx4 %9, %7 offset:1024\n\t"
-                         "global_load_lds_dwordx4 %10, %7 offset:2048\n\t"
-                         "global_load_lds_dwordx4 %11, %7 offset:3072"
-                         :
-                         : "s"(dst_k), "s"(bk), "v"(lane_kb[0]), "v"(lane_kb[1]), "v"(lane_kb[2]), "v"(lane_kb[3]),
-                           "s"(dst_v), "s"(bv), "v"(lane_vb[0]), "v"(lane_vb[1]), "v"(lane_vb[2]), "v"(lane_vb[3])
-                         : "memory", "m0");
-        } else {
-            issue_k(s);
-            issue_v(s);
-        }
     };
     // clear the rows this wave loaded that do not exist (after its loads have landed, before the barrier)
     auto clear_rows = [&](int tile, uint32_t dst) PF_INLINE {
@@ -361,7 +338,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 
     // ---- first subtile: S^T, mask, row maximum; K operands of the second; V^T of the first k-step ----
     read_k(t0 - 1, ka);
-    read_v(t0, 0, va0);
     PF_FENCE();
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) sb[0] = M::mma(ka[ks], qreg[ks], ks == 0 ? ref : sb[0]);
@@ -423,7 +399,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         for (int ks = 0; ks < KS; ++ks) {
             s_nx = M::mma(ka[ks], qreg[ks], ks == 0 ? ref : s_nx);
             PF_FENCE();
-            if (!(ks & 1)) read_v_one(g, 1, ks >> 1, va1[ks >> 1]);  // second k-step's V^T: consumed in (c)
+            // V^T of this subtile: the first k-step's (consumed in (b)) behind the first eight products, the second's
+            // (consumed in (c)) behind the others
+            if (ks < 8) read_v_one(g, 0, ks, va0[ks]);
+            else read_v_one(g, 1, ks - 8, va1[ks - 8]);
             if (ks & 1) exp_piece(ks >> 1);
             PF_FENCE();
         }
@@ -435,11 +414,11 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         // the loads of stage g+4, one behind each product of (b); a group that reaches past the end of the pool
         // takes the per-lane path here instead
         const int slot_k = __builtin_amdgcn_readfirstlane(pre_k), slot_v = __builtin_amdgcn_readfirstlane(pre_v);
-        const bool fast = max(slot_k, slot_v) <= slot_max;
+        const bool fast = !CHECKED || max(slot_k, slot_v) <= slot_max;
         const uint32_t dst_k = lds_base + stage_ofs(g + 4) + wave_rows, dst_v = dst_k + TENSOR;
         const char *bk = pf_scalar_ptr(pool_kb + (uint64_t)(uint32_t)slot_k * (uint32_t)tok_stride);
         const char *bv = pf_scalar_ptr(pool_vb + (uint64_t)(uint32_t)slot_v * (uint32_t)tok_stride);
-        if (__builtin_expect(!fast, 0)) { issue_k(g + 4); issue_v(g + 4); }
+        if (CHECKED && __builtin_expect(!fast, 0)) { issue_k(g + 4); issue_v(g + 4); }
         prefetch_entries(g + 5);
         PF_FENCE();
         // ---- (b) O^T += V^T . P^T, first k-step ----
@@ -463,7 +442,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             for (int dt = 0; dt < DT; ++dt) {
                 o[dt] = M::mma(va1[dt], pb, o[dt]);
                 PF_FENCE();
-                read_v_one(g + 1, 0, dt, va0[dt]);  // first k-step's V^T of the next subtile
                 read_k_one(g + 1, 8 + dt, ka[8 + dt]);
                 if (dt == 1) max_piece(s_nx, 0, mx);
                 if (dt == 3) max_piece(s_nx, 1, mx);
@@ -497,6 +475,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 }
 
 // nullptr unless the element type has this kernel
-prefill_mfma_fn pa_prefill_d256_kernel(int dtype);
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked);
 
 }  // namespace pa_decode_detail

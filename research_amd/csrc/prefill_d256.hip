@@ -3,9 +3,9 @@
 
 namespace pa_decode_detail {
 
-prefill_mfma_fn pa_prefill_d256_kernel(int dtype) {
-    if (dtype == PA_BF16) return prefill_d256_kernel<pa_bf16>;
-    if (dtype == PA_F16) return prefill_d256_kernel<pa_f16>;
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked) {
+    if (dtype == PA_BF16) return checked ? prefill_d256_kernel<pa_bf16, true> : prefill_d256_kernel<pa_bf16, false>;
+    if (dtype == PA_F16) return checked ? prefill_d256_kernel<pa_f16, true> : prefill_d256_kernel<pa_f16, false>;
     return nullptr;
 }
 
