@@ -5,7 +5,7 @@ namespace pa_decode_detail {
 constexpr int kPaCapTiles = 1600;  // (prefill_asm.h)
 prefill_mfma_fn pa_prefill_asm_kernel(int dtype, bool lower_bounds);
 constexpr int kWdTasks = 4, kWdCapGroups = 6144;  // (prefill_d256.h)
-prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked);
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked, bool lower_bounds);
 }
 
 using namespace pa_decode_detail;
@@ -63,7 +63,7 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     int tasks_per_wg = kPfTasks;
     if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) && num_blocks > 0 &&
         num_blocks * (int64_t)block_size < (1ll << 31) && bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16) {
-        mfma = pa_prefill_d256_kernel(dtype, block_size % 16 != 0);
+        mfma = pa_prefill_d256_kernel(dtype, block_size % 16 != 0, window > 0 || row_first_key != nullptr);
         tasks_per_wg = kWdTasks;
     }
     if (mfma) {

@@ -25,6 +25,7 @@
 // visible key multiplies exact zeros.
 #pragma once
 #include "prefill_mfma.h"
+#include "prefill_d256_loop.inc"
 
 namespace pa_decode_detail {
 
@@ -33,7 +34,7 @@ constexpr int kWdStages = 4;
 constexpr int kWdTasks = kPfWaves;   // tasks (32 query rows of one head) per workgroup: one per wave
 constexpr int kWdCapGroups = 6144;   // 16-key groups the slot tables hold: contexts of up to 98304 keys
 
-template <typename T, bool CHECKED>
+template <typename T, bool CHECKED, bool ASM>
 __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
@@ -47,11 +48,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     constexpr int CAP = kWdCapGroups;       // entry CAP of both tables: a group of which nothing exists
     constexpr int NL = 4;                   // direct loads per wave, stage and tensor (2 rows each)
     typedef __attribute__((address_space(3))) char lds_char;
-    __shared__ __attribute__((aligned(1024))) char s_mem[kRingBytes + (CAP + 2) * 4 + (CAP + 2)];
+    constexpr int kTabEntries = CAP + 4;    // (entries CAP .. CAP+3: groups of which nothing exists)
+    __shared__ __attribute__((aligned(1024))) char s_mem[kRingBytes + kTabEntries * 4 + kTabEntries];
     __shared__ int s_special[kPfWaves];
     const uint32_t lds_base = (uint32_t)(size_t)(lds_char *)s_mem;
     int32_t *tab_a = reinterpret_cast<int32_t *>(s_mem + kRingBytes);            // pool slot of the group's first key
-    uint8_t *tab_b = reinterpret_cast<uint8_t *>(s_mem + kRingBytes + (CAP + 2) * 4);  // rows of the group that exist
+    uint8_t *tab_b = reinterpret_cast<uint8_t *>(s_mem + kRingBytes + kTabEntries * 4);  // rows of the group that exist
 
     const PoolArgs &p = a.p;
     const int tid = threadIdx.x;
@@ -134,7 +136,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             tab_b[i] = (uint8_t)rows;
             if (rows < 16) first_special = min(first_special, i / 2);
         }
-        if (tid == 0) { tab_a[CAP] = 0; tab_b[CAP] = 0; }
+        if (tid < 4) { tab_a[CAP + tid] = 0; tab_b[CAP + tid] = 0; }
         if (2 * n_tiles > CAP) first_special = min(first_special, CAP / 2);
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) first_special = min(first_special, __shfl_xor(first_special, d, 64));
@@ -451,9 +453,48 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         l_run += sum;
         PF_FENCE();
     };
-    for (int g = t0; g < n_tiles; g += 2) {
-        subtile(g, PfBool<false>{});
-        if (g + 1 < n_tiles) subtile(g + 1, PfBool<true>{});
+    if constexpr (ASM) {
+        // The subtile loop as scheduled assembly (prefill_d256_loop.inc): no lower bounds, so the workgroup starts
+        // at tile 0 and every row has seen key 0.  S^T of the first subtile becomes relative to its row maximum,
+        // which is the reference from here on; the loop takes the first half of the first V^T operands read.
+        static_assert(!CHECKED && kWdStages == 4 && kWdKeys == 32 && CAP == 2 * 3072, "the assembly loop is written for this shape");
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            sb[0][i] -= mx;
+            ref[i] = -mx;
+        }
+        mx = 0.f;
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt) read_v_one(t0, 0, dt, va0[dt]);
+        f32x16 &sb0 = sb[0];
+        auto uni = [](int v) PF_INLINE { return __builtin_amdgcn_readfirstlane(v); };
+        int n_left = uni(n_tiles - t0 - 1);  // tiles after the current one
+        uint32_t s_t = (uint32_t)uni(t0 + 4), s_p = (uint32_t)uni(t0 + 1);
+        int s_rem = uni(mask_from - kWdKeys * t0);
+        const uint32_t tab_a_w = lds_base + kRingBytes + 4 * wave_group;
+        const uint32_t tab_b_w = lds_base + kRingBytes + kTabEntries * 4 + wave_group;
+        const uint32_t sp_lo = (uint32_t)uni(max(first_special - 1, 0)), mask_from_u = (uint32_t)uni(mask_from);
+        const uint32_t m0w = lds_base + wave_rows, lane16 = (uint32_t)lane * 16, arow_u = (uint32_t)arow0;
+        uint32_t kad[KS / 2], vad[DT / 2];
+#pragma unroll
+        for (int ks = 0; ks < KS / 2; ++ks) kad[ks] = lds_base + k_ofs[ks];
+#pragma unroll
+        for (int dt = 0; dt < DT / 2; ++dt) vad[dt] = lds_base + v_ofs[dt];
+        const uint64_t pk = reinterpret_cast<uint64_t>(pool_kb), pv = reinterpret_cast<uint64_t>(pool_vb);
+        const uint32_t pklo = uni((uint32_t)pk), pkhi = uni((uint32_t)(pk >> 32));
+        const uint32_t pvlo = uni((uint32_t)pv), pvhi = uni((uint32_t)(pv >> 32));
+        const uint32_t stride = (uint32_t)tok_stride;
+        const float slack = kPfSlack;
+        if constexpr (std::is_same<T, pa_bf16>::value) {
+            asm volatile(WD_LOOP_ASM_BF16 WD_LOOP_OPERANDS);
+        } else {
+            asm volatile(WD_LOOP_ASM_F16 WD_LOOP_OPERANDS);
+        }
+    } else {
+        for (int g = t0; g < n_tiles; g += 2) {
+            subtile(g, PfBool<false>{});
+            if (g + 1 < n_tiles) subtile(g + 1, PfBool<true>{});
+        }
     }
     pf_wait_loads<0>();  // (loads of the stages past the last tile: nothing may arrive after the workgroup has ended)
 
@@ -475,6 +516,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 }
 
 // nullptr unless the element type has this kernel
-prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked);
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked, bool lower_bounds);
 
 }  // namespace pa_decode_detail

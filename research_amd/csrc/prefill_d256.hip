@@ -3,9 +3,15 @@
 
 namespace pa_decode_detail {
 
-prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked) {
-    if (dtype == PA_BF16) return checked ? prefill_d256_kernel<pa_bf16, true> : prefill_d256_kernel<pa_bf16, false>;
-    if (dtype == PA_F16) return checked ? prefill_d256_kernel<pa_f16, true> : prefill_d256_kernel<pa_f16, false>;
+// `checked`: block sizes that are not multiples of 16; `lower_bounds`: a sliding window or per-row first keys.
+// With neither, the instance whose subtile loop is scheduled assembly.
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked, bool lower_bounds) {
+    if (dtype == PA_BF16)
+        return checked ? prefill_d256_kernel<pa_bf16, true, false>
+                       : lower_bounds ? prefill_d256_kernel<pa_bf16, false, false> : prefill_d256_kernel<pa_bf16, false, true>;
+    if (dtype == PA_F16)
+        return checked ? prefill_d256_kernel<pa_f16, true, false>
+                       : lower_bounds ? prefill_d256_kernel<pa_f16, false, false> : prefill_d256_kernel<pa_f16, false, true>;
     return nullptr;
 }
 

@@ -202,14 +202,16 @@ def test_error_text_is_cleared_by_a_good_call():
     assert _lib.last_error() == ""
 
 
-def test_generated_prefill_loop_is_current(tmp_path):
-    """research_amd/csrc/prefill_mfma_loop.inc is what gen_prefill_loop.py writes (the generator also checks the
-    instruction distances the hardware does not interlock, so a schedule that violates one cannot be committed)."""
+@pytest.mark.parametrize("script,generated", [("gen_prefill_loop.py", "prefill_mfma_loop.inc"),
+                                              ("gen_prefill_loop_d256.py", "prefill_d256_loop.inc")])
+def test_generated_prefill_loop_is_current(tmp_path, script, generated):
+    """The committed assembly loops (head_dim 128: prefill_mfma_loop.inc; head_dim 256: prefill_d256_loop.inc) are
+    what their generators write (the generators also check the instruction distances the hardware does not
+    interlock, so a schedule that violates one cannot be committed)."""
     import os
     import subprocess
     import sys
     csrc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "research_amd", "csrc")
     out = tmp_path / "loop.inc"
-    subprocess.run([sys.executable, os.path.join(csrc, "gen_prefill_loop.py"), str(out)], check=True,
-                   stdout=subprocess.DEVNULL)
-    assert out.read_text() == open(os.path.join(csrc, "prefill_mfma_loop.inc")).read()
+    subprocess.run([sys.executable, os.path.join(csrc, script), str(out)], check=True, stdout=subprocess.DEVNULL)
+    assert out.read_text() == open(os.path.join(csrc, generated)).read()

@@ -135,23 +135,24 @@ def test_absent_blocks_and_short_tables(dtype):
 
 
 def test_long_context_and_table_limit():
-    """A 70 000-key context (4 375 slot-table entries) through the matrix-core kernel, and a table just past what
-    its LDS tables hold (the host then launches the vector kernel): both against the vector kernel on the
-    chunk's rows."""
+    """A 70 000-key context (4 375 slot-table entries) through the matrix-core kernel; a table just past what
+    its LDS tables hold (the host then launches the vector kernel); and that context with a table cut to exactly
+    what they hold (the matrix-core kernel again: the keys past the table are absent, and the loop's look-ups
+    run past the tables' last tile).  All against the vector kernel on the chunk's rows."""
     announce("prefill d256 long context")
     rng = np.random.default_rng(904)
     hq, hkv, bs = 4, 1, 16
-    for ctx in (70000, 6144 * 16 + 40):
+    for ctx, table_len in ((70000, None), (6144 * 16 + 40, None), (6144 * 16 + 40, 6144)):
         chunk = 48
         nblk = -(-ctx // bs)
         kc = _randn(rng, (nblk * bs, hkv, D), torch.bfloat16).to(DEV)
         vc = _randn(rng, (nblk * bs, hkv, D), torch.bfloat16).to(DEV)
         q = _randn(rng, (chunk, hq, D), torch.bfloat16, 0.3).to(DEV)
-        table = torch.from_numpy(rng.permutation(nblk).astype(np.int32)).reshape(1, -1).to(DEV)
+        table = torch.from_numpy(rng.permutation(nblk).astype(np.int32)[:table_len]).reshape(1, -1).contiguous().to(DEV)
         args = (q, kc, vc, table, _i32([ctx]), _i32([chunk]), _i32([0]), chunk, bs, D ** -0.5)
         got = ops.prefill_paged(*args).float().cpu()
         want = ops.prefill_paged(*args, rowwise=True).float().cpu()
-        assert_close(got, want, 2e-2, f"context of {ctx} keys")
+        assert_close(got, want, 2e-2, f"context of {ctx} keys, table of {table.shape[1]} entries")
 
 
 def test_c3_shape_at_head_dim_256_full_size():
