@@ -40,14 +40,26 @@ Usage: python3 gen_prefill_loop.py [output file]   (default: prefill_mfma_loop.i
 import os
 import sys
 
-NC, KS, DT = 2, 8, 4
-RB = 256                # bytes of a K / V row (head_dim 128, 16-bit elements)
-TENSOR = 64 * RB        # one tensor's tile of 64 keys
-STAGE = 2 * TENSOR      # K tile + V tile
-NSTAGE = 4
-GAPS = 33               # places for other instructions around the 32 products of a subtile
-SYNC_GAP = int(os.environ.get("PF_GEN_SYNCGAP", "16"))  # where tile t+1 is published in a tile's first subtile
+NC, NSTAGE = 2, 4
 X = set(os.environ.get("PF_GEN_X", "").split(","))  # experiment switches
+
+
+def configure(head_dim):
+    """The shape constants of a head size (128 or 64; 16-bit elements)."""
+    global D, KS, DT, RB, TENSOR, STAGE, M_A, M_B, GAPS, SYNC_GAP, NG, MAX_GAP
+    D = head_dim
+    KS, DT = D // 16, D // 32   # k-steps of S^T = K . Q^T, 32-wide d tiles of O^T
+    RB = 2 * D                   # bytes of a K / V row
+    TENSOR = 64 * RB             # one tensor's tile of 64 keys
+    STAGE = 2 * TENSOR           # K tile + V tile
+    M_A, M_B = NC * KS, NC * DT  # products of S^T, and of one k-step of O^T, per subtile
+    GAPS = M_A + 2 * M_B + 1     # places for other instructions around the products of a subtile
+    SYNC_GAP = M_A               # where tile t+1 is published in a tile's first subtile
+    NG = RB // 64                # direct loads per wave, tile and tensor (a tensor's tile is 64 * RB bytes, a wave load 1 KiB, 4 waves)
+    MAX_GAP = {128: 21, 64: 11}[D]  # first gap of the row maxima (far enough behind the last S^T product)
+
+
+configure(128)
 
 
 def areg(base, n):
@@ -59,11 +71,11 @@ def vreg(base, n):
 
 
 def O(c, dt):
-    return areg(16 * (4 * c + dt), 16)
+    return areg(16 * (DT * c + dt), 16)
 
 
 def Q(c, ks):
-    return areg(128 + 4 * (8 * c + ks), 4)
+    return areg(128 + 4 * (KS * c + ks), 4)
 
 
 def KA(ks):
@@ -102,9 +114,9 @@ class Ins:
 
 
 class Op:
-    def __init__(self, ins, earliest=0, latest=GAPS - 1):
+    def __init__(self, ins, earliest=0, latest=None):
         self.ins = ins if isinstance(ins, list) else [ins]
-        self.earliest, self.latest = earliest, latest
+        self.earliest, self.latest = earliest, GAPS - 1 if latest is None else latest
         self.units = sum(i.units for i in self.ins)
 
 
@@ -183,13 +195,13 @@ def subtile_ops(ty, j, kt):
             lds.append(Op(Ins(f"ds_read_b64_tr_b16 {areg(VA(step, dt) + 2, 2)}, {reg} offset:{base + 8 * RB}", kind="lds",
                               issue=f"va{step}_{dt}"), gap + 1, gap + 1))
 
-    v_reads(0, j, kt, 0)   # first k-step of this subtile: consumed from product 16 on
-    v_reads(1, j, kt, 8)   # second k-step: consumed from product 24 on
+    v_reads(0, j, kt, 0)       # first k-step of this subtile: consumed from product M_A on
+    v_reads(1, j, kt, 2 * DT)  # second k-step: consumed from product M_A + M_B on
     if kt == 0:
         # tile j+1 becomes visible: this wave's loads of it have landed, then every wave's
         # (a tile in [splo, splo + spspan) has rows past the context end or in absent blocks: the wave clears the
         # rows it loaded itself; unsigned compare of the distance covers both ends)
-        lds.append(Op(Ins("s_waitcnt vmcnt(8)\n\ts_sub_u32 s56, %[sP], %[splo]\n\ts_cmp_lt_u32 s56, %[spspan]\n"
+        lds.append(Op(Ins(f"s_waitcnt vmcnt({2 * NG})\n\ts_sub_u32 s56, %[sP], %[splo]\n\ts_cmp_lt_u32 s56, %[spspan]\n"
                           f"\ts_cbranch_scc1 .Lpf_fix_{j}_%=\n.Lpf_fixed_{j}_%=:\n"
                           "\ts_add_u32 %[sP], %[sP], 1\n\t" + ("s_nop 0" if "nobarrier" in X else "s_barrier"),
                           kind="sync", units=6, n=6), SYNC_GAP, SYNC_GAP))
@@ -199,7 +211,7 @@ def subtile_ops(ty, j, kt):
     for ks in range(KS):
         reg, imm = k_addr(nstage, ks)
         lds.append(Op(Ins(f"ds_read_b128 {areg(KA(ks), 4)}, {reg} offset:{imm + kt * 32 * RB}", kind="lds", issue=f"ka{ks}"),
-                      17 + ks, 17 + ks))
+                      SYNC_GAP + 1 + ks, SYNC_GAP + 1 + ks))
     streams["lds"] = lds
 
     # ---- exponentials: piece n covers S^T values 2j', 2j'+1 of column tile c (n = 2j' + c) ----
@@ -229,7 +241,7 @@ def subtile_ops(ty, j, kt):
         return out
 
     def deadline(n):  # a whole gap before the product that reads the word
-        return 14 if n < 8 else 22
+        return M_A - 2 if n < 8 else M_A + M_B - 2
 
     # (every instruction is placed on its own; the order keeps the four instructions of the next piece between an
     # exponential and the conversion that reads it)
@@ -267,7 +279,7 @@ def subtile_ops(ty, j, kt):
     if LO:
         check += f"\ts_cmp_gt_i32 %[slo], {32 * (kt + 1)}\n\ts_cbranch_scc1 .Lpf_mask_{j}{kt}_%=\n"
     mx.append(Op(Ins(check + f".Lpf_masked_{j}{kt}_%=:", kind="salu", units=4 if LO else 2, n=4 if LO else 2,
-                     reads=[f"v{S(nb, c) + i}" for c in range(NC) for i in range(16)]), 21))
+                     reads=[f"v{S(nb, c) + i}" for c in range(NC) for i in range(16)]), MAX_GAP))
     for c in range(NC):
         s = S(nb, c)
         r = lambda i: f"v{s + i}"
@@ -277,17 +289,17 @@ def subtile_ops(ty, j, kt):
                              writes=(f"v{m[c]}",)))
         chain.append(Ins(f"v_max_f32_e32 v{m[c]}, v{m[c]}, {r(15)}", reads=(f"v{m[c]}", r(15)), writes=(f"v{m[c]}",)))
         for ins in chain:
-            mx.append(Op(ins, 21))
-        mx.append(Op(Ins(f"v_mov_b32_e32 v{w[c]}, v{m[c]}", reads=(f"v{m[c]}",), writes=(f"v{w[c]}",)), 21))
+            mx.append(Op(ins, MAX_GAP))
+        mx.append(Op(Ins(f"v_mov_b32_e32 v{w[c]}, v{m[c]}", reads=(f"v{m[c]}",), writes=(f"v{w[c]}",)), MAX_GAP))
     for c in range(NC):
         mx.append(Op(Ins(f"v_permlane32_swap_b32_e32 v{m[c]}, v{w[c]}", kind="swap", reads=(f"v{m[c]}", f"v{w[c]}"),
-                         writes=(f"v{m[c]}", f"v{w[c]}")), 21))
-        mx.append(Op(Ins(f"v_max_f32_e32 %[mx{c}], v{m[c]}, v{w[c]}", reads=(f"v{m[c]}", f"v{w[c]}")), 21))
+                         writes=(f"v{m[c]}", f"v{w[c]}")), MAX_GAP))
+        mx.append(Op(Ins(f"v_max_f32_e32 %[mx{c}], v{m[c]}, v{w[c]}", reads=(f"v{m[c]}", f"v{w[c]}")), MAX_GAP))
     # does a row's maximum exceed its reference by more than the slack?  (read at the start of the next subtile)
     # (with lower bounds a row may not have seen a key yet: its threshold thr is a large negative number until
     # it has, so that its first maximum, whatever its sign, becomes its reference)
-    mx.append(Op(Ins(f"v_cmp_gt_f32_e64 s[60:61], %[mx0], {'%[thr0]' if LO else '%[slack]'}"), 21))
-    mx.append(Op(Ins(f"v_cmp_gt_f32_e64 s[62:63], %[mx1], {'%[thr1]' if LO else '%[slack]'}"), 21))
+    mx.append(Op(Ins(f"v_cmp_gt_f32_e64 s[60:61], %[mx0], {'%[thr0]' if LO else '%[slack]'}"), MAX_GAP))
+    mx.append(Op(Ins(f"v_cmp_gt_f32_e64 s[62:63], %[mx1], {'%[thr1]' if LO else '%[slack]'}"), MAX_GAP))
     # (order: chain 0, copy 0, chain 1, copy 1, swap 0, max 0, swap 1, max 1: two instructions between a copy and its swap)
     streams["max"] = mx
 
@@ -301,12 +313,15 @@ def subtile_ops(ty, j, kt):
                        Ins("s_lshl4_add_u32 s55, s55, %[tabA]", kind="salu"),
                        Ins("s_add_u32 %[sT], %[sT], 1", kind="salu"),
                        Ins("v_mov_b32_e32 v92, s55", writes=("v92",))], first))
-        ldr.append(Op(Ins("ds_read_b128 v[88:91], v92", kind="lds", reads=("v92",), issue="tab"), first))
-        for n in range(4):
-            ldr.append(Op(Ins(f"v_readfirstlane_b32 s{40 + n}, v{88 + n}", reads=(f"v{88 + n}",), need=("tab",)), max(22, SYNC_GAP + 5)))
-    groups = (0, 1) if kt == 0 else (2, 3)
+        # (head_dim 128: a wave loads four rows of each of the tile's four 16-key groups; head_dim 64: eight rows of
+        # two of them, groups w/2 and w/2 + 2 - the wave's first group is folded into tabA)
+        read = "ds_read_b128 v[88:91], v92" if NG == 4 else "ds_read2_b32 v[88:89], v92 offset1:2"
+        ldr.append(Op(Ins(read, kind="lds", reads=("v92",), issue="tab"), first))
+        for n in range(NG):
+            ldr.append(Op(Ins(f"v_readfirstlane_b32 s{40 + n}, v{88 + n}", reads=(f"v{88 + n}",), need=("tab",)), SYNC_GAP + 6))
+    groups = range(NG // 2) if kt == 0 else range(NG // 2, NG)
     for n in groups:
-        e = max(24, SYNC_GAP + 7) if kt == 0 else 0
+        e = SYNC_GAP + 8 if kt == 0 else 0
         # slot * row stride (64 bits), then per tensor: LDS destination into m0, pool base + offset, load.  The
         # two additions between the write of m0 and the load are the wait state that write needs.
         ldr.append(Op([Ins(f"s_mul_i32 s44, s{40 + n}, %[stride]", kind="salu"),
@@ -386,13 +401,15 @@ def fixup():
            "v_mov_b32_e32 v99, s57",
            "ds_read_b32 v99, v99",
            "s_and_b32 s58, %[sP], 3",
-           "s_lshl_b32 s58, s58, 15",
+           f"s_lshl_b32 s58, s58, {STAGE.bit_length() - 1}",
            "s_add_u32 s58, s58, %[m0w]",
            "s_waitcnt lgkmcnt(0)",
            "v_readfirstlane_b32 s57, v99",
            "v_add_u32_e32 v99, s58, %[lane16]"]
-    for n in range(4):
-        out += [f"s_bfe_u32 s59, s57, {8 * n | (8 << 16)}",
+    if NG < 4:  # (the wave's first group is not group 0: its byte moves down to bit 0)
+        out.append("s_lshr_b32 s57, s57, %[bshift]")
+    for n in range(NG):
+        out += [f"s_bfe_u32 s59, s57, {8 * (4 // NG) * n | (8 << 16)}",
                 "v_cmp_le_u32_e32 vcc, s59, %[arow]",
                 "s_nop 1",
                 "s_and_saveexec_b64 s[52:53], vcc",
@@ -501,7 +518,7 @@ def rescale(ty):
             for i in range(16):
                 out.append(f"v_sub_f32_e32 v{S(buf, c) + i}, v{S(buf, c) + i}, v97")
         for dt in range(DT):
-            base = 16 * (4 * c + dt)
+            base = 16 * (DT * c + dt)
             for i in range(0, 16, 2):
                 out += [f"v_accvgpr_read_b32 v93, a{base + i}", f"v_accvgpr_read_b32 v94, a{base + i + 1}",
                         "v_mul_f32_e32 v93, v93, v98", "v_mul_f32_e32 v94, v94, v98",
@@ -567,16 +584,20 @@ def main():
              "// as inline assembly; the register map and the schedule are described in the generator.",
              ""]
     global LO
-    for lo in (False, True):
-        LO = lo
-        for name in ("bf16", "f16"):
-            lines, stats = loop_text(Types(name))
-            per_tile = {k: v // NSTAGE for k, v in sorted(stats.items())}
-            parts.append(f"// {name}{', with lower bounds' if lo else ''}: instructions per 64-key tile: {per_tile}")
-            parts.append(f"#define PF_LOOP_ASM_{name.upper()}{'_LO' if lo else ''} \\")
-            body = c_string(lines).split("\n")
-            parts.append(" \\\n".join(body))
-            parts.append("")
+    for head_dim in (128, 64):
+        configure(head_dim)
+        for lo in (False, True):
+            LO = lo
+            for name in ("bf16", "f16"):
+                lines, stats = loop_text(Types(name))
+                per_tile = {k: v // NSTAGE for k, v in sorted(stats.items())}
+                what = f"{name}{', with lower bounds' if lo else ''}" + ("" if head_dim == 128 else f", head_dim {head_dim}")
+                parts.append(f"// {what}: instructions per 64-key tile: {per_tile}")
+                parts.append(f"#define PF_LOOP_ASM_{'' if head_dim == 128 else f'D{head_dim}_'}{name.upper()}{'_LO' if lo else ''} \\")
+                body = c_string(lines).split("\n")
+                parts.append(" \\\n".join(body))
+                parts.append("")
+    configure(128)
     with open(path, "w") as f:
         f.write("\n".join(parts))
     print("wrote", path)

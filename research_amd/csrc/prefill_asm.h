@@ -29,14 +29,18 @@ constexpr int kPaCapTiles = 1600;  // tiles of 64 keys the slot tables hold: con
 
 // LO: the instance that also applies lower bounds (sliding window, per-row first keys): the workgroup starts at
 // the tile of the first key its first row sees, everything the loop counts in is relative to that tile.
-template <typename T, bool LO>
+template <typename T, bool LO, int D>
 __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
-    constexpr int D = 128;
+    static_assert(D == 128 || D == 64, "the assembly loops are generated for these head sizes");
     using G = PfTile<D>;
     constexpr int KS = D / 16, DT = D / 32, NC = kPfCols;
     constexpr int GPT = kPfKeys / 16;  // 16-key groups per tile
+    // A wave-wide direct load covers 1 KiB = RPL rows.  head_dim 128: wave w fetches four rows of each of the tile's
+    // four groups (NG = 4 loads per tensor: groups 0, 1, 2, 3); head_dim 64: eight rows of two of them (NG = 2:
+    // groups w/2 and w/2 + 2).  Either way load n lands 4 KiB behind load n-1.
+    constexpr int NG = G::LOADS / kPfWaves, GSTEP = GPT / NG;
     typedef __attribute__((address_space(3))) char lds_char;
     constexpr int kRingBytes = kPfStages * 2 * G::BYTES;
     constexpr int kTabABytes = kPaCapTiles * GPT * 4, kTabBBytes = (kPaCapTiles + 1) * GPT;
@@ -176,35 +180,39 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     const int first_special =
         __builtin_amdgcn_readfirstlane(min(min(s_special[0], s_special[1]), min(s_special[2], s_special[3])));
 
-    // ---- loads of a tile: wave w fetches rows 4w .. 4w+3 of each of the tile's four 16-key groups ----
+    // ---- loads of a tile: wave w fetches rows w*RPL .. w*RPL + RPL-1 of the tile and, NG-1 times, the rows 4*RPL on ----
     const int64_t tok_stride = (int64_t)p.hkv * D * 2;
     const char *pool_k = reinterpret_cast<const char *>(p.k) + (int64_t)kvh * D * 2;
     const char *pool_v = reinterpret_cast<const char *>(p.v) + (int64_t)kvh * D * 2;
     const int ld_row = lane / G::CPR, ld_slot = lane % G::CPR;
-    const int arow = wave * G::RPL + ld_row;  // this lane's row inside a 16-key group
-    const uint32_t lane_k = (uint32_t)(arow * tok_stride) + (uint32_t)((ld_slot ^ G::swz_k(arow)) * 16);
-    const uint32_t lane_v = (uint32_t)(arow * tok_stride) + (uint32_t)((ld_slot ^ G::swz_v(arow)) * 16);
+    const int tile_row = wave * G::RPL + ld_row;  // this lane's row of the tile in the wave's first load
+    const int g0 = (wave * G::RPL) / 16;          // the 16-key group of that load; load n: group g0 + n * GSTEP
+    const int arow = tile_row % 16;               // this lane's row inside its 16-key group
+    const uint32_t lane_k = (uint32_t)(arow * tok_stride) + (uint32_t)((ld_slot ^ G::swz_k(tile_row)) * 16);
+    const uint32_t lane_v = (uint32_t)(arow * tok_stride) + (uint32_t)((ld_slot ^ G::swz_v(tile_row)) * 16);
     const uint32_t m0w = lds_base + (uint32_t)wave * (G::RPL * G::RB);
+    constexpr int kLoadStep = kPfWaves * G::RPL * G::RB;  // LDS bytes between a wave's consecutive loads
+    static_assert(kLoadStep == 4096, "the assembly loops place a wave's loads 4 KiB apart");
     auto issue = [&](int tile) PF_INLINE {
         const int src = tile < n_real ? tile : 0;
         const uint32_t dst0 = m0w + (uint32_t)(tile % kPfStages) * 2 * G::BYTES;
 #pragma unroll
-        for (int n = 0; n < GPT; ++n) {
-            const uint32_t slot = (uint32_t)__builtin_amdgcn_readfirstlane(tab_a[src * GPT + n]);
+        for (int n = 0; n < NG; ++n) {
+            const uint32_t slot = (uint32_t)__builtin_amdgcn_readfirstlane(tab_a[src * GPT + g0 + n * GSTEP]);
             const uint64_t ofs = (uint64_t)slot * (uint32_t)tok_stride;
-            pf_dma16(dst0 + n * 16 * G::RB, pf_scalar_ptr(pool_k + ofs), lane_k);
-            pf_dma16(dst0 + G::BYTES + n * 16 * G::RB, pf_scalar_ptr(pool_v + ofs), lane_v);
+            pf_dma16(dst0 + n * kLoadStep, pf_scalar_ptr(pool_k + ofs), lane_k);
+            pf_dma16(dst0 + G::BYTES + n * kLoadStep, pf_scalar_ptr(pool_v + ofs), lane_v);
         }
     };
     issue(0);
     issue(1);
     issue(2);
-    pf_wait_loads<4 * GPT>();  // tile 0 has landed
+    pf_wait_loads<4 * NG>();  // tile 0 has landed
     if (first_special == 0) {  // clear the rows of tile 0 that do not exist (the loop does it for later tiles)
 #pragma unroll
-        for (int n = 0; n < GPT; ++n)
-            if (arow >= tab_b[n]) {
-                const uint32_t at = (m0w - lds_base) + n * 16 * G::RB + lane * 16;
+        for (int n = 0; n < NG; ++n)
+            if (arow >= tab_b[g0 + n * GSTEP]) {
+                const uint32_t at = (m0w - lds_base) + n * kLoadStep + lane * 16;
                 *reinterpret_cast<uint4 *>(s_mem + at) = uint4{0, 0, 0, 0};
                 *reinterpret_cast<uint4 *>(s_mem + at + G::BYTES) = uint4{0, 0, 0, 0};
             }
@@ -297,7 +305,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         uint32_t s_t = 3, s_p = 1;
         int s_rem = uni(mask_from - kPfKeys * t0);  // mask_from - 64 * (absolute) tile
         int s_lo = uni(lo_mask_until - kPfKeys * t0);  // the same for the lower bound
-        const uint32_t tab_a_base = lds_base + kRingBytes, tab_b_base = tab_a_base + kTabABytes;
+        const uint32_t tab_a_base = lds_base + kRingBytes + 4 * g0;  // (the wave's first group folded in)
+        const uint32_t tab_b_base = lds_base + kRingBytes + kTabABytes;
         const uint32_t sp_lo = (uint32_t)uni(first_special), sp_span = (uint32_t)uni(n_tiles - first_special);
         const uint32_t n_real_u = (uint32_t)uni(n_real), cap_tiles = (uint32_t)uni(cap_rel), mask_from_u = (uint32_t)uni(mask_from);
         const uint32_t lane16 = (uint32_t)lane * 16, arow_u = (uint32_t)arow;
@@ -306,25 +315,16 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         const uint32_t pvlo = __builtin_amdgcn_readfirstlane((uint32_t)pv), pvhi = __builtin_amdgcn_readfirstlane((uint32_t)(pv >> 32));
         const uint32_t stride = (uint32_t)tok_stride;
         const float slack = kPfSlack;  // in the units of S^T here: log2 of the factor a row's reference may lag by
-#define PA_LOOP_OPERANDS(MORE_OUT, MORE_IN)                                                                           \
-    : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[0][2]), "+{a[48:63]}"(o[0][3]),                    \
-      "+{a[64:79]}"(o[1][0]), "+{a[80:95]}"(o[1][1]), "+{a[96:111]}"(o[1][2]), "+{a[112:127]}"(o[1][3]),                \
+#define PA_LOOP_COMMON_OUT(...)                                                                                      \
       "+{v[0:15]}"(s0[0]), "+{v[16:31]}"(s0[1]), "+{v[118:133]}"(ref[0]), "+{v[134:149]}"(ref[1]),                    \
-      "+{a[192:195]}"(ka[0]), "+{a[196:199]}"(ka[1]), "+{a[200:203]}"(ka[2]), "+{a[204:207]}"(ka[3]),                   \
-      "+{a[208:211]}"(ka[4]), "+{a[212:215]}"(ka[5]), "+{a[216:219]}"(ka[6]), "+{a[220:223]}"(ka[7]),                   \
       [mx0] "+&v"(mx[0]), [mx1] "+&v"(mx[1]), [l0] "+&v"(l_run[0]), [l1] "+&v"(l_run[1]),                             \
-      [ntiles] "+&s"(n_left), [sT] "+&s"(s_t), [sP] "+&s"(s_p), [srem] "+&s"(s_rem) MORE_OUT                                \
-    : "{a[128:131]}"(qreg[0][0]), "{a[132:135]}"(qreg[0][1]), "{a[136:139]}"(qreg[0][2]), "{a[140:143]}"(qreg[0][3]),   \
-      "{a[144:147]}"(qreg[0][4]), "{a[148:151]}"(qreg[0][5]), "{a[152:155]}"(qreg[0][6]), "{a[156:159]}"(qreg[0][7]),   \
-      "{a[160:163]}"(qreg[1][0]), "{a[164:167]}"(qreg[1][1]), "{a[168:171]}"(qreg[1][2]), "{a[172:175]}"(qreg[1][3]),   \
-      "{a[176:179]}"(qreg[1][4]), "{a[180:183]}"(qreg[1][5]), "{a[184:187]}"(qreg[1][6]), "{a[188:191]}"(qreg[1][7]),   \
-      [kad0] "v"(kad[0]), [kad1] "v"(kad[1]), [kad2] "v"(kad[2]), [kad3] "v"(kad[3]), [kad4] "v"(kad[4]),               \
-      [kad5] "v"(kad[5]), [kad6] "v"(kad[6]), [kad7] "v"(kad[7]), [vad0] "v"(vad[0]), [vad1] "v"(vad[1]),               \
-      [vad2] "v"(vad[2]), [vad3] "v"(vad[3]), [lanek] "v"(lane_k), [lanev] "v"(lane_v), [lane16] "v"(lane16),           \
+      [ntiles] "+&s"(n_left), [sT] "+&s"(s_t), [sP] "+&s"(s_p), [srem] "+&s"(s_rem) __VA_ARGS__
+#define PA_LOOP_COMMON_IN(...)                                                                                        \
+      [lanek] "v"(lane_k), [lanev] "v"(lane_v), [lane16] "v"(lane16),                                                   \
       [arow] "v"(arow_u), [lim0] "v"(lim[0]), [lim1] "v"(lim[1]), [slack] "s"(slack),                                   \
       [pklo] "s"(pklo), [pkhi] "s"(pkhi), [pvlo] "s"(pvlo), [pvhi] "s"(pvhi), [stride] "s"(stride), [m0w] "s"(m0w),     \
       [nreal] "s"(n_real_u), [tabA] "s"(tab_a_base), [tabB] "s"(tab_b_base), [splo] "s"(sp_lo),                       \
-      [spspan] "s"(sp_span), [captiles] "s"(cap_tiles), [maskfrom] "s"(mask_from_u) MORE_IN                           \
+      [spspan] "s"(sp_span), [captiles] "s"(cap_tiles), [maskfrom] "s"(mask_from_u) __VA_ARGS__                       \
     : "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47",  \
       "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63",  \
       "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79",  \
@@ -335,25 +335,68 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
       "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255", "s40", "s41", "s42",     \
       "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58",  \
       "s59", "s60", "s61", "s62", "s63", "vcc", "scc", "memory"
+// head_dim 128: o[c][dt] at a[16*(4c+dt)], q[c][ks] at a[128 + 4*(8c+ks)], ka[ks] at a[192 + 4*ks]
+#define PA_LOOP_OPERANDS(MORE_OUT, MORE_IN)                                                                           \
+    : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[0][2]), "+{a[48:63]}"(o[0][3]),                    \
+      "+{a[64:79]}"(o[1][0]), "+{a[80:95]}"(o[1][1]), "+{a[96:111]}"(o[1][2]), "+{a[112:127]}"(o[1][3]),                \
+      "+{a[192:195]}"(ka[0]), "+{a[196:199]}"(ka[1]), "+{a[200:203]}"(ka[2]), "+{a[204:207]}"(ka[3]),                   \
+      "+{a[208:211]}"(ka[4]), "+{a[212:215]}"(ka[5]), "+{a[216:219]}"(ka[6]), "+{a[220:223]}"(ka[7]),                   \
+      PA_LOOP_COMMON_OUT(MORE_OUT)                                                                                    \
+    : "{a[128:131]}"(qreg[0][0]), "{a[132:135]}"(qreg[0][1]), "{a[136:139]}"(qreg[0][2]), "{a[140:143]}"(qreg[0][3]),   \
+      "{a[144:147]}"(qreg[0][4]), "{a[148:151]}"(qreg[0][5]), "{a[152:155]}"(qreg[0][6]), "{a[156:159]}"(qreg[0][7]),   \
+      "{a[160:163]}"(qreg[1][0]), "{a[164:167]}"(qreg[1][1]), "{a[168:171]}"(qreg[1][2]), "{a[172:175]}"(qreg[1][3]),   \
+      "{a[176:179]}"(qreg[1][4]), "{a[180:183]}"(qreg[1][5]), "{a[184:187]}"(qreg[1][6]), "{a[188:191]}"(qreg[1][7]),   \
+      [kad0] "v"(kad[0]), [kad1] "v"(kad[1]), [kad2] "v"(kad[2]), [kad3] "v"(kad[3]), [kad4] "v"(kad[4]),               \
+      [kad5] "v"(kad[5]), [kad6] "v"(kad[6]), [kad7] "v"(kad[7]), [vad0] "v"(vad[0]), [vad1] "v"(vad[1]),               \
+      [vad2] "v"(vad[2]), [vad3] "v"(vad[3]), PA_LOOP_COMMON_IN(MORE_IN)
+// head_dim 64: o[c][dt] at a[16*(2c+dt)], q[c][ks] at a[128 + 4*(4c+ks)], ka[ks] at a[192 + 4*ks]; bshift: the bit
+// of the wave's first group in a tile's row of table B
+#define PA_LOOP_OPERANDS_D64(MORE_OUT, MORE_IN)                                                                       \
+    : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[1][0]), "+{a[48:63]}"(o[1][1]),                    \
+      "+{a[192:195]}"(ka[0]), "+{a[196:199]}"(ka[1]), "+{a[200:203]}"(ka[2]), "+{a[204:207]}"(ka[3]),                   \
+      PA_LOOP_COMMON_OUT(MORE_OUT)                                                                                    \
+    : "{a[128:131]}"(qreg[0][0]), "{a[132:135]}"(qreg[0][1]), "{a[136:139]}"(qreg[0][2]), "{a[140:143]}"(qreg[0][3]),   \
+      "{a[144:147]}"(qreg[1][0]), "{a[148:151]}"(qreg[1][1]), "{a[152:155]}"(qreg[1][2]), "{a[156:159]}"(qreg[1][3]),   \
+      [kad0] "v"(kad[0]), [kad1] "v"(kad[1]), [kad2] "v"(kad[2]), [kad3] "v"(kad[3]), [vad0] "v"(vad[0]),               \
+      [vad1] "v"(vad[1]), [bshift] "s"(b_shift), PA_LOOP_COMMON_IN(MORE_IN)
 #define PA_NOTHING
 #define PA_LO_OUT , [thr0] "+&v"(thr[0]), [thr1] "+&v"(thr[1]), [slo] "+&s"(s_lo)
 #define PA_LO_IN , [lo0] "v"(lo[0]), [lo1] "v"(lo[1]), [negbig] "s"(neg_big)
         const float neg_big = kNegBig;
-        if constexpr (LO) {
-            if constexpr (std::is_same<T, pa_bf16>::value) {
+        constexpr bool BF = std::is_same<T, pa_bf16>::value;
+        if constexpr (D == 128 && LO) {
+            if constexpr (BF) {
                 asm volatile(PF_LOOP_ASM_BF16_LO PA_LOOP_OPERANDS(PA_LO_OUT, PA_LO_IN));
             } else {
                 asm volatile(PF_LOOP_ASM_F16_LO PA_LOOP_OPERANDS(PA_LO_OUT, PA_LO_IN));
             }
-        } else {
+        } else if constexpr (D == 128) {
             (void)s_lo; (void)neg_big;
-            if constexpr (std::is_same<T, pa_bf16>::value) {
+            if constexpr (BF) {
                 asm volatile(PF_LOOP_ASM_BF16 PA_LOOP_OPERANDS(PA_NOTHING, PA_NOTHING));
             } else {
                 asm volatile(PF_LOOP_ASM_F16 PA_LOOP_OPERANDS(PA_NOTHING, PA_NOTHING));
             }
+        } else if constexpr (LO) {
+            const uint32_t b_shift = (uint32_t)uni(8 * g0);
+            if constexpr (BF) {
+                asm volatile(PF_LOOP_ASM_D64_BF16_LO PA_LOOP_OPERANDS_D64(PA_LO_OUT, PA_LO_IN));
+            } else {
+                asm volatile(PF_LOOP_ASM_D64_F16_LO PA_LOOP_OPERANDS_D64(PA_LO_OUT, PA_LO_IN));
+            }
+        } else {
+            (void)s_lo; (void)neg_big;
+            const uint32_t b_shift = (uint32_t)uni(8 * g0);
+            if constexpr (BF) {
+                asm volatile(PF_LOOP_ASM_D64_BF16 PA_LOOP_OPERANDS_D64(PA_NOTHING, PA_NOTHING));
+            } else {
+                asm volatile(PF_LOOP_ASM_D64_F16 PA_LOOP_OPERANDS_D64(PA_NOTHING, PA_NOTHING));
+            }
         }
 #undef PA_LOOP_OPERANDS
+#undef PA_LOOP_OPERANDS_D64
+#undef PA_LOOP_COMMON_OUT
+#undef PA_LOOP_COMMON_IN
 #undef PA_NOTHING
 #undef PA_LO_OUT
 #undef PA_LO_IN
@@ -376,7 +419,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
                 uint2 w;
                 w.x = M::pack(o[c][dt][4 * g] * inv, o[c][dt][4 * g + 1] * inv);
                 w.y = M::pack(o[c][dt][4 * g + 2] * inv, o[c][dt][4 * g + 3] * inv);
-                *reinterpret_cast<uint2 *>(rowp + (((4 * dt + g) ^ (col & 15)) * 16) + 8 * half) = w;
+                *reinterpret_cast<uint2 *>(rowp + (((4 * dt + g) ^ (col & (QCPR - 1))) * 16) + 8 * half) = w;
             }
     }
     // (a wave reads only what it wrote itself: no barrier, the compiler waits for the LDS writes)
@@ -389,7 +432,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 #pragma unroll
             for (int i = 0; i < 32 / QRPI; ++i) {
                 const int r = i * QRPI + r_in;
-                const uint4 v = *reinterpret_cast<const uint4 *>(s_mem + out_stage + (c * 32 + r) * QRB + ((chunk ^ (r & 15)) * 16));
+                const uint4 v = *reinterpret_cast<const uint4 *>(s_mem + out_stage + (c * 32 + r) * QRB + ((chunk ^ (r & (QCPR - 1))) * 16));
                 if (row0[c] + r < q_len)
                     *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(obase + (int64_t)r * p.hq * D) + chunk * 16) = v;
             }
@@ -399,6 +442,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 
 // nullptr unless the element type has this kernel; `lower_bounds`: the instance for sliding windows and per-row
 // first keys
-prefill_mfma_fn pa_prefill_asm_kernel(int dtype, bool lower_bounds);
+prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds);
 
 }  // namespace pa_decode_detail

@@ -240,16 +240,17 @@ def test_packed_documents_chunked_prefill_over_a_prefix():
     assert_close(out.reshape(2, cmax, hq, d), want, 2e-2, "chunked documents")
 
 
+@pytest.mark.parametrize("d", [128, 64])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype):
-    """head_dim 128 takes the kernel whose tile loop is scheduled assembly.  Block ids of -1 or past the pool, and
+def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype, d):
+    """head_dim 128 and 64 take the kernel whose tile loop is scheduled assembly.  Block ids of -1 or past the pool, and
     contexts longer than the table, stand for zero key / value rows there as in the vector kernel (which is the
     statement of that rule: flex_backend.py:272-277 leaves rows of absent blocks zero); the two kernels must
     agree on every row, for 16-token and 64-token blocks, with the bad entries in the first tile, in the middle
     and at the end."""
-    announce(f"prefill assembly loop, absent blocks {dtype}")
+    announce(f"prefill assembly loop, absent blocks {dtype} d={d}")
     rng = np.random.default_rng(77)
-    hq, hkv, d = 8, 2, 128
+    hq, hkv = 8, 2
     for bs in (16, 64):
         prefix = [200, 0, 333, 64]
         chunk = [100, 190, 31, 64]
@@ -279,13 +280,14 @@ def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype):
                 assert_close(got[b, :c], want[b, :c], 2e-2, f"block_size {bs} sequence {b} window {window}")
 
 
-def test_assembly_loop_kernel_long_context_and_table_limit():
+@pytest.mark.parametrize("d", [128, 64])
+def test_assembly_loop_kernel_long_context_and_table_limit(d):
     """A 70 000-key context (more than a thousand tiles of slot-table entries) through the assembly-loop kernel,
     and a table just past what that kernel's LDS tables hold (the host then launches the other matrix-core
     kernel): both against the vector kernel on the chunk's rows."""
-    announce("prefill assembly loop, long context")
+    announce(f"prefill assembly loop, long context d={d}")
     rng = np.random.default_rng(78)
-    hq, hkv, d, bs = 4, 1, 128, 16
+    hq, hkv, bs = 4, 1, 16
     for ctx in (70000, 1600 * 64 + 40):
         chunk = 48
         nblk = -(-ctx // bs)
@@ -305,8 +307,8 @@ def test_logits_that_grow_along_the_context(d):
     """Keys whose logits rise steeply with the key index (about 9 in base-2 units per 32 keys, from far below
     zero to far above), so that every row's reference maximum is outgrown by more than the lazy-rescale slack
     again and again, by some rows of a wave earlier than by others; then the same keys in falling order (the
-    first subtile holds the maximum, nothing is ever rescaled).  All three matrix-core kernels (head_dim 64
-    compiled, 128 assembly loop, 256), chunked over a prefix, against the checker."""
+    first subtile holds the maximum, nothing is ever rescaled).  The assembly loops of head_dim 64, 128 and 256
+    (and, with a window, their instances with lower bounds), chunked over a prefix, against the checker."""
     announce(f"prefill rescale paths d={d}")
     rng = np.random.default_rng(500 + d)
     hq, hkv, bs = 4, 2, 16
