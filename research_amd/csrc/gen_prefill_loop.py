@@ -1,12 +1,15 @@
 #!/usr/bin/env python3
-"""Writes prefill_mfma_loop.inc: the tile loop of prefill_asm_kernel (head_dim 128) as one inline-assembly
-block per element type (bf16, fp16).
+"""Writes prefill_mfma_loop.inc: the tile loop of prefill_asm_kernel as one inline-assembly block per head size
+(128, 64), element type (bf16, fp16) and variant (without / with lower bounds).
 
 Why assembly: with one wave per SIMD nothing hides latency except the wave's own instruction order, and a
-wave issues one instruction per 4 cycles (a matrix product takes two issue slots, an exponential two).  A
-32-key subtile is 32 products = 1024 cycles = 256 issue slots, and the softmax arithmetic, operand reads and
-tile loads around them need about 230: the loop only runs near the matrix unit's rate if next to nothing
-else is issued and the other instructions are spread evenly between the products.  This script fixes the
+wave issues one instruction per 4 cycles (a matrix product takes two issue slots, an exponential two).  At
+head_dim 128 a 32-key subtile is 32 products = 1024 cycles = 256 issue slots, and the softmax arithmetic,
+operand reads and tile loads around them need about 230: the loop only runs near the matrix unit's rate if next
+to nothing else is issued and the other instructions are spread evenly between the products.  At head_dim 64
+the subtile has 16 products and nearly the same softmax arithmetic (it goes with keys x rows, not with the head
+size): about 200 slots of other instructions against 512 cycles of products, so the issue rate bounds that
+loop and every instruction saved counts in full.  This script fixes the
 register assignment, places every instruction, derives the `s_waitcnt lgkmcnt` values from the order of the
 LDS reads and checks the distances the hardware does not interlock (matrix result -> vector read,
 transcendental -> vector read, vector write -> lane swap).
@@ -20,11 +23,13 @@ wave needs it for.  A wave whose rows end before the workgroup's last tile keeps
 masked (its probabilities are exact zeros), and loads past the last tile fetch tile 0 again, so that every
 wave executes the same barriers and the same number of loads per tile.
 
-Register map (per lane; the kernel pins its variables to the same registers):
-  a[0:127]    O^T accumulators  o[c][dt]   at 16*(4c+dt)
-  a[128:191]  Q^T operands      q[c][ks]   at 128 + 4*(8c+ks)
+Register map (per lane; the kernel pins its variables to the same registers; KS = head_dim / 16 k-steps of
+S^T, DT = head_dim / 32 d tiles of O^T; the ranges are those of head_dim 128, head_dim 64 uses the first half
+of each):
+  a[0:127]    O^T accumulators  o[c][dt]   at 16*(DT*c + dt)
+  a[128:191]  Q^T operands      q[c][ks]   at 128 + 4*(KS*c + ks)
   a[192:223]  K operands        ka[ks]     at 192 + 4*ks
-  a[224:239]  V^T operands of the first k-step, a[240:255] of the second
+  a[224:239]  V^T operands of the first k-step (d tile dt at 224 + 4*dt), a[240:255] of the second
   v[0:63]     S^T: buffer b, column tile c at 16*(2b+c); a tile starts with its first subtile in buffer 0
   v[64:79]    P^T operand words pp[c][j] at 64 + 8c + j
   v[80:87]    exponentials in flight, v[88:91] four table entries, v92 table address, v[93:96] maxima
@@ -580,7 +585,7 @@ def c_string(lines):
 def main():
     path = sys.argv[1] if len(sys.argv) > 1 else os.path.join(os.path.dirname(os.path.abspath(__file__)),
                                                                "prefill_mfma_loop.inc")
-    parts = ["// Generated by gen_prefill_loop.py - do not edit.  The tile loop of prefill_asm_kernel (head_dim 128)",
+    parts = ["// Generated by gen_prefill_loop.py - do not edit.  The tile loops of prefill_asm_kernel (head_dim 128 and 64)",
              "// as inline assembly; the register map and the schedule are described in the generator.",
              ""]
     global LO

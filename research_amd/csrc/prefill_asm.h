@@ -1,12 +1,13 @@
-// Causal prefill attention over a paged context for head_dim 128 (bf16 / fp16) with the whole tile loop in
+// Causal prefill attention over a paged context for head_dim 128 and 64 (bf16 / fp16) with the whole tile loop in
 // scheduled assembly (prefill_mfma_loop.inc, written by gen_prefill_loop.py).
 //
 // Same computation, work split, LDS ring and operand layouts as prefill_mfma_kernel (prefill_mfma.h); what
 // differs is what surrounds the loop:
 //   * the pool slots of the context's 16-key groups are looked up once per workgroup and kept in LDS behind the
 //     ring (table A: slot of the group's first key; table B: first row of the group that does not exist, 16 =
-//     none), so a tile's loads are a table read, four scalar multiplies and eight direct loads, for any block
-//     size that is a multiple of 16;
+//     none), so a tile's loads are a table read, a scalar multiply per group and one direct load per group and
+//     tensor (head_dim 128: eight per wave and tile, head_dim 64: four), for any block size that is a multiple
+//     of 16;
 //   * rows past the context end and absent blocks are loaded from a slot that exists (the group's own block,
 //     or slot 0) and cleared in LDS before the tile is published; a zero key takes part with logit 0 and a
 //     zero value row, which is what the other kernels do for absent blocks;
