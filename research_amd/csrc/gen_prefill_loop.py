@@ -421,6 +421,34 @@ def fixup():
                 f"ds_write_b128 v99, v[112:115] offset:{n * 4096}",
                 f"ds_write_b128 v99, v[112:115] offset:{n * 4096 + TENSOR}",
                 "s_mov_b64 exec, s[52:53]"]
+    # The one 16-key group of a workgroup that reaches past the end of the pool (the last rows of the pool's last
+    # block, when blocks are not multiples of 16 keys long): its direct loads fetched 16 rows from a slot where 16
+    # exist, and the rows of it that exist are copied here, lane by lane, from where they are.  edgetile = its
+    # tile (-1 = none), edgeslot = its first row, edgerows = how many exist, edgeofs = LDS offset of this wave's
+    # load of that group (-1 = this wave loads no row of it).  (v88..v92 are free here: the table entries were
+    # consumed in the previous tile, the next table address is formed behind the barrier.)
+    out += ["s_cmp_lg_u32 %[sP], %[edgetile]",
+            "s_cbranch_scc1 .Lpf_noedge_%=",
+            "s_cmp_eq_u32 %[edgeofs], -1",
+            "s_cbranch_scc1 .Lpf_noedge_%=",
+            "s_mul_i32 s44, %[edgeslot], %[stride]",
+            "s_mul_hi_u32 s45, %[edgeslot], %[stride]",
+            "s_add_u32 s46, %[pklo], s44",
+            "s_addc_u32 s47, %[pkhi], s45",
+            "s_add_u32 s48, %[pvlo], s44",
+            "s_addc_u32 s49, %[pvhi], s45",
+            "v_cmp_gt_u32_e32 vcc, %[edgerows], %[arow]",
+            "s_nop 1",
+            "s_and_saveexec_b64 s[52:53], vcc",
+            "global_load_dwordx4 v[88:91], %[lanek], s[46:47]",
+            "v_add_u32_e32 v92, %[edgeofs], v99",
+            "s_waitcnt vmcnt(0)",
+            "ds_write_b128 v92, v[88:91]",
+            "global_load_dwordx4 v[88:91], %[lanev], s[48:49]",
+            "s_waitcnt vmcnt(0)",
+            f"ds_write_b128 v92, v[88:91] offset:{TENSOR}",
+            "s_mov_b64 exec, s[52:53]",
+            ".Lpf_noedge_%=:"]
     out += ["s_waitcnt lgkmcnt(0)", "s_setpc_b64 s[50:51]"]
     return out
 

@@ -16,8 +16,11 @@
 //   * sliding windows and per-row first keys have an instance of their own (LO): the out-of-line mask block also
 //     applies the lower bound, a row that has seen no key yet takes its first maximum as reference, and the
 //     workgroup starts at the tile of the first key its first row sees;
-//   * the host launches prefill_mfma_kernel for other head sizes, block sizes that are not multiples of 16 and
-//     tables past kPaCapTiles.
+//   * block sizes that are not multiples of 16 are taken with one block per sequence (what dense prefill passes):
+//     a group's load then runs into the next block's rows, which are cleared like rows past the context end,
+//     and the one group at the end of the pool is fetched lane by lane when its tile is published;
+//   * the host launches prefill_mfma_kernel for other head sizes, for tables of several blocks that are not
+//     multiples of 16 keys long and for tables past kPaCapTiles.
 // Only the set-up, the first subtile's S^T and the write-out are compiled code, so the register allocator sees
 // one asm statement with pinned operands and little else.
 #pragma once
@@ -135,6 +138,25 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         }
     }
     // ---- slot tables (in flight together with the Q rows) ----
+    const int64_t pool_rows = p.num_blocks * p.bs;  // >= 16, < 2^31 (the host checks)
+    // Blocks that are not multiples of 16 keys long (one block per sequence, as dense prefill passes its rows):
+    // a 16-key group may run into the rows of the next block - harmless, they are cleared before the tile is
+    // published - but the last group of the pool's last block would run past the end of the pool.  That one
+    // group (at most one per workgroup) is loaded from slot 0 instead and its existing rows are copied from
+    // where they are, lane by lane, when its tile is published.
+    int edge_tile = -1, edge_group = 0, edge_rows = 0;  // tile relative to t0
+    int64_t edge_slot = 0;
+    if (p.bs % 16 != 0) {  // (then bt_stride is 1)
+        const int64_t bid = p.bt[(int64_t)b * p.bt_stride];
+        const int n_keys = min(ctx_len, p.bs);
+        const int key_last = (n_keys - 1) / 16 * 16;
+        if (bid >= 0 && bid < p.num_blocks && bid * p.bs + key_last + 16 > pool_rows && key_last / kPfKeys >= t0) {
+            edge_tile = key_last / kPfKeys - t0;
+            edge_group = key_last / 16 % GPT;
+            edge_rows = n_keys - key_last;
+            edge_slot = bid * p.bs + key_last;
+        }
+    }
     {
         const int32_t *bt_seq = p.bt + (int64_t)b * p.bt_stride;
         const int n_entries = max(n_real, 1) * GPT;  // (the loads of tiles past the last fetch tile 0 again: it has entries)
@@ -144,8 +166,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             int64_t bid = -1;
             if (blk < p.bt_stride) bid = bt_seq[blk];
             const bool present = bid >= 0 && bid < p.num_blocks;
-            const int rows = present ? min(max(ctx_len - key, 0), 16) : 0;  // rows of the group that exist
-            tab_a[i] = present ? (int32_t)(bid * p.bs + key % p.bs) : 0;
+            // rows of the group that exist: inside the context and inside the group's block (a block that is not
+            // a multiple of 16 keys long is the only block of its sequence: what follows it is absent)
+            const int rows = present ? min(max(min(ctx_len, (blk + 1) * p.bs) - key, 0), 16) : 0;
+            int64_t slot = present ? bid * p.bs + key % p.bs : 0;
+            if (slot + 16 > pool_rows) slot = 0;  // (the group at the end of the pool: see edge_tile below)
+            tab_a[i] = (int32_t)slot;
             tab_b[i] = (uint8_t)rows;
             if (rows < 16) first_special = min(first_special, i / GPT);
         }
@@ -217,6 +243,15 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
                 *reinterpret_cast<uint4 *>(s_mem + at) = uint4{0, 0, 0, 0};
                 *reinterpret_cast<uint4 *>(s_mem + at + G::BYTES) = uint4{0, 0, 0, 0};
             }
+    }
+    // this wave's load of the group at the end of the pool, as an LDS offset behind the wave's first load (-1: none)
+    const int edge_n = edge_group - g0;
+    const int edge_ofs = edge_tile >= 0 && edge_n >= 0 && edge_n % GSTEP == 0 ? edge_n / GSTEP * kLoadStep : -1;
+    if (edge_tile == 0 && edge_ofs >= 0 && arow < edge_rows) {  // (in tile 0; the loop does it for later tiles)
+        const uint32_t at = (m0w - lds_base) + edge_ofs + lane * 16;
+        *reinterpret_cast<uint4 *>(s_mem + at) = *reinterpret_cast<const uint4 *>(pool_k + edge_slot * tok_stride + lane_k);
+        *reinterpret_cast<uint4 *>(s_mem + at + G::BYTES) =
+            *reinterpret_cast<const uint4 *>(pool_v + edge_slot * tok_stride + lane_v);
     }
     __syncthreads();  // tile 0 is visible
 
@@ -315,6 +350,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         const uint32_t pklo = __builtin_amdgcn_readfirstlane((uint32_t)pk), pkhi = __builtin_amdgcn_readfirstlane((uint32_t)(pk >> 32));
         const uint32_t pvlo = __builtin_amdgcn_readfirstlane((uint32_t)pv), pvhi = __builtin_amdgcn_readfirstlane((uint32_t)(pv >> 32));
         const uint32_t stride = (uint32_t)tok_stride;
+        const uint32_t edge_tile_u = (uint32_t)uni(edge_tile), edge_slot_u = (uint32_t)uni((int)edge_slot);
+        const uint32_t edge_rows_u = (uint32_t)uni(edge_rows), edge_ofs_u = (uint32_t)uni(edge_ofs);
         const float slack = kPfSlack;  // in the units of S^T here: log2 of the factor a row's reference may lag by
 #define PA_LOOP_COMMON_OUT(...)                                                                                      \
       "+{v[0:15]}"(s0[0]), "+{v[16:31]}"(s0[1]), "+{v[118:133]}"(ref[0]), "+{v[134:149]}"(ref[1]),                    \
@@ -325,7 +362,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
       [arow] "v"(arow_u), [lim0] "v"(lim[0]), [lim1] "v"(lim[1]), [slack] "s"(slack),                                   \
       [pklo] "s"(pklo), [pkhi] "s"(pkhi), [pvlo] "s"(pvlo), [pvhi] "s"(pvhi), [stride] "s"(stride), [m0w] "s"(m0w),     \
       [nreal] "s"(n_real_u), [tabA] "s"(tab_a_base), [tabB] "s"(tab_b_base), [splo] "s"(sp_lo),                       \
-      [spspan] "s"(sp_span), [captiles] "s"(cap_tiles), [maskfrom] "s"(mask_from_u) __VA_ARGS__                       \
+      [spspan] "s"(sp_span), [captiles] "s"(cap_tiles), [maskfrom] "s"(mask_from_u),                                \
+      [edgetile] "s"(edge_tile_u), [edgeslot] "s"(edge_slot_u), [edgerows] "s"(edge_rows_u),                          \
+      [edgeofs] "s"(edge_ofs_u) __VA_ARGS__                       \
     : "v32", "v33", "v34", "v35", "v36", "v37", "v38", "v39", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47",  \
       "v48", "v49", "v50", "v51", "v52", "v53", "v54", "v55", "v56", "v57", "v58", "v59", "v60", "v61", "v62", "v63",  \
       "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74", "v75", "v76", "v77", "v78", "v79",  \

@@ -302,6 +302,33 @@ def test_assembly_loop_kernel_long_context_and_table_limit(d):
             assert_close(got, want, 2e-2, f"context of {ctx} keys, window {window}")
 
 
+@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_assembly_loop_kernel_dense_rows_of_any_length(dtype, d):
+    """Dense rows handed over as one block per sequence whose length is not a multiple of 16 (what
+    `_prefill_attention`, flex_backend.py:144-185, gets for an ordinary prompt): a sequence's last 16-key group
+    runs into the next sequence's rows, and the last groups of the last sequences would run past the end of the
+    pool (with 6-token sequences, two of the three sequences' only group).  With per-row first keys (packed
+    documents, attention/mask.py:141-191), a sliding window, both, and neither; against the checker."""
+    announce(f"prefill assembly loop, dense rows {dtype} d={d}")
+    rng = np.random.default_rng(79)
+    hq, hkv = 8, 2
+    for b, t, doc_lens in ((2, 700, (1, 31, 32, 0, 64, 65, 300, 207)), (3, 6, (2, 4)), (1, 33, (33,)), (4, 129, (100, 29))):
+        q, k, v = (torch.from_numpy(rng.standard_normal((b, t, h, d)).astype(np.float32)).to(dtype) for h in (hq, hkv, hkv))
+        ident = torch.arange(b, dtype=torch.int32, device=DEV).reshape(b, 1).contiguous()
+        lens = _i32([t] * b)
+        bounds = np.asarray(po.document_boundaries(doc_lens))
+        first = bounds[np.searchsorted(bounds[1:], np.arange(t), side="right")].astype(np.int32)
+        first = torch.from_numpy(np.tile(first, b)).to(DEV)
+        for docs in (None, doc_lens):
+            for window in (0, 40):
+                got = ops.prefill_paged(q.reshape(b * t, hq, d).to(DEV), k.reshape(b * t, hkv, d).to(DEV),
+                                        v.reshape(b * t, hkv, d).to(DEV), ident, lens, lens, _i32(np.arange(b) * t), t, t,
+                                        d ** -0.5, window=window, row_first_key=first if docs else None)
+                want = po.dense_prefill(q, k, v, d ** -0.5, window=window, doc_lens=docs)
+                assert_close(got.reshape(b, t, hq, d), want, 2e-2, f"{b} x {t}, documents {docs}, window {window}")
+
+
 @pytest.mark.parametrize("d", [64, 128, 256])
 def test_logits_that_grow_along_the_context(d):
     """Keys whose logits rise steeply with the key index (about 9 in base-2 units per 32 keys, from far below
