@@ -162,3 +162,27 @@ def test_random_matrix_core_prefill(seed):
     if not with_absent and not with_first:
         want = po.paged_prefill_chunk(q, k, v, tables, prefix, chunk, bs, d ** -0.5, window=window)
         assert_close(got, want, 2e-2, "against the checker")
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_dense_prefill_of_any_length(seed):
+    """Dense causal prefill the way `_prefill_attention` hands it over (flex_backend.py:144-185): a pool of B blocks
+    of T rows with the identity table, T of any length (so 16-key groups run into the next sequence's rows and, at
+    the end of the pool, past it), head sizes 64 / 128 / 256, with and without a sliding window; against the
+    checker."""
+    rng = np.random.default_rng(9700 + seed)
+    d = int(rng.choice([64, 128, 256]))
+    hkv = int(rng.choice([1, 2, 4]))
+    hq = hkv * int(rng.choice([1, 2, 4, 7]))
+    dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
+    b = int(rng.integers(1, 5))
+    t = int(rng.choice([rng.integers(1, 40), rng.integers(40, 300), rng.integers(300, 900)]))
+    window = int(rng.choice([0, 0, 13, 100]))
+    announce(f"random dense prefill seed={seed} hq={hq} hkv={hkv} d={d} {dtype} batch={b} length={t} window={window}")
+    q, k, v = (torch.from_numpy(rng.standard_normal((b, t, h, d)).astype(np.float32)).to(dtype) for h in (hq, hkv, hkv))
+    i32 = lambda x: torch.tensor(list(x), dtype=torch.int32, device=DEV)
+    ident = torch.arange(b, dtype=torch.int32, device=DEV).reshape(b, 1).contiguous()
+    got = ops.prefill_paged(q.reshape(b * t, hq, d).to(DEV), k.reshape(b * t, hkv, d).to(DEV), v.reshape(b * t, hkv, d).to(DEV),
+                            ident, i32([t] * b), i32([t] * b), i32(np.arange(b) * t), t, t, d ** -0.5, window=window)
+    want = po.dense_prefill(q, k, v, d ** -0.5, window=window)
+    assert_close(got.reshape(b, t, hq, d), want, 2e-2, "against the checker")
