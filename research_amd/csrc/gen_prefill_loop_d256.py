@@ -1,6 +1,7 @@
 #!/usr/bin/env python3
-"""Writes prefill_d256_loop.inc: the subtile loop of prefill_d256_asm_kernel (head_dim 256, no lower bounds, block
-sizes that are multiples of 16) as one inline-assembly block per element type (bf16, fp16).
+"""Writes prefill_d256_loop.inc: the subtile loop of the assembly instances of prefill_d256_kernel (head_dim 256,
+block sizes that are multiples of 16) as one inline-assembly block per element type (bf16, fp16) and variant
+(without / with lower bounds: sliding window, per-row first keys).
 
 The instruction classes, the placement of the other instructions into the gaps around a subtile's 32 products,
 the derivation of the `s_waitcnt lgkmcnt` values and the hazard checks are those of gen_prefill_loop.py; what
@@ -43,6 +44,7 @@ TENSOR = 32 * RB         # one tensor's 32 keys
 STAGE = 2 * TENSOR       # K of tile s+1, then V of tile s
 NSLOT = 4
 SYNC_GAP = 16
+LO = False                # the variant being generated also applies lower bounds (sliding window, per-row first keys)
 CAP_TILES = 3072         # tiles the slot tables hold (kWdCapGroups / 2); the entries of four more groups follow, all absent
 STUBS = []
 
@@ -183,10 +185,19 @@ def subtile_ops(ty, j):
            "v_subrev_u32_e32 v95, 32, v95"]
     for i in range(16):
         blk += [f"v_cmp_gt_i32_e32 vcc, {8 * (i >> 2) + (i & 3)}, v95", f"v_cndmask_b32_e32 v{s + i}, v{s + i}, v116, vcc"]
+    if LO:
+        # slo = (first key the wave's last row sees) - 32*g: S^T(g+1) also needs the mask if it starts below that
+        # key: slo > 32; a value is then also masked below lo - first key of the subtile
+        blk += ["v_subrev_u32_e32 v95, %[maskfrom], %[lo0]", "v_add_u32_e32 v95, %[srem], v95", "v_subrev_u32_e32 v95, 32, v95"]
+        for i in range(16):
+            blk += [f"v_cmp_lt_i32_e32 vcc, {8 * (i >> 2) + (i & 3)}, v95", f"v_cndmask_b32_e32 v{s + i}, v{s + i}, v116, vcc"]
     blk.append(f"s_branch .Lwd_masked_{j}_%=")
     STUBS.append(blk)
-    mx.append(Op(Ins(f"s_cmp_lt_i32 %[srem], 64\n\ts_cbranch_scc1 .Lwd_mask_{j}_%=\n.Lwd_masked_{j}_%=:", kind="salu",
-                     units=2, n=2, reads=[f"v{s + i}" for i in range(16)]), 21))
+    check = f"s_cmp_lt_i32 %[srem], 64\n\ts_cbranch_scc1 .Lwd_mask_{j}_%=\n"
+    if LO:
+        check += f"\ts_cmp_gt_i32 %[slo], 32\n\ts_cbranch_scc1 .Lwd_mask_{j}_%=\n"
+    mx.append(Op(Ins(check + f".Lwd_masked_{j}_%=:", kind="salu", units=4 if LO else 2, n=4 if LO else 2,
+                     reads=[f"v{s + i}" for i in range(16)]), 21))
     r = lambda i: f"v{s + i}"
     chain = [Ins(f"v_max3_f32 v93, {r(0)}, {r(1)}, {r(2)}", reads=(r(0), r(1), r(2)), writes=("v93",))]
     for i in range(3, 15, 2):
@@ -198,7 +209,9 @@ def subtile_ops(ty, j):
     mx.append(Op(Ins("s_nop 1", kind="salu", n=2), 21))  # (two wait states between the copy and the swap)
     mx.append(Op(Ins("v_permlane32_swap_b32_e32 v93, v95", kind="swap", reads=("v93", "v95"), writes=("v93", "v95")), 21))
     mx.append(Op(Ins("v_max_f32_e32 %[mx0], v93, v95", reads=("v93", "v95")), 21))
-    mx.append(Op(Ins("v_cmp_gt_f32_e64 s[60:61], %[mx0], %[slack]"), 21))
+    # (with lower bounds a row may not have seen a key yet: its threshold thr is a large negative number until it
+    # has, so that its first maximum, whatever its sign, becomes its reference)
+    mx.append(Op(Ins(f"v_cmp_gt_f32_e64 s[60:61], %[mx0], {'%[thr0]' if LO else '%[slack]'}"), 21))
     streams["max"] = mx
 
     # ---- loads of stage g+4 into slot j: two table entries, then four K loads and four V loads ----
@@ -263,11 +276,26 @@ def rescale():
     moves up by delta = max(maximum, 0): the reference tile, both S^T buffers and the maximum shift by -delta,
     the sum and the accumulators shrink by 2^-delta."""
     out = ["s_nop 7", "s_nop 7", "s_nop 7"]  # products still writing the accumulators
-    out += ["v_max_f32_e32 v97, 0, %[mx0]",
-            "v_exp_f32_e64 v98, -v97",
-            "v_sub_f32_e32 %[mx0], %[mx0], v97",
-            "s_nop 0",
-            "v_mul_f32_e32 %[l0], %[l0], v98"]
+    if LO:
+        # a row that had seen no key so far (thr still the large negative number; sum and accumulators zero)
+        # takes its first maximum as reference whatever its sign, and nothing of it is scaled
+        out += ["v_max_f32_e32 v97, 0, %[mx0]",
+                "v_cmp_lt_f32_e64 s[54:55], %[negbig], %[mx0]",       # this maximum is of visible keys
+                "v_cndmask_b32_e64 v99, 0, %[mx0], s[54:55]",
+                "v_cmp_eq_f32_e64 vcc, %[negbig], %[thr0]",            # no reference yet
+                "v_cndmask_b32_e32 v97, v97, v99, vcc",
+                "v_exp_f32_e64 v98, -v97",
+                "v_sub_f32_e32 %[mx0], %[mx0], v97",
+                "v_mov_b32_e32 v99, %[slack]",
+                "v_cndmask_b32_e64 %[thr0], %[thr0], v99, s[54:55]",
+                "v_cndmask_b32_e64 v98, v98, 1.0, vcc",
+                "v_mul_f32_e32 %[l0], %[l0], v98"]
+    else:
+        out += ["v_max_f32_e32 v97, 0, %[mx0]",
+                "v_exp_f32_e64 v98, -v97",
+                "v_sub_f32_e32 %[mx0], %[mx0], v97",
+                "s_nop 0",
+                "v_mul_f32_e32 %[l0], %[l0], v98"]
     for i in range(16):
         out.append(f"v_sub_f32_e32 v{CT + i}, v{CT + i}, v97")
     for buf in range(2):
@@ -294,11 +322,13 @@ def loop_text(ty):
     for dt in range(4):
         lines.append(f"v_add_u32_e32 v{108 + dt}, {2 * STAGE}, %[vad{dt}]")
     lines += [f"v_mov_b32_e32 v{r}, 0" for r in range(112, 116)]
-    lines += ["v_mov_b32_e32 v116, 0xff800000", "v_cmp_gt_f32_e64 s[60:61], %[mx0], %[slack]", "s_waitcnt lgkmcnt(0)", "s_nop 3"]
+    lines += ["v_mov_b32_e32 v116, 0xff800000", f"v_cmp_gt_f32_e64 s[60:61], %[mx0], {'%[thr0]' if LO else '%[slack]'}",
+              "s_waitcnt lgkmcnt(0)", "s_nop 3"]
     for j in range(NSLOT):
         lines.append(f".Lwd_tile{j}_%=:")
         lines += [ins.text for ins in bodies[j]]
-        lines += ["s_sub_u32 %[srem], %[srem], 32", "s_sub_u32 %[ntiles], %[ntiles], 1", "s_cbranch_scc1 .Lwd_done_%="]
+        lines += ["s_sub_u32 %[srem], %[srem], 32"] + (["s_sub_u32 %[slo], %[slo], 32"] if LO else [])
+        lines += ["s_sub_u32 %[ntiles], %[ntiles], 1", "s_cbranch_scc1 .Lwd_done_%="]
     lines.append("s_branch .Lwd_tile0_%=")
     for stub in STUBS:
         lines += stub
@@ -322,13 +352,13 @@ def operands():
     outs += [f'"+{{a[{KA(ks)}:{KA(ks) + 3}]}}"(ka[{ks}])' for ks in range(KS)]
     outs += [f'"+{{v[{VA0(dt)}:{VA0(dt) + 3}]}}"(va0[{dt}])' for dt in range(4)]
     outs += ['[mx0] "+&v"(mx)', '[l0] "+&v"(l_run)', '[ntiles] "+&s"(n_left)', '[sT] "+&s"(s_t)', '[sP] "+&s"(s_p)',
-             '[srem] "+&s"(s_rem)']
+             '[srem] "+&s"(s_rem) MORE_OUT']
     ins = [f'"{{a[{128 + 4 * ks}:{131 + 4 * ks}]}}"(qreg[{ks}])' for ks in range(KS)]
     ins += [f'[kad{ks}] "v"(kad[{ks}])' for ks in range(8)] + [f'[vad{dt}] "v"(vad[{dt}])' for dt in range(4)]
     ins += [f'[lanek{n}] "v"(lane_kb[{n}])' for n in range(4)] + [f'[lanev{n}] "v"(lane_vb[{n}])' for n in range(4)]
     ins += ['[lane16] "v"(lane16)', '[arow] "v"(arow_u)', '[lim0] "v"(lim)', '[slack] "s"(slack)', '[pklo] "s"(pklo)',
             '[pkhi] "s"(pkhi)', '[pvlo] "s"(pvlo)', '[pvhi] "s"(pvhi)', '[stride] "s"(stride)', '[m0w] "s"(m0w)',
-            '[tabA] "s"(tab_a_w)', '[tabB] "s"(tab_b_w)', '[splo] "s"(sp_lo)', '[maskfrom] "s"(mask_from_u)']
+            '[tabA] "s"(tab_a_w)', '[tabB] "s"(tab_b_w)', '[splo] "s"(sp_lo)', '[maskfrom] "s"(mask_from_u) MORE_IN']
     clob = [f"v{r}" for r in list(range(16, 32)) + list(range(48, 118)) + list(range(150, 182))]
     clob += [f"s{r}" for r in range(40, 64)] + ["vcc", "scc", "memory"]
 
@@ -342,22 +372,25 @@ def operands():
         rows.append(cur[:-len(sep)])
         return " \\\n      ".join(rows)
 
-    return (f"#define WD_LOOP_OPERANDS \\\n    : {wrap(outs)} \\\n    : {wrap(ins)} \\\n    : "
+    return (f"#define WD_LOOP_OPERANDS(MORE_OUT, MORE_IN) \\\n    : {wrap(outs)} \\\n    : {wrap(ins)} \\\n    : "
             + wrap([f'"{c}"' for c in clob]))
 
 
 def main():
     path = sys.argv[1] if len(sys.argv) > 1 else os.path.join(os.path.dirname(os.path.abspath(__file__)),
                                                                "prefill_d256_loop.inc")
-    parts = ["// Generated by gen_prefill_loop_d256.py - do not edit.  The subtile loop of prefill_d256_asm_kernel as",
-             "// inline assembly; the register map and the schedule are described in the generator.", ""]
-    for name in ("bf16", "f16"):
-        lines, stats = loop_text(Types(name))
-        per = {k: v // NSLOT for k, v in sorted(stats.items())}
-        parts.append(f"// {name}: instructions per 32-key subtile: {per}")
-        parts.append(f"#define WD_LOOP_ASM_{name.upper()} \\")
-        parts.append(" \\\n".join(c_string(lines).split("\n")))
-        parts.append("")
+    parts = ["// Generated by gen_prefill_loop_d256.py - do not edit.  The subtile loop of prefill_d256_kernel's assembly",
+             "// instances as inline assembly; the register map and the schedule are described in the generator.", ""]
+    global LO
+    for lo in (False, True):
+        LO = lo
+        for name in ("bf16", "f16"):
+            lines, stats = loop_text(Types(name))
+            per = {k: v // NSLOT for k, v in sorted(stats.items())}
+            parts.append(f"// {name}{', with lower bounds' if lo else ''}: instructions per 32-key subtile: {per}")
+            parts.append(f"#define WD_LOOP_ASM_{name.upper()}{'_LO' if lo else ''} \\")
+            parts.append(" \\\n".join(c_string(lines).split("\n")))
+            parts.append("")
     parts.append(operands())
     parts.append("")
     with open(path, "w") as f:

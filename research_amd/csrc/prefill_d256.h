@@ -19,8 +19,11 @@
 // stage is published, so every wave issues the same number of loads per stage and the waits are plain counts.
 // A group must lie inside one pool block: block sizes that are multiples of 16, or one block per sequence.
 // CHECKED: the instance for block sizes that are not multiples of 16 (one block per sequence), where a sequence's
-// last group can reach past the end of the pool: such a group is fetched lane by lane with clamped rows.  With
-// blocks of a multiple of 16 keys no group can, and the other instance carries neither the test nor that path.
+// last group can reach past the end of the pool: such a group is fetched lane by lane with clamped rows; its
+// subtile loop is compiled code with the instruction order written out and fenced.  With blocks of a multiple of
+// 16 keys no group can reach past the pool, and the subtile loop is scheduled assembly (ASM; prefill_d256_loop.inc,
+// written by gen_prefill_loop_d256.py), in one instance without and one with lower bounds (LO: sliding window,
+// per-row first keys).
 // Every wave runs every subtile of the workgroup, with the masks applied where needed: a wave past its last
 // visible key multiplies exact zeros.
 #pragma once
@@ -34,7 +37,7 @@ constexpr int kWdStages = 4;
 constexpr int kWdTasks = kPfWaves;   // tasks (32 query rows of one head) per workgroup: one per wave
 constexpr int kWdCapGroups = 6144;   // 16-key groups the slot tables hold: contexts of up to 98304 keys
 
-template <typename T, bool CHECKED, bool ASM>
+template <typename T, bool CHECKED, bool ASM, bool LO>
 __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
@@ -202,7 +205,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             }
         }
     };
-    auto stage_ofs = [&](int s) PF_INLINE { return (uint32_t)(s & (kWdStages - 1)) * STAGE; };
+    // (ring slots are counted from the workgroup's first tile: the assembly loop starts in slot 0)
+    auto stage_ofs = [&](int s) PF_INLINE { return (uint32_t)((s - t0) & (kWdStages - 1)) * STAGE; };
     auto issue_k = [&](int s) PF_INLINE { issue_rows(pool_k, lane_k, 15, s + 1, stage_ofs(s) + wave_rows); };
     auto issue_v = [&](int s) PF_INLINE { issue_rows(pool_v, lane_v, 3, s, stage_ofs(s) + TENSOR + wave_rows); };
     // The same inside the loop, trimmed: the two table entries are read one subtile ahead (pre_k, pre_v), and the
@@ -454,16 +458,21 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         PF_FENCE();
     };
     if constexpr (ASM) {
-        // The subtile loop as scheduled assembly (prefill_d256_loop.inc): no lower bounds, so the workgroup starts
-        // at tile 0 and every row has seen key 0.  S^T of the first subtile becomes relative to its row maximum,
-        // which is the reference from here on; the loop takes the first half of the first V^T operands read.
+        // The subtile loop as scheduled assembly (prefill_d256_loop.inc).  S^T of the first subtile becomes relative
+        // to its row maximum, which is the reference from here on.  Without lower bounds every row has seen key
+        // 0; with them a row may have seen nothing yet: its reference stays unset (thr = a large negative number
+        // instead of the slack) until a maximum of visible keys arrives (see prefill_asm_kernel).  The loop takes
+        // the first half of the first V^T operands read.
         static_assert(!CHECKED && kWdStages == 4 && kWdKeys == 32 && CAP == 2 * 3072, "the assembly loop is written for this shape");
+        const bool seen = mx > kNegBig;
+        const float m0 = seen ? mx : 0.f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            sb[0][i] -= mx;
-            ref[i] = -mx;
+            sb[0][i] -= m0;
+            ref[i] = -m0;
         }
-        mx = 0.f;
+        if (seen) mx = 0.f;
+        float thr = seen ? kPfSlack : kNegBig;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) read_v_one(t0, 0, dt, va0[dt]);
         f32x16 &sb0 = sb[0];
@@ -471,6 +480,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         int n_left = uni(n_tiles - t0 - 1);  // tiles after the current one
         uint32_t s_t = (uint32_t)uni(t0 + 4), s_p = (uint32_t)uni(t0 + 1);
         int s_rem = uni(mask_from - kWdKeys * t0);
+        int s_lo = uni(lo_mask_until - kWdKeys * t0);
         const uint32_t tab_a_w = lds_base + kRingBytes + 4 * wave_group;
         const uint32_t tab_b_w = lds_base + kRingBytes + kTabEntries * 4 + wave_group;
         const uint32_t sp_lo = (uint32_t)uni(max(first_special - 1, 0)), mask_from_u = (uint32_t)uni(mask_from);
@@ -484,12 +494,28 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         const uint32_t pklo = uni((uint32_t)pk), pkhi = uni((uint32_t)(pk >> 32));
         const uint32_t pvlo = uni((uint32_t)pv), pvhi = uni((uint32_t)(pv >> 32));
         const uint32_t stride = (uint32_t)tok_stride;
-        const float slack = kPfSlack;
-        if constexpr (std::is_same<T, pa_bf16>::value) {
-            asm volatile(WD_LOOP_ASM_BF16 WD_LOOP_OPERANDS);
+        const float slack = kPfSlack, neg_big = kNegBig;
+#define WD_NOTHING
+#define WD_LO_OUT , [thr0] "+&v"(thr), [slo] "+&s"(s_lo)
+#define WD_LO_IN , [lo0] "v"(lo_lim), [negbig] "s"(neg_big)
+        constexpr bool BF = std::is_same<T, pa_bf16>::value;
+        if constexpr (LO) {
+            if constexpr (BF) {
+                asm volatile(WD_LOOP_ASM_BF16_LO WD_LOOP_OPERANDS(WD_LO_OUT, WD_LO_IN));
+            } else {
+                asm volatile(WD_LOOP_ASM_F16_LO WD_LOOP_OPERANDS(WD_LO_OUT, WD_LO_IN));
+            }
         } else {
-            asm volatile(WD_LOOP_ASM_F16 WD_LOOP_OPERANDS);
+            (void)thr; (void)s_lo; (void)neg_big;
+            if constexpr (BF) {
+                asm volatile(WD_LOOP_ASM_BF16 WD_LOOP_OPERANDS(WD_NOTHING, WD_NOTHING));
+            } else {
+                asm volatile(WD_LOOP_ASM_F16 WD_LOOP_OPERANDS(WD_NOTHING, WD_NOTHING));
+            }
         }
+#undef WD_NOTHING
+#undef WD_LO_OUT
+#undef WD_LO_IN
     } else {
         for (int g = t0; g < n_tiles; g += 2) {
             subtile(g, PfBool<false>{});
