@@ -8,7 +8,7 @@ JSON line; with the default workload the line also carries short runs of the
 other configurations (c2, c5 decode, c3 append + chunked prefill) under
 ``secondary``.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1|c3|c3-d256|engine] [--no-secondary]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1|c3|c3-d256|c3-d64|engine] [--no-secondary]
     python bench.py --traffic-from-pmc NAME KERNEL FETCH.csv WRITE.csv   # refresh profiles/traffic.json
 """
 
@@ -89,7 +89,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c3-d256", "c4", "c5", "engine"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c3-d256", "c3-d64", "c4", "c5", "engine"])
     ap.add_argument("--preheat-s", type=float, default=0.5,
                     help="seconds of untimed steps before the warmup steps: an idle GPU sits at its lowest clocks "
                          "and takes a few hundred milliseconds of work to leave them")
@@ -315,13 +315,20 @@ def bench_prefill_c3(args, dev) -> dict:
     return result
 
 
-def bench_prefill_d256(args, dev) -> dict:
-    """The c3 shape with 16 query / 8 kv heads of 256 (32 x (2048 shared + 256 own) tokens, 16-token blocks,
-    bf16): the chunked-prefill kernel for that head size alone, against the bf16 matrix-core peak."""
+# the c3 shape at other head sizes: workload -> (query heads, kv heads, head_dim, seed, kernel)
+PREFILL_HEAD_SHAPES = {"c3-d256": (16, 8, 256, 1006, "prefill_d256_kernel"),
+                       "c3-d64": (32, 8, 64, 1007, "prefill_asm_kernel")}
+
+
+def bench_prefill_head(args, dev, name) -> dict:
+    """The c3 shape (32 x (2048 shared + 256 own) tokens, 16-token blocks, bf16) with 16 query / 8 kv heads of 256
+    or 32 query / 8 kv heads of 64: the chunked-prefill kernel for that head size alone, against the bf16
+    matrix-core peak."""
     from research_amd import ops
     from research_amd.workloads import make_prefill_c3
 
-    w = make_prefill_c3(num_q_heads=16, num_kv_heads=8, head_dim=256, seed=1006)
+    hq, hkv, head_dim, seed, kernel = PREFILL_HEAD_SHAPES[name]
+    w = make_prefill_c3(num_q_heads=hq, num_kv_heads=hkv, head_dim=head_dim, seed=seed)
     S, C, P = w.num_seqs, w.chunk_len, w.prefix_len
     shape = (w.num_blocks * w.block_size, w.num_kv_heads, w.head_dim)
     kc = torch.zeros(shape, dtype=w.dtype, device=dev)
@@ -357,13 +364,13 @@ def bench_prefill_d256(args, dev) -> dict:
         "tokens_per_s": S * C / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_median": ms_step_median,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": "c3 shape at head_dim 256: chunked prefill, 32 x (2048 + 256), 16 q / 8 kv heads, bf16",
+        "config": {"workload": f"c3 shape at head_dim {head_dim}: chunked prefill, 32 x (2048 + 256), {hq} q / {hkv} kv heads, bf16",
                    "num_seqs": S, "prefix_len": P, "chunk_len": C, "num_q_heads": w.num_q_heads,
                    "num_kv_heads": w.num_kv_heads, "head_dim": w.head_dim, "block_size": w.block_size,
-                   "attention_flops": flops, "seed": 1006},
-        "roofline": {"bound": "mfma", "kernel": "prefill_d256_kernel", "achieved": achieved,
+                   "attention_flops": flops, "seed": seed},
+        "roofline": {"bound": "mfma", "kernel": kernel, "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
-                     "traffic": measured_traffic("c3-d256"), "kernel_ms": ms_kernel,
+                     "traffic": measured_traffic(name), "kernel_ms": ms_kernel,
                      "kernel_launches": max(args.steps, KERNEL_LAUNCHES)},
     }
 
@@ -598,8 +605,8 @@ def secondary(args, dev) -> dict:
     short.copy_calibration = False
     short.secondary_run = True
     out = {}
-    for name in ("c2", "c5", "c3", "c3-d256"):
-        r = (bench_prefill_c3(short, dev) if name == "c3" else bench_prefill_d256(short, dev) if name == "c3-d256"
+    for name in ("c2", "c5", "c3", "c3-d256", "c3-d64"):
+        r = (bench_prefill_c3(short, dev) if name == "c3" else bench_prefill_head(short, dev, name) if name in PREFILL_HEAD_SHAPES
              else bench_decode(name, short, dev))
         keep = ("metric", "value", "unit", "ms_per_step", "ms_per_step_median", "steps", "warmup", "tokens_per_s",
                 "dtype", "roofline", "cpu_baseline", "append", "pct_of_hbm_peak")
@@ -627,8 +634,8 @@ def main() -> int:
     torch.cuda.set_device(dev)
     if args.workload == "engine":
         return bench_engine(args, dev)
-    if args.workload == "c3-d256":
-        result = bench_prefill_d256(args, dev)
+    if args.workload in PREFILL_HEAD_SHAPES:
+        result = bench_prefill_head(args, dev, args.workload)
     else:
         result = bench_prefill_c3(args, dev) if args.workload == "c3" else bench_decode(args.workload, args, dev)
     if args.workload == "c4" and not args.no_secondary:
