@@ -330,6 +330,29 @@ def test_assembly_loop_kernel_dense_rows_of_any_length(dtype, d):
 
 
 @pytest.mark.parametrize("d", [64, 128, 256])
+def test_one_short_block_per_sequence_and_a_longer_context(d):
+    """One block per sequence that is not a multiple of 16 keys long, with contexts that run past it (the keys
+    behind the block are absent: zero rows, as in the vector kernel, which states that rule) and chunks that do
+    not start at key 0; the last sequence's block ends the pool.  Matrix-core kernels against the vector kernel."""
+    announce(f"prefill, one short block per sequence d={d}")
+    rng = np.random.default_rng(81 + d)
+    hq, hkv = 4, 2
+    for bs, ctx, chunk in ((33, [40, 33, 20], [40, 10, 20]), (100, [130, 100, 7], [60, 100, 7]), (17, [17, 30], [17, 30])):
+        b = len(ctx)
+        cmax = max(chunk)
+        kc = torch.from_numpy(rng.standard_normal((b * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+        vc = torch.from_numpy(rng.standard_normal((b * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+        q = torch.from_numpy(rng.standard_normal((b * cmax, hq, d)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+        ident = torch.from_numpy(rng.permutation(b).astype(np.int32)).reshape(b, 1).contiguous().to(DEV)
+        args = (q, kc, vc, ident, _i32(ctx), _i32(chunk), _i32(np.arange(b) * cmax), cmax, bs, d ** -0.5)
+        for window in (0, 12):
+            got = ops.prefill_paged(*args, window=window).float().cpu().reshape(b, cmax, hq, d)
+            want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu().reshape(b, cmax, hq, d)
+            for i, c in enumerate(chunk):
+                assert_close(got[i, :c], want[i, :c], 2e-2, f"block_size {bs} sequence {i} window {window}")
+
+
+@pytest.mark.parametrize("d", [64, 128, 256])
 def test_logits_that_grow_along_the_context(d):
     """Keys whose logits rise steeply with the key index (about 9 in base-2 units per 32 keys, from far below
     zero to far above), so that every row's reference maximum is outgrown by more than the lazy-rescale slack
