@@ -879,7 +879,7 @@ struct KernelSet {
 };
 
 template <typename KV, typename QT, int D> KernelSet kernels_for_d(int nrep_t) {
-    constexpr int U = sizeof(KV) == 1 ? 4 : 8;
+    constexpr int U = sizeof(KV) == 1 && D == 32 ? 4 : 8;  // token steps in flight per wave (the fp8 pools' generic loop at head_dim 32 would spill with 8)
     KernelSet k;
     switch (nrep_t) {
     case 1: k.reduce = decode_reduce_kernel<QT, D, 1>; k.reduce_wave = decode_reduce_wave_kernel<QT, D, 1>; k.split = decode_split_kernel<KV, QT, D, 1, U>; k.rowwise = prefill_rowwise_kernel<KV, QT, D, 1, U>; break;
