@@ -177,7 +177,7 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     if ((phases & kPhaseReduce) && !a.merge_in_split) {
         // Many rows and therefore few pieces per sequence: one wave per row.
         const int64_t rows = (int64_t)batch * num_q_heads;
-        if (rows >= 4 * (int64_t)grid)
+        if (rows >= 2 * (int64_t)grid)
             ks.reduce_wave<<<dim3((unsigned)((rows + kWaves - 1) / kWaves)), dim3(kThreads), 0, s>>>(a);
         else
             ks.reduce<<<dim3((unsigned)rows), dim3(kThreads), 0, s>>>(a);
