@@ -316,6 +316,10 @@ def test_decode_step_in_a_hip_graph():
     (6, 2, 64, "bf16"),    # two kv heads of D=64: 4 tokens per load
     (8, 1, 128, "fp8"),    # fp8 rows of 8 lanes, 8 tokens per load, two blocks per iteration
     (4, 1, 256, "fp8"),
+    (8, 2, 128, "fp8"),    # 4 tokens per load: the eight steps in flight come from two blocks
+    (8, 4, 128, "fp8"),    # 2 tokens per load: eight steps are one block
+    (4, 2, 64, "fp8"),     # fp8 rows of 4 lanes, 8 tokens per load
+    (32, 8, 128, "fp8"),   # the long-context workload's layout: one token per load, 16 steps per block
 ])
 def test_few_kv_heads_with_blocks_of_16(hq, hkv, d, kv):
     """Layouts whose loop takes several blocks per iteration: ragged lengths around block and iteration
