@@ -138,11 +138,9 @@ class Types:
             self.ones = "0x3c003c00"
 
     def pack(self, dst, a, b):
-        if self.name == "bf16":
-            return [Ins(f"v_cvt_pk_bf16_f32 v{dst}, v{a}, v{b}", reads=(f"v{a}", f"v{b}"), writes=(f"v{dst}",))]
-        return [Ins(f"v_cvt_f16_f32_e32 v{a}, v{a}", reads=(f"v{a}",), writes=(f"v{a}",)),
-                Ins(f"v_cvt_f16_f32_e32 v{b}, v{b}", reads=(f"v{b}",), writes=(f"v{b}",)),
-                Ins(f"v_pack_b32_f16 v{dst}, v{a}, v{b}", reads=(f"v{a}", f"v{b}"), writes=(f"v{dst}",))]
+        # (gfx950 converts a pair to either 16-bit type in one instruction, round to nearest even)
+        op = "v_cvt_pk_bf16_f32" if self.name == "bf16" else "v_cvt_pk_f16_f32"
+        return [Ins(f"{op} v{dst}, v{a}, v{b}", reads=(f"v{a}", f"v{b}"), writes=(f"v{dst}",))]
 
 
 def k_addr(stage, ks):
