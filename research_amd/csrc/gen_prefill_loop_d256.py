@@ -267,6 +267,30 @@ def fixup():
                     "s_and_saveexec_b64 s[52:53], vcc",
                     f"ds_write_b128 v99, v[112:115] offset:{n * 2 * RB + ofs}",
                     "s_mov_b64 exec, s[52:53]"]
+    # The one 16-key group of a workgroup that reaches past the end of the pool (blocks that are not multiples of
+    # 16 keys long: the last rows of the pool's last block): its direct loads fetched 16 rows from slot 0 instead,
+    # and the rows of it that exist are copied here, lane by lane, from where they are - as K when the stage
+    # holds its tile's K (tile sP+1), as V when it holds its V (tile sP).  edgetile = its tile for the waves that
+    # load its rows (no tile for the others), edgeslot = its first row, edgerows = how many exist.
+    # (v72..v75 are not used by the loop.)
+    for name, tile_ofs, lanes, ofs in (("k", 1, "lanek", 0), ("v", 0, "lanev", TENSOR)):
+        out += [f"s_add_u32 s56, %[sP], {tile_ofs}",
+                "s_cmp_lg_u32 s56, %[edgetile]",
+                f"s_cbranch_scc1 .Lwd_noedge_{name}_%=",
+                "s_mul_i32 s44, %[edgeslot], %[stride]",
+                "s_mul_hi_u32 s45, %[edgeslot], %[stride]",
+                f"s_add_u32 s46, %[p{name}lo], s44",
+                f"s_addc_u32 s47, %[p{name}hi], s45"]
+        for n in range(4):
+            out += [f"v_add_u32_e32 v92, {2 * n}, %[arow]",
+                    "v_cmp_gt_u32_e32 vcc, %[edgerows], v92",
+                    "s_nop 1",
+                    "s_and_saveexec_b64 s[52:53], vcc",
+                    f"global_load_dwordx4 v[72:75], %[{lanes}{n}], s[46:47] offset:{1024 * n}",
+                    "s_waitcnt vmcnt(0)",
+                    f"ds_write_b128 v99, v[72:75] offset:{n * 2 * RB + ofs}",
+                    "s_mov_b64 exec, s[52:53]"]
+        out.append(f".Lwd_noedge_{name}_%=:")
     out += ["s_waitcnt lgkmcnt(0)", "s_setpc_b64 s[50:51]"]
     return out
 
@@ -358,7 +382,8 @@ def operands():
     ins += [f'[lanek{n}] "v"(lane_kb[{n}])' for n in range(4)] + [f'[lanev{n}] "v"(lane_vb[{n}])' for n in range(4)]
     ins += ['[lane16] "v"(lane16)', '[arow] "v"(arow_u)', '[lim0] "v"(lim)', '[slack] "s"(slack)', '[pklo] "s"(pklo)',
             '[pkhi] "s"(pkhi)', '[pvlo] "s"(pvlo)', '[pvhi] "s"(pvhi)', '[stride] "s"(stride)', '[m0w] "s"(m0w)',
-            '[tabA] "s"(tab_a_w)', '[tabB] "s"(tab_b_w)', '[splo] "s"(sp_lo)', '[maskfrom] "s"(mask_from_u) MORE_IN']
+            '[tabA] "s"(tab_a_w)', '[tabB] "s"(tab_b_w)', '[splo] "s"(sp_lo)', '[maskfrom] "s"(mask_from_u)',
+            '[edgetile] "s"(edge_tile_u)', '[edgeslot] "s"(edge_slot_u)', '[edgerows] "s"(edge_rows_u) MORE_IN']
     clob = [f"v{r}" for r in list(range(16, 32)) + list(range(48, 118)) + list(range(150, 182))]
     clob += [f"s{r}" for r in range(40, 64)] + ["vcc", "scc", "memory"]
 

@@ -65,7 +65,8 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     int tasks_per_wg = kPfTasks;
     if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) && num_blocks > 0 &&
         num_blocks * (int64_t)block_size < (1ll << 31) && bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16) {
-        mfma = pa_prefill_d256_kernel(dtype, block_size % 16 != 0, window > 0 || row_first_key != nullptr);
+        // (a pool of fewer than 16 rows has no slot a whole group could be loaded from: the compiled instance)
+        mfma = pa_prefill_d256_kernel(dtype, num_blocks * (int64_t)block_size < 16, window > 0 || row_first_key != nullptr);
         tasks_per_wg = kWdTasks;
     }
     if (mfma) {

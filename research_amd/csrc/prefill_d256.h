@@ -119,7 +119,24 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         }
     }
     // ---- slot tables (in flight together with the Q rows) ----
-    const int64_t pool_rows = p.num_blocks * p.bs;  // < 2^31 (the host checks)
+    const int64_t pool_rows = p.num_blocks * p.bs;  // >= 16, < 2^31 (the host checks)
+    // Blocks that are not multiples of 16 keys long (one block per sequence): the last 16-key group of the pool's
+    // last block would be loaded from past the end of the pool.  The assembly instances load that one group (at
+    // most one per workgroup) from slot 0 instead and copy its existing rows from where they are, lane by lane,
+    // when the stages that hold it are published (see prefill_asm_kernel).
+    int edge_tile = -1, edge_group = 0, edge_rows = 0;
+    int64_t edge_slot = 0;
+    if (ASM && p.bs % 16 != 0) {  // (then bt_stride is 1)
+        const int64_t bid = p.bt[(int64_t)b * p.bt_stride];
+        const int n_keys = min(ctx_len, p.bs);
+        const int key_last = (n_keys - 1) / 16 * 16;
+        if (bid >= 0 && bid < p.num_blocks && bid * p.bs + key_last + 16 > pool_rows) {
+            edge_tile = key_last / kWdKeys;
+            edge_group = key_last / 16 % 2;
+            edge_rows = n_keys - key_last;
+            edge_slot = bid * p.bs + key_last;
+        }
+    }
     // (entries of kLookahead tiles past the workgroup's last one follow as groups of which nothing exists: the
     // loads run that far ahead and past the end, so that every wave issues the same loads per stage)
     constexpr int kLookahead = 6;
@@ -135,7 +152,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             // rows of the group that exist: inside the context and inside the group's block (a block that is not
             // a multiple of 16 keys long is the only block of its sequence: what follows it is absent)
             const int rows = present ? min(min(max(ctx_len - key, 0), 16), (blk + 1) * p.bs - key) : 0;
-            tab_a[i] = present ? (int32_t)(bid * p.bs + key % p.bs) : 0;
+            int64_t slot = present ? bid * p.bs + key % p.bs : 0;
+            if (ASM && slot + 16 > pool_rows) slot = 0;  // (the group at the end of the pool: see edge_tile below)
+            tab_a[i] = (int32_t)slot;
             tab_b[i] = (uint8_t)rows;
             if (rows < 16) first_special = min(first_special, i / 2);
         }
@@ -236,8 +255,23 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         for (int n = 0; n < NL; ++n)
             if (arow0 + 2 * n >= rows) *reinterpret_cast<uint4 *>(s_mem + dst + n * 2 * RB + lane * 16) = uint4{0, 0, 0, 0};
     };
-    auto fix_k = [&](int s) PF_INLINE { if (s + 1 >= first_special) clear_rows(s + 1, stage_ofs(s) + wave_rows); };
-    auto fix_v = [&](int s) PF_INLINE { if (s >= first_special) clear_rows(s, stage_ofs(s) + TENSOR + wave_rows); };
+    // the rows of the group at the end of the pool that this wave holds, copied from where they are
+    auto edge_copy = [&](const char *pool, const uint32_t (&lane_ofs)[NL], uint32_t dst) PF_INLINE {
+        if (wave_group != edge_group) return;
+#pragma unroll
+        for (int n = 0; n < NL; ++n)
+            if (arow0 + 2 * n < edge_rows)
+                *reinterpret_cast<uint4 *>(s_mem + dst + n * 2 * RB + lane * 16) =
+                    *reinterpret_cast<const uint4 *>(pool + edge_slot * tok_stride + lane_ofs[n]);
+    };
+    auto fix_k = [&](int s) PF_INLINE {
+        if (s + 1 >= first_special) clear_rows(s + 1, stage_ofs(s) + wave_rows);
+        if (ASM && s + 1 == edge_tile) edge_copy(pool_k, lane_k, stage_ofs(s) + wave_rows);
+    };
+    auto fix_v = [&](int s) PF_INLINE {
+        if (s >= first_special) clear_rows(s, stage_ofs(s) + TENSOR + wave_rows);
+        if (ASM && s == edge_tile) edge_copy(pool_v, lane_v, stage_ofs(s) + TENSOR + wave_rows);
+    };
 
     // ---- per-lane byte offsets of the operand reads inside a stage ----
     // K operand of k-step ks: key row `col`, chunk 2*ks + half; k-steps 8..15 are 256 bytes behind 0..7
@@ -494,6 +528,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         const uint32_t pklo = uni((uint32_t)pk), pkhi = uni((uint32_t)(pk >> 32));
         const uint32_t pvlo = uni((uint32_t)pv), pvhi = uni((uint32_t)(pv >> 32));
         const uint32_t stride = (uint32_t)tok_stride;
+        // (only the waves that load rows of the group at the end of the pool see its tile)
+        const uint32_t edge_tile_u = (uint32_t)uni(wave_group == edge_group ? edge_tile : -1);
+        const uint32_t edge_slot_u = (uint32_t)uni((int)edge_slot), edge_rows_u = (uint32_t)uni(edge_rows);
         const float slack = kPfSlack, neg_big = kNegBig;
 #define WD_NOTHING
 #define WD_LO_OUT , [thr0] "+&v"(thr), [slo] "+&s"(s_lo)
