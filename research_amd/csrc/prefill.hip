@@ -5,7 +5,7 @@ namespace pa_decode_detail {
 constexpr int kPaCapTiles = 1600;  // (prefill_asm.h)
 prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds);
 constexpr int kWdTasks = 4, kWdCapGroups = 6144;  // (prefill_d256.h)
-prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked, bool lower_bounds);
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool lower_bounds);
 }
 
 using namespace pa_decode_detail;
@@ -63,10 +63,11 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // head_dim 256: one 32-row task per wave, loads driven by a table of 16-key groups - which must lie inside one
     // pool block (block sizes that are multiples of 16, or a single block per sequence) - that LDS can hold
     int tasks_per_wg = kPfTasks;
-    if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) && num_blocks > 0 &&
-        num_blocks * (int64_t)block_size < (1ll << 31) && bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16) {
-        // (a pool of fewer than 16 rows has no slot a whole group could be loaded from: the compiled instance)
-        mfma = pa_prefill_d256_kernel(dtype, num_blocks * (int64_t)block_size < 16, window > 0 || row_first_key != nullptr);
+    // (a pool of fewer than 16 rows has no slot a whole group could be loaded from: the vector kernel)
+    if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) &&
+        num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
+        bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16) {
+        mfma = pa_prefill_d256_kernel(dtype, window > 0 || row_first_key != nullptr);
         tasks_per_wg = kWdTasks;
     }
     if (mfma) {

@@ -17,13 +17,14 @@
 // up once per workgroup and kept in LDS behind the ring (with the number of rows of the group that exist); rows
 // past the context end or in absent blocks are fetched from a slot that exists and cleared in LDS before the
 // stage is published, so every wave issues the same number of loads per stage and the waits are plain counts.
-// A group must lie inside one pool block: block sizes that are multiples of 16, or one block per sequence.
-// CHECKED: the instance for block sizes that are not multiples of 16 (one block per sequence), where a sequence's
-// last group can reach past the end of the pool: such a group is fetched lane by lane with clamped rows; its
-// subtile loop is compiled code with the instruction order written out and fenced.  With blocks of a multiple of
-// 16 keys no group can reach past the pool, and the subtile loop is scheduled assembly (ASM; prefill_d256_loop.inc,
-// written by gen_prefill_loop_d256.py), in one instance without and one with lower bounds (LO: sliding window,
-// per-row first keys).
+// A group must lie inside one pool block: block sizes that are multiples of 16, or one block per sequence of any
+// length (what dense prefill passes).  In the second case a group's load may run into the next block's rows -
+// they are cleared like rows past the context end - and the one group at the end of the pool is fetched lane
+// by lane when the stages that hold it are published.
+//
+// The subtile loop is scheduled assembly (prefill_d256_loop.inc, written by gen_prefill_loop_d256.py), in one
+// instance without and one with lower bounds (LO: sliding window, per-row first keys); the set-up, the first
+// subtile's S^T and the write-out are compiled code.
 // Every wave runs every subtile of the workgroup, with the masks applied where needed: a wave past its last
 // visible key multiplies exact zeros.
 #pragma once
@@ -37,7 +38,7 @@ constexpr int kWdStages = 4;
 constexpr int kWdTasks = kPfWaves;   // tasks (32 query rows of one head) per workgroup: one per wave
 constexpr int kWdCapGroups = 6144;   // 16-key groups the slot tables hold: contexts of up to 98304 keys
 
-template <typename T, bool CHECKED, bool ASM, bool LO>
+template <typename T, bool LO>
 __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
@@ -126,7 +127,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     // when the stages that hold it are published (see prefill_asm_kernel).
     int edge_tile = -1, edge_group = 0, edge_rows = 0;
     int64_t edge_slot = 0;
-    if (ASM && p.bs % 16 != 0) {  // (then bt_stride is 1)
+    if (p.bs % 16 != 0) {  // (then bt_stride is 1)
         const int64_t bid = p.bt[(int64_t)b * p.bt_stride];
         const int n_keys = min(ctx_len, p.bs);
         const int key_last = (n_keys - 1) / 16 * 16;
@@ -153,7 +154,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             // a multiple of 16 keys long is the only block of its sequence: what follows it is absent)
             const int rows = present ? min(min(max(ctx_len - key, 0), 16), (blk + 1) * p.bs - key) : 0;
             int64_t slot = present ? bid * p.bs + key % p.bs : 0;
-            if (ASM && slot + 16 > pool_rows) slot = 0;  // (the group at the end of the pool: see edge_tile below)
+            if (slot + 16 > pool_rows) slot = 0;  // (the group at the end of the pool: see edge_tile below)
             tab_a[i] = (int32_t)slot;
             tab_b[i] = (uint8_t)rows;
             if (rows < 16) first_special = min(first_special, i / 2);
@@ -205,35 +206,20 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     const int wave_group = wave >> 1;
     auto entry_of = [&](int tile) PF_INLINE { return min(2 * tile + wave_group, CAP); };
     // one tensor's rows of one tile into LDS at byte offset `dst` of s_mem (always NL direct loads)
-    auto issue_rows = [&](const char *pool, const uint32_t (&lane_ofs)[NL], int chunk_swz_mask, int tile, uint32_t dst) PF_INLINE {
+    auto issue_rows = [&](const char *pool, const uint32_t (&lane_ofs)[NL], int tile, uint32_t dst) PF_INLINE {
         const int slot = __builtin_amdgcn_readfirstlane(tab_a[entry_of(tile)]);
-        if (!CHECKED || __builtin_expect((int64_t)slot + 16 <= pool_rows, 1)) {
-            const uint64_t ofs = (uint64_t)(uint32_t)slot * (uint32_t)tok_stride;  // 32 x 32 -> 64 bits, scalar
-            const char *base = pf_scalar_ptr(pool + ofs);
+        const uint64_t ofs = (uint64_t)(uint32_t)slot * (uint32_t)tok_stride;  // 32 x 32 -> 64 bits, scalar
+        const char *base = pf_scalar_ptr(pool + ofs);
 #pragma unroll
-            for (int n = 0; n < NL; ++n) pf_dma16(lds_base + dst + n * 2 * RB, base, lane_ofs[n]);
-        } else {
-            // the group reaches past the end of the pool (its last rows do not exist): such lanes fetch the
-            // pool's last row instead; the rows are cleared before the stage is published
-#pragma unroll
-            for (int n = 0; n < NL; ++n) {
-                const int r = arow0 + 2 * n;
-                const int64_t row = min((int64_t)slot + r, pool_rows - 1);
-                const int swz = chunk_swz_mask == 15 ? (r & 15) : (r & 3) * 4;
-                pf_dma16(lds_base + dst + n * 2 * RB, pool + row * tok_stride + ((ld_slot ^ swz) * 16));
-            }
-        }
+        for (int n = 0; n < NL; ++n) pf_dma16(lds_base + dst + n * 2 * RB, base, lane_ofs[n]);
     };
     // (ring slots are counted from the workgroup's first tile: the assembly loop starts in slot 0)
     auto stage_ofs = [&](int s) PF_INLINE { return (uint32_t)((s - t0) & (kWdStages - 1)) * STAGE; };
-    auto issue_k = [&](int s) PF_INLINE { issue_rows(pool_k, lane_k, 15, s + 1, stage_ofs(s) + wave_rows); };
-    auto issue_v = [&](int s) PF_INLINE { issue_rows(pool_v, lane_v, 3, s, stage_ofs(s) + TENSOR + wave_rows); };
-    // The same inside the loop, trimmed: the two table entries are read one subtile ahead (pre_k, pre_v), and the
-    // eight loads of a stage are one block of instructions.  A direct load adds its immediate offset to the LDS
-    // address and to the global address alike, so with the global side compensated in the per-lane offsets the
-    // four loads of a tensor share one LDS base (one write of m0).
-    int pre_k = 0, pre_v = 0;
-    auto prefetch_entries = [&](int s) PF_INLINE { pre_k = tab_a[entry_of(s + 1)]; pre_v = tab_a[entry_of(s)]; };
+    auto issue_k = [&](int s) PF_INLINE { issue_rows(pool_k, lane_k, s + 1, stage_ofs(s) + wave_rows); };
+    auto issue_v = [&](int s) PF_INLINE { issue_rows(pool_v, lane_v, s, stage_ofs(s) + TENSOR + wave_rows); };
+    // The loop's loads: a direct load adds its immediate offset to the LDS address and to the global address alike,
+    // so with the global side compensated in the per-lane offsets the four loads of a tensor share one LDS base
+    // (one write of m0).
     uint32_t lane_kb[NL], lane_vb[NL];
 #pragma unroll
     for (int n = 0; n < NL; ++n) {
@@ -241,13 +227,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         lane_vb[n] = lane_v[n] + (NL - 1 - n) * 2 * RB;
     }
     const char *pool_kb = pool_k - (NL - 1) * 2 * RB, *pool_vb = pool_v - (NL - 1) * 2 * RB;
-    const int slot_max = (int)max(pool_rows - 16, (int64_t)-1);  // last slot a whole group can start at
-    auto dma_one = [&](uint32_t dst, const char *base, uint32_t lane_ofs, int n) PF_INLINE {
-        if (n == 0) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:0" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
-        if (n == 1) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:1024" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
-        if (n == 2) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:2048" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
-        if (n == 3) asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %1 offset:3072" : : "s"(dst), "s"(base), "v"(lane_ofs) : "memory", "m0");
-    };
     // clear the rows this wave loaded that do not exist (after its loads have landed, before the barrier)
     auto clear_rows = [&](int tile, uint32_t dst) PF_INLINE {
         const int rows = tab_b[entry_of(tile)];
@@ -266,11 +245,11 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     };
     auto fix_k = [&](int s) PF_INLINE {
         if (s + 1 >= first_special) clear_rows(s + 1, stage_ofs(s) + wave_rows);
-        if (ASM && s + 1 == edge_tile) edge_copy(pool_k, lane_k, stage_ofs(s) + wave_rows);
+        if (s + 1 == edge_tile) edge_copy(pool_k, lane_k, stage_ofs(s) + wave_rows);
     };
     auto fix_v = [&](int s) PF_INLINE {
         if (s >= first_special) clear_rows(s, stage_ofs(s) + TENSOR + wave_rows);
-        if (ASM && s == edge_tile) edge_copy(pool_v, lane_v, stage_ofs(s) + TENSOR + wave_rows);
+        if (s == edge_tile) edge_copy(pool_v, lane_v, stage_ofs(s) + TENSOR + wave_rows);
     };
 
     // ---- per-lane byte offsets of the operand reads inside a stage ----
@@ -295,24 +274,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
                                                 (const lds_char *)(size_t)adr + (ks >> 3) * 256));
         }
     };
-    auto read_v = [&](int s, int step, X8 (&va)[DT]) PF_INLINE {  // V^T of keys 16*step .. +16 of tile s
-        const uint32_t base = lds_base + stage_ofs(s);
-#pragma unroll
-        for (int dt = 0; dt < DT; ++dt) {
-            const lds_char *at = (const lds_char *)(size_t)(base + v_ofs[dt & 3]) + (dt >> 2) * 256 + 16 * step * RB;
-            const X4 lo = __builtin_bit_cast(X4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((pa_s16x4 __attribute__((address_space(3))) *)at));
-            const X4 hi = __builtin_bit_cast(
-                X4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((pa_s16x4 __attribute__((address_space(3))) *)(at + 8 * RB)));
-#pragma unroll
-            for (int e = 0; e < 4; ++e) { va[dt][e] = lo[e]; va[dt][4 + e] = hi[e]; }
-        }
-    };
-    // the same reads one operand at a time (the loop spreads them between the products)
-    auto read_k_one = [&](int s, int ks, X8 &dst) PF_INLINE {
-        const uint32_t adr = lds_base + stage_ofs(s) + k_ofs[ks & 7];
-        dst = __builtin_bit_cast(X8, *reinterpret_cast<const __attribute__((address_space(3))) uint4 *>(
-                                         (const lds_char *)(size_t)adr + (ks >> 3) * 256));
-    };
+    // V^T of keys 16*step .. +16 of tile s, d tile dt (two transposing reads)
     auto read_v_one = [&](int s, int step, int dt, X8 &dst) PF_INLINE {
         const lds_char *at = (const lds_char *)(size_t)(lds_base + stage_ofs(s) + v_ofs[dt & 3]) + (dt >> 2) * 256 + 16 * step * RB;
         const X4 lo = __builtin_bit_cast(X4, __builtin_amdgcn_ds_read_tr16_b64_v4i16((pa_s16x4 __attribute__((address_space(3))) *)at));
@@ -368,148 +330,50 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         for (int i = 0; i < 16; ++i) o[dt][i] = 0.f;
     // S^T is kept relative to the row's reference maximum (see prefill_mfma_kernel): the first product of a
     // subtile accumulates onto ref = minus the reference in all 16 registers, the exponentials take S^T as it
-    // is, mx is relative too; m_thr is what mx must exceed for a rescale (kNegBig until the row has seen a key).
+    // is, mx is relative too.
     f32x16 ref;
 #pragma unroll
     for (int i = 0; i < 16; ++i) ref[i] = 0.f;
-    float m_thr = kNegBig, l_run = 0.f, mx = kNegBig;
-    X8 ka[KS], va0[DT], va1[DT];
-    f32x16 sb[2];  // S^T of the current and of the next subtile, swapping roles every subtile
+    float l_run = 0.f, mx = kNegBig;
+    X8 ka[KS], va0[DT / 2];
+    f32x16 sb0;  // S^T of the first subtile
 
     // ---- first subtile: S^T, mask, row maximum; K operands of the second; V^T of the first k-step ----
     read_k(t0 - 1, ka);
     PF_FENCE();
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) sb[0] = M::mma(ka[ks], qreg[ks], ks == 0 ? ref : sb[0]);
+    for (int ks = 0; ks < KS; ++ks) sb0 = M::mma(ka[ks], qreg[ks], ks == 0 ? ref : sb0);
     PF_FENCE();
     read_k(t0, ka);
     PF_FENCE();
-    if (32 * (t0 + 1) > mask_from || 32 * t0 < lo_mask_until) mask_s(sb[0], 32 * t0);
-    max_piece(sb[0], 0, mx);
-    max_piece(sb[0], 1, mx);
+    if (32 * (t0 + 1) > mask_from || 32 * t0 < lo_mask_until) mask_s(sb0, 32 * t0);
+    max_piece(sb0, 0, mx);
+    max_piece(sb0, 1, mx);
     PF_FENCE();
     // every wave has read K of tile t0: its slot takes stage t0+3
     __builtin_amdgcn_s_waitcnt((15) | (7 << 4) | (0 << 8) | (3 << 14));  // lgkmcnt(0)
     __syncthreads();
     issue_k(t0 + 3); issue_v(t0 + 3);
-    prefetch_entries(t0 + 4);
     PF_FENCE();
 
-    // One subtile g (= tile g, stage g); PAR = parity of g - t0: which S^T buffer is the current one.
-    auto subtile = [&](int g, auto par_tag) PF_INLINE {
-        constexpr int PAR = decltype(par_tag)::value ? 1 : 0;
-        f32x16 &s = sb[PAR];
-        f32x16 &s_nx = sb[PAR ^ 1];
-        const bool mask_next = 32 * (g + 2) > mask_from || 32 * (g + 1) < lo_mask_until;
-        uint32_t pp[8];
-        float sum = 0.f;
-        // exponentials of S^T values 2*j, 2*j+1, packed as a P^T operand word
-        auto exp_piece = [&](int j) PF_INLINE {
-            const float p0 = __builtin_amdgcn_exp2f(s[2 * j]);
-            const float p1 = __builtin_amdgcn_exp2f(s[2 * j + 1]);
-            sum += p0 + p1;
-            uint32_t w = M::pack(p0, p1);
-            asm volatile("" : "+v"(w), "+v"(sum));
-            pp[j] = w;
-        };
-        // ---- the row maximum outgrew its reference by more than the slack (rare): rescale ----
-        if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m_thr) != 0, 0)) {
-            // the reference moves by delta: up to the new maximum, or - for a row that had seen no key so far
-            // (sum and accumulators still zero) - to its first maximum, whatever its sign
-            const bool unset = m_thr == kNegBig;
-            const bool seen = mx > kNegBig;
-            const float delta = unset ? (seen ? mx : 0.f) : fmaxf(mx, 0.f);
-            const float alpha = unset ? 1.f : __builtin_amdgcn_exp2f(-delta);
-            l_run *= alpha;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) o[dt][i] *= alpha;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                ref[i] -= delta;
-                s[i] -= delta;  // formed against the old reference
-            }
-            mx -= delta;
-            if (seen) m_thr = kPfSlack;
-        }
-        PF_FENCE();
-        // ---- (a) S^T of subtile g+1, with the exponentials of subtile g between the products ----
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-            s_nx = M::mma(ka[ks], qreg[ks], ks == 0 ? ref : s_nx);
-            PF_FENCE();
-            // V^T of this subtile: the first k-step's (consumed in (b)) behind the first eight products, the second's
-            // (consumed in (c)) behind the others
-            if (ks < 8) read_v_one(g, 0, ks, va0[ks]);
-            else read_v_one(g, 1, ks - 8, va1[ks - 8]);
-            if (ks & 1) exp_piece(ks >> 1);
-            PF_FENCE();
-        }
-        // ---- publish stage g+1; the loads of stage g+4 go into the slot of stage g (every read of it is done) ----
-        pf_wait_loads<4 * NL>();  // loads in flight, oldest first: stages g+1, g+2, g+3
-        fix_k(g + 1); fix_v(g + 1);
-        __builtin_amdgcn_s_waitcnt((15) | (7 << 4) | (0 << 8) | (3 << 14));  // lgkmcnt(0): this wave's reads of stage g
-        __syncthreads();
-        // the loads of stage g+4, one behind each product of (b); a group that reaches past the end of the pool
-        // takes the per-lane path here instead
-        const int slot_k = __builtin_amdgcn_readfirstlane(pre_k), slot_v = __builtin_amdgcn_readfirstlane(pre_v);
-        const bool fast = !CHECKED || max(slot_k, slot_v) <= slot_max;
-        const uint32_t dst_k = lds_base + stage_ofs(g + 4) + wave_rows, dst_v = dst_k + TENSOR;
-        const char *bk = pf_scalar_ptr(pool_kb + (uint64_t)(uint32_t)slot_k * (uint32_t)tok_stride);
-        const char *bv = pf_scalar_ptr(pool_vb + (uint64_t)(uint32_t)slot_v * (uint32_t)tok_stride);
-        if (CHECKED && __builtin_expect(!fast, 0)) { issue_k(g + 4); issue_v(g + 4); }
-        prefetch_entries(g + 5);
-        PF_FENCE();
-        // ---- (b) O^T += V^T . P^T, first k-step ----
-        {
-            const X8 pb = __builtin_bit_cast(X8, uint4{pp[0], pp[1], pp[2], pp[3]});
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                o[dt] = M::mma(va0[dt], pb, o[dt]);
-                PF_FENCE();
-                if (fast) dma_one(dt < 4 ? dst_k : dst_v, dt < 4 ? bk : bv, dt < 4 ? lane_kb[dt & 3] : lane_vb[dt & 3], dt & 3);
-                read_k_one(g + 1, dt, ka[dt]);  // K of subtile g+2 (k-steps 0..7 here, 8..15 in (c)): consumed in (a) of g+1
-                PF_FENCE();
-            }
-        }
-        if (mask_next) mask_s(s_nx, 32 * (g + 1));
-        PF_FENCE();
-        // ---- (c) second k-step, with the next subtile's row maximum ----
-        {
-            const X8 pb = __builtin_bit_cast(X8, uint4{pp[4], pp[5], pp[6], pp[7]});
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                o[dt] = M::mma(va1[dt], pb, o[dt]);
-                PF_FENCE();
-                read_k_one(g + 1, 8 + dt, ka[8 + dt]);
-                if (dt == 1) max_piece(s_nx, 0, mx);
-                if (dt == 3) max_piece(s_nx, 1, mx);
-                PF_FENCE();
-            }
-        }
-        l_run += sum;
-        PF_FENCE();
-    };
-    if constexpr (ASM) {
+    {
         // The subtile loop as scheduled assembly (prefill_d256_loop.inc).  S^T of the first subtile becomes relative
         // to its row maximum, which is the reference from here on.  Without lower bounds every row has seen key
         // 0; with them a row may have seen nothing yet: its reference stays unset (thr = a large negative number
         // instead of the slack) until a maximum of visible keys arrives (see prefill_asm_kernel).  The loop takes
         // the first half of the first V^T operands read.
-        static_assert(!CHECKED && kWdStages == 4 && kWdKeys == 32 && CAP == 2 * 3072, "the assembly loop is written for this shape");
+        static_assert(kWdStages == 4 && kWdKeys == 32 && CAP == 2 * 3072, "the assembly loop is written for this shape");
         const bool seen = mx > kNegBig;
         const float m0 = seen ? mx : 0.f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            sb[0][i] -= m0;
+            sb0[i] -= m0;
             ref[i] = -m0;
         }
         if (seen) mx = 0.f;
         float thr = seen ? kPfSlack : kNegBig;
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) read_v_one(t0, 0, dt, va0[dt]);
-        f32x16 &sb0 = sb[0];
         auto uni = [](int v) PF_INLINE { return __builtin_amdgcn_readfirstlane(v); };
         int n_left = uni(n_tiles - t0 - 1);  // tiles after the current one
         uint32_t s_t = (uint32_t)uni(t0 + 4), s_p = (uint32_t)uni(t0 + 1);
@@ -553,11 +417,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 #undef WD_NOTHING
 #undef WD_LO_OUT
 #undef WD_LO_IN
-    } else {
-        for (int g = t0; g < n_tiles; g += 2) {
-            subtile(g, PfBool<false>{});
-            if (g + 1 < n_tiles) subtile(g + 1, PfBool<true>{});
-        }
     }
     pf_wait_loads<0>();  // (loads of the stages past the last tile: nothing may arrive after the workgroup has ended)
 
@@ -578,7 +437,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         }
 }
 
-// nullptr unless the element type has this kernel
-prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool checked, bool lower_bounds);
+// nullptr unless the element type has this kernel; `lower_bounds`: the instance for sliding windows and per-row
+// first keys
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool lower_bounds);
 
 }  // namespace pa_decode_detail
