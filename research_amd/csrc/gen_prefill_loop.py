@@ -1,6 +1,6 @@
 #!/usr/bin/env python3
 """Writes prefill_mfma_loop.inc: the tile loop of prefill_asm_kernel as one inline-assembly block per head size
-(128, 64), element type (bf16, fp16) and variant (without / with lower bounds).
+(128, 64, 32), element type (bf16, fp16) and variant (without / with lower bounds).
 
 Why assembly: with one wave per SIMD nothing hides latency except the wave's own instruction order, and a
 wave issues one instruction per 4 cycles (a matrix product takes two issue slots, an exponential two).  At
@@ -25,7 +25,7 @@ wave executes the same barriers and the same number of loads per tile.
 
 Register map (per lane; the kernel pins its variables to the same registers; KS = head_dim / 16 k-steps of
 S^T, DT = head_dim / 32 d tiles of O^T; the ranges are those of head_dim 128, head_dim 64 uses the first half
-of each):
+of each, head_dim 32 the first quarter):
   a[0:127]    O^T accumulators  o[c][dt]   at 16*(DT*c + dt)
   a[128:191]  Q^T operands      q[c][ks]   at 128 + 4*(KS*c + ks)
   a[192:223]  K operands        ka[ks]     at 192 + 4*ks
@@ -50,7 +50,7 @@ X = set(os.environ.get("PF_GEN_X", "").split(","))  # experiment switches
 
 
 def configure(head_dim):
-    """The shape constants of a head size (128 or 64; 16-bit elements)."""
+    """The shape constants of a head size (128, 64 or 32; 16-bit elements)."""
     global D, KS, DT, RB, TENSOR, STAGE, M_A, M_B, GAPS, SYNC_GAP, NG, MAX_GAP
     D = head_dim
     KS, DT = D // 16, D // 32   # k-steps of S^T = K . Q^T, 32-wide d tiles of O^T
@@ -61,7 +61,7 @@ def configure(head_dim):
     GAPS = M_A + 2 * M_B + 1     # places for other instructions around the products of a subtile
     SYNC_GAP = M_A               # where tile t+1 is published in a tile's first subtile
     NG = RB // 64                # direct loads per wave, tile and tensor (a tensor's tile is 64 * RB bytes, a wave load 1 KiB, 4 waves)
-    MAX_GAP = {128: 21, 64: 11}[D]  # first gap of the row maxima (far enough behind the last S^T product)
+    MAX_GAP = {128: 21, 64: 11, 32: 5}[D]  # first gap of the row maxima (far enough behind the last S^T product)
 
 
 configure(128)
@@ -321,10 +321,10 @@ def subtile_ops(ty, j, kt):
         read = "ds_read_b128 v[88:91], v92" if NG == 4 else "ds_read2_b32 v[88:89], v92 offset1:2"
         ldr.append(Op(Ins(read, kind="lds", reads=("v92",), issue="tab"), first))
         for n in range(NG):
-            ldr.append(Op(Ins(f"v_readfirstlane_b32 s{40 + n}, v{88 + n}", reads=(f"v{88 + n}",), need=("tab",)), SYNC_GAP + 6))
+            ldr.append(Op(Ins(f"v_readfirstlane_b32 s{40 + n}, v{88 + n}", reads=(f"v{88 + n}",), need=("tab",)), min(SYNC_GAP + 6, GAPS - 1)))
     groups = range(NG // 2) if kt == 0 else range(NG // 2, NG)
     for n in groups:
-        e = SYNC_GAP + 8 if kt == 0 else 0
+        e = min(SYNC_GAP + 8, GAPS - 1) if kt == 0 else 0
         # slot * row stride (64 bits), then per tensor: LDS destination into m0, pool base + offset, load.  The
         # two additions between the write of m0 and the load are the wait state that write needs.
         ldr.append(Op([Ins(f"s_mul_i32 s44, s{40 + n}, %[stride]", kind="salu"),
@@ -611,11 +611,11 @@ def c_string(lines):
 def main():
     path = sys.argv[1] if len(sys.argv) > 1 else os.path.join(os.path.dirname(os.path.abspath(__file__)),
                                                                "prefill_mfma_loop.inc")
-    parts = ["// Generated by gen_prefill_loop.py - do not edit.  The tile loops of prefill_asm_kernel (head_dim 128 and 64)",
+    parts = ["// Generated by gen_prefill_loop.py - do not edit.  The tile loops of prefill_asm_kernel (head_dim 128, 64, 32)",
              "// as inline assembly; the register map and the schedule are described in the generator.",
              ""]
     global LO
-    for head_dim in (128, 64):
+    for head_dim in (128, 64, 32):
         configure(head_dim)
         for lo in (False, True):
             LO = lo

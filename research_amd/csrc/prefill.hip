@@ -53,10 +53,10 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // (the matrix-core softmax takes the running maximum of the unscaled logits, which needs scale > 0)
     prefill_mfma_fn mfma =
         force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
-    // head_dim 128 or 64, blocks of a multiple of 16 tokens (or one block per sequence, as dense prefill passes its
+    // head_dim 128, 64 or 32, blocks of a multiple of 16 tokens (or one block per sequence, as dense prefill passes its
     // rows) and a table the kernel's LDS copy can hold: the kernel whose whole tile loop is scheduled assembly
     // (one instance without, one with sliding window / per-row first keys)
-    if (mfma && (head_dim == 128 || head_dim == 64) && (block_size % 16 == 0 || bt_stride == 1) &&
+    if (mfma && (head_dim == 128 || head_dim == 64 || head_dim == 32) && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
         bt_stride * (int64_t)block_size <= (int64_t)kPaCapTiles * kPfKeys)
         mfma = pa_prefill_asm_kernel(dtype, head_dim, window > 0 || row_first_key != nullptr);

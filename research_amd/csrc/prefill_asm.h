@@ -1,4 +1,4 @@
-// Causal prefill attention over a paged context for head_dim 128 and 64 (bf16 / fp16) with the whole tile loop in
+// Causal prefill attention over a paged context for head_dim 128, 64 and 32 (bf16 / fp16) with the whole tile loop in
 // scheduled assembly (prefill_mfma_loop.inc, written by gen_prefill_loop.py).
 //
 // Same computation, work split, LDS ring and operand layouts as prefill_mfma_kernel (prefill_mfma.h); what
@@ -6,7 +6,7 @@
 //   * the pool slots of the context's 16-key groups are looked up once per workgroup and kept in LDS behind the
 //     ring (table A: slot of the group's first key; table B: first row of the group that does not exist, 16 =
 //     none), so a tile's loads are a table read, a scalar multiply per group and one direct load per group and
-//     tensor (head_dim 128: eight per wave and tile, head_dim 64: four), for any block size that is a multiple
+//     tensor (head_dim 128: eight per wave and tile, head_dim 64: four, head_dim 32: two), for any block size that is a multiple
 //     of 16;
 //   * rows past the context end and absent blocks are loaded from a slot that exists (the group's own block,
 //     or slot 0) and cleared in LDS before the tile is published; a zero key takes part with logit 0 and a
@@ -37,13 +37,13 @@ template <typename T, bool LO, int D>
 __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
-    static_assert(D == 128 || D == 64, "the assembly loops are generated for these head sizes");
+    static_assert(D == 128 || D == 64 || D == 32, "the assembly loops are generated for these head sizes");
     using G = PfTile<D>;
     constexpr int KS = D / 16, DT = D / 32, NC = kPfCols;
     constexpr int GPT = kPfKeys / 16;  // 16-key groups per tile
     // A wave-wide direct load covers 1 KiB = RPL rows.  head_dim 128: wave w fetches four rows of each of the tile's
     // four groups (NG = 4 loads per tensor: groups 0, 1, 2, 3); head_dim 64: eight rows of two of them (NG = 2:
-    // groups w/2 and w/2 + 2).  Either way load n lands 4 KiB behind load n-1.
+    // groups w/2 and w/2 + 2); head_dim 32: all sixteen rows of group w (NG = 1).  Load n lands 4 KiB behind load n-1.
     constexpr int NG = G::LOADS / kPfWaves, GSTEP = GPT / NG;
     typedef __attribute__((address_space(3))) char lds_char;
     constexpr int kRingBytes = kPfStages * 2 * G::BYTES;
@@ -399,6 +399,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
       "{a[144:147]}"(qreg[1][0]), "{a[148:151]}"(qreg[1][1]), "{a[152:155]}"(qreg[1][2]), "{a[156:159]}"(qreg[1][3]),   \
       [kad0] "v"(kad[0]), [kad1] "v"(kad[1]), [kad2] "v"(kad[2]), [kad3] "v"(kad[3]), [vad0] "v"(vad[0]),               \
       [vad1] "v"(vad[1]), [bshift] "s"(b_shift), PA_LOOP_COMMON_IN(MORE_IN)
+// head_dim 32: o[c][0] at a[16*c], q[c][ks] at a[128 + 4*(2c+ks)], ka[ks] at a[192 + 4*ks]
+#define PA_LOOP_OPERANDS_D32(MORE_OUT, MORE_IN)                                                                       \
+    : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[1][0]), "+{a[192:195]}"(ka[0]), "+{a[196:199]}"(ka[1]),                    \
+      PA_LOOP_COMMON_OUT(MORE_OUT)                                                                                    \
+    : "{a[128:131]}"(qreg[0][0]), "{a[132:135]}"(qreg[0][1]), "{a[136:139]}"(qreg[1][0]), "{a[140:143]}"(qreg[1][1]),   \
+      [kad0] "v"(kad[0]), [kad1] "v"(kad[1]), [vad0] "v"(vad[0]), [bshift] "s"(b_shift), PA_LOOP_COMMON_IN(MORE_IN)
 #define PA_NOTHING
 #define PA_LO_OUT , [thr0] "+&v"(thr[0]), [thr1] "+&v"(thr[1]), [slo] "+&s"(s_lo)
 #define PA_LO_IN , [lo0] "v"(lo[0]), [lo1] "v"(lo[1]), [negbig] "s"(neg_big)
@@ -416,6 +422,21 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
                 asm volatile(PF_LOOP_ASM_BF16 PA_LOOP_OPERANDS(PA_NOTHING, PA_NOTHING));
             } else {
                 asm volatile(PF_LOOP_ASM_F16 PA_LOOP_OPERANDS(PA_NOTHING, PA_NOTHING));
+            }
+        } else if constexpr (D == 32 && LO) {
+            const uint32_t b_shift = (uint32_t)uni(8 * g0);
+            if constexpr (BF) {
+                asm volatile(PF_LOOP_ASM_D32_BF16_LO PA_LOOP_OPERANDS_D32(PA_LO_OUT, PA_LO_IN));
+            } else {
+                asm volatile(PF_LOOP_ASM_D32_F16_LO PA_LOOP_OPERANDS_D32(PA_LO_OUT, PA_LO_IN));
+            }
+        } else if constexpr (D == 32) {
+            (void)s_lo; (void)neg_big;
+            const uint32_t b_shift = (uint32_t)uni(8 * g0);
+            if constexpr (BF) {
+                asm volatile(PF_LOOP_ASM_D32_BF16 PA_LOOP_OPERANDS_D32(PA_NOTHING, PA_NOTHING));
+            } else {
+                asm volatile(PF_LOOP_ASM_D32_F16 PA_LOOP_OPERANDS_D32(PA_NOTHING, PA_NOTHING));
             }
         } else if constexpr (LO) {
             const uint32_t b_shift = (uint32_t)uni(8 * g0);
@@ -435,6 +456,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         }
 #undef PA_LOOP_OPERANDS
 #undef PA_LOOP_OPERANDS_D64
+#undef PA_LOOP_OPERANDS_D32
 #undef PA_LOOP_COMMON_OUT
 #undef PA_LOOP_COMMON_IN
 #undef PA_NOTHING

@@ -1,4 +1,4 @@
-// Instantiates the prefill kernels whose tile loop is scheduled assembly (head_dim 128 and 64; bf16 / fp16).
+// Instantiates the prefill kernels whose tile loop is scheduled assembly (head_dim 128, 64 and 32; bf16 / fp16).
 #include "prefill_asm.h"
 
 namespace pa_decode_detail {
@@ -14,6 +14,7 @@ template <int D> prefill_mfma_fn pick(int dtype, bool lower_bounds) {
 prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds) {
     if (head_dim == 128) return pick<128>(dtype, lower_bounds);
     if (head_dim == 64) return pick<64>(dtype, lower_bounds);
+    if (head_dim == 32) return pick<32>(dtype, lower_bounds);
     return nullptr;
 }
 

@@ -240,10 +240,10 @@ def test_packed_documents_chunked_prefill_over_a_prefix():
     assert_close(out.reshape(2, cmax, hq, d), want, 2e-2, "chunked documents")
 
 
-@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("d", [128, 64, 32])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype, d):
-    """head_dim 128 and 64 take the kernel whose tile loop is scheduled assembly.  Block ids of -1 or past the pool, and
+    """head_dim 128, 64 and 32 take the kernel whose tile loop is scheduled assembly.  Block ids of -1 or past the pool, and
     contexts longer than the table, stand for zero key / value rows there as in the vector kernel (which is the
     statement of that rule: flex_backend.py:272-277 leaves rows of absent blocks zero); the two kernels must
     agree on every row, for 16-token and 64-token blocks, with the bad entries in the first tile, in the middle
@@ -280,7 +280,7 @@ def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype, d):
                 assert_close(got[b, :c], want[b, :c], 2e-2, f"block_size {bs} sequence {b} window {window}")
 
 
-@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("d", [128, 64, 32])
 def test_assembly_loop_kernel_long_context_and_table_limit(d):
     """A 70 000-key context (more than a thousand tiles of slot-table entries) through the assembly-loop kernel,
     and a table just past what that kernel's LDS tables hold (the host then launches the other matrix-core
@@ -302,7 +302,7 @@ def test_assembly_loop_kernel_long_context_and_table_limit(d):
             assert_close(got, want, 2e-2, f"context of {ctx} keys, window {window}")
 
 
-@pytest.mark.parametrize("d", [128, 64])
+@pytest.mark.parametrize("d", [128, 64, 32])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_assembly_loop_kernel_dense_rows_of_any_length(dtype, d):
     """Dense rows handed over as one block per sequence whose length is not a multiple of 16 (what
@@ -329,7 +329,7 @@ def test_assembly_loop_kernel_dense_rows_of_any_length(dtype, d):
                 assert_close(got.reshape(b, t, hq, d), want, 2e-2, f"{b} x {t}, documents {docs}, window {window}")
 
 
-@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_one_short_block_per_sequence_and_a_longer_context(d):
     """One block per sequence that is not a multiple of 16 keys long, with contexts that run past it (the keys
     behind the block are absent: zero rows, as in the vector kernel, which states that rule) and chunks that do
@@ -352,12 +352,12 @@ def test_one_short_block_per_sequence_and_a_longer_context(d):
                 assert_close(got[i, :c], want[i, :c], 2e-2, f"block_size {bs} sequence {i} window {window}")
 
 
-@pytest.mark.parametrize("d", [64, 128, 256])
+@pytest.mark.parametrize("d", [32, 64, 128, 256])
 def test_logits_that_grow_along_the_context(d):
     """Keys whose logits rise steeply with the key index (about 9 in base-2 units per 32 keys, from far below
     zero to far above), so that every row's reference maximum is outgrown by more than the lazy-rescale slack
     again and again, by some rows of a wave earlier than by others; then the same keys in falling order (the
-    first subtile holds the maximum, nothing is ever rescaled).  The assembly loops of head_dim 64, 128 and 256
+    first subtile holds the maximum, nothing is ever rescaled).  The assembly loops of head_dim 32, 64, 128 and 256
     (and, with a window, their instances with lower bounds), chunked over a prefix, against the checker."""
     announce(f"prefill rescale paths d={d}")
     rng = np.random.default_rng(500 + d)

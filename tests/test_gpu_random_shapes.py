@@ -109,13 +109,13 @@ def test_random_chunked_prefill(seed):
 
 @pytest.mark.parametrize("seed", range(24))
 def test_random_matrix_core_prefill(seed):
-    """Shapes the table-driven matrix-core prefill kernels take (head_dim 64 and 128: the assembly loop with and
+    """Shapes the table-driven matrix-core prefill kernels take (head_dim 32, 64 and 128: the assembly loop with and
     without lower bounds; head_dim 256), drawn at random: block sizes that are multiples of 16, ragged prefixes and
     chunks, sliding windows, per-row first keys, absent blocks.  Every case against the vector kernel (which
     states the zero-row rule of absent blocks), cases without absent blocks and first keys also against the
     checker."""
     rng = np.random.default_rng(9500 + seed)
-    d = int(rng.choice([64, 128, 128, 256]))
+    d = int(rng.choice([32, 64, 128, 128, 256]))
     hkv = int(rng.choice([1, 2, 4]))
     n_rep = int(rng.choice([1, 2, 3, 4, 8]))
     hq = hkv * n_rep
@@ -168,10 +168,10 @@ def test_random_matrix_core_prefill(seed):
 def test_random_dense_prefill_of_any_length(seed):
     """Dense causal prefill the way `_prefill_attention` hands it over (flex_backend.py:144-185): a pool of B blocks
     of T rows with the identity table, T of any length (so 16-key groups run into the next sequence's rows and, at
-    the end of the pool, past it), head sizes 64 / 128 / 256, with and without a sliding window; against the
+    the end of the pool, past it), head sizes 32 / 64 / 128 / 256, with and without a sliding window; against the
     checker."""
     rng = np.random.default_rng(9700 + seed)
-    d = int(rng.choice([64, 128, 256]))
+    d = int(rng.choice([32, 64, 128, 256]))
     hkv = int(rng.choice([1, 2, 4]))
     hq = hkv * int(rng.choice([1, 2, 4, 7]))
     dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
