@@ -2,7 +2,6 @@
 #include "prefill_mfma.h"
 
 namespace pa_decode_detail {
-constexpr int kPaCapTiles = 1600;  // (prefill_asm.h)
 prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds);
 constexpr int kWdTasks = 4, kWdCapGroups = 6144;  // (prefill_d256.h)
 prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool lower_bounds);
@@ -58,7 +57,7 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // (one instance without, one with sliding window / per-row first keys)
     if (mfma && (head_dim == 128 || head_dim == 64 || head_dim == 32) && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
-        bt_stride * (int64_t)block_size <= (int64_t)kPaCapTiles * kPfKeys)
+        bt_stride * (int64_t)block_size <= (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys)
         mfma = pa_prefill_asm_kernel(dtype, head_dim, window > 0 || row_first_key != nullptr);
     // head_dim 256: one 32-row task per wave, loads driven by a table of 16-key groups - which must lie inside one
     // pool block (block sizes that are multiples of 16, or a single block per sequence) - that LDS can hold

@@ -20,7 +20,7 @@
 //     a group's load then runs into the next block's rows, which are cleared like rows past the context end,
 //     and the one group at the end of the pool is fetched lane by lane when its tile is published;
 //   * the host launches prefill_mfma_kernel for other head sizes, for tables of several blocks that are not
-//     multiples of 16 keys long and for tables past kPaCapTiles.
+//     multiples of 16 keys long and for tables past pa_asm_cap_tiles().
 // Only the set-up, the first subtile's S^T and the write-out are compiled code, so the register allocator sees
 // one asm statement with pinned operands and little else.
 #pragma once
@@ -29,7 +29,6 @@
 
 namespace pa_decode_detail {
 
-constexpr int kPaCapTiles = 1600;  // tiles of 64 keys the slot tables hold: contexts of up to 102400 keys
 
 // LO: the instance that also applies lower bounds (sliding window, per-row first keys): the workgroup starts at
 // the tile of the first key its first row sees, everything the loop counts in is relative to that tile.
@@ -47,6 +46,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     constexpr int NG = G::LOADS / kPfWaves, GSTEP = GPT / NG;
     typedef __attribute__((address_space(3))) char lds_char;
     constexpr int kRingBytes = kPfStages * 2 * G::BYTES;
+    constexpr int kPaCapTiles = pa_asm_cap_tiles(D);
     constexpr int kTabABytes = kPaCapTiles * GPT * 4, kTabBBytes = (kPaCapTiles + 1) * GPT;
     static_assert(kPfStages == 4 && kPfKeys == 64 && kPfWaves == 4 && NC == 2, "the assembly loop is written for this shape");
     __shared__ __attribute__((aligned(1024))) char s_mem[kRingBytes + kTabABytes + kTabBBytes];
