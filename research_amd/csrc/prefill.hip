@@ -57,7 +57,11 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // (one instance without, one with sliding window / per-row first keys)
     if (mfma && (head_dim == 128 || head_dim == 64 || head_dim == 32) && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
-        bt_stride * (int64_t)block_size <= (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys)
+        (bt_stride * (int64_t)block_size <= (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys ||
+         // (under a sliding window the rows of a workgroup - at most kPfTasks blocks of kPfRows - see a bounded
+         // stretch of keys, whatever the table's length; the kernel's table starts at the workgroup's first tile)
+         (window > 0 &&
+          (int64_t)window + kPfTasks * kPfRows + 3 * kPfKeys <= (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys)))
         mfma = pa_prefill_asm_kernel(dtype, head_dim, window > 0 || row_first_key != nullptr);
     // head_dim 256: one 32-row task per wave, loads driven by a table of 16-key groups - which must lie inside one
     // pool block (block sizes that are multiples of 16, or a single block per sequence) - that LDS can hold
@@ -65,7 +69,9 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // (a pool of fewer than 16 rows has no slot a whole group could be loaded from: the vector kernel)
     if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
-        bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16) {
+        (bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16 ||
+         // (a workgroup's kWdTasks blocks of kPfRows rows under a sliding window, and the tiles its loads run ahead)
+         (window > 0 && (int64_t)window + kWdTasks * kPfRows + 10 * 32 <= (int64_t)kWdCapGroups * 16))) {
         mfma = pa_prefill_d256_kernel(dtype, window > 0 || row_first_key != nullptr);
         tasks_per_wg = kWdTasks;
     }

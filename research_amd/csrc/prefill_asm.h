@@ -117,8 +117,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     }
     // tiles the loop runs (>= 1), those of them with table entries, and the table's limit, all relative to t0
     const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys - t0;
-    const int n_real = max(min(n_tiles + t0, kPaCapTiles) - t0, 0);
-    const int cap_rel = max(kPaCapTiles - t0, 0);
+    // (the tables hold the kPaCapTiles tiles from t0 on: the host launches this kernel when the whole block table
+    // fits, or when a sliding window bounds the tiles a workgroup can see)
+    const int n_real = min(n_tiles, kPaCapTiles);
+    const int cap_rel = kPaCapTiles;
 
     // ---- Q^T operands, staged through the (still empty) ring as whole rows: see prefill_mfma_kernel ----
     constexpr int QRB = D * 2, QCPR = QRB / 16, QRPI = 64 / QCPR;

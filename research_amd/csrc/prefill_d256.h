@@ -36,7 +36,7 @@ namespace pa_decode_detail {
 constexpr int kWdKeys = 32;          // keys per ring stage
 constexpr int kWdStages = 4;
 constexpr int kWdTasks = kPfWaves;   // tasks (32 query rows of one head) per workgroup: one per wave
-constexpr int kWdCapGroups = 6144;   // 16-key groups the slot tables hold: contexts of up to 98304 keys
+constexpr int kWdCapGroups = 6144;   // 16-key groups the slot tables hold, from the workgroup's first tile on
 
 template <typename T, bool LO>
 __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseArgs a) {
@@ -141,14 +141,17 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     // (entries of kLookahead tiles past the workgroup's last one follow as groups of which nothing exists: the
     // loads run that far ahead and past the end, so that every wave issues the same loads per stage)
     constexpr int kLookahead = 6;
-    const int n_entries = min(2 * (n_tiles + kLookahead), CAP);
+    // The tables start at the workgroup's first tile t0 (entry i: keys 16 * (2 * t0 + i) ..): the host launches this
+    // kernel when the whole block table fits, or when a sliding window bounds the tiles a workgroup can see.
+    const int n_own = n_tiles - t0;  // tiles the loop runs
+    const int n_entries = min(2 * (n_own + kLookahead), CAP);
     {
         const int32_t *bt_seq = p.bt + (int64_t)b * p.bt_stride;
-        int first_special = n_tiles;
+        int first_special = n_own;
         for (int i = tid; i < n_entries; i += kPfThreads) {
-            const int key = 16 * i, blk = key / p.bs;
+            const int key = 16 * (2 * t0 + i), blk = key / p.bs;
             int64_t bid = -1;
-            if (i < 2 * n_tiles && blk < p.bt_stride) bid = bt_seq[blk];
+            if (i < 2 * n_own && blk < p.bt_stride) bid = bt_seq[blk];
             const bool present = bid >= 0 && bid < p.num_blocks;
             // rows of the group that exist: inside the context and inside the group's block (a block that is not
             // a multiple of 16 keys long is the only block of its sequence: what follows it is absent)
@@ -160,7 +163,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             if (rows < 16) first_special = min(first_special, i / 2);
         }
         if (tid < 4) { tab_a[CAP + tid] = 0; tab_b[CAP + tid] = 0; }
-        if (2 * n_tiles > CAP) first_special = min(first_special, CAP / 2);
+        if (2 * n_own > CAP) first_special = min(first_special, CAP / 2);
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) first_special = min(first_special, __shfl_xor(first_special, d, 64));
         if (lane == 0) s_special[wave] = first_special;
@@ -183,8 +186,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qreg[ks]));  // (product operands live in AGPRs)
     __syncthreads();  // the tables are complete and the staged rows have been read: the ring may overwrite them
     // first tile with a row that does not exist; every tile from there on is checked before it is published
-    const int first_special =
+    const int first_special_rel =
         __builtin_amdgcn_readfirstlane(min(min(s_special[0], s_special[1]), min(s_special[2], s_special[3])));
+    const int first_special = t0 + first_special_rel;
 
     // ---- loads: wave w fetches rows 8w .. 8w+7 of a stage's K and V, two rows (1 KiB) per direct load ----
     const int64_t tok_stride = (int64_t)p.hkv * RB;
@@ -204,7 +208,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     const uint32_t wave_rows = (uint32_t)wave * (8 * RB);  // the wave's rows inside a tensor of a stage
     // table entry of the wave's group of tile `tile` (>= 0, at most kLookahead - 1 past the last tile)
     const int wave_group = wave >> 1;
-    auto entry_of = [&](int tile) PF_INLINE { return min(2 * tile + wave_group, CAP); };
+    auto entry_of = [&](int tile) PF_INLINE { return min(2 * (tile - t0) + wave_group, CAP); };
     // one tensor's rows of one tile into LDS at byte offset `dst` of s_mem (always NL direct loads)
     auto issue_rows = [&](const char *pool, const uint32_t (&lane_ofs)[NL], int tile, uint32_t dst) PF_INLINE {
         const int slot = __builtin_amdgcn_readfirstlane(tab_a[entry_of(tile)]);
@@ -375,13 +379,13 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) read_v_one(t0, 0, dt, va0[dt]);
         auto uni = [](int v) PF_INLINE { return __builtin_amdgcn_readfirstlane(v); };
-        int n_left = uni(n_tiles - t0 - 1);  // tiles after the current one
-        uint32_t s_t = (uint32_t)uni(t0 + 4), s_p = (uint32_t)uni(t0 + 1);
+        int n_left = uni(n_own - 1);  // tiles after the current one
+        uint32_t s_t = 4, s_p = 1;   // (the loop counts tiles from t0, as the tables do)
         int s_rem = uni(mask_from - kWdKeys * t0);
         int s_lo = uni(lo_mask_until - kWdKeys * t0);
         const uint32_t tab_a_w = lds_base + kRingBytes + 4 * wave_group;
         const uint32_t tab_b_w = lds_base + kRingBytes + kTabEntries * 4 + wave_group;
-        const uint32_t sp_lo = (uint32_t)uni(max(first_special - 1, 0)), mask_from_u = (uint32_t)uni(mask_from);
+        const uint32_t sp_lo = (uint32_t)uni(max(first_special_rel - 1, 0)), mask_from_u = (uint32_t)uni(mask_from);
         const uint32_t m0w = lds_base + wave_rows, lane16 = (uint32_t)lane * 16, arow_u = (uint32_t)arow0;
         uint32_t kad[KS / 2], vad[DT / 2];
 #pragma unroll
@@ -393,7 +397,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         const uint32_t pvlo = uni((uint32_t)pv), pvhi = uni((uint32_t)(pv >> 32));
         const uint32_t stride = (uint32_t)tok_stride;
         // (only the waves that load rows of the group at the end of the pool see its tile)
-        const uint32_t edge_tile_u = (uint32_t)uni(wave_group == edge_group ? edge_tile : -1);
+        const uint32_t edge_tile_u = (uint32_t)uni(wave_group == edge_group && edge_tile >= t0 ? edge_tile - t0 : -1);
         const uint32_t edge_slot_u = (uint32_t)uni((int)edge_slot), edge_rows_u = (uint32_t)uni(edge_rows);
         const float slack = kPfSlack, neg_big = kNegBig;
 #define WD_NOTHING

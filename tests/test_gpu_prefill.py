@@ -284,7 +284,8 @@ def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype, d):
 def test_assembly_loop_kernel_long_context_and_table_limit(d):
     """A 70 000-key context (more than a thousand tiles of slot-table entries) through the assembly-loop kernel,
     and a table just past what that kernel's LDS tables hold (the host then launches the other matrix-core
-    kernel): both against the vector kernel on the chunk's rows."""
+    kernel; under a sliding window the assembly-loop kernel still runs, its tables starting at the workgroup's
+    first tile): both against the vector kernel on the chunk's rows."""
     announce(f"prefill assembly loop, long context d={d}")
     rng = np.random.default_rng(78)
     hq, hkv, bs = 4, 1, 16
@@ -301,6 +302,33 @@ def test_assembly_loop_kernel_long_context_and_table_limit(d):
             got = ops.prefill_paged(*args, window=window).float().cpu()
             want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu()
             assert_close(got, want, 2e-2, f"context of {ctx} keys, window {window}")
+
+
+@pytest.mark.parametrize("d", [256, 128, 64])
+def test_assembly_loop_kernel_window_over_a_table_longer_than_its_tables(d):
+    """Sliding window over contexts whose block table is longer than the kernel's slot tables: a chunk of 600 rows
+    with one query head per kv head (a workgroup then spans the most rows it can), and the last 300 rows of a
+    sequence whose context is one block of a length that is no multiple of 16; against the vector kernel."""
+    announce(f"prefill assembly loop, window over a long table d={d}")
+    rng = np.random.default_rng(80)
+    cap_keys = {256: 6144 * 16, 128: 1600 * 64, 64: 4096 * 64}[d]  # keys the kernel's slot tables hold at this head size
+    hq = hkv = 1
+    mk = lambda *shape: torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    ctx, chunk, bs = cap_keys + 5000, 600, 16
+    nblk = -(-ctx // bs)
+    table = torch.from_numpy(rng.permutation(nblk).astype(np.int32)).reshape(1, -1).to(DEV)
+    args = (0.3 * mk(chunk, hq, d), mk(nblk * bs, hkv, d), mk(nblk * bs, hkv, d), table, _i32([ctx]), _i32([chunk]), _i32([0]),
+            chunk, bs, d ** -0.5)
+    for window in (1000, 1):
+        got = ops.prefill_paged(*args, window=window).float().cpu()
+        want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu()
+        assert_close(got, want, 2e-2, f"paged, window {window}")
+    t = cap_keys + 1111
+    args = (0.3 * mk(300, hq, d), mk(t, hkv, d), mk(t, hkv, d), torch.zeros(1, 1, dtype=torch.int32, device=DEV), _i32([t]), _i32([300]),
+            _i32([0]), 300, t, d ** -0.5)
+    got = ops.prefill_paged(*args, window=500).float().cpu()
+    want = ops.prefill_paged(*args, window=500, rowwise=True).float().cpu()
+    assert_close(got, want, 2e-2, "one block of the whole context, window 500")
 
 
 @pytest.mark.parametrize("d", [128, 64, 32])
