@@ -374,11 +374,12 @@ def operands():
     outs = [f'"+{{a[{16 * dt}:{16 * dt + 15}]}}"(o[{dt}])' for dt in range(DT)]
     outs += ['"+{v[0:15]}"(sb0)', '"+{v[118:133]}"(ref)']
     outs += [f'"+{{a[{KA(ks)}:{KA(ks) + 3}]}}"(ka[{ks}])' for ks in range(KS)]
+    # (Q^T is only read; as read-write operands the registers stay where they are when the statement sits in a loop)
+    outs += [f'"+{{a[{128 + 4 * ks}:{131 + 4 * ks}]}}"(qreg[{ks}])' for ks in range(KS)]
     outs += [f'"+{{v[{VA0(dt)}:{VA0(dt) + 3}]}}"(va0[{dt}])' for dt in range(4)]
     outs += ['[mx0] "+&v"(mx)', '[l0] "+&v"(l_run)', '[ntiles] "+&s"(n_left)', '[sT] "+&s"(s_t)', '[sP] "+&s"(s_p)',
              '[srem] "+&s"(s_rem) MORE_OUT']
-    ins = [f'"{{a[{128 + 4 * ks}:{131 + 4 * ks}]}}"(qreg[{ks}])' for ks in range(KS)]
-    ins += [f'[kad{ks}] "v"(kad[{ks}])' for ks in range(8)] + [f'[vad{dt}] "v"(vad[{dt}])' for dt in range(4)]
+    ins = [f'[kad{ks}] "v"(kad[{ks}])' for ks in range(8)] + [f'[vad{dt}] "v"(vad[{dt}])' for dt in range(4)]
     ins += [f'[lanek{n}] "v"(lane_kb[{n}])' for n in range(4)] + [f'[lanev{n}] "v"(lane_vb[{n}])' for n in range(4)]
     ins += ['[lane16] "v"(lane16)', '[arow] "v"(arow_u)', '[lim0] "v"(lim)', '[slack] "s"(slack)', '[pklo] "s"(pklo)',
             '[pkhi] "s"(pkhi)', '[pvlo] "s"(pvlo)', '[pvhi] "s"(pvhi)', '[stride] "s"(stride)', '[m0w] "s"(m0w)',

@@ -2,9 +2,9 @@
 #include "prefill_mfma.h"
 
 namespace pa_decode_detail {
-prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds);
+prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds, bool long_table);
 constexpr int kWdTasks = 4, kWdCapGroups = 6144;  // (prefill_d256.h)
-prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool lower_bounds);
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool lower_bounds, bool long_table);
 }
 
 using namespace pa_decode_detail;
@@ -53,26 +53,33 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     prefill_mfma_fn mfma =
         force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
     // head_dim 128, 64 or 32, blocks of a multiple of 16 tokens (or one block per sequence, as dense prefill passes its
-    // rows) and a table the kernel's LDS copy can hold: the kernel whose whole tile loop is scheduled assembly
-    // (one instance without, one with sliding window / per-row first keys)
+    // rows): the kernel whose whole tile loop is scheduled assembly (one instance without, one with sliding window /
+    // per-row first keys).  Its LDS copy of the table holds pa_asm_cap_tiles() tiles from the workgroup's first tile
+    // on, which bounds the table's length - or, under a sliding window, the stretch of keys that the rows of a
+    // workgroup (at most kPfTasks blocks of kPfRows) see; at head_dim 128 longer tables take the instance that fills
+    // its copy again on the way.
     if (mfma && (head_dim == 128 || head_dim == 64 || head_dim == 32) && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
-        (bt_stride * (int64_t)block_size <= (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys ||
-         // (under a sliding window the rows of a workgroup - at most kPfTasks blocks of kPfRows - see a bounded
-         // stretch of keys, whatever the table's length; the kernel's table starts at the workgroup's first tile)
-         (window > 0 &&
-          (int64_t)window + kPfTasks * kPfRows + 3 * kPfKeys <= (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys)))
-        mfma = pa_prefill_asm_kernel(dtype, head_dim, window > 0 || row_first_key != nullptr);
+        bt_stride * (int64_t)block_size < (1ll << 31)) {
+        const int64_t cap_keys = (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys;
+        const bool fits = bt_stride * (int64_t)block_size <= cap_keys ||
+                          (window > 0 && (int64_t)window + kPfTasks * kPfRows + 3 * kPfKeys <= cap_keys);
+        if (fits || head_dim == 128)
+            mfma = pa_prefill_asm_kernel(dtype, head_dim, window > 0 || row_first_key != nullptr, !fits);
+    }
     // head_dim 256: one 32-row task per wave, loads driven by a table of 16-key groups - which must lie inside one
-    // pool block (block sizes that are multiples of 16, or a single block per sequence) - that LDS can hold
+    // pool block (block sizes that are multiples of 16, or a single block per sequence); the kernel fills its table
+    // again whenever the context is longer than what LDS can hold of it
     int tasks_per_wg = kPfTasks;
     // (a pool of fewer than 16 rows has no slot a whole group could be loaded from: the vector kernel)
     if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
-        (bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16 ||
-         // (a workgroup's kWdTasks blocks of kPfRows rows under a sliding window, and the tiles its loads run ahead)
-         (window > 0 && (int64_t)window + kWdTasks * kPfRows + 10 * 32 <= (int64_t)kWdCapGroups * 16))) {
-        mfma = pa_prefill_d256_kernel(dtype, window > 0 || row_first_key != nullptr);
+        bt_stride * (int64_t)block_size < (1ll << 31)) {
+        // (the tables hold kWdCapGroups groups of 16 keys from the workgroup's first tile on; under a sliding window
+        // a workgroup's kWdTasks blocks of kPfRows rows, and the tiles its loads run ahead, bound what it needs)
+        const bool fits = bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16 ||
+                          (window > 0 && (int64_t)window + kWdTasks * kPfRows + 10 * 32 <= (int64_t)kWdCapGroups * 16);
+        mfma = pa_prefill_d256_kernel(dtype, window > 0 || row_first_key != nullptr, !fits);
         tasks_per_wg = kWdTasks;
     }
     if (mfma) {

@@ -19,8 +19,10 @@
 //   * block sizes that are not multiples of 16 are taken with one block per sequence (what dense prefill passes):
 //     a group's load then runs into the next block's rows, which are cleared like rows past the context end,
 //     and the one group at the end of the pool is fetched lane by lane when its tile is published;
+//   * the tables hold pa_asm_cap_tiles() tiles from the workgroup's first tile on; the LONG instance fills them
+//     again on the way when the workgroup runs more tiles than that (instantiated for head_dim 128);
 //   * the host launches prefill_mfma_kernel for other head sizes, for tables of several blocks that are not
-//     multiples of 16 keys long and for tables past pa_asm_cap_tiles().
+//     multiples of 16 keys long and, at head_dim 64 and 32, for tables past pa_asm_cap_tiles().
 // Only the set-up, the first subtile's S^T and the write-out are compiled code, so the register allocator sees
 // one asm statement with pinned operands and little else.
 #pragma once
@@ -32,7 +34,9 @@ namespace pa_decode_detail {
 
 // LO: the instance that also applies lower bounds (sliding window, per-row first keys): the workgroup starts at
 // the tile of the first key its first row sees, everything the loop counts in is relative to that tile.
-template <typename T, bool LO, int D>
+// LONG: the instance for workgroups that run more tiles than the tables hold (the same code with a loop around the
+// assembly that fills the tables again, which costs registers in the set-up).
+template <typename T, bool LO, int D, bool LONG = false>
 __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
@@ -115,11 +119,13 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 #pragma unroll
         for (int c = 0; c < NC; ++c) lo[c] = row_first(row0[c] + col) - 4 * half;
     }
-    // tiles the loop runs (>= 1), those of them with table entries, and the table's limit, all relative to t0
+    // tiles the loop runs (>= 1), counted from t0 like every tile number below
     const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys - t0;
-    // (the tables hold the kPaCapTiles tiles from t0 on: the host launches this kernel when the whole block table
-    // fits, or when a sliding window bounds the tiles a workgroup can see)
-    const int n_real = min(n_tiles, kPaCapTiles);
+    // The tables hold kPaCapTiles tiles from a first tile `base` on.  They are filled for base = 0 here and, in the
+    // LONG instance, again every kSegTiles tiles: the assembly loop is left and entered again, which is free of side
+    // conditions because every pass of its body leaves the state the next one starts from.  (The host launches the
+    // other instance when the whole block table fits, or when a sliding window bounds the tiles a workgroup can see.)
+    constexpr int kSegTiles = (kPaCapTiles - kPfStages) / kPfStages * kPfStages;  // (the loop starts in ring slot 0)
     const int cap_rel = kPaCapTiles;
 
     // ---- Q^T operands, staged through the (still empty) ring as whole rows: see prefill_mfma_kernel ----
@@ -159,12 +165,14 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             edge_slot = bid * p.bs + key_last;
         }
     }
-    {
+    auto fill_tables = [&](int base) PF_INLINE {
         const int32_t *bt_seq = p.bt + (int64_t)b * p.bt_stride;
-        const int n_entries = max(n_real, 1) * GPT;  // (the loads of tiles past the last fetch tile 0 again: it has entries)
-        int first_special = n_tiles;
+        const int n_rest = n_tiles - base;             // tiles still to run (>= 1)
+        const int n_real = min(n_rest, kPaCapTiles);   // those of them with table entries
+        const int n_entries = n_real * GPT;  // (the loads of tiles past the last fetch tile 0 again: it has entries)
+        int first_special = n_rest;
         for (int i = tid; i < n_entries; i += kPfThreads) {
-            const int key = 16 * (t0 * GPT + i), blk = key / p.bs;
+            const int key = 16 * ((t0 + base) * GPT + i), blk = key / p.bs;
             int64_t bid = -1;
             if (blk < p.bt_stride) bid = bt_seq[blk];
             const bool present = bid >= 0 && bid < p.num_blocks;
@@ -178,12 +186,17 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             if (rows < 16) first_special = min(first_special, i / GPT);
         }
         if (tid < GPT) tab_b[cap_rel * GPT + tid] = 0;  // tiles past the tables: nothing exists
-        if (n_tiles > n_real) first_special = min(first_special, n_real);
-        // minimum over the wave here, over the waves behind the barrier below
+        if (n_rest > n_real) first_special = min(first_special, n_real);
+        // minimum over the wave here, over the waves behind the next barrier (read_special)
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) first_special = min(first_special, __shfl_xor(first_special, d, 64));
         if (lane == 0) s_special[wave] = first_special;
-    }
+    };
+    // first tile (counted from the tables' base) with a row that does not exist
+    auto read_special = [&]() PF_INLINE {
+        return __builtin_amdgcn_readfirstlane(min(min(s_special[0], s_special[1]), min(s_special[2], s_special[3])));
+    };
+    fill_tables(0);
     pf_wait_loads<0>();
     const float sc = p.scale_log2;
     X8 qreg[NC][KS];
@@ -206,8 +219,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qreg[c][ks]));
     __syncthreads();  // the tables are complete and the staged rows have been read: the ring may overwrite them
-    const int first_special =
-        __builtin_amdgcn_readfirstlane(min(min(s_special[0], s_special[1]), min(s_special[2], s_special[3])));
+    int first_special = read_special();
 
     // ---- loads of a tile: wave w fetches rows w*RPL .. w*RPL + RPL-1 of the tile and, NG-1 times, the rows 4*RPL on ----
     const int64_t tok_stride = (int64_t)p.hkv * D * 2;
@@ -223,7 +235,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     constexpr int kLoadStep = kPfWaves * G::RPL * G::RB;  // LDS bytes between a wave's consecutive loads
     static_assert(kLoadStep == 4096, "the assembly loops place a wave's loads 4 KiB apart");
     auto issue = [&](int tile) PF_INLINE {
-        const int src = tile < n_real ? tile : 0;
+        const int src = tile < min(n_tiles, kPaCapTiles) ? tile : 0;
         const uint32_t dst0 = m0w + (uint32_t)(tile % kPfStages) * 2 * G::BYTES;
 #pragma unroll
         for (int n = 0; n < NG; ++n) {
@@ -339,20 +351,15 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     {
         // (wave-uniform values the compiler may hold in vector registers are moved to scalar ones for the "s" operands)
         auto uni = [](int v) PF_INLINE { return __builtin_amdgcn_readfirstlane(v); };
-        int n_left = uni(n_tiles - 1);  // tiles after the current one
-        uint32_t s_t = 3, s_p = 1;
-        int s_rem = uni(mask_from - kPfKeys * t0);  // mask_from - 64 * (absolute) tile
-        int s_lo = uni(lo_mask_until - kPfKeys * t0);  // the same for the lower bound
         const uint32_t tab_a_base = lds_base + kRingBytes + 4 * g0;  // (the wave's first group folded in)
         const uint32_t tab_b_base = lds_base + kRingBytes + kTabABytes;
-        const uint32_t sp_lo = (uint32_t)uni(first_special), sp_span = (uint32_t)uni(n_tiles - first_special);
-        const uint32_t n_real_u = (uint32_t)uni(n_real), cap_tiles = (uint32_t)uni(cap_rel), mask_from_u = (uint32_t)uni(mask_from);
+        const uint32_t cap_tiles = (uint32_t)uni(cap_rel), mask_from_u = (uint32_t)uni(mask_from);
         const uint32_t lane16 = (uint32_t)lane * 16, arow_u = (uint32_t)arow;
         const uint64_t pk = reinterpret_cast<uint64_t>(pool_k), pv = reinterpret_cast<uint64_t>(pool_v);
         const uint32_t pklo = __builtin_amdgcn_readfirstlane((uint32_t)pk), pkhi = __builtin_amdgcn_readfirstlane((uint32_t)(pk >> 32));
         const uint32_t pvlo = __builtin_amdgcn_readfirstlane((uint32_t)pv), pvhi = __builtin_amdgcn_readfirstlane((uint32_t)(pv >> 32));
         const uint32_t stride = (uint32_t)tok_stride;
-        const uint32_t edge_tile_u = (uint32_t)uni(edge_tile), edge_slot_u = (uint32_t)uni((int)edge_slot);
+        const uint32_t edge_slot_u = (uint32_t)uni((int)edge_slot);
         const uint32_t edge_rows_u = (uint32_t)uni(edge_rows), edge_ofs_u = (uint32_t)uni(edge_ofs);
         const float slack = kPfSlack;  // in the units of S^T here: log2 of the factor a row's reference may lag by
 #define PA_LOOP_COMMON_OUT(...)                                                                                      \
@@ -377,18 +384,19 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
       "a245", "a246", "a247", "a248", "a249", "a250", "a251", "a252", "a253", "a254", "a255", "s40", "s41", "s42",     \
       "s43", "s44", "s45", "s46", "s47", "s48", "s49", "s50", "s51", "s52", "s53", "s54", "s55", "s56", "s57", "s58",  \
       "s59", "s60", "s61", "s62", "s63", "vcc", "scc", "memory"
-// head_dim 128: o[c][dt] at a[16*(4c+dt)], q[c][ks] at a[128 + 4*(8c+ks)], ka[ks] at a[192 + 4*ks]
+// head_dim 128: o[c][dt] at a[16*(4c+dt)], q[c][ks] at a[128 + 4*(8c+ks)], ka[ks] at a[192 + 4*ks] (Q^T is only read;
+// as read-write operands its registers stay where they are when the statement sits in a loop)
 #define PA_LOOP_OPERANDS(MORE_OUT, MORE_IN)                                                                           \
     : "+{a[0:15]}"(o[0][0]), "+{a[16:31]}"(o[0][1]), "+{a[32:47]}"(o[0][2]), "+{a[48:63]}"(o[0][3]),                    \
       "+{a[64:79]}"(o[1][0]), "+{a[80:95]}"(o[1][1]), "+{a[96:111]}"(o[1][2]), "+{a[112:127]}"(o[1][3]),                \
       "+{a[192:195]}"(ka[0]), "+{a[196:199]}"(ka[1]), "+{a[200:203]}"(ka[2]), "+{a[204:207]}"(ka[3]),                   \
       "+{a[208:211]}"(ka[4]), "+{a[212:215]}"(ka[5]), "+{a[216:219]}"(ka[6]), "+{a[220:223]}"(ka[7]),                   \
+      "+{a[128:131]}"(qreg[0][0]), "+{a[132:135]}"(qreg[0][1]), "+{a[136:139]}"(qreg[0][2]), "+{a[140:143]}"(qreg[0][3]), \
+      "+{a[144:147]}"(qreg[0][4]), "+{a[148:151]}"(qreg[0][5]), "+{a[152:155]}"(qreg[0][6]), "+{a[156:159]}"(qreg[0][7]), \
+      "+{a[160:163]}"(qreg[1][0]), "+{a[164:167]}"(qreg[1][1]), "+{a[168:171]}"(qreg[1][2]), "+{a[172:175]}"(qreg[1][3]), \
+      "+{a[176:179]}"(qreg[1][4]), "+{a[180:183]}"(qreg[1][5]), "+{a[184:187]}"(qreg[1][6]), "+{a[188:191]}"(qreg[1][7]), \
       PA_LOOP_COMMON_OUT(MORE_OUT)                                                                                    \
-    : "{a[128:131]}"(qreg[0][0]), "{a[132:135]}"(qreg[0][1]), "{a[136:139]}"(qreg[0][2]), "{a[140:143]}"(qreg[0][3]),   \
-      "{a[144:147]}"(qreg[0][4]), "{a[148:151]}"(qreg[0][5]), "{a[152:155]}"(qreg[0][6]), "{a[156:159]}"(qreg[0][7]),   \
-      "{a[160:163]}"(qreg[1][0]), "{a[164:167]}"(qreg[1][1]), "{a[168:171]}"(qreg[1][2]), "{a[172:175]}"(qreg[1][3]),   \
-      "{a[176:179]}"(qreg[1][4]), "{a[180:183]}"(qreg[1][5]), "{a[184:187]}"(qreg[1][6]), "{a[188:191]}"(qreg[1][7]),   \
-      [kad0] "v"(kad[0]), [kad1] "v"(kad[1]), [kad2] "v"(kad[2]), [kad3] "v"(kad[3]), [kad4] "v"(kad[4]),               \
+    : [kad0] "v"(kad[0]), [kad1] "v"(kad[1]), [kad2] "v"(kad[2]), [kad3] "v"(kad[3]), [kad4] "v"(kad[4]),               \
       [kad5] "v"(kad[5]), [kad6] "v"(kad[6]), [kad7] "v"(kad[7]), [vad0] "v"(vad[0]), [vad1] "v"(vad[1]),               \
       [vad2] "v"(vad[2]), [vad3] "v"(vad[3]), PA_LOOP_COMMON_IN(MORE_IN)
 // head_dim 64: o[c][dt] at a[16*(2c+dt)], q[c][ks] at a[128 + 4*(4c+ks)], ka[ks] at a[192 + 4*ks]; bshift: the bit
@@ -412,6 +420,19 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 #define PA_LO_IN , [lo0] "v"(lo[0]), [lo1] "v"(lo[1]), [negbig] "s"(neg_big)
         const float neg_big = kNegBig;
         constexpr bool BF = std::is_same<T, pa_bf16>::value;
+        const int n_tiles_u = uni(n_tiles);
+        for (int base = 0;;) {  // one pass per fill of the tables (uniform control flow, stated to the compiler)
+        const int n_rest = n_tiles_u - base;
+        const int n_seg = LONG ? uni(min(n_rest, kSegTiles)) : n_rest;  // tiles of this pass
+        int n_left = uni(n_seg - 1);  // tiles after the current one
+        uint32_t s_t = 3, s_p = 1;    // (the loop counts tiles from the tables' base)
+        int s_rem = uni(mask_from - kPfKeys * (t0 + base));      // mask_from - 64 * (absolute) tile
+        int s_lo = uni(lo_mask_until - kPfKeys * (t0 + base));   // the same for the lower bound
+        // tiles in [sp_lo, sp_lo + sp_span) are checked before they are published (the pass publishes tiles 1 .. n_seg)
+        const uint32_t sp_lo = (uint32_t)uni(first_special);
+        const uint32_t sp_span = (uint32_t)uni(max(min(n_rest, n_seg + 1) - first_special, 0));
+        const uint32_t n_real_u = (uint32_t)uni(min(n_rest, kPaCapTiles));
+        const uint32_t edge_tile_u = (uint32_t)uni(edge_tile >= base ? edge_tile - base : -1);
         if constexpr (D == 128 && LO) {
             if constexpr (BF) {
                 asm volatile(PF_LOOP_ASM_BF16_LO PA_LOOP_OPERANDS(PA_LO_OUT, PA_LO_IN));
@@ -455,6 +476,14 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             } else {
                 asm volatile(PF_LOOP_ASM_D64_F16 PA_LOOP_OPERANDS_D64(PA_NOTHING, PA_NOTHING));
             }
+        }
+        if constexpr (!LONG) break;
+        base = uni(base + n_seg);
+        if (base >= n_tiles_u) break;
+        __syncthreads();  // every wave has left the loop: nobody reads the tables
+        fill_tables(base);
+        __syncthreads();
+        first_special = read_special();
         }
 #undef PA_LOOP_OPERANDS
 #undef PA_LOOP_OPERANDS_D64
@@ -505,7 +534,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 }
 
 // nullptr unless the element type has this kernel; `lower_bounds`: the instance for sliding windows and per-row
-// first keys
-prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds);
+// first keys; `long_table`: the instance that fills its tables more than once (head_dim 128 only)
+prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds, bool long_table);
 
 }  // namespace pa_decode_detail

@@ -38,7 +38,9 @@ constexpr int kWdStages = 4;
 constexpr int kWdTasks = kPfWaves;   // tasks (32 query rows of one head) per workgroup: one per wave
 constexpr int kWdCapGroups = 6144;   // 16-key groups the slot tables hold, from the workgroup's first tile on
 
-template <typename T, bool LO>
+// LONG: the instance for workgroups that run more tiles than the tables hold (it fills them again on the way; the
+// other instance is the same code without that loop around the assembly, which costs it registers in the set-up).
+template <typename T, bool LO, bool LONG>
 __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseArgs a) {
     using M = Mfma16<T>;
     using X8 = typename M::x8;
@@ -141,17 +143,21 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     // (entries of kLookahead tiles past the workgroup's last one follow as groups of which nothing exists: the
     // loads run that far ahead and past the end, so that every wave issues the same loads per stage)
     constexpr int kLookahead = 6;
-    // The tables start at the workgroup's first tile t0 (entry i: keys 16 * (2 * t0 + i) ..): the host launches this
-    // kernel when the whole block table fits, or when a sliding window bounds the tiles a workgroup can see.
-    const int n_own = n_tiles - t0;  // tiles the loop runs
-    const int n_entries = min(2 * (n_own + kLookahead), CAP);
-    {
+    // The tables hold the groups of kWdCapGroups / 2 tiles, counted from a first tile `base` (entry i: keys
+    // 16 * (2 * base + i) ..).  They are filled for base = t0 here, and in the LONG instance again every kSegTiles
+    // tiles: the loop below is left and entered again, which is free of side conditions because every pass of its
+    // body leaves the state the next one starts from.  (The host launches the other instance when the whole block
+    // table fits, or when a sliding window bounds the tiles a workgroup can see.)
+    constexpr int kSegTiles = (CAP / 2 - kLookahead - 2) / kWdStages * kWdStages;  // (the loop starts in ring slot 0)
+    auto fill_tables = [&](int base) PF_INLINE {
+        const int n_rest = n_tiles - base;  // tiles still to run
+        const int n_entries = min(2 * (n_rest + kLookahead), CAP);
         const int32_t *bt_seq = p.bt + (int64_t)b * p.bt_stride;
-        int first_special = n_own;
+        int first_special = n_rest;
         for (int i = tid; i < n_entries; i += kPfThreads) {
-            const int key = 16 * (2 * t0 + i), blk = key / p.bs;
+            const int key = 16 * (2 * base + i), blk = key / p.bs;
             int64_t bid = -1;
-            if (i < 2 * n_own && blk < p.bt_stride) bid = bt_seq[blk];
+            if (i < 2 * n_rest && blk < p.bt_stride) bid = bt_seq[blk];
             const bool present = bid >= 0 && bid < p.num_blocks;
             // rows of the group that exist: inside the context and inside the group's block (a block that is not
             // a multiple of 16 keys long is the only block of its sequence: what follows it is absent)
@@ -163,11 +169,17 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             if (rows < 16) first_special = min(first_special, i / 2);
         }
         if (tid < 4) { tab_a[CAP + tid] = 0; tab_b[CAP + tid] = 0; }
-        if (2 * n_own > CAP) first_special = min(first_special, CAP / 2);
+        if (2 * n_rest > CAP) first_special = min(first_special, CAP / 2);
 #pragma unroll
         for (int d = 32; d >= 1; d >>= 1) first_special = min(first_special, __shfl_xor(first_special, d, 64));
         if (lane == 0) s_special[wave] = first_special;
-    }
+    };
+    // first tile (counted from the tables' base) with a row that does not exist; every tile from there on is checked
+    // before it is published.  Valid behind a barrier after fill_tables.
+    auto read_special = [&]() PF_INLINE {
+        return __builtin_amdgcn_readfirstlane(min(min(s_special[0], s_special[1]), min(s_special[2], s_special[3])));
+    };
+    fill_tables(t0);
     pf_wait_loads<0>();
     X8 qreg[KS];
 #pragma unroll
@@ -185,9 +197,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qreg[ks]));  // (product operands live in AGPRs)
     __syncthreads();  // the tables are complete and the staged rows have been read: the ring may overwrite them
-    // first tile with a row that does not exist; every tile from there on is checked before it is published
-    const int first_special_rel =
-        __builtin_amdgcn_readfirstlane(min(min(s_special[0], s_special[1]), min(s_special[2], s_special[3])));
+    int first_special_rel = read_special();
     const int first_special = t0 + first_special_rel;
 
     // ---- loads: wave w fetches rows 8w .. 8w+7 of a stage's K and V, two rows (1 KiB) per direct load ----
@@ -366,7 +376,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         // 0; with them a row may have seen nothing yet: its reference stays unset (thr = a large negative number
         // instead of the slack) until a maximum of visible keys arrives (see prefill_asm_kernel).  The loop takes
         // the first half of the first V^T operands read.
-        static_assert(kWdStages == 4 && kWdKeys == 32 && CAP == 2 * 3072, "the assembly loop is written for this shape");
+        static_assert(kWdStages == 4 && kWdKeys == 32 && CAP == 2 * 3072 && kSegTiles % kWdStages == 0,
+                      "the assembly loop is written for this shape");
         const bool seen = mx > kNegBig;
         const float m0 = seen ? mx : 0.f;
 #pragma unroll
@@ -379,13 +390,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 #pragma unroll
         for (int dt = 0; dt < 4; ++dt) read_v_one(t0, 0, dt, va0[dt]);
         auto uni = [](int v) PF_INLINE { return __builtin_amdgcn_readfirstlane(v); };
-        int n_left = uni(n_own - 1);  // tiles after the current one
-        uint32_t s_t = 4, s_p = 1;   // (the loop counts tiles from t0, as the tables do)
-        int s_rem = uni(mask_from - kWdKeys * t0);
-        int s_lo = uni(lo_mask_until - kWdKeys * t0);
         const uint32_t tab_a_w = lds_base + kRingBytes + 4 * wave_group;
         const uint32_t tab_b_w = lds_base + kRingBytes + kTabEntries * 4 + wave_group;
-        const uint32_t sp_lo = (uint32_t)uni(max(first_special_rel - 1, 0)), mask_from_u = (uint32_t)uni(mask_from);
+        const uint32_t mask_from_u = (uint32_t)uni(mask_from);
         const uint32_t m0w = lds_base + wave_rows, lane16 = (uint32_t)lane * 16, arow_u = (uint32_t)arow0;
         uint32_t kad[KS / 2], vad[DT / 2];
 #pragma unroll
@@ -396,27 +403,43 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         const uint32_t pklo = uni((uint32_t)pk), pkhi = uni((uint32_t)(pk >> 32));
         const uint32_t pvlo = uni((uint32_t)pv), pvhi = uni((uint32_t)(pv >> 32));
         const uint32_t stride = (uint32_t)tok_stride;
-        // (only the waves that load rows of the group at the end of the pool see its tile)
-        const uint32_t edge_tile_u = (uint32_t)uni(wave_group == edge_group && edge_tile >= t0 ? edge_tile - t0 : -1);
         const uint32_t edge_slot_u = (uint32_t)uni((int)edge_slot), edge_rows_u = (uint32_t)uni(edge_rows);
         const float slack = kPfSlack, neg_big = kNegBig;
 #define WD_NOTHING
 #define WD_LO_OUT , [thr0] "+&v"(thr), [slo] "+&s"(s_lo)
 #define WD_LO_IN , [lo0] "v"(lo_lim), [negbig] "s"(neg_big)
         constexpr bool BF = std::is_same<T, pa_bf16>::value;
-        if constexpr (LO) {
-            if constexpr (BF) {
-                asm volatile(WD_LOOP_ASM_BF16_LO WD_LOOP_OPERANDS(WD_LO_OUT, WD_LO_IN));
+        const int n_tiles_u = uni(n_tiles);
+        for (int base = uni(t0);;) {  // one pass per fill of the tables (uniform control flow, stated to the compiler)
+            const int n_seg = uni(min(n_tiles_u - base, kSegTiles));
+            int n_left = uni(n_seg - 1);  // tiles after the current one
+            uint32_t s_t = 4, s_p = 1;    // (the loop counts tiles from the tables' base)
+            int s_rem = uni(mask_from - kWdKeys * base);
+            int s_lo = uni(lo_mask_until - kWdKeys * base);
+            const uint32_t sp_lo = (uint32_t)uni(max(first_special_rel - 1, 0));
+            // (only the waves that load rows of the group at the end of the pool see its tile)
+            const uint32_t edge_tile_u = (uint32_t)uni(wave_group == edge_group && edge_tile >= base ? edge_tile - base : -1);
+            if constexpr (LO) {
+                if constexpr (BF) {
+                    asm volatile(WD_LOOP_ASM_BF16_LO WD_LOOP_OPERANDS(WD_LO_OUT, WD_LO_IN));
+                } else {
+                    asm volatile(WD_LOOP_ASM_F16_LO WD_LOOP_OPERANDS(WD_LO_OUT, WD_LO_IN));
+                }
             } else {
-                asm volatile(WD_LOOP_ASM_F16_LO WD_LOOP_OPERANDS(WD_LO_OUT, WD_LO_IN));
+                (void)thr; (void)s_lo; (void)neg_big;
+                if constexpr (BF) {
+                    asm volatile(WD_LOOP_ASM_BF16 WD_LOOP_OPERANDS(WD_NOTHING, WD_NOTHING));
+                } else {
+                    asm volatile(WD_LOOP_ASM_F16 WD_LOOP_OPERANDS(WD_NOTHING, WD_NOTHING));
+                }
             }
-        } else {
-            (void)thr; (void)s_lo; (void)neg_big;
-            if constexpr (BF) {
-                asm volatile(WD_LOOP_ASM_BF16 WD_LOOP_OPERANDS(WD_NOTHING, WD_NOTHING));
-            } else {
-                asm volatile(WD_LOOP_ASM_F16 WD_LOOP_OPERANDS(WD_NOTHING, WD_NOTHING));
-            }
+            if constexpr (!LONG) break;
+            base = uni(base + n_seg);
+            if (base >= n_tiles_u) break;
+            __syncthreads();  // every wave has left the loop: nobody reads the tables
+            fill_tables(base);
+            __syncthreads();
+            first_special_rel = read_special();
         }
 #undef WD_NOTHING
 #undef WD_LO_OUT
@@ -442,7 +465,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 }
 
 // nullptr unless the element type has this kernel; `lower_bounds`: the instance for sliding windows and per-row
-// first keys
-prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool lower_bounds);
+// first keys; `long_table`: the instance that fills its tables more than once
+prefill_mfma_fn pa_prefill_d256_kernel(int dtype, bool lower_bounds, bool long_table);
+prefill_mfma_fn pa_prefill_d256_kernel_long(int dtype, bool lower_bounds);
 
 }  // namespace pa_decode_detail

@@ -283,9 +283,10 @@ def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype, d):
 @pytest.mark.parametrize("d", [128, 64, 32])
 def test_assembly_loop_kernel_long_context_and_table_limit(d):
     """A 70 000-key context (more than a thousand tiles of slot-table entries) through the assembly-loop kernel,
-    and a table just past what that kernel's LDS tables hold (the host then launches the other matrix-core
-    kernel; under a sliding window the assembly-loop kernel still runs, its tables starting at the workgroup's
-    first tile): both against the vector kernel on the chunk's rows."""
+    and a table just past what that kernel's LDS tables hold (at head_dim 128 the instance that fills its tables
+    again runs, below that the host launches the other matrix-core kernel; under a sliding window the
+    assembly-loop kernel runs in any case, its tables starting at the workgroup's first tile): both against the
+    vector kernel on the chunk's rows."""
     announce(f"prefill assembly loop, long context d={d}")
     rng = np.random.default_rng(78)
     hq, hkv, bs = 4, 1, 16
@@ -302,6 +303,36 @@ def test_assembly_loop_kernel_long_context_and_table_limit(d):
             got = ops.prefill_paged(*args, window=window).float().cpu()
             want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu()
             assert_close(got, want, 2e-2, f"context of {ctx} keys, window {window}")
+
+
+def test_assembly_loop_kernel_table_refills_at_head_dim_128():
+    """Contexts longer than what the head_dim 128 kernel's LDS tables hold of them (it fills them again every 1 596
+    tiles of 64 keys): two refills with blocks missing on either side of the second and one block id past the pool;
+    a window that starts the workgroup far into such a context; and a context that is one block of a length that
+    is no multiple of 16, whose last group lies in the third fill.  Against the vector kernel on the chunk's rows."""
+    announce("prefill assembly loop, table refills d=128")
+    rng = np.random.default_rng(81)
+    d, hq, hkv, bs, chunk = 128, 4, 1, 16, 80
+    seg = 1596 * 64  # keys per fill of the tables
+    mk = lambda *shape: torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    ctx = 2 * seg + 5000
+    nblk = -(-ctx // bs)
+    blocks = rng.permutation(nblk).astype(np.int32)
+    blocks[2 * seg // bs - 3 : 2 * seg // bs + 2] = -1
+    blocks[seg // bs + 1] = nblk + 5
+    table = torch.from_numpy(blocks).reshape(1, -1).contiguous().to(DEV)
+    args = (0.3 * mk(chunk, hq, d), mk(nblk * bs, hkv, d), mk(nblk * bs, hkv, d), table, _i32([ctx]), _i32([chunk]), _i32([0]),
+            chunk, bs, d ** -0.5)
+    for window in (0, seg + 7000):
+        got = ops.prefill_paged(*args, window=window).float().cpu()
+        want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu()
+        assert_close(got, want, 2e-2, f"context of {ctx} keys, window {window}")
+    ctx = 2 * seg + 1111
+    args = (0.3 * mk(chunk, hq, d), mk(ctx, hkv, d), mk(ctx, hkv, d), torch.zeros(1, 1, dtype=torch.int32, device=DEV), _i32([ctx]),
+            _i32([chunk]), _i32([0]), chunk, ctx, d ** -0.5)
+    got = ops.prefill_paged(*args).float().cpu()
+    want = ops.prefill_paged(*args, rowwise=True).float().cpu()
+    assert_close(got, want, 2e-2, f"one block of {ctx} keys")
 
 
 @pytest.mark.parametrize("d", [256, 128, 64])

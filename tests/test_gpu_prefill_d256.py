@@ -134,25 +134,41 @@ def test_absent_blocks_and_short_tables(dtype):
             assert_close(got[b, :c], want[b, :c], 2e-2, f"block_size {bs} sequence {b}")
 
 
-def test_long_context_and_table_limit():
-    """A 70 000-key context (4 375 slot-table entries) through the matrix-core kernel; a table just past what
-    its LDS tables hold (the host then launches the vector kernel); and that context with a table cut to exactly
-    what they hold (the matrix-core kernel again: the keys past the table are absent, and the loop's look-ups
-    run past the tables' last tile).  All against the vector kernel on the chunk's rows."""
+def test_long_context_and_table_refills():
+    """A 70 000-key context (4 375 slot-table entries) through the matrix-core kernel; contexts longer than what
+    its LDS tables hold of them (the kernel fills the tables again every 3 064 tiles of 32 keys: one refill, and
+    two refills with blocks missing on either side of the second); a table cut short of the context (the keys past
+    it are absent); a window that starts the workgroup far into such a context; and a context that is one block of
+    a length that is no multiple of 16, whose last group lies in the third fill.  All against the vector kernel
+    on the chunk's rows."""
     announce("prefill d256 long context")
     rng = np.random.default_rng(904)
     hq, hkv, bs = 4, 1, 16
-    for ctx, table_len in ((70000, None), (6144 * 16 + 40, None), (6144 * 16 + 40, 6144)):
+    seg = 3064 * 32  # keys per fill of the tables
+    for ctx, table_len, window in ((70000, None, 0), (6144 * 16 + 40, None, 0), (6144 * 16 + 40, 6144, 0),
+                                   (2 * seg + 5000, None, 0), (2 * seg + 5000, None, seg + 7000)):
         chunk = 48
         nblk = -(-ctx // bs)
         kc = _randn(rng, (nblk * bs, hkv, D), torch.bfloat16).to(DEV)
         vc = _randn(rng, (nblk * bs, hkv, D), torch.bfloat16).to(DEV)
         q = _randn(rng, (chunk, hq, D), torch.bfloat16, 0.3).to(DEV)
-        table = torch.from_numpy(rng.permutation(nblk).astype(np.int32)[:table_len]).reshape(1, -1).contiguous().to(DEV)
+        blocks = rng.permutation(nblk).astype(np.int32)[:table_len]
+        if ctx > 2 * seg:  # blocks missing around the second refill, and one block id past the pool
+            blocks[2 * seg // bs - 3 : 2 * seg // bs + 2] = -1
+            blocks[seg // bs + 1] = nblk + 5
+        table = torch.from_numpy(blocks).reshape(1, -1).contiguous().to(DEV)
         args = (q, kc, vc, table, _i32([ctx]), _i32([chunk]), _i32([0]), chunk, bs, D ** -0.5)
-        got = ops.prefill_paged(*args).float().cpu()
-        want = ops.prefill_paged(*args, rowwise=True).float().cpu()
-        assert_close(got, want, 2e-2, f"context of {ctx} keys, table of {table.shape[1]} entries")
+        got = ops.prefill_paged(*args, window=window).float().cpu()
+        want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu()
+        assert_close(got, want, 2e-2, f"context of {ctx} keys, table of {table.shape[1]} entries, window {window}")
+    ctx, chunk = 2 * seg + 1111, 48
+    kc = _randn(rng, (ctx, hkv, D), torch.bfloat16).to(DEV)
+    vc = _randn(rng, (ctx, hkv, D), torch.bfloat16).to(DEV)
+    q = _randn(rng, (chunk, hq, D), torch.bfloat16, 0.3).to(DEV)
+    args = (q, kc, vc, torch.zeros(1, 1, dtype=torch.int32, device=DEV), _i32([ctx]), _i32([chunk]), _i32([0]), chunk, ctx, D ** -0.5)
+    got = ops.prefill_paged(*args).float().cpu()
+    want = ops.prefill_paged(*args, rowwise=True).float().cpu()
+    assert_close(got, want, 2e-2, f"one block of {ctx} keys")
 
 
 def test_c3_shape_at_head_dim_256_full_size():
