@@ -56,16 +56,15 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // rows): the kernel whose whole tile loop is scheduled assembly (one instance without, one with sliding window /
     // per-row first keys).  Its LDS copy of the table holds pa_asm_cap_tiles() tiles from the workgroup's first tile
     // on, which bounds the table's length - or, under a sliding window, the stretch of keys that the rows of a
-    // workgroup (at most kPfTasks blocks of kPfRows) see; at head_dim 128 longer tables take the instance that fills
-    // its copy again on the way.
+    // workgroup (at most kPfTasks blocks of kPfRows) see; longer tables take the instance that fills its copy again on
+    // the way.
     if (mfma && (head_dim == 128 || head_dim == 64 || head_dim == 32) && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
         bt_stride * (int64_t)block_size < (1ll << 31)) {
         const int64_t cap_keys = (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys;
         const bool fits = bt_stride * (int64_t)block_size <= cap_keys ||
                           (window > 0 && (int64_t)window + kPfTasks * kPfRows + 3 * kPfKeys <= cap_keys);
-        if (fits || head_dim == 128)
-            mfma = pa_prefill_asm_kernel(dtype, head_dim, window > 0 || row_first_key != nullptr, !fits);
+        mfma = pa_prefill_asm_kernel(dtype, head_dim, window > 0 || row_first_key != nullptr, !fits);
     }
     // head_dim 256: one 32-row task per wave, loads driven by a table of 16-key groups - which must lie inside one
     // pool block (block sizes that are multiples of 16, or a single block per sequence); the kernel fills its table

@@ -20,9 +20,8 @@
 //     a group's load then runs into the next block's rows, which are cleared like rows past the context end,
 //     and the one group at the end of the pool is fetched lane by lane when its tile is published;
 //   * the tables hold pa_asm_cap_tiles() tiles from the workgroup's first tile on; the LONG instance fills them
-//     again on the way when the workgroup runs more tiles than that (instantiated for head_dim 128);
-//   * the host launches prefill_mfma_kernel for other head sizes, for tables of several blocks that are not
-//     multiples of 16 keys long and, at head_dim 64 and 32, for tables past pa_asm_cap_tiles().
+//     again on the way when the workgroup runs more tiles than that;
+//   * the host launches prefill_mfma_kernel for tables of several blocks that are not multiples of 16 keys long.
 // Only the set-up, the first subtile's S^T and the write-out are compiled code, so the register allocator sees
 // one asm statement with pinned operands and little else.
 #pragma once
@@ -534,7 +533,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 }
 
 // nullptr unless the element type has this kernel; `lower_bounds`: the instance for sliding windows and per-row
-// first keys; `long_table`: the instance that fills its tables more than once (head_dim 128 only)
+// first keys; `long_table`: the instance that fills its tables more than once
 prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds, bool long_table);
 
 }  // namespace pa_decode_detail

@@ -78,8 +78,8 @@ constexpr float kPfSlack = 8.f;  // log2 of the factor by which a row's referenc
 
 // LDS tile geometry and swizzles for head_dim D (rows of D*2 bytes = CPR chunks of 16 bytes).
 // Tiles of 64 keys the slot tables of prefill_asm_kernel hold (they live in LDS behind the ring, which is 128 KiB at
-// head_dim 128 and smaller below), from the workgroup's first tile on: contexts of up to 102 400 keys at head_dim 128,
-// 262 144 at 64 and 32, longer ones under a sliding window.
+// head_dim 128 and smaller below), from the workgroup's first tile on: 102 400 keys at head_dim 128, 262 144 at 64 and
+// 32.  Workgroups that run more tiles take the instance that fills the tables again on the way.
 constexpr int pa_asm_cap_tiles(int head_dim) { return head_dim == 128 ? 1600 : 4096; }
 
 template <int D> struct PfTile {

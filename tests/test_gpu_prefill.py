@@ -283,10 +283,9 @@ def test_assembly_loop_kernel_absent_blocks_and_short_tables(dtype, d):
 @pytest.mark.parametrize("d", [128, 64, 32])
 def test_assembly_loop_kernel_long_context_and_table_limit(d):
     """A 70 000-key context (more than a thousand tiles of slot-table entries) through the assembly-loop kernel,
-    and a table just past what that kernel's LDS tables hold (at head_dim 128 the instance that fills its tables
-    again runs, below that the host launches the other matrix-core kernel; under a sliding window the
-    assembly-loop kernel runs in any case, its tables starting at the workgroup's first tile): both against the
-    vector kernel on the chunk's rows."""
+    and a table just past what that kernel's LDS tables hold (the instance that fills its tables again runs;
+    under a sliding window the other instance, its tables starting at the workgroup's first tile): both against
+    the vector kernel on the chunk's rows."""
     announce(f"prefill assembly loop, long context d={d}")
     rng = np.random.default_rng(78)
     hq, hkv, bs = 4, 1, 16
@@ -305,15 +304,16 @@ def test_assembly_loop_kernel_long_context_and_table_limit(d):
             assert_close(got, want, 2e-2, f"context of {ctx} keys, window {window}")
 
 
-def test_assembly_loop_kernel_table_refills_at_head_dim_128():
-    """Contexts longer than what the head_dim 128 kernel's LDS tables hold of them (it fills them again every 1 596
-    tiles of 64 keys): two refills with blocks missing on either side of the second and one block id past the pool;
+@pytest.mark.parametrize("d", [128, 64, 32])
+def test_assembly_loop_kernel_table_refills(d):
+    """Contexts longer than what the kernel's LDS tables hold of them (it fills them again every 1 596 tiles of 64
+    keys at head_dim 128, every 4 092 below): two refills with blocks missing on either side of the second and one block id past the pool;
     a window that starts the workgroup far into such a context; and a context that is one block of a length that
     is no multiple of 16, whose last group lies in the third fill.  Against the vector kernel on the chunk's rows."""
-    announce("prefill assembly loop, table refills d=128")
+    announce(f"prefill assembly loop, table refills d={d}")
     rng = np.random.default_rng(81)
-    d, hq, hkv, bs, chunk = 128, 4, 1, 16, 80
-    seg = 1596 * 64  # keys per fill of the tables
+    hq, hkv, bs, chunk = 4, 1, 16, 80
+    seg = (1596 if d == 128 else 4092) * 64  # keys per fill of the tables
     mk = lambda *shape: torch.from_numpy(rng.standard_normal(shape).astype(np.float32)).to(torch.bfloat16).to(DEV)
     ctx = 2 * seg + 5000
     nblk = -(-ctx // bs)
