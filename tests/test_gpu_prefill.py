@@ -327,6 +327,12 @@ def test_assembly_loop_kernel_table_refills(d):
         got = ops.prefill_paged(*args, window=window).float().cpu()
         want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu()
         assert_close(got, want, 2e-2, f"context of {ctx} keys, window {window}")
+    # per-row first keys: the chunk's first half belongs to a document that starts at key 1000, the rest to one that
+    # starts with row 40
+    first = torch.tensor([1000] * 40 + [ctx - chunk + 40] * (chunk - 40), dtype=torch.int32, device=DEV)
+    got = ops.prefill_paged(*args, row_first_key=first).float().cpu()
+    want = ops.prefill_paged(*args, row_first_key=first, rowwise=True).float().cpu()
+    assert_close(got, want, 2e-2, f"context of {ctx} keys, per-row first keys")
     ctx = 2 * seg + 1111
     args = (0.3 * mk(chunk, hq, d), mk(ctx, hkv, d), mk(ctx, hkv, d), torch.zeros(1, 1, dtype=torch.int32, device=DEV), _i32([ctx]),
             _i32([chunk]), _i32([0]), chunk, ctx, d ** -0.5)

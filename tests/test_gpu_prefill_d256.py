@@ -161,6 +161,12 @@ def test_long_context_and_table_refills():
         got = ops.prefill_paged(*args, window=window).float().cpu()
         want = ops.prefill_paged(*args, window=window, rowwise=True).float().cpu()
         assert_close(got, want, 2e-2, f"context of {ctx} keys, table of {table.shape[1]} entries, window {window}")
+    # per-row first keys over the last of these contexts: a document that starts at key 1000, then one that starts
+    # with row 20
+    first = torch.tensor([1000] * 20 + [ctx - chunk + 20] * (chunk - 20), dtype=torch.int32, device=DEV)
+    got = ops.prefill_paged(*args, row_first_key=first).float().cpu()
+    want = ops.prefill_paged(*args, row_first_key=first, rowwise=True).float().cpu()
+    assert_close(got, want, 2e-2, f"context of {ctx} keys, per-row first keys")
     ctx, chunk = 2 * seg + 1111, 48
     kc = _randn(rng, (ctx, hkv, D), torch.bfloat16).to(DEV)
     vc = _randn(rng, (ctx, hkv, D), torch.bfloat16).to(DEV)
