@@ -8,7 +8,7 @@ JSON line; with the default workload the line also carries short runs of the
 other configurations (c2, c5 decode, c3 append + chunked prefill) under
 ``secondary``.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1|c3|c3-d256|c3-d64|engine] [--no-secondary]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1|c3|c3-d256|c3-d64|long-d128|long-d256|engine] [--no-secondary]
     python bench.py --traffic-from-pmc NAME KERNEL FETCH.csv WRITE.csv   # refresh profiles/traffic.json
 """
 
@@ -89,7 +89,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c3-d256", "c3-d64", "c4", "c5", "engine"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c3-d256", "c3-d64", "long-d128", "long-d256", "c4", "c5", "engine"])
     ap.add_argument("--preheat-s", type=float, default=0.5,
                     help="seconds of untimed steps before the warmup steps: an idle GPU sits at its lowest clocks "
                          "and takes a few hundred milliseconds of work to leave them")
@@ -375,6 +375,62 @@ def bench_prefill_head(args, dev, name) -> dict:
     }
 
 
+# one long sequence: workload -> (query heads, kv heads, head_dim, seed, kernel)
+PREFILL_LONG_SHAPES = {"long-d128": (8, 2, 128, 1008, "prefill_asm_kernel"),
+                       "long-d256": (8, 2, 256, 1009, "prefill_d256_kernel")}
+
+
+def bench_prefill_long(args, dev, name) -> dict:
+    """A 2048-token chunk of ONE sequence behind 200 000 cached keys (16-token blocks in random pool order, bf16,
+    8 query / 2 kv heads): more keys than the prefill kernels' LDS slot tables hold, so the instances that fill them
+    again on the way run; few rows, so the launch has 64 (head_dim 128) or 128 (256) workgroups for 256 CUs."""
+    from research_amd import ops
+
+    hq, hkv, head_dim, seed, kernel = PREFILL_LONG_SHAPES[name]
+    P, C, bs = 200_000, 2048, 16
+    nblk = -(-(P + C) // bs)
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    kc = torch.randn(nblk * bs, hkv, head_dim, device=dev, dtype=torch.bfloat16, generator=gen)
+    vc = torch.randn(nblk * bs, hkv, head_dim, device=dev, dtype=torch.bfloat16, generator=gen)
+    q = torch.randn(C, hq, head_dim, device=dev, dtype=torch.bfloat16, generator=gen)
+    tables = torch.randperm(nblk, device=dev, generator=gen).to(torch.int32).reshape(1, -1).contiguous()
+    ctx = torch.tensor([P + C], dtype=torch.int32, device=dev)
+    ql = torch.tensor([C], dtype=torch.int32, device=dev)
+    qs = torch.zeros(1, dtype=torch.int32, device=dev)
+    out = torch.empty_like(q)
+    scale = head_dim ** -0.5
+
+    def prefill():
+        ops.prefill_paged(q, kc, vc, tables, ctx, ql, qs, C, bs, scale, out=out)
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    preheat(prefill, args.preheat_s)
+    for _ in range(args.warmup):
+        prefill()
+    ms_step, ms_step_median = timed_steps(prefill, args.steps)
+    ms_kernel = timed_ms(prefill, max(args.steps, KERNEL_LAUNCHES))
+    flops = 4 * head_dim * hq * (C * P + C * (C + 1) // 2)  # two products, every visible (row, key) pair
+    achieved = flops / (ms_kernel * 1e-3) / 1e12
+    return {
+        "metric": "prefill-attn TFLOP/s", "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "tokens_per_s": C / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_median": ms_step_median,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"one sequence, chunked prefill, 200000 + 2048, {hq} q / {hkv} kv heads of {head_dim}, bf16",
+                   "num_seqs": 1, "prefix_len": P, "chunk_len": C, "num_q_heads": hq, "num_kv_heads": hkv,
+                   "head_dim": head_dim, "block_size": bs, "attention_flops": flops, "seed": seed},
+        "roofline": {"bound": "mfma", "kernel": kernel, "achieved": achieved,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": measured_traffic(name), "kernel_ms": ms_kernel,
+                     "kernel_launches": max(args.steps, KERNEL_LAUNCHES)},
+    }
+
+
 def bench_engine(args, dev) -> int:
     """The engine loop on a Qwen2.5-0.5B-shaped model with random weights (24 layers, 14 query / 2 kv heads of
     64, vocabulary 151 936, bf16): 8 prompts of 512 tokens, 16 rollouts each, 64 new tokens per rollout at
@@ -636,6 +692,8 @@ def main() -> int:
         return bench_engine(args, dev)
     if args.workload in PREFILL_HEAD_SHAPES:
         result = bench_prefill_head(args, dev, args.workload)
+    elif args.workload in PREFILL_LONG_SHAPES:
+        result = bench_prefill_long(args, dev, args.workload)
     else:
         result = bench_prefill_c3(args, dev) if args.workload == "c3" else bench_decode(args.workload, args, dev)
     if args.workload == "c4" and not args.no_secondary:
