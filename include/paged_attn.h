@@ -45,7 +45,7 @@ extern "C" {
 #define PA_F16 2
 #define PA_FP8_E4M3 3 /* OCP e4m3fn, KV pool only; q/out stay 16- or 32-bit */
 
-/* Library ABI version (bumped when an entry point is added or a signature changes; now 4). */
+/* Library ABI version (bumped when an entry point is added or a signature or contract changes; now 5). */
 int pa_version(void);
 
 /* Text of the calling thread's most recent error; "" if none. */
@@ -94,10 +94,15 @@ int pa_kv_gather(const void *k_cache, const void *v_cache, void *k_out, void *v_
  * grid of workgroups; a sequence whose blocks fall into several workgroups
  * leaves one partial result per piece in the workspace.  The size depends on
  * the shapes only, never on the sequence lengths, so one allocation serves
- * every step of a model.  Alignment: 256 bytes.  Contents need not be
- * initialised (a call recognises what an earlier call or nobody left there);
- * calls that share a workspace must not overlap in time.
+ * every step of a model.  Alignment: 256 bytes.  The first
+ * PA_DECODE_TICKET_BYTES bytes hold the arrival counters of the merge inside
+ * the split pass: zero-fill them once after allocating the workspace (before
+ * its first use; outside any stream capture) and leave them to the library
+ * afterwards - every call returns them to "nothing arrived", whatever its
+ * shapes, so captured graphs replay without clearing anything.  The rest need
+ * not be initialised.  Calls that share a workspace must not overlap in time.
  */
+#define PA_DECODE_TICKET_BYTES (512u << 10)
 size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads, int head_dim,
                                  int kv_dtype);
 
@@ -132,8 +137,8 @@ int pa_decode_passes(int batch, int num_q_heads, int num_kv_heads, int head_dim,
  *                   seq_lens[b]-1; blocks wholly before the window are never read.  The reference's own
  *                   decode applies a window only through a caller-built ctx.block_mask
  *                   (flex_backend.py:220-225).  Not combinable with extra_zero_keys.
- *   batch         : at most 8192 sequences per call
- *   workspace     : pa_decode_workspace_bytes(...) bytes
+ *   batch         : any; more than 8192 sequences are taken 8192 at a time, one after the other on the stream
+ *   workspace     : pa_decode_workspace_bytes(...) bytes, its first PA_DECODE_TICKET_BYTES zero-filled once
  *   A sequence of length 0 yields zeros.
  */
 int pa_decode(const void *q, const void *k_cache, const void *v_cache, void *out,

@@ -46,6 +46,7 @@ using namespace pa_decode_detail;
 
 namespace {
 
+static_assert(PA_DECODE_TICKET_BYTES == kPlanTicketBytes, "paged_attn.h and decode_plan.h disagree on the ticket region");
 constexpr int kMaxSplitGrid = kPlanMaxSplitGrid;  // upper bound of the split pass's grid, fixes the workspace size
 
 constexpr int kMaxDevices = 64;
@@ -120,9 +121,6 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     if (!ks.split)
         return pa_fail(PA_ERR_UNSUPPORTED, "pa_decode: no kernel for q_dtype=%d kv_dtype=%d head_dim=%d", q_dtype,
                        kv_dtype, head_dim);
-    PA_REQUIRE(batch <= kMaxBatch, "batch=%d above the %d sequences one call handles", batch, kMaxBatch);
-    PA_REQUIRE(plan_split_lds_bytes(batch, head_dim, pa_dtype_bytes(kv_dtype), nrep_t) <= 65536,
-               "batch=%d needs more than 64 KB of LDS per workgroup", batch);
     if (batch == 0) return PA_OK;
     PA_REQUIRE(q && out && seq_lens, "NULL q / out / seq_lens");
     PA_REQUIRE(k_cache && v_cache, "NULL cache pointer");
@@ -130,6 +128,23 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     PA_REQUIRE(kv_dtype != PA_FP8_E4M3 || (k_scale && v_scale), "fp8 KV needs k_scale and v_scale");
     PA_REQUIRE(pa_aligned16(k_cache) && pa_aligned16(v_cache) && pa_aligned16(q),
                "q and cache pointers must be 16-byte aligned");
+    if (batch > kMaxBatch) {
+        // The block prefix sums of a launch live in LDS: a larger batch is taken kMaxBatch sequences at a time, one
+        // after the other on the stream, all through the same workspace (sized for kMaxBatch sequences).
+        const size_t q_row = (size_t)num_q_heads * head_dim * pa_dtype_bytes(q_dtype);
+        for (int at = 0; at < batch; at += kMaxBatch) {
+            const int rc = decode_launch(
+                phases, (const char *)q + at * q_row, k_cache, v_cache, (char *)out + at * q_row,
+                block_tables ? block_tables + (int64_t)at * bt_stride : nullptr, bt_stride, seq_lens + at,
+                extra_zero_keys ? extra_zero_keys + at : nullptr, k_scale, v_scale,
+                batch - at < kMaxBatch ? batch - at : kMaxBatch, num_q_heads, num_kv_heads, head_dim, block_size,
+                num_blocks, scale, window, q_dtype, kv_dtype, workspace, workspace_bytes, stream, use_static);
+            if (rc != PA_OK) return rc;
+        }
+        return PA_OK;
+    }
+    PA_REQUIRE(plan_split_lds_bytes(batch, head_dim, pa_dtype_bytes(kv_dtype), nrep_t) <= 65536,
+               "batch=%d needs more than 64 KB of LDS per workgroup", batch);
     const int grid = split_grid();
     // A caller's workspace is sized without asking the device (kMaxSplitGrid workgroups); the library's own
     // scratch is laid out for the grid this device really gets, which is what makes its fixed size go far.
@@ -162,11 +177,11 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     a.tickets = (unsigned long long *)(ws + w.ticket_off);
     a.part_ml = (float *)(ws + w.ml_off);
     a.part_acc = (float *)(ws + w.acc_off);
-    // Batches that leave a sequence few pieces are finished by the split pass alone; the tag tells this launch's
-    // tickets from whatever the workspace held before.
+    // Batches that leave a sequence few pieces are finished by the split pass alone; the tag (the launch number,
+    // 1 .. 2^40 - 1) tells this launch's tickets from those of the launches before it.
     static std::atomic<unsigned long long> launches{0};
     a.merge_in_split = phases == (kPhaseSplit | kPhaseReduce) && plan_merge_in_split(batch, plan, grid) ? 1 : 0;
-    a.ticket_tag = ((launches.fetch_add(1, std::memory_order_relaxed) + 1) * 0x9E3779B97F4A7C15ull) >> 24;
+    a.ticket_tag = launches.fetch_add(1, std::memory_order_relaxed) % ((1ull << 40) - 1) + 1;
 
     hipStream_t s = (hipStream_t)stream;
     a.split_grid = grid;
@@ -203,13 +218,14 @@ extern "C" size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_
         return 0;
     }
     const HeadPlan plan = plan_heads(num_q_heads, num_kv_heads, head_dim, pa_dtype_bytes(kv_dtype));
-    return plan_workspace(batch, plan, head_dim, kMaxSplitGrid).total;
+    return plan_workspace(batch < kMaxBatch ? batch : kMaxBatch, plan, head_dim, kMaxSplitGrid).total;
 }
 
 extern "C" int pa_decode_passes(int batch, int num_q_heads, int num_kv_heads, int head_dim, int kv_dtype) {
     pa_clear_error();
     const HeadPlan plan = plan_heads(num_q_heads, num_kv_heads, head_dim, pa_dtype_bytes(kv_dtype));
     if (batch < 0 || !plan.nrep_t) return pa_fail(PA_ERR_UNSUPPORTED, "pa_decode_passes: no kernel for these shapes");
+    if (batch > kMaxBatch) batch = kMaxBatch;  // launches per group of kMaxBatch sequences
     return plan_merge_in_split(batch, plan, split_grid()) ? 1 : 2;
 }
 

@@ -67,7 +67,7 @@ struct DecodeArgs {
     float *part_ml;         // [slot_cap][hpw*NREP][2]
     int32_t *block_prefix;  // [batch+1], written by the split pass for the reduction pass
     unsigned long long *tickets;  // [planes*batch]: (launch tag << 24) | pieces of the (plane, sequence) that have arrived
-    unsigned long long ticket_tag;  // 40-bit tag of this launch: a ticket with another tag counts as zero
+    unsigned long long ticket_tag;  // 40-bit tag of this launch (never 0): a ticket with another tag counts as zero
     int merge_in_split;     // the workgroup that delivers a sequence's last piece merges the pieces (no second pass)
 };
 
@@ -444,17 +444,22 @@ __device__ __forceinline__ float2 ld_coherent(const float *p) {
                                                    __HIP_MEMORY_SCOPE_AGENT);
     return float2{__builtin_bit_cast(float, (uint32_t)v), __builtin_bit_cast(float, (uint32_t)(v >> 32))};
 }
+// Every memory access this thread has issued is complete (a device-scope store has then reached the memory side),
+// and the compiler moves no access across this point.
+__device__ __forceinline__ void wait_all_memory() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void compiler_fence() { asm volatile("" ::: "memory"); }
 
 // One piece of a (plane, sequence) has been written to the workspace: count it; true for the arrival that completes
-// the sequence.  A ticket is (tag of the launch << 24 | arrivals so far); a ticket carrying another tag is left
-// over from an earlier launch (or was never written) and counts as zero, so the workspace needs no initialisation,
-// and the completing arrival stores zero arrivals, so a replay of the same launch (a captured graph replays with
-// the same tag) starts clean as well.  Called by one thread, after the workgroup's stores were fenced.
+// the sequence.  A ticket is (tag of the launch << 24 | arrivals so far).  The ticket region is zero when the
+// workspace is first used; the completing arrival stores zero arrivals under its own tag, and a ticket carrying
+// another launch's tag counts as zero, so every launch - also a replay of a captured graph, which carries the tag
+// it was recorded with - finds every ticket at zero arrivals.  Tags are consecutive launch numbers, so a launch
+// never meets its own tag from an earlier one.  Called by one thread, after the workgroup's stores are complete.
 __device__ __forceinline__ bool piece_arrived_last(unsigned long long *ticket, unsigned long long tag, int n_pieces) {
     unsigned long long old = __hip_atomic_load(ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     for (;;) {  // ends after at most n_pieces rounds: a failed exchange means another piece was counted
         const unsigned long long cnt = (old >> 24) == tag ? (old & 0xffffffull) : 0ull;
-        const bool last = cnt + 1 == (unsigned long long)n_pieces;
+        const bool last = cnt + 1 >= (unsigned long long)n_pieces;
         const unsigned long long neu = (tag << 24) | (last ? 0ull : cnt + 1);
         if (__hip_atomic_compare_exchange_strong(ticket, &old, neu, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
                                                  __HIP_MEMORY_SCOPE_AGENT))
@@ -646,11 +651,12 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
                 // the piece; the workgroup whose piece completes the sequence reads all of them back and merges.
                 const int64_t u0 = plane * per_plane + s_prefix[b];
                 const int w0 = owner_of(u0, total, grid), w1 = owner_of(u0 + nblk - 1, total, grid);
-                __builtin_amdgcn_s_waitcnt(0);  // this thread's stores have reached the memory side
+                wait_all_memory();  // this thread's stores have reached the memory side
                 __syncthreads();
                 if (tid == 0)
                     s_last = piece_arrived_last(a.tickets + ((int64_t)plane * B + b), a.ticket_tag, w1 - w0 + 1);
                 __syncthreads();
+                compiler_fence();  // the pieces are read after the count, never before
                 if (s_last) merge_pieces<QT, D, NREP>(a, plane, b, hg, rep0, w0, w1, tid);  // uniform
             }
         }

@@ -17,6 +17,11 @@ namespace pa_decode_detail {
 constexpr int kPlanMaxBatch = 8192;      // sequences per call (their block prefix sum lives in LDS)
 constexpr int kPlanMaxSplitGrid = 4096;  // upper bound of the split pass's grid, fixes the caller's workspace size
 constexpr int kPlanMinUnitsPerWorkgroup = 4;
+// Arrival tickets of the merge inside the split pass: one 64-bit word per (plane, sequence), in a region of fixed
+// size at the start of every workspace so that calls of any shape use the same bytes for the same purpose and
+// nothing else is ever written there.  The caller zero-fills the region once; every call leaves it counting zero.
+constexpr int kPlanTicketSlots = 65536;
+constexpr size_t kPlanTicketBytes = (size_t)kPlanTicketSlots * 8;
 
 // How the heads are spread over wave loads and planes (a plane = one group of hpw kv heads x one group of <= nrep_t
 // query heads per kv head).  lpr lanes of 16 bytes hold one K/V row; a wave load covers rpw = 64/lpr rows, mapped
@@ -74,7 +79,7 @@ PA_PLAN_FN int plan_effective_grid(int64_t total, int grid) {
 // order both w and plane*batch + sequence only grow.
 PA_PLAN_FN int64_t plan_slot(int w, int plane, int batch, int b) { return (int64_t)w + (int64_t)plane * batch + b; }
 
-// workspace = [block_prefix int32[batch+1]] [tickets uint64[planes*batch]] [part_ml float[slots][heads][2]]
+// workspace = [tickets uint64[kPlanTicketSlots]] [block_prefix int32[batch+1]] [part_ml float[slots][heads][2]]
 //             [part_acc float[slots][heads][D]], heads = hpw*nrep_t query heads of one plane,
 // slots = grid_cap + planes*batch (slot indices stay below grid + planes*batch - 1).
 struct WsPlan {
@@ -87,9 +92,9 @@ PA_PLAN_FN WsPlan plan_workspace(int batch, const HeadPlan &h, int head_dim, int
     const size_t heads = (size_t)h.heads_per_slot();
     const size_t keys = (size_t)h.planes() * (size_t)batch;
     w.slots = (int64_t)grid_cap + (int64_t)keys;
-    w.prefix_off = 0;
-    w.ticket_off = plan_align_up((size_t)(batch + 1) * 4, 256);
-    w.ml_off = w.ticket_off + plan_align_up(keys * 8, 256);
+    w.ticket_off = 0;
+    w.prefix_off = kPlanTicketBytes;
+    w.ml_off = w.prefix_off + plan_align_up((size_t)(batch + 1) * 4, 256);
     w.acc_off = w.ml_off + plan_align_up((size_t)w.slots * heads * 2 * 4, 256);
     w.total = w.acc_off + plan_align_up((size_t)w.slots * heads * (size_t)head_dim * 4, 256);
     return w;
@@ -124,7 +129,8 @@ PA_PLAN_FN constexpr size_t plan_split_lds_bytes(int batch, int head_dim, int kv
 // round trip to the memory side before its next part - and a few long sequences spread over the whole grid are
 // merged much faster by the second launch, whose workgroups take one output row each.
 PA_PLAN_FN bool plan_merge_in_split(int batch, const HeadPlan &h, int grid) {
-    return (int64_t)grid <= 2 * (int64_t)h.planes() * batch;
+    const int64_t keys = (int64_t)h.planes() * batch;  // one ticket each
+    return (int64_t)grid <= 2 * keys && keys <= kPlanTicketSlots;
 }
 
 }  // namespace pa_decode_detail

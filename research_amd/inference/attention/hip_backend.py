@@ -35,10 +35,12 @@ Differences of ``HipPagedAttentionBackend`` from the reference, all deliberate:
   the default ``True`` attends the last ``window`` keys, consistent with prefill.
 * ``ctx.block_mask`` takes the ``PagedMask`` objects of ``attention/mask.py``
   (causal, sliding window, packed documents): a window becomes the kernels'
-  ``window`` argument and documents become one first key per query row.  Any
-  other object (a FlexAttention ``BlockMask``, an arbitrary predicate) raises
+  ``window`` argument and documents become one first key per query row.  A
+  ``mask_mod(b, h, q_idx, kv_idx)`` callable, or an object that carries one (a
+  FlexAttention ``BlockMask``), is evaluated once per context, packed into bits
+  and applied by the general masked kernel.  Anything else raises
   ``NotImplementedError`` instead of being ignored.  A document mask describes
-  packed prefill rows; in decode it raises as well.
+  packed prefill rows; in decode it raises.
 """
 
 from __future__ import annotations
@@ -339,7 +341,8 @@ class HipPagedAttentionBackend:
             if self._workspace is not None:
                 have = self._workspace.numel()
                 self._retired_workspaces.append(self._workspace)
-            self._workspace = torch.empty(max(nbytes, 2 * have, 1 << 20), dtype=torch.uint8,
+            # zero-filled: the arrival counters at the start of a workspace must read zero before its first use
+            self._workspace = torch.zeros(max(nbytes, 2 * have, 1 << 20), dtype=torch.uint8,
                                           device=self.k_cache.device)
         return self._workspace
 
@@ -474,12 +477,18 @@ class HipPagedAttentionBackend:
                     raise TypeError("a device-resident seq_lens must be a contiguous int32 tensor")
                 step.seq_lens = ctx.seq_lens[:batch]
                 if self.pad_zero_keys and batch > 0:
-                    step.extra_zero = (step.seq_lens.max() - step.seq_lens).to(torch.int32)
+                    step.extra_zero = torch.zeros(batch, dtype=torch.int32, device=step.seq_lens.device)
             else:
                 lens = self._lens(ctx.seq_lens, batch)
                 step.seq_lens = self._to_device(lens.astype(np.int32))
                 if self.pad_zero_keys and batch > 0:
                     step.extra_zero = self._to_device((lens.max() - lens).astype(np.int32))
+        if (self.pad_zero_keys and batch > 0 and layer_idx == 0 and isinstance(ctx.seq_lens, Tensor)
+                and ctx.seq_lens.device.type == "cuda"):
+            # Lengths that live on the device may have been rewritten since the last pass (a caller replaying a
+            # captured graph does exactly that), so the padding counts are recomputed from them at the first
+            # layer of every pass, into the buffer every layer reads: a capture records these two operations.
+            torch.sub(step.seq_lens.max(), step.seq_lens, out=step.extra_zero)
         q3 = q.contiguous().view(batch, num_heads, head_dim)
         ws = self._workspace_for(
             ops.decode_workspace_bytes(batch, num_heads, cfg.num_kv_heads, head_dim, self.k_cache.dtype))

@@ -70,10 +70,11 @@ def decode_workspace_bytes(batch: int, num_q_heads: int, num_kv_heads: int, head
 
 
 def decode_workspace(q: Tensor, k_cache: Tensor) -> Tensor:
-    """A fresh workspace tensor sized for ``decode(q, k_cache, ...)``."""
+    """A fresh workspace tensor sized for ``decode(q, k_cache, ...)``, zero-filled: the library's arrival
+    counters at its start must read zero before the first call that uses them."""
     batch, hq, d = q.shape
     n = decode_workspace_bytes(batch, hq, k_cache.shape[1], d, k_cache.dtype)
-    return torch.empty(n, dtype=torch.uint8, device=q.device)
+    return torch.zeros(n, dtype=torch.uint8, device=q.device)
 
 
 def decode(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, seq_lens: Tensor, block_size: int,

@@ -41,9 +41,10 @@ extern "C" int pa_plan_replay(const int32_t *seq_lens, int batch, int num_q_head
     stats[7] = (int64_t)ws.total;
     if (plan_split_lds_bytes(batch, head_dim, kv_elem_bytes, h.nrep_t) > 65536) FAIL("workgroup LDS above 64 KB");
     // layout: regions in order, aligned, inside the total
-    if (!(ws.prefix_off == 0 && ws.ticket_off >= (size_t)(batch + 1) * 4 && ws.ml_off >= ws.ticket_off + (size_t)planes * batch * 8 &&
+    if (!(ws.ticket_off == 0 && ws.prefix_off >= kPlanTicketBytes && ws.ml_off >= ws.prefix_off + (size_t)(batch + 1) * 4 &&
+          (!plan_merge_in_split(batch, h, launch_grid) || (size_t)planes * batch * 8 <= kPlanTicketBytes) &&
           ws.acc_off >= ws.ml_off + (size_t)ws.slots * h.heads_per_slot() * 8 &&
-          ws.total >= ws.acc_off + (size_t)ws.slots * h.heads_per_slot() * head_dim * 4 && ws.ticket_off % 256 == 0 &&
+          ws.total >= ws.acc_off + (size_t)ws.slots * h.heads_per_slot() * head_dim * 4 && ws.prefix_off % 256 == 0 &&
           ws.ml_off % 256 == 0 && ws.acc_off % 256 == 0))
         FAIL("workspace regions overlap or are misaligned");
     if (total == 0) return 0;

@@ -33,7 +33,7 @@ def test_binding_table_matches_header():
 
 def test_version_and_dtype_sizes():
     lib = _lib.load()
-    assert lib.pa_version() == 4
+    assert lib.pa_version() == 5
     assert [lib.pa_dtype_bytes(c) for c in (0, 1, 2, 3, 4, -1)] == [4, 2, 2, 1, 0, 0]
 
 
@@ -99,8 +99,12 @@ def test_decode_argument_errors():
     assert rc == _lib.PA_ERR_WORKSPACE and "need" in msg
     rc, msg = _status("pa_decode", *_decode_args(ws=None))
     assert rc == _lib.PA_ERR_WORKSPACE
-    rc, msg = _status("pa_decode", *_decode_args(batch=10000))
-    assert rc == _lib.PA_ERR_INVALID_ARG and "sequences one call handles" in msg
+    # more than 8192 sequences are taken 8192 at a time through a workspace sized for 8192
+    lib = _lib.load()
+    assert (lib.pa_decode_workspace_bytes(10000, 32, 8, 128, _lib.PA_BF16)
+            == lib.pa_decode_workspace_bytes(8192, 32, 8, 128, _lib.PA_BF16))
+    rc, msg = _status("pa_decode", *_decode_args(batch=10000, ws_bytes=1024))
+    assert rc == _lib.PA_ERR_WORKSPACE
     rc, msg = _status("pa_decode", *_decode_args(q=None))
     assert rc == _lib.PA_ERR_INVALID_ARG and "NULL" in msg
     assert _status("pa_decode", *_decode_args(batch=0, q=None, ws=None, ws_bytes=0))[0] == _lib.PA_OK

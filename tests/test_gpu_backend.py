@@ -492,3 +492,52 @@ def test_fp8_blocks_dequantise_bit_exact_and_chunked_prefill_over_an_fp8_pool():
     want = po.paged_prefill_chunk(q, kd, vd, tables, prefix, chunk, bs, backend.scale)
     for b, c in enumerate(chunk):
         assert_close(out[b, :c], want[b, :c], 6e-2, f"sequence {b}")
+
+
+def test_reference_numerics_replayed_from_a_graph_with_lengths_rewritten_in_place():
+    """``FlexAttentionBackend`` (zero-padded ragged decode) on a context whose lengths live on the device: an eager
+    warm-up on the same context object, then a captured two-layer decode pass replayed with the lengths rewritten
+    between the replays.  The padding counts follow the lengths of each replay."""
+    announce("backend pad_zero_keys decode from a graph")
+    w = make_decode("c2", batch=7, len_range=(20, 300), seed=12)
+    config = CacheConfig(num_layers=2, num_kv_heads=8, head_dim=128, num_blocks=w.num_blocks, block_size=16,
+                         device="cuda", dtype=torch.bfloat16)
+    backend = FlexAttentionBackend(config)
+    backend.set_num_heads(16)
+    for layer in range(2):
+        backend.k_cache[layer].copy_(w.k_pool.cuda())
+        backend.v_cache[layer].copy_(w.v_pool.cuda())
+    tables = [t.tolist() for t in w.block_tables]
+    lens_dev = torch.zeros(7, dtype=torch.int32, device="cuda")  # the warm-up sees empty sequences
+    ctx = InferenceContext(is_prefill=False, block_tables=torch.from_numpy(w.padded_tables().astype(np.int32)).cuda(),
+                           seq_lens=lens_dev)
+    q = torch.zeros(7, 1, 16, 128, dtype=torch.bfloat16, device="cuda")
+    outs = [torch.empty_like(q) for _ in range(2)]
+
+    def one_pass():
+        for layer in range(2):
+            outs[layer].copy_(backend.forward(q, None, None, layer, ctx))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        one_pass()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        one_pass()
+    rng = np.random.default_rng(4)
+    full = np.asarray(w.seq_lens)
+    for it in range(4):
+        lens = np.maximum(1, full - rng.integers(0, 19, 7) * (it + 1)).astype(np.int32)
+        qh = torch.from_numpy(rng.standard_normal((7, 16, 128)).astype(np.float32)).to(torch.bfloat16)
+        q.copy_(qh[:, None].cuda())
+        lens_dev.copy_(torch.from_numpy(lens).cuda())
+        graph.replay()
+        torch.cuda.synchronize()
+        want = po.paged_decode(qh, w.k_pool, w.v_pool, tables, lens.tolist(), 16, w.scale, pad_zero_keys=True)
+        for layer in range(2):
+            assert_close(outs[layer][:, 0], want, 2e-2, f"replay {it} layer {layer}")
+        exact = po.paged_decode(qh, w.k_pool, w.v_pool, tables, lens.tolist(), 16, w.scale)
+        assert np.abs(exact - want).max() > 1e-3  # the two semantics differ on this batch, so the test can tell
+        (torch.ones(1000, device="cuda") * 2).sum().item()
