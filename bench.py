@@ -130,7 +130,9 @@ def cpu_baseline(w, budget_s: float):
         done_tokens += int(lens[sl].sum())
         at = (at + n) % len(lens)
     dt = time.perf_counter() - t0
-    kv_size = w.q.element_size()
+    # the same bytes per key as the GPU figure counts: one per element of an fp8 pool (the CPU path itself reads
+    # the dequantised 16-bit copy)
+    kv_size = 1 if w.kv_format == "fp8_e4m3" else w.q.element_size()
     sample_bytes = done_tokens * w.num_kv_heads * w.head_dim * 2 * kv_size
     return {
         "value": sample_bytes / dt / 1e9,
@@ -244,7 +246,7 @@ def bench_prefill_c3(args, dev) -> dict:
     preheat(step, args.preheat_s)
     for _ in range(args.warmup):
         step()
-    ms_step, ms_step_median = timed_steps(step, args.steps)
+    ms_step_mean, ms_step = timed_steps(step, args.steps)
     ms_prefill = timed_ms(prefill, max(args.steps, KERNEL_LAUNCHES))
     ms_append = timed_ms(append, max(args.steps, KERNEL_LAUNCHES))
     # The same append with the rotary embedding of q and k fused in (the step a model runs right before this
@@ -274,7 +276,7 @@ def bench_prefill_c3(args, dev) -> dict:
     result = {
         "metric": "prefill-attn TFLOP/s", "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
         "tokens_per_s": S * C / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_median": ms_step_median,
+        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_mean": ms_step_mean, "step_statistic": "median of the timed steps",
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic",
         "config": {"workload": "c3 shared-prefix chunked prefill + KV append, 32 x (2048 + 256), bf16",
@@ -355,14 +357,14 @@ def bench_prefill_head(args, dev, name) -> dict:
     preheat(prefill, args.preheat_s)
     for _ in range(args.warmup):
         prefill()
-    ms_step, ms_step_median = timed_steps(prefill, args.steps)
+    ms_step_mean, ms_step = timed_steps(prefill, args.steps)
     ms_kernel = timed_ms(prefill, max(args.steps, KERNEL_LAUNCHES))
     flops = w.attention_flops()
     achieved = flops / (ms_kernel * 1e-3) / 1e12
     return {
         "metric": "prefill-attn TFLOP/s", "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
         "tokens_per_s": S * C / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_median": ms_step_median,
+        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_mean": ms_step_mean, "step_statistic": "median of the timed steps",
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"c3 shape at head_dim {head_dim}: chunked prefill, 32 x (2048 + 256), {hq} q / {hkv} kv heads, bf16",
                    "num_seqs": S, "prefix_len": P, "chunk_len": C, "num_q_heads": w.num_q_heads,
@@ -412,14 +414,14 @@ def bench_prefill_long(args, dev, name) -> dict:
     preheat(prefill, args.preheat_s)
     for _ in range(args.warmup):
         prefill()
-    ms_step, ms_step_median = timed_steps(prefill, args.steps)
+    ms_step_mean, ms_step = timed_steps(prefill, args.steps)
     ms_kernel = timed_ms(prefill, max(args.steps, KERNEL_LAUNCHES))
     flops = 4 * head_dim * hq * (C * P + C * (C + 1) // 2)  # two products, every visible (row, key) pair
     achieved = flops / (ms_kernel * 1e-3) / 1e12
     return {
         "metric": "prefill-attn TFLOP/s", "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
         "tokens_per_s": C / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_median": ms_step_median,
+        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_mean": ms_step_mean, "step_statistic": "median of the timed steps",
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"one sequence, chunked prefill, 200000 + 2048, {hq} q / {hkv} kv heads of {head_dim}, bf16",
                    "num_seqs": 1, "prefix_len": P, "chunk_len": C, "num_q_heads": hq, "num_kv_heads": hkv,
@@ -539,7 +541,7 @@ def bench_decode(name, args, dev) -> dict:
         step()
     torch.cuda.synchronize()
     wall = time.perf_counter()
-    ms_step, ms_step_median = timed_steps(step, args.steps)
+    ms_step_mean, ms_step = timed_steps(step, args.steps)
     wall = time.perf_counter() - wall
     n_kernel = max(args.steps, KERNEL_LAUNCHES)
     # the dominant kernel alone: the split pass (with one launch per step it IS the step)
@@ -615,13 +617,15 @@ def bench_decode(name, args, dev) -> dict:
         "warmup": args.warmup,
         "preheat_s": args.preheat_s,
         "ms_per_step": ms_step,
-        "ms_per_step_median": ms_step_median,
-        "value_at_median": alg_bytes / (ms_step_median * 1e-3) / 1e9,
+        "ms_per_step_mean": ms_step_mean,
+        "step_statistic": "median of the timed steps",
+        "value_at_mean": alg_bytes / (ms_step_mean * 1e-3) / 1e9,
         "wall_ms_per_step": wall * 1e3 / args.steps,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16" if w.dtype == torch.bfloat16 else str(w.dtype).replace("torch.", ""),
+        "dtype": ("fp8-e4m3 KV, bf16 q" if w.kv_format == "fp8_e4m3" else
+                  "bf16" if w.dtype == torch.bfloat16 else str(w.dtype).replace("torch.", "")),
         "data": "synthetic",
         "config": {
             "workload": {"c1": "c1 fp32 decode B=4", "c2": "c2 Qwen3-0.6B-shaped decode B=64 bf16",
@@ -664,7 +668,7 @@ def secondary(args, dev) -> dict:
     for name in ("c2", "c5", "c3", "c3-d256", "c3-d64"):
         r = (bench_prefill_c3(short, dev) if name == "c3" else bench_prefill_head(short, dev, name) if name in PREFILL_HEAD_SHAPES
              else bench_decode(name, short, dev))
-        keep = ("metric", "value", "unit", "ms_per_step", "ms_per_step_median", "steps", "warmup", "tokens_per_s",
+        keep = ("metric", "value", "unit", "ms_per_step", "ms_per_step_mean", "steps", "warmup", "tokens_per_s",
                 "dtype", "roofline", "cpu_baseline", "append", "pct_of_hbm_peak")
         entry = {k: r[k] for k in keep if k in r}
         entry["workload"] = r["config"]["workload"]

@@ -86,6 +86,8 @@ def _padded_tables(block_tables: Sequence[Sequence[int]]) -> np.ndarray:
 
 
 class HipPagedAttentionBackend:
+    _mask_round_elems = 1 << 28  # (sequence, head, row, key) entries of a mask predicate evaluated per round
+
     def __init__(self, config: CacheConfig, pad_zero_keys: bool = False, window_in_decode: bool = True) -> None:
         self._lib = _lib.load()  # raises if the HIP library has not been built
         self.config = config
@@ -172,12 +174,26 @@ class HipPagedAttentionBackend:
             b = torch.arange(batch, device=dev)[:, None, None, None]
             h = torch.arange(heads, device=dev)[None, :, None, None]
             kv = torch.arange(n_keys, device=dev)[None, None, None, :]
-            keep = torch.as_tensor(mod(b, h, q_pos.to(dev)[:, None, :, None], kv), device=dev).to(torch.bool)
-            while keep.dim() < 4:
-                keep = keep[None]
-            keep = keep.expand(batch, keep.shape[1], q_pos.shape[1], n_keys)
-            rows = keep.permute(0, 2, 1, 3).reshape(batch * q_pos.shape[1], keep.shape[1], n_keys)
-            step.mask_words, step.mask_keys = ops.pack_mask(rows), n_keys
+            q_pos = q_pos.to(dev)
+            rows_per_seq = q_pos.shape[1]
+            # a bounded number of query rows at a time: the dense boolean result of one round stays near 256 MiB
+            # even when the predicate looks at the head (a whole 8192-row step would be gigabytes)
+            chunk = max(1, self._mask_round_elems // max(1, batch * heads * max(n_keys, 1)))
+            parts = []
+            for at in range(0, rows_per_seq, chunk):
+                qi = q_pos[:, None, at: at + chunk, None]
+                keep = torch.as_tensor(mod(b, h, qi, kv), device=dev).to(torch.bool)
+                while keep.dim() < 4:
+                    keep = keep[None]
+                keep = keep.expand(batch, keep.shape[1], qi.shape[2], n_keys)  # one head when `h` is not looked at
+                parts.append(ops.pack_mask(keep.permute(0, 2, 1, 3).reshape(batch * qi.shape[2], keep.shape[1], n_keys)))
+            words = parts[0].shape[-1]
+            if len(parts) == 1:
+                packed = parts[0]
+            else:  # rows of a sequence are contiguous in the step: interleave the rounds back into that order
+                packed = torch.cat([p.view(batch, -1, p.shape[1], words) for p in parts], dim=1)
+                packed = packed.reshape(batch * rows_per_seq, -1, words).contiguous()
+            step.mask_words, step.mask_keys = packed, n_keys
         return step.mask_words
 
     def _mask_first_keys(self, mask: object, step: _StepTensors, batch: int, seq_len: int,

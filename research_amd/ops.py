@@ -139,14 +139,27 @@ def prefill_paged(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Ten
 
 def pack_mask(keep: Tensor) -> Tensor:
     """Bits of a boolean mask ``[rows, heads (or 1), keys]`` as int32 words ``[rows, heads, ceil(keys / 32)]``
-    (bit j of word j // 32 = keep[..., j]), the layout ``attend_masked`` takes."""
+    (bit j of word j // 32 = keep[..., j]), the layout ``attend_masked`` takes.  Packed with byte arithmetic, a
+    bounded number of rows at a time: the temporaries stay near the size of the boolean input."""
     rows, heads, keys = keep.shape
     words = max(1, -(-keys // 32))
-    padded = torch.zeros((rows, heads, words * 32), dtype=torch.int64, device=keep.device)
-    padded[..., :keys] = keep
-    weights = torch.ones(32, dtype=torch.int64, device=keep.device) << torch.arange(32, device=keep.device)
-    packed = (padded.view(rows, heads, words, 32) * weights).sum(-1)
-    return torch.where(packed >= 2 ** 31, packed - 2 ** 32, packed).to(torch.int32).contiguous()
+    out = torch.empty((rows, heads, words), dtype=torch.int32, device=keep.device)
+    per_row = max(1, heads * words * 32)
+    chunk = max(1, (1 << 27) // per_row)  # about 128 MiB of bytes per round
+    for at in range(0, rows, chunk):
+        part = keep[at: at + chunk]
+        n = part.shape[0]
+        if keys == words * 32:
+            bits = part.contiguous().view(torch.uint8) if part.dtype == torch.bool else part.to(torch.uint8)
+        else:
+            bits = torch.zeros((n, heads, words * 32), dtype=torch.uint8, device=keep.device)
+            bits[..., :keys] = part
+        bits = bits.reshape(n, heads, words * 4, 8)
+        byte = bits[..., 0].clone()
+        for k in range(1, 8):
+            byte |= bits[..., k] << k
+        out[at: at + n] = byte.contiguous().view(torch.int32).view(n, heads, words)  # little-endian: byte 0 = bits 0..7
+    return out
 
 
 def attend_masked(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, ctx_lens: Tensor, q_lens: Tensor,

@@ -201,3 +201,27 @@ def test_prefill_passes():
     # splitting would not remove enough padding (chunks of similar length): one pass
     assert prefill_passes([0, 16, 0, 16], [40, 30, 38, 35]) == [[0, 1, 2, 3]]
     assert prefill_passes([], []) == [[]]
+
+
+def test_pack_mask_bit_layout():
+    """Bit j of word j // 32 is keep[..., j] (two's-complement int32 words), for key counts around word
+    boundaries, broadcast (stride 0) head dimensions and many rows."""
+    from research_amd import ops
+
+    g = torch.Generator().manual_seed(3)
+    for rows, heads, keys in [(1, 1, 1), (3, 2, 31), (4, 1, 32), (5, 3, 33), (2, 2, 100), (7, 1, 0)]:
+        keep = torch.rand((rows, heads, keys), generator=g) < 0.5
+        words = ops.pack_mask(keep)
+        assert words.dtype == torch.int32 and tuple(words.shape) == (rows, heads, max(1, -(-keys // 32)))
+        for r in range(rows):
+            for h in range(heads):
+                for w in range(words.shape[2]):
+                    want = sum(1 << j for j in range(32) if w * 32 + j < keys and keep[r, h, w * 32 + j])
+                    assert int(words[r, h, w]) & 0xFFFFFFFF == want
+    shared = (torch.rand((6, 1, 64), generator=g) < 0.5).expand(6, 4, 64)
+    assert torch.equal(ops.pack_mask(shared), ops.pack_mask(shared.contiguous()))
+    tall = torch.rand((70000, 1, 64), generator=g) < 0.5
+    words = ops.pack_mask(tall)
+    for r in (0, 32767, 32768, 69999):
+        want = sum(1 << j for j in range(32) if tall[r, 0, j])
+        assert int(words[r, 0, 0]) & 0xFFFFFFFF == want

@@ -82,6 +82,11 @@ def test_predicates_through_the_backend():
     out = be.forward(q.cuda(), k.cuda(), v.cuda(), 0, InferenceContext(is_prefill=True, block_mask=per_head))
     keep = np.stack([np.stack([(qi >= ki) & (qi - ki <= h + b) for h in range(H)], 1) for b in range(B)])
     assert_close(out, dense(keep), 1e-5, "per-head windows")
+    # the same predicate evaluated a few query rows at a time (what bounds the memory of long steps)
+    small = _backend()
+    small._mask_round_elems = B * H * T * 4  # four rows per round: six rounds
+    out = small.forward(q.cuda(), k.cuda(), v.cuda(), 0, InferenceContext(is_prefill=True, block_mask=per_head))
+    assert_close(out, dense(keep), 1e-5, "per-head windows, evaluated in rounds of rows")
 
     # (3) the causal predicate and the reference's own mask object give the causal kernels' result
     causal = be.forward(q.cuda(), k.cuda(), v.cuda(), 0, InferenceContext(is_prefill=True))
