@@ -262,11 +262,16 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
         (sizeof(KV) == 2 && std::is_same<KV, QT>::value && (D == 64 || D == 128 || D == 256)) ||
         (sizeof(KV) == 1 && sizeof(QT) == 2 && (D == 64 || D == 128 || D == 256));
 
+    // Blocks [blk_first, blk_end) of the row are shared out among the `n_waves` waves of the workgroup; this is
+    // wave `wave`'s share: alternate blocks in the generic and the several-blocks-per-iteration loops, alternate
+    // chunks of a block (the U token steps of one iteration) in the packed loop when `by_chunk` asks for it.
     static __device__ __forceinline__ RowState<NREP, S::EPL> run(const PoolArgs &p, const QT *qrow,
                                                                   const int32_t *bt_row, int k_lo, int L,
-                                                                  int blk_begin, int blk_end, int blk_step,
-                                                                  const LaneRole &role, int lane, int kvh, int rep0) {
+                                                                  int blk_first, int blk_end, int wave, int n_waves,
+                                                                  bool by_chunk, const LaneRole &role, int lane,
+                                                                  int kvh, int rep0) {
         RowState<NREP, S::EPL> out;
+        const int blk_begin = blk_first + wave, blk_step = n_waves;
         if constexpr (kPacked) {
             using HS = HeadScatter<NREP, S::LPR>;
             constexpr int NW = S::EPL / 2;  // packed pairs per lane
@@ -293,10 +298,11 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
                 attend_blocks_pk_multi<KV, QT, D, NREP, U, 2>(st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step,
                                                               lane, lane_voff, kvh, role.tok_local == 0);
             else if (p.tpw * U > p.bs)
-                attend_blocks_pk<KV, QT, D, NREP, U, true>(st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step,
-                                                           lane, lane_voff, kvh, role.tok_local == 0);
+                attend_blocks_pk<KV, QT, D, NREP, U, true>(st, qpk, p, bt_row, k_lo, L, blk_first, blk_end, wave, n_waves,
+                                                           1, false, lane, lane_voff, kvh, role.tok_local == 0);
             else
-                attend_blocks_pk<KV, QT, D, NREP, U, false>(st, qpk, p, bt_row, k_lo, L, blk_begin, blk_end, blk_step,
+                attend_blocks_pk<KV, QT, D, NREP, U, false>(st, qpk, p, bt_row, k_lo, L, blk_first, blk_end, wave,
+                                                            n_waves, (p.bs + p.tpw * U - 1) / (p.tpw * U), by_chunk,
                                                             lane, lane_voff, kvh, role.tok_local == 0);
             StaticFor<NREP>::run([&](auto h) {
                 out.m[h.value] = HS::template bcast<h.value>(st.m);
@@ -523,6 +529,26 @@ __device__ __forceinline__ void merge_pieces(const DecodeArgs &a, int plane, int
     }
 }
 
+// Launches with at most this many blocks per workgroup deal a run of blocks out to the waves chunk by chunk.
+constexpr int kChunkDealUnits = 64;
+
+// Batches up to this size get their block prefix sum from every wave on its own (no barrier); larger ones from the
+// workgroup's scan through LDS.
+constexpr int kWaveScanBatch = 512;
+
+// Inclusive prefix sum of x over the 64 lanes of a wave: four shifted adds inside each row of 16 lanes (a lane
+// with no source in its row adds 0), then the totals of the rows before a lane's own, read through scalars.
+__device__ __forceinline__ int wave_inclusive_scan(int x, int lane) {
+    x += __builtin_amdgcn_update_dpp(0, x, 0x111, 0xf, 0xf, false);  // row_shr:1
+    x += __builtin_amdgcn_update_dpp(0, x, 0x112, 0xf, 0xf, false);  // row_shr:2
+    x += __builtin_amdgcn_update_dpp(0, x, 0x114, 0xf, 0xf, false);  // row_shr:4
+    x += __builtin_amdgcn_update_dpp(0, x, 0x118, 0xf, 0xf, false);  // row_shr:8
+    const int t0 = __builtin_amdgcn_readlane(x, 15), t1 = __builtin_amdgcn_readlane(x, 31),
+              t2 = __builtin_amdgcn_readlane(x, 47);
+    const int row = lane >> 4;
+    return x + (row >= 1 ? t0 : 0) + (row >= 2 ? t1 : 0) + (row >= 3 ? t2 : 0);
+}
+
 // Split pass.  The (plane, sequence, block) space - plane = (rep group, head
 // group) - is flattened in that order and cut into gridDim.x equal ranges, one
 // per workgroup, so every workgroup streams the same number of pool blocks
@@ -546,11 +572,33 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
     const int B = a.batch;
 
     // ---- block prefix sum over the batch --------------------------------
-    {
+    // blocks of sequence b that hold visible keys: [first_key(b) / bs, ceil(L / bs))
+    auto blocks_of = [&](int b) { return plan_blocks_of(a.seq_lens[b], p.bs, p.window); };
+    if (B <= kWaveScanBatch) {
+        // Every wave computes the whole prefix sum by itself: lane l of round c holds sequence 64 c + l, the lengths
+        // of all rounds are requested at once, a round is scanned with data-parallel moves and the rounds are
+        // chained through a scalar.  All four waves store the same values to the same LDS words and each reads
+        // back what it has itself written, so no barrier stands between the lengths and the first table entry.
+        int n[kWaveScanBatch / PA_WAVE];
+#pragma unroll
+        for (int c = 0; c < kWaveScanBatch / PA_WAVE; ++c) {
+            const int b = c * PA_WAVE + lane;
+            n[c] = c * PA_WAVE < B && b < B ? blocks_of(b) : 0;
+        }
+        int carry = 0;
+#pragma unroll
+        for (int c = 0; c < kWaveScanBatch / PA_WAVE; ++c) {
+            if (c * PA_WAVE >= B) break;  // uniform
+            const int x = wave_inclusive_scan(n[c], lane);
+            if (c * PA_WAVE + lane < B) s_prefix[c * PA_WAVE + lane] = carry + x - n[c];
+            carry += __builtin_amdgcn_readlane(x, PA_WAVE - 1);
+        }
+        if (lane == 0) s_prefix[B] = carry;
+        if (blockIdx.x == 0 && wave == 0)
+            for (int b = lane; b <= B; b += PA_WAVE) a.block_prefix[b] = s_prefix[b];
+    } else {
         const int per = (B + kThreads - 1) / kThreads;
         const int lo = min(B, tid * per), hi = min(B, lo + per);
-        // blocks of sequence b that hold visible keys: [first_key(b) / bs, ceil(L / bs))
-        auto blocks_of = [&](int b) { return plan_blocks_of(a.seq_lens[b], p.bs, p.window); };
         int sum = 0;
         for (int b = lo; b < hi; ++b) sum += blocks_of(b);
         s_scan[tid] = sum;
@@ -589,6 +637,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
 
     int64_t cur = unit_begin(blockIdx.x, total, grid);
     const int64_t end = unit_begin((int64_t)blockIdx.x + 1, total, grid);
+    const bool by_chunk = total <= (int64_t)kChunkDealUnits * grid;  // short launches: see attend_blocks_pk
     while (cur < end) {
         const int plane = (int)(cur / per_plane);
         const int off = (int)(cur - plane * per_plane);
@@ -611,7 +660,7 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
 
         RowState<NREP, S::EPL> st = Attender<KV, QT, D, NREP, U>::run(
             p, reinterpret_cast<const QT *>(a.q) + (int64_t)b * p.hq * D, p.bt + (int64_t)b * p.bt_stride, k_lo, L,
-            fb + blk0 + wave, fb + blk1, kWaves, role, lane, kvh, rep0);
+            fb + blk0, fb + blk1, wave, kWaves, by_chunk, role, lane, kvh, rep0);
         if (blk0 == 0 && blk1 == nblk) {
             // the whole sequence is ours: write the output row
             const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
@@ -863,7 +912,7 @@ __global__ __launch_bounds__(kThreads) void prefill_rowwise_kernel(const Rowwise
     k_lo = max(k_lo, 0);
     RowState<NREP, S::EPL> st = Attender<KV, QT, D, NREP, U>::run(
         p, reinterpret_cast<const QT *>(a.q) + qrow * p.hq * D, p.bt + (int64_t)b * p.bt_stride, k_lo, L,
-        k_lo / p.bs + wave, nblk, kWaves, role, lane, kvh, rep0);
+        k_lo / p.bs, nblk, wave, kWaves, false, role, lane, kvh, rep0);
     QT *orow = reinterpret_cast<QT *>(a.out) + qrow * p.hq * D;
     merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
                             [&](int qh, int d, const float (&num)[4], float M, float den) {

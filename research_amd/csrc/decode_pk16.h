@@ -173,6 +173,12 @@ template <int NREP, int LPR> struct HeadScatter {
     }
 };
 
+// A 64-bit value that is the same in every lane, as two scalar halves.
+__device__ __forceinline__ int64_t uniform64(int64_t x) {
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)x), hi = __builtin_amdgcn_readfirstlane((uint32_t)((uint64_t)x >> 32));
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+
 template <int NREP, int VPL, int EPL> struct PkState {
     float m[VPL], l[VPL];
     float acc[NREP][EPL];
@@ -198,17 +204,29 @@ template <> struct StaticFor<0> {
     template <typename F> static __device__ __forceinline__ void run(F &&) {}
 };
 
-// Attend keys [k_lo, L) of blocks blk_begin, blk_begin+blk_step, ... < blk_end.
+// Attend keys [k_lo, L) of this wave's share of blocks [blk_first, blk_end), which the n_waves waves of the
+// workgroup divide among themselves.  A chunk is the U token steps a wave keeps in flight (p.tpw * U tokens); a
+// block holds cpb = ceil(block_size / chunk) of them.  The largest multiple of n_waves blocks is dealt out block by
+// block (a wave streams whole blocks: one table entry and one descriptor per block) and the up to n_waves - 1
+// blocks left over chunk by chunk, so the waves' shares differ by one chunk at most however short the run is
+// (the waves meet at a barrier behind every run).  With `by_chunk` the whole run is dealt chunk by chunk: the
+// chunks of a block are then requested by neighbouring waves at the same time instead of by one wave one after
+// the other.  Measured on MI355X (32 query / 8 kv heads of 128): dealing everything by chunk takes about 2 us off
+// a bf16 launch whatever its length (16 sequences of 4 096 to 65 536 keys; the 64-sequence ragged batch of
+// 0.14 M keys: 99.4 -> 96.5 us) but costs the 256-sequence batch of 0.84 M keys 0.8 % (540 -> 545 us), so the
+// split pass asks for it in launches of at most kChunkDealUnits blocks per workgroup; dealing only the left-over
+// blocks by chunk took 3 us off the long-context fp8 launch (274 -> 271 us).
 // qpk[r][i]: packed pairs of this lane's query elements of head r (raw bits of the query type AT).
 // lane_kvh: the kv head this lane's row belongs to (selects the fp8 scales).
-// SHORT: a token step of the wave (tpw tokens) times U exceeds the block, so whole steps can lie past the
-// block's end; they are skipped under uniform branches.  The straight-line form (SHORT = false) keeps the
-// loop free of branches for the layouts where every step of a full block is live.
+// SHORT: a chunk exceeds the block (cpb = 1), so whole token steps can lie past the block's end; they are skipped
+// under uniform branches.  The straight-line form (SHORT = false) keeps the loop free of branches for the layouts
+// where every step of a full chunk is live.
 template <typename KV, typename AT, int D, int NREP, int U, bool SHORT>
 __device__ __forceinline__ void attend_blocks_pk(
     PkState<NREP, HeadScatter<NREP, D * (int)sizeof(KV) / 16>::VPL, 2 * PoolWords<KV, AT>::NW> &st,
     const uint32_t (&qpk)[NREP][PoolWords<KV, AT>::NW], const PoolArgs &p, const int32_t *bt_row, int k_lo, int L,
-    int blk_begin, int blk_end, int blk_step, int lane, int lane_voff, int lane_kvh, bool count_zero_keys) {
+    int blk_first, int blk_end, int wave, int n_waves, int cpb, bool by_chunk, int lane, int lane_voff, int lane_kvh,
+    bool count_zero_keys) {
     static_assert(U % 2 == 0, "tokens are consumed in pairs");
     constexpr int LPR = D * (int)sizeof(KV) / 16;
     constexpr bool kFp8 = sizeof(KV) == 1;
@@ -219,46 +237,65 @@ __device__ __forceinline__ void attend_blocks_pk(
     constexpr int VPL = HS::VPL;
     const int tok_stride = p.hkv * D * (int)sizeof(KV);  // bytes between tokens
     const int tok_local = (lane / LPR) / p.hpw;
+    const int chunk = p.tpw * U;                          // tokens per chunk
 
-    // the table entry of a block is requested one iteration ahead, so its latency is off the wave's critical path
-    int64_t bid_next = blk_begin < blk_end && blk_begin < p.bt_stride ? (int64_t)bt_row[blk_begin] : -1;
-    for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
-        const int ntok = min(p.bs, L - blk * p.bs);
-        const int tlo = max(0, k_lo - blk * p.bs);  // tokens below it lie before the window (first block only)
-        const int64_t bid = bid_next;
+    int voff[U];  // byte offset of this lane's 16 bytes in token step u of a chunk
+#pragma unroll
+    for (int u = 0; u < U; ++u) voff[u] = lane_voff + u * p.tpw * tok_stride;
+    // chunk-by-chunk dealing indexes chunks with shifts, so it needs a power-of-two number of chunks per block
+    const bool can_chunk = cpb > 1 && (cpb & (cpb - 1)) == 0;
+    const int whole = !can_chunk ? blk_end - blk_first : by_chunk ? 0 : (blk_end - blk_first) / n_waves * n_waves;
+    // phase 0: whole blocks, wave w takes blocks first+w, first+w+n_waves, ...; phase 1: the chunks of the blocks
+    // not dealt out in phase 0, wave w takes chunks w, w+n_waves, ... of them.  One loop serves both: its index o
+    // counts blocks (shift 0, a span of one block) or chunks (shift log2 cpb, a span of one chunk).
+    for (int phase = 0; phase < 2; ++phase) {
+    const int sh = phase == 0 ? 0 : __builtin_ctz(cpb);
+    const int span = phase == 0 ? p.bs : chunk;
+    const int o_begin = phase == 0 ? blk_first + wave : ((blk_first + whole) << sh) + wave;
+    const int o_end = phase == 0 ? blk_first + whole : blk_end << sh;
+    // the table entry of a step's block is requested one step ahead, so its latency is off the wave's critical path
+    int64_t bid_next = o_begin < o_end && (o_begin >> sh) < p.bt_stride ? (int64_t)bt_row[o_begin >> sh] : -1;
+    for (int o = o_begin; o < o_end; o += n_waves) {
+        const int cur_blk = o >> sh;
+        const int64_t bid = uniform64(bid_next);  // (a scalar from here on: the address arithmetic stays off the vector unit)
         {
-            const int nb = blk + blk_step;
-            bid_next = nb < blk_end && nb < p.bt_stride ? (int64_t)bt_row[nb] : -1;
+            const int nb = (o + n_waves) >> sh;
+            bid_next = o + n_waves < o_end && nb < p.bt_stride ? (int64_t)bt_row[nb] : -1;
         }
+        const int ntok = min(p.bs, L - cur_blk * p.bs);
+        const int tlo = max(0, k_lo - cur_blk * p.bs);  // tokens below it lie before the window (first block only)
+        const int t_begin = (o - (cur_blk << sh)) * chunk, t_end = min(ntok, t_begin + span);  // this step's tokens
         if (bid < 0 || bid >= p.num_blocks) {
-            if (count_zero_keys) st.zero_keys += max(0, ntok - tlo);
+            if (count_zero_keys) st.zero_keys += max(0, t_end - max(tlo, t_begin));
             continue;
         }
-        // descriptor of the valid part of this block: reads past it return 0
         const int64_t block_off = bid * p.bs * (int64_t)tok_stride;
-        const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(reinterpret_cast<const char *>(p.k) + block_off), 0, ntok * tok_stride, 0x00020000);
-        const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(reinterpret_cast<const char *>(p.v) + block_off), 0, ntok * tok_stride, 0x00020000);
         float k_sc = p.scale_log2, v_sc = 1.f;  // logit scale (with the K scale folded in) and V scale of this block
         if (kFp8) {
             k_sc *= p.k_scale[bid * p.hkv + lane_kvh];
             v_sc = p.v_scale[bid * p.hkv + lane_kvh];
         }
 
-        for (int t0 = 0; t0 < ntok; t0 += p.tpw * U) {
+        for (int t0 = t_begin; t0 < t_end; t0 += chunk) {
+            if (t0 + chunk <= tlo) continue;  // the whole chunk lies before the window
+            // descriptors of the valid rows of the block from t0 on: reads past them return 0.  The per-lane
+            // offsets of the U token steps are loop invariants (voff), so a load costs no address arithmetic.
+            const int64_t chunk_off = block_off + (int64_t)t0 * tok_stride;
+            const int valid = (ntok - t0) * tok_stride;
+            const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(reinterpret_cast<const char *>(p.k) + chunk_off), 0, valid, 0x00020000);
+            const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
+                (void *)(reinterpret_cast<const char *>(p.v) + chunk_off), 0, valid, 0x00020000);
             pa_u4 kraw[U], vraw[U];
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                kraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rk, lane_voff + (t0 + u * p.tpw) * tok_stride, 0, kStreamPolicy);
+            for (int u = 0; u < U; ++u) kraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rk, voff[u], 0, kStreamPolicy);
 #pragma unroll
-            for (int u = 0; u < U; ++u)
-                vraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rv, lane_voff + (t0 + u * p.tpw) * tok_stride, 0, kStreamPolicy);
+            for (int u = 0; u < U; ++u) vraw[u] = __builtin_amdgcn_raw_buffer_load_b128(rv, voff[u], 0, kStreamPolicy);
 
             // ---- logits: one (token, head) per lane -----------------------
             float sv[U][VPL];
-            const int rem = ntok - t0;                         // tokens of the block from t0 on (uniform)
-            const bool partial = rem < p.tpw * U || t0 < tlo;  // uniform
+            const int rem = ntok - t0;                   // tokens of the block from t0 on (uniform)
+            const bool partial = rem < chunk || t0 < tlo;  // uniform
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 if (SHORT && u * p.tpw >= rem) {  // uniform: the whole token step lies past the block
@@ -348,6 +385,7 @@ __device__ __forceinline__ void attend_blocks_pk(
             }
         }
     }
+    }  // phase
 }
 
 // The same loop for layouts where a token step of the wave covers several tokens and a block holds only SPB
