@@ -102,7 +102,7 @@ int pa_kv_gather(const void *k_cache, const void *v_cache, void *k_out, void *v_
  * shapes, so captured graphs replay without clearing anything.  The rest need
  * not be initialised.  Calls that share a workspace must not overlap in time.
  */
-#define PA_DECODE_TICKET_BYTES (512u << 10)
+#define PA_DECODE_TICKET_BYTES (640u << 10)
 size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_kv_heads, int head_dim,
                                  int kv_dtype);
 

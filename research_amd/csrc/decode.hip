@@ -4,7 +4,6 @@
 // decode_inst_*.hip.
 #include <stdlib.h>
 
-#include <atomic>
 #include <mutex>
 
 #include "decode_impl.h"
@@ -177,11 +176,9 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     a.tickets = (unsigned long long *)(ws + w.ticket_off);
     a.part_ml = (float *)(ws + w.ml_off);
     a.part_acc = (float *)(ws + w.acc_off);
-    // Batches that leave a sequence few pieces are finished by the split pass alone; the tag (the launch number,
-    // 1 .. 2^40 - 1) tells this launch's tickets from those of the launches before it.
-    static std::atomic<unsigned long long> launches{0};
+    // Batches that leave a sequence few pieces are finished by the split pass alone.
+    a.group_tickets = (unsigned long long *)(ws + kPlanGroupTicketOff);
     a.merge_in_split = phases == (kPhaseSplit | kPhaseReduce) && plan_merge_in_split(batch, plan, grid) ? 1 : 0;
-    a.ticket_tag = launches.fetch_add(1, std::memory_order_relaxed) % ((1ull << 40) - 1) + 1;
 
     hipStream_t s = (hipStream_t)stream;
     a.split_grid = grid;

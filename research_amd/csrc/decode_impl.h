@@ -66,8 +66,8 @@ struct DecodeArgs {
     float *part_acc;        // [slot_cap][hpw*NREP][D]
     float *part_ml;         // [slot_cap][hpw*NREP][2]
     int32_t *block_prefix;  // [batch+1], written by the split pass for the reduction pass
-    unsigned long long *tickets;  // [planes*batch]: (launch tag << 24) | pieces of the (plane, sequence) that have arrived
-    unsigned long long ticket_tag;  // 40-bit tag of this launch (never 0): a ticket with another tag counts as zero
+    unsigned long long *tickets;        // [planes*batch]: arrivals per (plane, sequence); zero between launches
+    unsigned long long *group_tickets;  // [2*split_grid]: arrivals per group of pieces of a many-piece sequence
     int merge_in_split;     // the workgroup that delivers a sequence's last piece merges the pieces (no second pass)
 };
 
@@ -455,49 +455,60 @@ __device__ __forceinline__ float2 ld_coherent(const float *p) {
 __device__ __forceinline__ void wait_all_memory() { asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory"); }
 __device__ __forceinline__ void compiler_fence() { asm volatile("" ::: "memory"); }
 
-// One piece of a (plane, sequence) has been written to the workspace: count it; true for the arrival that completes
-// the sequence.  A ticket is (tag of the launch << 24 | arrivals so far).  The ticket region is zero when the
-// workspace is first used; the completing arrival stores zero arrivals under its own tag, and a ticket carrying
-// another launch's tag counts as zero, so every launch - also a replay of a captured graph, which carries the tag
-// it was recorded with - finds every ticket at zero arrivals.  Tags are consecutive launch numbers, so a launch
-// never meets its own tag from an earlier one.  Called by one thread, after the workgroup's stores are complete.
-__device__ __forceinline__ bool piece_arrived_last(unsigned long long *ticket, unsigned long long tag, int n_pieces) {
-    unsigned long long old = __hip_atomic_load(ticket, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    for (;;) {  // ends after at most n_pieces rounds: a failed exchange means another piece was counted
-        const unsigned long long cnt = (old >> 24) == tag ? (old & 0xffffffull) : 0ull;
-        const bool last = cnt + 1 >= (unsigned long long)n_pieces;
-        const unsigned long long neu = (tag << 24) | (last ? 0ull : cnt + 1);
-        if (__hip_atomic_compare_exchange_strong(ticket, &old, neu, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
-                                                 __HIP_MEMORY_SCOPE_AGENT))
-            return last;
-    }
+// Arrival counting.  A ticket is a 64-bit counter in the zero-filled region at the start of the workspace.  One
+// thread of a workgroup, after the workgroup's stores are complete, adds one; the arrival that brings the count to
+// `expected` is the last one: it puts the counter back to zero (nobody else touches it any more in this launch),
+// so every launch - also a replay of a captured graph - finds every ticket at zero.
+__device__ __forceinline__ bool arrive_is_last(unsigned long long *ticket, int expected) {
+    const unsigned long long old = __hip_atomic_fetch_add(ticket, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const bool last = old + 1 >= (unsigned long long)expected;
+    if (last) __hip_atomic_store(ticket, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return last;
 }
 
-// The workgroup that delivered the last piece of (plane, sequence b) merges the pieces of workgroups w0..w1 and
-// writes the plane's output rows: one thread per (query head, four consecutive d), the loads of four pieces in
-// flight at a time.
-template <typename QT, int D, int NREP>
-__device__ __forceinline__ void merge_pieces(const DecodeArgs &a, int plane, int b, int hg, int rep0, int w0, int w1,
-                                             int tid) {
+// How the pieces w0..w1 of one (plane, sequence) are merged inside the split pass.  Up to kInlinePieces pieces: the
+// workgroup that delivers the last of them merges them all.  More (one sequence that dominates its batch is cut
+// into hundreds): the pieces form groups of `group` consecutive workgroups, the last arrival of a group merges the
+// group into the slot of the group's first piece, and the last group to finish merges the groups - two levels of
+// at most 32 partials each instead of one workgroup reading hundreds.
+constexpr int kInlinePieces = 8;
+struct PieceTree {
+    int pieces, group, n_groups;
+};
+__device__ __forceinline__ PieceTree piece_tree(int pieces) {
+    PieceTree t;
+    t.pieces = pieces;
+    t.group = pieces <= kInlinePieces ? pieces : pieces <= 64 ? 8 : pieces <= 256 ? 16 : 32;
+    t.n_groups = (pieces + t.group - 1) / t.group;
+    return t;
+}
+
+// Merge `count` partials of (plane, sequence b) - the slots of workgroups w_first, w_first + stride, ... - one
+// thread per (query head, four consecutive d), the loads of PIPE partials in flight at a time.  FINAL: normalise and
+// write the plane's output rows; otherwise leave the merged partial in the slot of workgroup w_first (every thread
+// overwrites exactly what it has itself read).
+template <typename QT, int D, int NREP, bool FINAL>
+__device__ __forceinline__ void merge_slots(const DecodeArgs &a, int plane, int b, int hg, int rep0, int w_first,
+                                            int count, int stride, int tid) {
     constexpr int PIPE = 4;
     const PoolArgs &p = a.p;
     const int stride_acc = p.hpw * NREP * D, stride_ml = p.hpw * NREP * 2;
     const int64_t key = (int64_t)plane * a.batch + b;
-    const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
+    const int ez = FINAL && a.extra_zero ? max(0, a.extra_zero[b]) : 0;
     QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * D;
     for (int item = tid; item < p.hpw * NREP * (D / 4); item += kThreads) {
         const int idx = item / (D / 4), d = (item - idx * (D / 4)) * 4;
         const int kv_local = idx / NREP, r = idx - kv_local * NREP;
         if (rep0 + r >= p.n_rep) continue;
-        const int qh = (hg * p.hpw + kv_local) * p.n_rep + rep0 + r;
         float M = kNegBig, den = 0.f, num[4] = {0.f, 0.f, 0.f, 0.f};
-        for (int w = w0; w <= w1; w += PIPE) {
+        for (int i = 0; i < count; i += PIPE) {
             float m[PIPE], l[PIPE];
             float4 x[PIPE];
 #pragma unroll
             for (int j = 0; j < PIPE; ++j) {
-                const bool have = w + j <= w1 && w + j + key < a.slot_cap;
-                const int64_t slot = (have ? w + j : w0) + key;
+                const int64_t want = (int64_t)w_first + (int64_t)(i + j) * stride + key;
+                const bool have = i + j < count && want < a.slot_cap;
+                const int64_t slot = have ? want : w_first + key;
                 const float2 ml = ld_coherent(a.part_ml + slot * stride_ml + idx * 2);
                 const float2 lo = ld_coherent(a.part_acc + slot * stride_acc + idx * D + d);
                 const float2 hi = ld_coherent(a.part_acc + slot * stride_acc + idx * D + d + 2);
@@ -524,9 +535,55 @@ __device__ __forceinline__ void merge_pieces(const DecodeArgs &a, int plane, int
             }
             M = mn;
         }
+        if (FINAL) {
+            const int qh = (hg * p.hpw + kv_local) * p.n_rep + rep0 + r;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) pa_scalar<QT>::store(orow + (int64_t)qh * D + d + j, finish_row(num[j], M, den, ez));
+            for (int j = 0; j < 4; ++j)
+                pa_scalar<QT>::store(orow + (int64_t)qh * D + d + j, finish_row(num[j], M, den, ez));
+        } else if ((int64_t)w_first + key < a.slot_cap) {
+            const int64_t slot = w_first + key;
+            st_coherent(a.part_acc + slot * stride_acc + idx * D + d, num[0], num[1]);
+            st_coherent(a.part_acc + slot * stride_acc + idx * D + d + 2, num[2], num[3]);
+            if (d == 0) st_coherent(a.part_ml + slot * stride_ml + idx * 2, M, den);
+        }
     }
+}
+
+// A piece of (plane, sequence b) that this workgroup has just stored; w0..w1 are the workgroups holding pieces of it.
+struct PieceRef {
+    int plane, b, hg, rep0, w0, w1;
+};
+
+// Count the piece and do whatever merging falls to this workgroup.  s_flag: one LDS word.
+template <typename QT, int D, int NREP>
+__device__ __forceinline__ void deliver_piece(const DecodeArgs &a, const PieceRef &pp, int *s_flag, int tid) {
+    const PieceTree t = piece_tree(pp.w1 - pp.w0 + 1);
+    const int me = (int)blockIdx.x - pp.w0;  // index of this workgroup's piece
+    const int g = me / t.group;
+    const int g_first = pp.w0 + g * t.group;                      // workgroup of the group's first piece
+    const int g_count = min(t.group, t.pieces - g * t.group);     // pieces of this group
+    unsigned long long *seq_ticket = a.tickets + ((int64_t)pp.plane * a.batch + pp.b);
+    // a group's ticket is found by the workgroup of its first piece; a workgroup can be that for the sequence that
+    // runs on into it (a later group of it) and for the sequence that starts in it (group 0 of it)
+    unsigned long long *grp_ticket = a.group_tickets + (2 * (int64_t)g_first + (g == 0 ? 1 : 0));
+    wait_all_memory();  // this thread's stores have reached the memory side
+    __syncthreads();
+    if (tid == 0) *s_flag = arrive_is_last(t.n_groups == 1 ? seq_ticket : grp_ticket, g_count);
+    __syncthreads();
+    compiler_fence();  // the pieces are read after the count, never before
+    if (!*s_flag) return;  // uniform
+    if (t.n_groups == 1) {
+        merge_slots<QT, D, NREP, true>(a, pp.plane, pp.b, pp.hg, pp.rep0, pp.w0, t.pieces, 1, tid);
+        return;
+    }
+    merge_slots<QT, D, NREP, false>(a, pp.plane, pp.b, pp.hg, pp.rep0, g_first, g_count, 1, tid);
+    wait_all_memory();
+    __syncthreads();
+    if (tid == 0) *s_flag = arrive_is_last(seq_ticket, t.n_groups);
+    __syncthreads();
+    compiler_fence();
+    if (!*s_flag) return;
+    merge_slots<QT, D, NREP, true>(a, pp.plane, pp.b, pp.hg, pp.rep0, pp.w0, t.n_groups, t.group, tid);
 }
 
 // Launches with at most this many blocks per workgroup deal a run of blocks out to the waves chunk by chunk.
@@ -696,17 +753,15 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
                                         });
             }
             if (a.merge_in_split) {
-                // Every thread's part of the partial is made visible to the whole device, then one thread counts
-                // the piece; the workgroup whose piece completes the sequence reads all of them back and merges.
+                // Count the piece; if it completes its sequence (or its group of pieces), merge.  Done right away
+                // and not behind the next run of blocks: a workgroup's first piece is the tail of a sequence whose
+                // head the workgroup before it delivers at its very end, so delivering early leaves that merge to
+                // the neighbour instead of stacking two merges at this workgroup's own end (measured: 0.7 % of
+                // the 256-sequence launch).
                 const int64_t u0 = plane * per_plane + s_prefix[b];
-                const int w0 = owner_of(u0, total, grid), w1 = owner_of(u0 + nblk - 1, total, grid);
-                wait_all_memory();  // this thread's stores have reached the memory side
-                __syncthreads();
-                if (tid == 0)
-                    s_last = piece_arrived_last(a.tickets + ((int64_t)plane * B + b), a.ticket_tag, w1 - w0 + 1);
-                __syncthreads();
-                compiler_fence();  // the pieces are read after the count, never before
-                if (s_last) merge_pieces<QT, D, NREP>(a, plane, b, hg, rep0, w0, w1, tid);  // uniform
+                const PieceRef piece = {plane, b, hg, rep0, owner_of(u0, total, grid),
+                                        owner_of(u0 + nblk - 1, total, grid)};
+                deliver_piece<QT, D, NREP>(a, piece, &s_last, tid);
             }
         }
         cur += blk1 - blk0;

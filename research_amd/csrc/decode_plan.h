@@ -17,11 +17,14 @@ namespace pa_decode_detail {
 constexpr int kPlanMaxBatch = 8192;      // sequences per call (their block prefix sum lives in LDS)
 constexpr int kPlanMaxSplitGrid = 4096;  // upper bound of the split pass's grid, fixes the caller's workspace size
 constexpr int kPlanMinUnitsPerWorkgroup = 4;
-// Arrival tickets of the merge inside the split pass: one 64-bit word per (plane, sequence), in a region of fixed
-// size at the start of every workspace so that calls of any shape use the same bytes for the same purpose and
-// nothing else is ever written there.  The caller zero-fills the region once; every call leaves it counting zero.
+// Arrival tickets of the merge inside the split pass: 64-bit counters in a region of fixed size at the start of
+// every workspace, so that calls of any shape use the same bytes for the same purpose and nothing else is ever
+// written there: kPlanTicketSlots counters per (plane, sequence), then 2 per workgroup of the largest grid for the
+// groups that the pieces of a many-piece sequence are merged in.  The caller zero-fills the region once; every call
+// leaves it at zero.
 constexpr int kPlanTicketSlots = 65536;
-constexpr size_t kPlanTicketBytes = (size_t)kPlanTicketSlots * 8;
+constexpr size_t kPlanGroupTicketOff = (size_t)kPlanTicketSlots * 8;
+constexpr size_t kPlanTicketBytes = kPlanGroupTicketOff + 2 * (size_t)kPlanMaxSplitGrid * 8 + 64 * 1024;  // 640 KiB
 
 // How the heads are spread over wave loads and planes (a plane = one group of hpw kv heads x one group of <= nrep_t
 // query heads per kv head).  lpr lanes of 16 bytes hold one K/V row; a wave load covers rpw = 64/lpr rows, mapped
@@ -122,12 +125,13 @@ PA_PLAN_FN constexpr size_t plan_split_lds_bytes(int batch, int head_dim, int kv
     return (size_t)(batch + 1) * 4 + kPlanThreads * 4 + (size_t)plan_merge_floats(head_dim, kv_elem_bytes, nrep_t) * 4 + 4;
 }
 
-// Whether the split pass merges the pieces of a sequence itself (the workgroup that delivers a sequence's last
-// outstanding piece merges them all) instead of leaving them to a second launch: when the batch is so large that a
-// (plane, sequence) has two pieces on average at most.  Measured on MI355X: 256 sequences (two pieces each) gain
-// 1 % over the two launches, 64 sequences (four pieces each) lose 2 % - delivering a piece costs the workgroup a
-// round trip to the memory side before its next part - and a few long sequences spread over the whole grid are
-// merged much faster by the second launch, whose workgroups take one output row each.
+// Whether the split pass merges the pieces of a sequence itself (the workgroup that delivers the last outstanding
+// piece of a sequence, or of a group of its pieces, merges) instead of leaving them to a second launch: when the
+// batch is so large that a (plane, sequence) has two pieces on average at most.  Measured on MI355X: 256 sequences
+// (two pieces each) gain 1 % over the two launches; 64 sequences (four pieces each) lose 2 % - delivering a piece
+// costs round trips to the memory side, about 9 us at the end of a 100 us launch where the second launch costs 7 -
+// and a few long sequences spread over the whole grid are merged much faster by the second launch, whose
+// workgroups take one output row each.
 PA_PLAN_FN bool plan_merge_in_split(int batch, const HeadPlan &h, int grid) {
     const int64_t keys = (int64_t)h.planes() * batch;  // one ticket each
     return (int64_t)grid <= 2 * keys && keys <= kPlanTicketSlots;

@@ -108,5 +108,5 @@ def test_merge_in_split_rule_and_layout_match_the_library():
     want = lib.pa_decode_workspace_bytes(256, 32, 8, 128, _lib.PA_BF16)
     slots = 4096 + 2 * 256
     align = lambda x: -(-x // 256) * 256
-    tickets = 512 * 1024  # the fixed region at the start (PA_DECODE_TICKET_BYTES)
+    tickets = 640 * 1024  # the fixed region at the start (PA_DECODE_TICKET_BYTES)
     assert want == tickets + align(257 * 4) + align(slots * 16 * 2 * 4) + align(slots * 16 * 128 * 4)

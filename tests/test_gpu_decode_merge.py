@@ -1,8 +1,8 @@
-"""Large decode batches: the split pass that merges a sequence's pieces itself, inside its one launch.
+"""Decode batches whose split pass merges a sequence's pieces itself, inside its one launch.
 
 With about 128 sequences or more (``pa_decode_passes`` == 1) a workgroup that finishes a piece of a sequence counts
-itself on the sequence's ticket, and the workgroup whose piece completes the sequence reads every piece back and
-writes the row.  Each case here is checked three ways: against the CPU checker (2e-2 for 16-bit pools, 1e-5 for
+itself on the sequence's ticket, and the workgroup whose piece completes the sequence (or a group of its pieces, when
+there are many) reads the pieces back and merges them.  Each case here is checked three ways: against the CPU checker (2e-2 for 16-bit pools, 1e-5 for
 fp32, 6e-2 for fp8 against dequantise-then-attend), against ``pa_decode_split`` + ``pa_decode_reduce`` on the same
 inputs (the same partials merged by the second launch, in another order: 1e-3), and for rows that must be exactly
 zero.  The graph tests replay a captured append + decode step of 256 sequences with lengths, slots and queries
@@ -169,6 +169,22 @@ def test_one_very_long_sequence_among_255_short_ones():
         timings[entry] = (time.perf_counter() - t0) / 5 * 1e6
     print(f"[timing] one launch {timings['pa_decode']:.1f} us, split + reduce {timings['two']:.1f} us", flush=True)
     assert timings["pa_decode"] < 4 * timings["two"] + 200, "the merge of the long sequence's pieces dominates the launch"
+
+
+@pytest.mark.parametrize("batch,long_len,short", [(200, 4000, 300), (128, 30000, 200), (160, 1500, 700)])
+def test_sequences_of_many_pieces_are_merged_in_groups(batch, long_len, short):
+    """A sequence cut into more than eight pieces is merged in two levels (groups of 8, 16 or 32 pieces, then the
+    groups); here one sequence takes about 20, about 150 and about 5 pieces beside sequences of one or two."""
+    announce(f"decode merge-in-split: groups of pieces, batch {batch}, one sequence of {long_len}")
+    rng = np.random.default_rng(batch)
+    lens = _ragged(rng, batch, short // 2, short)
+    lens[batch // 3] = long_len
+    b = Batch(lens, 32, 8, 128, "bf16", seed=batch)
+    _three_ways(b, what=f"batch {batch} with one sequence of {long_len}")
+    # (an fp8 pool of 8 kv heads is one plane: it takes the one-launch path from 64 sequences on)
+    kv = "fp8" if _passes(batch, 32, 8, 128, torch.float8_e4m3fn) == 1 else "f16"
+    b = Batch(lens, 32, 8, 128, kv, seed=batch + 1)
+    _three_ways(b, extra_zero=[max(b.lens) - n for n in b.lens], what=f"{kv}, batch {batch}, extra zero keys")
 
 
 def test_more_sequences_than_one_launch_takes():
