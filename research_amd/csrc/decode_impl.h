@@ -278,8 +278,11 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
             uint32_t qpk[NREP][NW];
 #pragma unroll
             for (int r = 0; r < NREP; ++r) {
-                const bool live = rep0 + r < p.n_rep;
-                const QT *qp = qrow + ((int64_t)kvh * p.n_rep + rep0 + r) * D + role.d0;
+                // local index r of this lane stands for head head_of(r, lane): the order that spares the
+                // reduce-scatter of the logits its selects
+                const int hr = HS::head_of(r, lane);
+                const bool live = rep0 + hr < p.n_rep;
+                const QT *qp = qrow + ((int64_t)kvh * p.n_rep + rep0 + hr) * D + role.d0;
 #pragma unroll
                 for (int i = 0; i < NW; i += 4) {
                     const uint4 raw = live ? ld16(qp + 2 * i) : uint4{0, 0, 0, 0};

@@ -110,29 +110,30 @@ template <int NREP, int LPR> struct HeadScatter {
     static constexpr int SC = NREP >= 4 ? 2 : (NREP == 2 ? 1 : 0);  // scatter steps (xor 1, xor 2)
     static constexpr int VPL = NREP >> SC;                            // values a lane keeps
 
+    // The scatter steps exchange between lane pairs (xor 1, then xor 2): a lane keeps half of its values and adds
+    // the partner's other half.  Which half a lane keeps would depend on its position in the quad - a select per
+    // value - so instead the lanes hold their query heads in different orders: local index j of a lane stands for
+    // head j ^ swizzle(lane).  Then every lane keeps its first half and receives the partner's second half, one
+    // DPP add per value, and ends up owning local values 0 .. VPL-1 = heads head_of(0 .. VPL-1, lane).
+    static __device__ __forceinline__ int swizzle(int lane) {
+        return (SC >= 1 ? (lane & 1) * (NREP / 2) : 0) ^ (SC == 2 ? ((lane >> 1) & 1) * VPL : 0);
+    }
+    static __device__ __forceinline__ int head_of(int j, int lane) { return j ^ swizzle(lane); }
+
+    // s[j]: this lane's partial dot product of head head_of(j, lane).
     static __device__ __forceinline__ void reduce(const float (&s)[NREP], float (&out)[VPL], int lane) {
         constexpr int H1 = SC >= 1 ? NREP / 2 : NREP;
         float t[H1];
         if (SC >= 1) {
-            const bool odd = lane & 1;
 #pragma unroll
-            for (int i = 0; i < H1; ++i) {
-                const float keep = odd ? s[i + H1] : s[i];
-                const float send = odd ? s[i] : s[i + H1];
-                t[i] = keep + dpp_mov<0xB1>(0.f, send);  // quad_perm [1,0,3,2]
-            }
+            for (int i = 0; i < H1; ++i) t[i] = s[i] + dpp_mov<0xB1>(0.f, s[i + H1]);  // quad_perm [1,0,3,2]
         } else {
 #pragma unroll
             for (int i = 0; i < H1; ++i) t[i] = s[i] + dpp_mov<0xB1>(0.f, s[i]);
         }
         if (SC == 2) {
-            const bool up = lane & 2;
 #pragma unroll
-            for (int i = 0; i < VPL; ++i) {
-                const float keep = up ? t[i + VPL] : t[i];
-                const float send = up ? t[i] : t[i + VPL];
-                out[i] = keep + dpp_mov<0x4E>(0.f, send);  // quad_perm [2,3,0,1]
-            }
+            for (int i = 0; i < VPL; ++i) out[i] = t[i] + dpp_mov<0x4E>(0.f, t[i + VPL]);  // quad_perm [2,3,0,1]
         } else {
 #pragma unroll
             for (int i = 0; i < VPL; ++i) out[i] = t[i] + dpp_mov<0x4E>(0.f, t[i]);
