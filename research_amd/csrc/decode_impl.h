@@ -771,16 +771,20 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
     }
 }
 
-// Reduction pass: one workgroup of 4 waves per (sequence, query head).  The
-// pieces of the sequence are dealt round-robin to the waves (a long sequence in
-// a small batch has one piece per workgroup of the split pass), each wave
-// merges its pieces online with lanes across d, and the four wave results are
-// merged through LDS.  Rows the split pass finished in place are skipped;
-// empty sequences get their zeros here.
+// Reduction pass: one workgroup per (sequence, query head).  A long sequence in a small batch has a piece in every
+// workgroup of the split pass, hundreds of them, and all of this pass is waiting for small loads, so the
+// workgroup spreads them wide: thread (p, v) takes pieces p, p + PL, ... and the four consecutive d of 16-byte
+// vector v, keeps kPipe pieces in flight (PL * kPipe pieces of the row per round trip), merges its pieces online,
+// and the PL partial merges are combined through LDS.  Rows the split pass finished in place are skipped; empty
+// sequences get their zeros here.
 template <typename QT, int D, int NREP>
 __global__ __launch_bounds__(kThreads) void decode_reduce_kernel(const DecodeArgs a) {
-    constexpr int DPL = (D + PA_WAVE - 1) / PA_WAVE;  // d values per lane
-    __shared__ float s_w[kWaves][D + 2];
+    constexpr int V4 = D / 4;             // 16-byte vectors of a row
+    constexpr int PL = kThreads / V4;     // pieces taken side by side
+    constexpr int kPipe = 8;
+    static_assert(D % 4 == 0 && kThreads % V4 == 0 && PL >= 1, "row shape");
+    __shared__ float s_num[PL][D];
+    __shared__ float s_m[PL], s_l[PL];
     const PoolArgs &p = a.p;
     const int hq = p.hq;
     const int b = blockIdx.x / hq;
@@ -793,10 +797,10 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_kernel(const DecodeArg
     const int64_t total = per_plane * p.n_hgroups * p.n_rgroups;
     const int nblk = a.block_prefix[b + 1] - a.block_prefix[b];
     const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
-    const int lane = threadIdx.x & (PA_WAVE - 1), wave = threadIdx.x / PA_WAVE;
+    const int tid = threadIdx.x;
     QT *orow = reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * D;
     if (nblk == 0) {
-        for (int d = threadIdx.x; d < D; d += kThreads) pa_scalar<QT>::store(orow + d, 0.f);
+        for (int d = tid; d < D; d += kThreads) pa_scalar<QT>::store(orow + d, 0.f);
         return;
     }
     const int64_t u0 = plane * per_plane + a.block_prefix[b];
@@ -807,27 +811,21 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_kernel(const DecodeArg
     const int stride_acc = p.hpw * NREP * D, stride_ml = p.hpw * NREP * 2;
     // every taking-part workgroup has units (effective_grid never exceeds the number of units), so every index
     // in [w0, w1] left a partial unless its slot fell outside the workspace
-    auto has_piece = [&](int w) { return w + key < a.slot_cap; };
-    float M = kNegBig, den = 0.f, num[DPL];
-#pragma unroll
-    for (int k = 0; k < DPL; ++k) num[k] = 0.f;
-    // the pieces of a long sequence in a small batch number in the hundreds: each wave keeps the loads of
-    // kPipe of its pieces in flight, then folds them in
-    constexpr int kPipe = 8;
-    for (int w = w0 + wave; w <= w1; w += kWaves * kPipe) {
-        float m[kPipe], l[kPipe], x[kPipe][DPL];
+    const int v = tid % V4, pl = tid / V4;
+    float M = kNegBig, den = 0.f, num[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int w = w0 + pl; w <= w1; w += PL * kPipe) {
+        float m[kPipe], l[kPipe];
+        float4 x[kPipe];
 #pragma unroll
         for (int j = 0; j < kPipe; ++j) {
-            const int wj = w + j * kWaves;
-            const bool have = wj <= w1 && has_piece(wj);
+            const int wj = w + j * PL;
+            const bool have = wj <= w1 && wj + key < a.slot_cap;
             const int64_t slot = (have ? wj : w0) + key;
-            m[j] = have ? a.part_ml[slot * stride_ml + idx * 2] : kNegBig;
-            l[j] = have ? a.part_ml[slot * stride_ml + idx * 2 + 1] : 0.f;
-#pragma unroll
-            for (int k = 0; k < DPL; ++k) {
-                const int d = lane + PA_WAVE * k;
-                x[j][k] = have && d < D ? a.part_acc[slot * stride_acc + idx * D + d] : 0.f;
-            }
+            const float2 ml = *reinterpret_cast<const float2 *>(a.part_ml + slot * stride_ml + idx * 2);
+            x[j] = *reinterpret_cast<const float4 *>(a.part_acc + slot * stride_acc + idx * D + 4 * v);
+            m[j] = have ? ml.x : kNegBig;
+            l[j] = have ? ml.y : 0.f;
+            if (!have) x[j] = float4{0.f, 0.f, 0.f, 0.f};
         }
         float mn = M;
 #pragma unroll
@@ -835,32 +833,35 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_kernel(const DecodeArg
         const float so = __builtin_amdgcn_exp2f(M - mn);
         den *= so;
 #pragma unroll
-        for (int k = 0; k < DPL; ++k) num[k] *= so;
+        for (int k = 0; k < 4; ++k) num[k] *= so;
 #pragma unroll
         for (int j = 0; j < kPipe; ++j) {
             const float sn = __builtin_amdgcn_exp2f(m[j] - mn);
             den = fmaf(l[j], sn, den);
-#pragma unroll
-            for (int k = 0; k < DPL; ++k) num[k] = fmaf(x[j][k], sn, num[k]);
+            num[0] = fmaf(x[j].x, sn, num[0]);
+            num[1] = fmaf(x[j].y, sn, num[1]);
+            num[2] = fmaf(x[j].z, sn, num[2]);
+            num[3] = fmaf(x[j].w, sn, num[3]);
         }
         M = mn;
     }
 #pragma unroll
-    for (int k = 0; k < DPL; ++k)
-        if (lane + PA_WAVE * k < D) s_w[wave][lane + PA_WAVE * k] = num[k];
-    if (lane == 0) {
-        s_w[wave][D] = M;
-        s_w[wave][D + 1] = den;
+    for (int k = 0; k < 4; ++k) s_num[pl][4 * v + k] = num[k];
+    if (v == 0) {
+        s_m[pl] = M;
+        s_l[pl] = den;
     }
     __syncthreads();
-    for (int d = threadIdx.x; d < D; d += kThreads) {
+    for (int d = tid; d < D; d += kThreads) {
         float Mt = kNegBig;
-        for (int w = 0; w < kWaves; ++w) Mt = fmaxf(Mt, s_w[w][D]);
+#pragma unroll
+        for (int q = 0; q < PL; ++q) Mt = fmaxf(Mt, s_m[q]);
         float n = 0.f, dn = 0.f;
-        for (int w = 0; w < kWaves; ++w) {
-            const float wgt = __builtin_amdgcn_exp2f(s_w[w][D] - Mt);
-            n = fmaf(wgt, s_w[w][d], n);
-            dn = fmaf(wgt, s_w[w][D + 1], dn);
+#pragma unroll
+        for (int q = 0; q < PL; ++q) {
+            const float wgt = __builtin_amdgcn_exp2f(s_m[q] - Mt);
+            n = fmaf(wgt, s_num[q][d], n);
+            dn = fmaf(wgt, s_l[q], dn);
         }
         pa_scalar<QT>::store(orow + d, finish_row(n, Mt, dn, ez));
     }

@@ -72,6 +72,14 @@ template <typename AT> struct PoolWords<AT, AT> {  // 16-bit pool: the raw dword
     static __device__ __forceinline__ void unpack(const pa_u4 &raw, uint32_t (&w)[NW]) {
         w[0] = raw[0]; w[1] = raw[1]; w[2] = raw[2]; w[3] = raw[3];
     }
+    // The rows of two tokens as pairs across the tokens: lo[i] = (t0[2i], t1[2i]), hi[i] = (t0[2i+1], t1[2i+1]).
+    static __device__ __forceinline__ void interleave(const pa_u4 &t0, const pa_u4 &t1, uint32_t (&lo)[NW], uint32_t (&hi)[NW]) {
+#pragma unroll
+        for (int i = 0; i < NW; ++i) {
+            lo[i] = __builtin_amdgcn_perm(t1[i], t0[i], 0x05040100u);
+            hi[i] = __builtin_amdgcn_perm(t1[i], t0[i], 0x07060302u);
+        }
+    }
 };
 template <> struct PoolWords<pa_fp8, pa_bf16> {
     static constexpr int NW = 8;
@@ -82,6 +90,20 @@ template <> struct PoolWords<pa_fp8, pa_bf16> {
             w[2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(raw[i], 1.0f, true));
         }
     }
+    // Pairs across two tokens: the bytes of the two rows are interleaved first (two byte permutes per dword of
+    // four elements) and widened after, so every widening delivers a finished pair - 6 instructions per four
+    // elements of both tokens instead of 4 widenings and 4 permutes of the widened words.
+    static __device__ __forceinline__ void interleave(const pa_u4 &t0, const pa_u4 &t1, uint32_t (&lo)[NW], uint32_t (&hi)[NW]) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t a = __builtin_amdgcn_perm(t1[k], t0[k], 0x05010400u);  // t0.b0 t1.b0 t0.b1 t1.b1
+            const uint32_t b = __builtin_amdgcn_perm(t1[k], t0[k], 0x07030602u);  // t0.b2 t1.b2 t0.b3 t1.b3
+            lo[2 * k] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(a, 1.0f, false));
+            hi[2 * k] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(a, 1.0f, true));
+            lo[2 * k + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b, 1.0f, false));
+            hi[2 * k + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(b, 1.0f, true));
+        }
+    }
 };
 template <> struct PoolWords<pa_fp8, pa_f16> {
     static constexpr int NW = 8;
@@ -90,6 +112,20 @@ template <> struct PoolWords<pa_fp8, pa_f16> {
         for (int i = 0; i < 4; ++i) {
             w[2 * i] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[i], 1.0f, false));
             w[2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(raw[i], 1.0f, true));
+        }
+    }
+    // Pairs across two tokens: the bytes of the two rows are interleaved first (two byte permutes per dword of
+    // four elements) and widened after, so every widening delivers a finished pair - 6 instructions per four
+    // elements of both tokens instead of 4 widenings and 4 permutes of the widened words.
+    static __device__ __forceinline__ void interleave(const pa_u4 &t0, const pa_u4 &t1, uint32_t (&lo)[NW], uint32_t (&hi)[NW]) {
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t a = __builtin_amdgcn_perm(t1[k], t0[k], 0x05010400u);  // t0.b0 t1.b0 t0.b1 t1.b1
+            const uint32_t b = __builtin_amdgcn_perm(t1[k], t0[k], 0x07030602u);  // t0.b2 t1.b2 t0.b3 t1.b3
+            lo[2 * k] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(a, 1.0f, false));
+            hi[2 * k] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(a, 1.0f, true));
+            lo[2 * k + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(b, 1.0f, false));
+            hi[2 * k + 1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_f16_fp8(b, 1.0f, true));
         }
     }
 };
@@ -366,15 +402,8 @@ __device__ __forceinline__ void attend_blocks_pk(
                     st.l[j] += p0 + p1;
                     ppk[j] = kFp8 ? PK::pack(p0 * v_sc, p1 * v_sc) : PK::pack(p0, p1);
                 }
-                uint32_t v0[NW], v1[NW];
-                PW::unpack(vraw[u], v0);
-                PW::unpack(vraw[u + 1], v1);
                 uint32_t lo[NW], hi[NW];  // (v_t0[2i], v_t1[2i]) and (v_t0[2i+1], v_t1[2i+1])
-#pragma unroll
-                for (int i = 0; i < NW; ++i) {
-                    lo[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x05040100u);
-                    hi[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x07060302u);
-                }
+                PW::interleave(vraw[u], vraw[u + 1], lo, hi);
                 StaticFor<NREP>::run([&](auto h) {
                     const uint32_t pb = HS::template bcast_u<h.value>(ppk);
 #pragma unroll
@@ -519,15 +548,8 @@ __device__ __forceinline__ void attend_blocks_pk_multi(
                 st.l[j] += p0 + p1;
                 ppk[j] = kFp8 ? PK::pack(p0 * v_sc[g], p1 * v_sc[g]) : PK::pack(p0, p1);
             }
-            uint32_t v0[NW], v1[NW];
-            PW::unpack(vraw[u], v0);
-            PW::unpack(vraw[u + 1], v1);
             uint32_t lo[NW], hi[NW];  // (v_t0[2i], v_t1[2i]) and (v_t0[2i+1], v_t1[2i+1])
-#pragma unroll
-            for (int i = 0; i < NW; ++i) {
-                lo[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x05040100u);
-                hi[i] = __builtin_amdgcn_perm(v1[i], v0[i], 0x07060302u);
-            }
+            PW::interleave(vraw[u], vraw[u + 1], lo, hi);
             StaticFor<NREP>::run([&](auto h) {
                 const uint32_t pb = HS::template bcast_u<h.value>(ppk);
 #pragma unroll
