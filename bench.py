@@ -385,7 +385,9 @@ PREFILL_LONG_SHAPES = {"long-d128": (8, 2, 128, 1008, "prefill_asm_kernel"),
 def bench_prefill_long(args, dev, name) -> dict:
     """A 2048-token chunk of ONE sequence behind 200 000 cached keys (16-token blocks in random pool order, bf16,
     8 query / 2 kv heads): more keys than the prefill kernels' LDS slot tables hold, so the instances that fill them
-    again on the way run; few rows, so the launch has 64 (head_dim 128) or 128 (256) workgroups for 256 CUs."""
+    again on the way run; few rows: 64 (head_dim 128) or 128 (256) workgroups for 256 CUs, so the call hands over a
+    workspace and the head_dim 128 launch runs every workgroup's keys in pieces (kernel_ms then covers the piece
+    kernel and the merge of the pieces)."""
     from research_amd import ops
 
     hq, hkv, head_dim, seed, kernel = PREFILL_LONG_SHAPES[name]
@@ -402,8 +404,13 @@ def bench_prefill_long(args, dev, name) -> dict:
     out = torch.empty_like(q)
     scale = head_dim ** -0.5
 
+    # few rows: with a workspace the library cuts every workgroup's keys into pieces run side by side
+    ws_bytes = ops.prefill_workspace_bytes(q, tables, C, bs, hkv)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    pieces = ws_bytes // (C * hq * (head_dim + 2) * 4)
+
     def prefill():
-        ops.prefill_paged(q, kc, vc, tables, ctx, ql, qs, C, bs, scale, out=out)
+        ops.prefill_paged(q, kc, vc, tables, ctx, ql, qs, C, bs, scale, out=out, workspace=ws)
 
     if args.copy_calibration:
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
@@ -425,7 +432,8 @@ def bench_prefill_long(args, dev, name) -> dict:
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"one sequence, chunked prefill, 200000 + 2048, {hq} q / {hkv} kv heads of {head_dim}, bf16",
                    "num_seqs": 1, "prefix_len": P, "chunk_len": C, "num_q_heads": hq, "num_kv_heads": hkv,
-                   "head_dim": head_dim, "block_size": bs, "attention_flops": flops, "seed": seed},
+                   "head_dim": head_dim, "block_size": bs, "attention_flops": flops, "seed": seed,
+                   "key_pieces_per_workgroup": max(1, pieces), "workspace_bytes": ws_bytes},
         "roofline": {"bound": "mfma", "kernel": kernel, "achieved": achieved,
                      "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
                      "traffic": measured_traffic(name), "kernel_ms": ms_kernel,

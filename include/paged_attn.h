@@ -45,7 +45,7 @@ extern "C" {
 #define PA_F16 2
 #define PA_FP8_E4M3 3 /* OCP e4m3fn, KV pool only; q/out stay 16- or 32-bit */
 
-/* Library ABI version (bumped when an entry point is added or a signature or contract changes; now 5). */
+/* Library ABI version (bumped when an entry point is added or a signature or contract changes; now 6). */
 int pa_version(void);
 
 /* Text of the calling thread's most recent error; "" if none. */
@@ -222,6 +222,32 @@ int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, vo
                      const int32_t *q_lens, const int32_t *q_starts, const int32_t *row_first_key,
                      int batch, int max_q_len, int num_q_heads, int num_kv_heads, int head_dim,
                      int block_size, int64_t num_blocks, float scale, int window, int dtype, void *stream);
+
+/*
+ * pa_prefill_paged with a workspace, for launches of few query rows.  The reference's SDPA call
+ * (attention/flex_backend.py:180-182) spreads one long row's keys over the machine however PyTorch likes; the
+ * matrix-core kernels here give a workgroup 256 row-head pairs and all their keys, so one 2048-row chunk behind a
+ * long cached context occupies a quarter of the compute units.  Given a workspace, such a launch cuts every
+ * workgroup's keys into up to 8 pieces run by workgroups of their own, which leave (maximum, sum, unnormalised
+ * output row) per piece in the workspace, and a second kernel merges them - the arithmetic of pa_decode's
+ * reduction pass.  Results equal pa_prefill_paged's to fp32 merge-order rounding.
+ *   total_q        : rows of q / out (every q_starts[b] + q_lens[b] <= total_q)
+ *   workspace      : pa_prefill_workspace_bytes(...) bytes, 256-byte aligned, contents need not be initialised;
+ *                    NULL or too small for any split: the call is pa_prefill_paged.  A smaller workspace is used
+ *                    for as many pieces as it holds.
+ * pa_prefill_workspace_bytes: what the split the library would choose for these shapes on the current device needs
+ * (0 when the launch fills the device anyway, or for shapes only the unsplit kernels take: head_dim 256, fp32,
+ * tables of several blocks that are not multiples of 16 keys long); host arithmetic plus one device-attribute query.
+ * bt_stride * block_size bounds the context length the split is sized for.
+ */
+size_t pa_prefill_workspace_bytes(int batch, int max_q_len, int64_t total_q, int64_t bt_stride, int block_size,
+                                  int window, int num_q_heads, int num_kv_heads, int head_dim, int dtype);
+int pa_prefill_paged_ws(const void *q, const void *k_cache, const void *v_cache, void *out,
+                        const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
+                        const int32_t *q_lens, const int32_t *q_starts, const int32_t *row_first_key,
+                        int batch, int max_q_len, int num_q_heads, int num_kv_heads, int head_dim,
+                        int block_size, int64_t num_blocks, float scale, int window, int dtype, void *stream,
+                        int64_t total_q, void *workspace, size_t workspace_bytes);
 
 /*
  * Attention under an arbitrary mask: what FlexAttentionBackend does with a ctx.block_mask built from any

@@ -83,6 +83,10 @@ SIGNATURES = {
 }
 SIGNATURES["pa_decode_split"] = SIGNATURES["pa_decode_reduce"] = SIGNATURES["pa_decode"]
 SIGNATURES["pa_prefill_paged_rowwise"] = SIGNATURES["pa_prefill_paged"]
+# pa_prefill_paged + total_q, workspace, workspace_bytes
+SIGNATURES["pa_prefill_paged_ws"] = (c_int, SIGNATURES["pa_prefill_paged"][1] + [c_int64, c_void_p, c_size_t])
+SIGNATURES["pa_prefill_workspace_bytes"] = (
+    c_size_t, [c_int, c_int, c_int64, c_int64, c_int, c_int, c_int, c_int, c_int, c_int])
 # pa_decode without the workspace pointer and size
 SIGNATURES["pa_decode_static"] = (c_int, SIGNATURES["pa_decode"][1][:-3] + [c_void_p])
 

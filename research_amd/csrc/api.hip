@@ -18,7 +18,7 @@ int pa_fail(int code, const char *fmt, ...) {
 
 void pa_clear_error() { g_last_error[0] = '\0'; }
 
-extern "C" int pa_version(void) { return 5; }
+extern "C" int pa_version(void) { return 6; }
 
 extern "C" const char *pa_last_error(void) { return g_last_error; }
 

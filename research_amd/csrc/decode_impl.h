@@ -79,6 +79,11 @@ struct RowwiseArgs {
     const int32_t *row_lo;  // per query row: first key it sees (NULL = none); non-decreasing along a sequence
     int batch;
     int max_q_len;
+    // Matrix-core kernels only: a workgroup's tiles cut into `splits` pieces, each run by a workgroup of its own
+    // (grid.y = groups * splits) that leaves (m, l) and the unnormalised O rows of its piece in the workspace for
+    // the merge kernel: part_o float [row][head][split][D], part_ml float [row][head][split][2].  1 = no split.
+    int splits;
+    float *part_o, *part_ml;
 };
 
 __device__ __forceinline__ uint4 ld16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }

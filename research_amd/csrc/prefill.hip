@@ -11,11 +11,87 @@ using namespace pa_decode_detail;
 
 namespace {
 
+// Compute units of the current device (asked once per device).
+int prefill_cus() {
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+    }
+    return n;
+}
+
+constexpr int kMaxPrefillSplits = 8;
+constexpr int kMinTilesPerSplit = 24;  // a piece's set-up and write-out cost about six tiles of its loop
+
+// Pieces to cut every workgroup's tiles into, from shapes alone.  The matrix-core kernels run one workgroup per
+// compute unit, each owning 256 (head_dim 256: 128) row-head pairs and all their keys, so a launch of few rows
+// leaves compute units idle however long the context is.  The launch takes rounds of `cus` workgroups, each lasting
+// a piece's tiles plus its fixed cost; the split with the shortest estimate wins (the smaller on ties), as long as a
+// piece keeps kMinTilesPerSplit tiles of the longest context the block tables can describe.
+int prefill_splits(int64_t workgroups, int cus, int64_t max_keys) {
+    const int64_t tiles = max_keys / kPfKeys;
+    constexpr int64_t kFixedTiles = 6;  // set-up and write-out of a workgroup, in tiles of its loop
+    int best = 1;
+    int64_t best_cost = 0;
+    for (int s = 1; s <= kMaxPrefillSplits; ++s) {
+        if (s > 1 && tiles / s < kMinTilesPerSplit) break;
+        const int64_t rounds = (workgroups * s + cus - 1) / cus;
+        const int64_t cost = rounds * (tiles / s + kFixedTiles);
+        if (s == 1 || cost < best_cost) {
+            best_cost = cost;
+            best = s;
+        }
+    }
+    return best;
+}
+
+size_t prefill_ws_bytes(int64_t total_q, int num_q_heads, int head_dim, int splits) {
+    return splits <= 1 ? 0 : (size_t)total_q * num_q_heads * splits * ((size_t)head_dim + 2) * sizeof(float);
+}
+
+// Merge of the pieces of a split prefill launch: one thread per (row, head, four consecutive d).
+template <typename T>
+__global__ __launch_bounds__(256) void prefill_merge_kernel(const float *part_o, const float *part_ml, T *out,
+                                                            const int32_t *q_lens, const int32_t *q_starts, int hq,
+                                                            int d_head, int splits) {
+    const int b = blockIdx.z, i = blockIdx.y;
+    if (i >= q_lens[b]) return;
+    const int item = blockIdx.x * 256 + threadIdx.x, v4 = d_head / 4;
+    if (item >= hq * v4) return;
+    const int h = item / v4, d = (item - h * v4) * 4;
+    const int64_t row = (int64_t)q_starts[b] + i;
+    const int64_t base = (row * hq + h) * splits;
+    float m_all = -1.0e30f;
+    for (int s = 0; s < splits; ++s)
+        if (part_ml[(base + s) * 2 + 1] > 0.f) m_all = fmaxf(m_all, part_ml[(base + s) * 2]);
+    float den = 0.f, num[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int s = 0; s < splits; ++s) {
+        const float l = part_ml[(base + s) * 2 + 1];
+        if (!(l > 0.f)) continue;  // a piece in which the row saw no key wrote no O row
+        const float w = __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - m_all);
+        const float4 o = *reinterpret_cast<const float4 *>(part_o + (base + s) * d_head + d);
+        den = fmaf(w, l, den);
+        num[0] = fmaf(w, o.x, num[0]);
+        num[1] = fmaf(w, o.y, num[1]);
+        num[2] = fmaf(w, o.z, num[2]);
+        num[3] = fmaf(w, o.w, num[3]);
+    }
+    const float inv = den > 0.f ? 1.f / den : 0.f;
+    T *op = out + (row * hq + h) * d_head + d;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) pa_scalar<T>::store(op + j, num[j] * inv);
+}
+
 int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const void *v_cache, void *out,
                    const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens, const int32_t *q_lens,
                    const int32_t *q_starts, const int32_t *row_first_key, int batch, int max_q_len, int num_q_heads,
                    int num_kv_heads, int head_dim, int block_size, int64_t num_blocks, float scale, int window,
-                   int dtype, void *stream) {
+                   int dtype, void *stream, int64_t total_q = 0, void *workspace = nullptr,
+                   size_t workspace_bytes = 0) {
     pa_clear_error();
     PA_REQUIRE(batch >= 0 && max_q_len >= 0, "batch=%d max_q_len=%d must be non-negative", batch, max_q_len);
     PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && head_dim > 0, "head counts / head_dim must be positive");
@@ -46,12 +122,14 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     a.q = q; a.out = out; a.ctx_lens = ctx_lens; a.q_lens = q_lens; a.q_starts = q_starts;
     a.row_lo = row_first_key;
     a.batch = batch; a.max_q_len = max_q_len;
+    a.splits = 1; a.part_o = nullptr; a.part_ml = nullptr;
     hipStream_t s = (hipStream_t)stream;
     // bf16 / fp16 with head_dim 32, 64, 128 (and 256, below) run on the matrix cores unless the caller asked for the
     // vector kernel
     // (the matrix-core softmax takes the running maximum of the unscaled logits, which needs scale > 0)
     prefill_mfma_fn mfma =
         force_rowwise || !(scale > 0.f) ? nullptr : pa_prefill_mfma_kernel(dtype, head_dim, block_size == 16);
+    int split = 1;  // pieces per workgroup (the kernels with the assembly loop, given a workspace)
     // head_dim 128, 64 or 32, blocks of a multiple of 16 tokens (or one block per sequence, as dense prefill passes its
     // rows): the kernel whose whole tile loop is scheduled assembly (one instance without, one with sliding window /
     // per-row first keys).  Its LDS copy of the table holds pa_asm_cap_tiles() tiles from the workgroup's first tile
@@ -64,12 +142,23 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
         const int64_t cap_keys = (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys;
         const bool fits = bt_stride * (int64_t)block_size <= cap_keys ||
                           (window > 0 && (int64_t)window + kPfTasks * kPfRows + 3 * kPfKeys <= cap_keys);
-        mfma = pa_prefill_asm_kernel(dtype, head_dim, window > 0 || row_first_key != nullptr, !fits);
+        // With a workspace, a launch that cannot fill the chip has every workgroup's tiles cut into pieces (the
+        // instance with lower bounds runs them: a piece is a later first tile and an earlier last key).
+        if (workspace) {
+            const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
+            const int64_t groups = (row_blocks * (int64_t)a.p.n_rep + kPfTasks - 1) / kPfTasks;
+            int want = prefill_splits((int64_t)num_kv_heads * groups * batch, prefill_cus(),
+                                      window > 0 ? (int64_t)window + kPfTasks * kPfRows : bt_stride * (int64_t)block_size);
+            while (want > 1 && prefill_ws_bytes(total_q, num_q_heads, head_dim, want) > workspace_bytes) --want;
+            split = want;
+        }
+        mfma = pa_prefill_asm_kernel(dtype, head_dim, split > 1 || window > 0 || row_first_key != nullptr, !fits);
     }
     // head_dim 256: one 32-row task per wave, loads driven by a table of 16-key groups - which must lie inside one
     // pool block (block sizes that are multiples of 16, or a single block per sequence); the kernel fills its table
     // again whenever the context is longer than what LDS can hold of it
     int tasks_per_wg = kPfTasks;
+    if (head_dim == 256) split = 1;
     // (a pool of fewer than 16 rows has no slot a whole group could be loaded from: the vector kernel)
     if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
@@ -85,9 +174,26 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
         PA_REQUIRE(pa_aligned16(q) && pa_aligned16(out), "q and out must be 16-byte aligned");
         const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
         const int groups = (row_blocks * a.p.n_rep + tasks_per_wg - 1) / tasks_per_wg;
-        PA_REQUIRE(groups <= 65535, "max_q_len=%d is too long for one launch", max_q_len);
-        mfma<<<dim3((unsigned)num_kv_heads, (unsigned)groups, (unsigned)batch), dim3(kPfThreads), 0, s>>>(a);
+        PA_REQUIRE((int64_t)groups * split <= 65535, "max_q_len=%d is too long for one launch", max_q_len);
+        if (split > 1) {
+            PA_REQUIRE(((uintptr_t)workspace & 255u) == 0, "workspace must be 256-byte aligned");
+            a.splits = split;
+            a.part_o = (float *)workspace;
+            a.part_ml = a.part_o + (size_t)total_q * num_q_heads * split * head_dim;
+        }
+        mfma<<<dim3((unsigned)num_kv_heads, (unsigned)(groups * split), (unsigned)batch), dim3(kPfThreads), 0, s>>>(a);
         PA_CHECK_LAUNCH("pa_prefill_paged (matrix-core kernel)");
+        if (split > 1) {
+            const unsigned gx = (unsigned)((num_q_heads * (head_dim / 4) + 255) / 256);
+            const dim3 mg(gx, (unsigned)max_q_len, (unsigned)batch);
+            if (dtype == PA_BF16)
+                prefill_merge_kernel<pa_bf16><<<mg, dim3(256), 0, s>>>(a.part_o, a.part_ml, (pa_bf16 *)out, q_lens, q_starts,
+                                                                     num_q_heads, head_dim, split);
+            else
+                prefill_merge_kernel<pa_f16><<<mg, dim3(256), 0, s>>>(a.part_o, a.part_ml, (pa_f16 *)out, q_lens, q_starts,
+                                                                    num_q_heads, head_dim, split);
+            PA_CHECK_LAUNCH("pa_prefill_paged_ws (merge of the pieces)");
+        }
         return PA_OK;
     }
     ks.rowwise<<<dim3((unsigned)(a.p.n_hgroups * a.p.n_rgroups), (unsigned)max_q_len, (unsigned)batch),
@@ -108,4 +214,34 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
         max_q_len, num_q_heads, num_kv_heads, head_dim, block_size, num_blocks, scale, window, dtype, stream
 
 extern "C" int pa_prefill_paged(PA_PREFILL_PARAMS) { return prefill_launch(false, PA_PREFILL_ARGS); }
+
+extern "C" size_t pa_prefill_workspace_bytes(int batch, int max_q_len, int64_t total_q, int64_t bt_stride,
+                                             int block_size, int window, int num_q_heads, int num_kv_heads,
+                                             int head_dim, int dtype) {
+    pa_clear_error();
+    if (batch < 0 || max_q_len < 0 || total_q < 0 || bt_stride < 0 || block_size <= 0 || window < 0 ||
+        num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0 || head_dim <= 0) {
+        pa_fail(PA_ERR_INVALID_ARG, "pa_prefill_workspace_bytes: negative size or inconsistent head counts");
+        return 0;
+    }
+    // only the 16-bit kernels with the assembly loop for head_dim 32 / 64 / 128 split; everything else needs none
+    if ((dtype != PA_BF16 && dtype != PA_F16) || (head_dim != 128 && head_dim != 64 && head_dim != 32) || batch == 0 ||
+        max_q_len == 0)
+        return 0;
+    const int n_rep = num_q_heads / num_kv_heads;
+    const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
+    const int64_t groups = (row_blocks * (int64_t)n_rep + kPfTasks - 1) / kPfTasks;
+    const int split = prefill_splits((int64_t)num_kv_heads * groups * batch, prefill_cus(),
+                                     window > 0 ? (int64_t)window + kPfTasks * kPfRows : bt_stride * (int64_t)block_size);
+    return prefill_ws_bytes(total_q, num_q_heads, head_dim, split);
+}
+
+extern "C" int pa_prefill_paged_ws(PA_PREFILL_PARAMS, int64_t total_q, void *workspace, size_t workspace_bytes) {
+    if (workspace && total_q <= 0) {
+        pa_clear_error();
+        return pa_fail(PA_ERR_INVALID_ARG, "pa_prefill_paged_ws: total_q=%lld must be positive with a workspace",
+                       (long long)total_q);
+    }
+    return prefill_launch(false, PA_PREFILL_ARGS, total_q, workspace, workspace_bytes);
+}
 extern "C" int pa_prefill_paged_rowwise(PA_PREFILL_PARAMS) { return prefill_launch(true, PA_PREFILL_ARGS); }

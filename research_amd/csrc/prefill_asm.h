@@ -67,10 +67,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     // workgroup -> (kv head, group of 8 tasks, sequence), heaviest groups first when the prefix is short
     // (the launch order of prefill_mfma_kernel)
     const int kvh = blockIdx.x;
-    const int n_groups = gridDim.y, n_seqs = gridDim.z;
-    const int lin = blockIdx.y + n_groups * blockIdx.z;
+    const int n_splits = a.splits;  // pieces a workgroup's tiles are cut into (1: none; more only in the LO instance)
+    const int piece = (int)blockIdx.y % n_splits, group_y = (int)blockIdx.y / n_splits;
+    const int n_groups = gridDim.y / n_splits, n_seqs = gridDim.z;
+    const int lin = group_y + n_groups * blockIdx.z;
     const bool group_major = a.ctx_lens[0] - a.q_lens[0] < a.q_lens[0];
-    const int group = group_major ? n_groups - 1 - lin / n_seqs : (int)blockIdx.y;
+    const int group = group_major ? n_groups - 1 - lin / n_seqs : group_y;
     const int b = group_major ? lin % n_seqs : (int)blockIdx.z;
     const int q_len = a.q_lens[b];
     const int ctx_len = a.ctx_lens[b];
@@ -92,7 +94,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         qh[c] = kvh * p.n_rep + rep;
     }
     const int last_task = min(n_tasks, task0 + kPfTasks) - 1;
-    const int wg_keys = min(ctx_len, prefix + min(q_len, (last_task / p.n_rep) * kPfRows + kPfRows));
+    int wg_keys = min(ctx_len, prefix + min(q_len, (last_task / p.n_rep) * kPfRows + kPfRows));
     // subtiles that reach past this key hold keys some row of the wave must not see
     const int mask_from = min(prefix + min(row0[0], row0[1]) + 1, ctx_len);
     // a lane's last visible key per column tile, less the 4 keys its half of the wave is ahead by
@@ -117,6 +119,29 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
         lo_mask_until = row_first(min(q_len, max(row0[0], row0[1]) + kPfRows) - 1);
 #pragma unroll
         for (int c = 0; c < NC; ++c) lo[c] = row_first(row0[c] + col) - 4 * half;
+    }
+    if constexpr (LO) {
+        if (n_splits > 1) {
+            // This workgroup runs piece `piece` of the tiles [t0, t0 + n_all): a later first tile and an earlier
+            // last key, nothing else changes (rows that see none of the piece's keys end with an empty sum).
+            const int n_all = (wg_keys + kPfKeys - 1) / kPfKeys - t0;
+            const int tb = t0 + (int)((int64_t)piece * n_all / n_splits);
+            const int te = t0 + (int)((int64_t)(piece + 1) * n_all / n_splits);
+            if (tb >= te) {  // uniform: fewer tiles than pieces - an empty partial for every row
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    const int row = row0[c] + col;
+                    if (live[c] && row < q_len && half == 0) {
+                        const int64_t at = ((((int64_t)a.q_starts[b] + row) * p.hq + qh[c]) * n_splits + piece) * 2;
+                        a.part_ml[at] = kNegBig;
+                        a.part_ml[at + 1] = 0.f;
+                    }
+                }
+                return;
+            }
+            t0 = tb;
+            wg_keys = min(wg_keys, te * kPfKeys);
+        }
     }
     // tiles the loop runs (>= 1), counted from t0 like every tile number below
     const int n_tiles = (wg_keys + kPfKeys - 1) / kPfKeys - t0;
@@ -494,6 +519,36 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 #undef PA_LO_IN
     }
 
+    if constexpr (LO) {
+        if (n_splits > 1) {
+            // ---- a piece: the row's reference maximum, sum and unnormalised O^T go to the workspace ----
+            // (the accumulators sit in the registers the assembly loop pins them to; they leave through a multiply
+            // by a one the compiler cannot see through, as they do through the normalisation in the write-out below -
+            // a plain copy of such an element is mis-selected by this compiler)
+            float one = 1.f;
+            asm volatile("" : "+v"(one));
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                const float l_tot = l_run[c] + __shfl_xor(l_run[c], 32, 64);
+                const int row = row0[c] + col;
+                if (!live[c] || row >= q_len) continue;
+                const int64_t at = (((int64_t)a.q_starts[b] + row) * p.hq + qh[c]) * n_splits + piece;
+                float *po = a.part_o + at * D + 4 * half;  // lane owns d = 32*dt + 8*g + 4*half + j
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g)
+                        *reinterpret_cast<float4 *>(po + 32 * dt + 8 * g) =
+                            float4{o[c][dt][4 * g] * one, o[c][dt][4 * g + 1] * one, o[c][dt][4 * g + 2] * one,
+                                   o[c][dt][4 * g + 3] * one};
+                if (half == 0) {
+                    a.part_ml[at * 2] = l_tot > 0.f ? -(ref[c][0] * one) : kNegBig;  // (a row that saw no key has no maximum)
+                    a.part_ml[at * 2 + 1] = l_tot;
+                }
+            }
+            return;
+        }
+    }
     // ---- normalise; rows go through LDS so that every store instruction writes whole 256-byte rows ----
     __syncthreads();  // every wave is done with the ring
     const uint32_t out_stage = (uint32_t)wave * (NC * 32 * QRB);  // this wave's 64 rows of 256 bytes

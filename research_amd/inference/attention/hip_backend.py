@@ -634,9 +634,12 @@ class HipPagedAttentionBackend:
             kc = ops.dequantize_blocks_e4m3(kc, self.k_scale[layer_idx], step.fp8_blocks, cfg.block_size, q.dtype)
             vc = ops.dequantize_blocks_e4m3(vc, self.v_scale[layer_idx], step.fp8_blocks, cfg.block_size, q.dtype)
             tables = step.fp8_tables
-        ops.prefill_paged(q.contiguous().view(batch * seq_len, num_heads, head_dim), kc, vc, tables,
-                          step.ctx_lens, step.q_lens, step.q_starts, step.max_q_len, cfg.block_size, self.scale,
-                          out=out.view(batch * seq_len, num_heads, head_dim), window=window, row_first_key=first)
+        q3 = q.contiguous().view(batch * seq_len, num_heads, head_dim)
+        # a step of few rows over a long context: with a workspace the kernel spreads its keys over the device
+        need = ops.prefill_workspace_bytes(q3, tables, step.max_q_len, cfg.block_size, cfg.num_kv_heads, window)
+        ops.prefill_paged(q3, kc, vc, tables, step.ctx_lens, step.q_lens, step.q_starts, step.max_q_len,
+                          cfg.block_size, self.scale, out=out.view(batch * seq_len, num_heads, head_dim), window=window,
+                          row_first_key=first, workspace=self._workspace_for(need) if need else None)
         return out
 
     # ------------------------------------------------------------------ fp8 pool

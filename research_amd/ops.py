@@ -115,25 +115,43 @@ def decode_static(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Ten
     return out
 
 
+def prefill_workspace_bytes(q: Tensor, block_tables: Tensor, max_q_len: int, block_size: int, num_kv_heads: int,
+                            window: int = 0) -> int:
+    """Bytes of workspace with which ``prefill_paged`` spreads a launch of few rows over the device (0: the launch
+    fills it anyway, or its shapes have no split kernel)."""
+    total_q, hq, d = q.shape
+    if q.dtype not in PA_DTYPE:
+        return 0
+    return int(_lib.load().pa_prefill_workspace_bytes(block_tables.shape[0], int(max_q_len), total_q,
+                                                      block_tables.shape[1], block_size, int(window), hq,
+                                                      num_kv_heads, d, PA_DTYPE[q.dtype]))
+
+
 def prefill_paged(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, ctx_lens: Tensor,
                   q_lens: Tensor, q_starts: Tensor, max_q_len: int, block_size: int, scale: float,
                   out: Optional[Tensor] = None, window: int = 0, row_first_key: Optional[Tensor] = None,
-                  rowwise: bool = False) -> Tensor:
+                  rowwise: bool = False, workspace: Optional[Tensor] = None) -> Tensor:
     """Causal prefill over a paged context; q ``[total_q, Hq, D]`` packed rows; ``window`` > 0 adds the
     sliding window (a row at position p sees keys p - window < j <= p); ``row_first_key`` (int32 per q row,
     non-decreasing along a sequence) adds a per-row first key, e.g. the start of the row's document;
-    ``rowwise`` selects the vector kernel (``pa_prefill_paged_rowwise``) also where a matrix-core kernel exists."""
+    ``rowwise`` selects the vector kernel (``pa_prefill_paged_rowwise``) also where a matrix-core kernel exists;
+    ``workspace`` (uint8, ``prefill_workspace_bytes`` or more) lets a launch of few rows split its keys over
+    several workgroups (``pa_prefill_paged_ws``)."""
     total_q, hq, d = q.shape
     if row_first_key is not None and (row_first_key.dtype != torch.int32 or row_first_key.numel() != total_q):
         raise ValueError("row_first_key must hold one int32 per q row")
     total_slots, hkv, _ = k_cache.shape
     if out is None:
         out = torch.empty_like(q)
-    _run("pa_prefill_paged_rowwise" if rowwise else "pa_prefill_paged", _ptr(q), _ptr(k_cache), _ptr(v_cache),
-         _ptr(out), _ptr(block_tables),
-         block_tables.shape[1], _ptr(ctx_lens), _ptr(q_lens), _ptr(q_starts),
-         _ptr(row_first_key) if row_first_key is not None else None, block_tables.shape[0], max_q_len, hq,
-         hkv, d, block_size, total_slots // block_size, float(scale), int(window), PA_DTYPE[q.dtype], _stream(q))
+    args = (_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_tables), block_tables.shape[1],
+            _ptr(ctx_lens), _ptr(q_lens), _ptr(q_starts), _ptr(row_first_key) if row_first_key is not None else None,
+            block_tables.shape[0], max_q_len, hq, hkv, d, block_size, total_slots // block_size, float(scale),
+            int(window), PA_DTYPE[q.dtype], _stream(q))
+    if workspace is not None and not rowwise:
+        # (``pa_prefill_paged_ws``: the launch is cut into pieces over the keys when it has too few rows for the device)
+        _run("pa_prefill_paged_ws", *args, total_q, _ptr(workspace), workspace.numel() * workspace.element_size())
+    else:
+        _run("pa_prefill_paged_rowwise" if rowwise else "pa_prefill_paged", *args)
     return out
 
 

@@ -33,7 +33,7 @@ def test_binding_table_matches_header():
 
 def test_version_and_dtype_sizes():
     lib = _lib.load()
-    assert lib.pa_version() == 5
+    assert lib.pa_version() == 6
     assert [lib.pa_dtype_bytes(c) for c in (0, 1, 2, 3, 4, -1)] == [4, 2, 2, 1, 0, 0]
 
 
