@@ -158,7 +158,6 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // pool block (block sizes that are multiples of 16, or a single block per sequence); the kernel fills its table
     // again whenever the context is longer than what LDS can hold of it
     int tasks_per_wg = kPfTasks;
-    if (head_dim == 256) split = 1;
     // (a pool of fewer than 16 rows has no slot a whole group could be loaded from: the vector kernel)
     if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
@@ -167,7 +166,15 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
         // a workgroup's kWdTasks blocks of kPfRows rows, and the tiles its loads run ahead, bound what it needs)
         const bool fits = bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16 ||
                           (window > 0 && (int64_t)window + kWdTasks * kPfRows + 10 * 32 <= (int64_t)kWdCapGroups * 16);
-        mfma = pa_prefill_d256_kernel(dtype, window > 0 || row_first_key != nullptr, !fits);
+        if (workspace) {  // (as above; a workgroup of this kernel holds kWdTasks tasks)
+            const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
+            const int64_t groups = (row_blocks * (int64_t)a.p.n_rep + kWdTasks - 1) / kWdTasks;
+            int want = prefill_splits((int64_t)num_kv_heads * groups * batch, prefill_cus(),
+                                      window > 0 ? (int64_t)window + kWdTasks * kPfRows : bt_stride * (int64_t)block_size);
+            while (want > 1 && prefill_ws_bytes(total_q, num_q_heads, head_dim, want) > workspace_bytes) --want;
+            split = want;
+        }
+        mfma = pa_prefill_d256_kernel(dtype, split > 1 || window > 0 || row_first_key != nullptr, !fits);
         tasks_per_wg = kWdTasks;
     }
     if (mfma) {
@@ -224,15 +231,16 @@ extern "C" size_t pa_prefill_workspace_bytes(int batch, int max_q_len, int64_t t
         pa_fail(PA_ERR_INVALID_ARG, "pa_prefill_workspace_bytes: negative size or inconsistent head counts");
         return 0;
     }
-    // only the 16-bit kernels with the assembly loop for head_dim 32 / 64 / 128 split; everything else needs none
-    if ((dtype != PA_BF16 && dtype != PA_F16) || (head_dim != 128 && head_dim != 64 && head_dim != 32) || batch == 0 ||
-        max_q_len == 0)
+    // only the 16-bit kernels with the assembly loop (head_dim 32 / 64 / 128 / 256) split; everything else needs none
+    if ((dtype != PA_BF16 && dtype != PA_F16) ||
+        (head_dim != 256 && head_dim != 128 && head_dim != 64 && head_dim != 32) || batch == 0 || max_q_len == 0)
         return 0;
     const int n_rep = num_q_heads / num_kv_heads;
     const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
-    const int64_t groups = (row_blocks * (int64_t)n_rep + kPfTasks - 1) / kPfTasks;
+    const int tasks = head_dim == 256 ? kWdTasks : kPfTasks;
+    const int64_t groups = (row_blocks * (int64_t)n_rep + tasks - 1) / tasks;
     const int split = prefill_splits((int64_t)num_kv_heads * groups * batch, prefill_cus(),
-                                     window > 0 ? (int64_t)window + kPfTasks * kPfRows : bt_stride * (int64_t)block_size);
+                                     window > 0 ? (int64_t)window + tasks * kPfRows : bt_stride * (int64_t)block_size);
     return prefill_ws_bytes(total_q, num_q_heads, head_dim, split);
 }
 

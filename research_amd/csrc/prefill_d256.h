@@ -69,10 +69,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 
     // workgroup -> (kv head, group of 4 tasks, sequence): the launch order of prefill_mfma_kernel
     const int kvh = blockIdx.x;
-    const int n_groups = gridDim.y, n_seqs = gridDim.z;
-    const int lin = blockIdx.y + n_groups * blockIdx.z;
+    const int n_splits = a.splits;  // pieces a workgroup's tiles are cut into (1: none; more only in the LO instances)
+    const int piece = (int)blockIdx.y % n_splits, group_y = (int)blockIdx.y / n_splits;
+    const int n_groups = gridDim.y / n_splits, n_seqs = gridDim.z;
+    const int lin = group_y + n_groups * blockIdx.z;
     const bool group_major = a.ctx_lens[0] - a.q_lens[0] < a.q_lens[0];
-    const int group = group_major ? n_groups - 1 - lin / n_seqs : (int)blockIdx.y;
+    const int group = group_major ? n_groups - 1 - lin / n_seqs : group_y;
     const int b = group_major ? lin % n_seqs : (int)blockIdx.z;
     const int q_len = a.q_lens[b];
     const int ctx_len = a.ctx_lens[b];
@@ -89,7 +91,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     const int qh = kvh * p.n_rep + (live ? task - rb * p.n_rep : 0);
     const int last_task = min(n_tasks, task0 + kWdTasks) - 1;
     const int wg_keys = min(ctx_len, prefix + min(q_len, (last_task / p.n_rep) * kPfRows + kPfRows));
-    const int n_tiles = (wg_keys + kWdKeys - 1) / kWdKeys;  // >= 1
+    int n_tiles = (wg_keys + kWdKeys - 1) / kWdKeys;  // >= 1; the workgroup runs tiles t0 .. n_tiles-1
     // lower bounds (sliding window, per-row first keys): see prefill_mfma_kernel
     const int win = p.window;
     const int32_t *rlo = a.row_lo ? a.row_lo + a.q_starts[b] : nullptr;
@@ -101,7 +103,27 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         return min(max(lo, 0), min(pos, ctx_len - 1));
     };
     const int wg_first_key = bounded ? row_first((task0 / p.n_rep) * kPfRows) : 0;
-    const int t0 = wg_first_key / kWdKeys;  // first tile of the workgroup (< n_tiles)
+    int t0 = wg_first_key / kWdKeys;  // first tile of the workgroup (< n_tiles)
+    if constexpr (LO) {
+        if (n_splits > 1) {
+            // This workgroup runs piece `piece` of the tiles [t0, n_tiles): a later first tile and an earlier last
+            // one, nothing else changes (rows that see none of the piece's keys end with an empty sum).
+            const int n_all = n_tiles - t0;
+            const int tb = t0 + (int)((int64_t)piece * n_all / n_splits);
+            const int te = t0 + (int)((int64_t)(piece + 1) * n_all / n_splits);
+            if (tb >= te) {  // uniform: fewer tiles than pieces - an empty partial for every row
+                const int row = row0 + col;
+                if (live && row < q_len && half == 0) {
+                    const int64_t at = ((((int64_t)a.q_starts[b] + row) * p.hq + qh) * n_splits + piece) * 2;
+                    a.part_ml[at] = kNegBig;
+                    a.part_ml[at + 1] = 0.f;
+                }
+                return;
+            }
+            t0 = tb;
+            n_tiles = te;
+        }
+    }
     const int mask_from = min(prefix + row0 + 1, ctx_len);  // subtiles reaching past this key are masked
     const int lo_mask_until = bounded ? row_first(min(q_len, row0 + kPfRows) - 1) : 0;  // subtiles starting below it too
     // a lane's last and first visible key, less the 4 keys its half of the wave is ahead by
@@ -452,6 +474,27 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
     const int row = row0 + col;
     if (!live || row >= q_len) return;
+    if constexpr (LO) {
+        if (n_splits > 1) {
+            // a piece: the row's reference maximum, sum and unnormalised O^T go to the workspace (through a multiply
+            // by a one the compiler cannot see through: see prefill_asm_kernel)
+            float one = 1.f;
+            asm volatile("" : "+v"(one));
+            const int64_t at = (((int64_t)a.q_starts[b] + row) * p.hq + qh) * n_splits + piece;
+            float *po = a.part_o + at * D + 4 * half;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    *reinterpret_cast<float4 *>(po + 32 * dt + 8 * g) =
+                        float4{o[dt][4 * g] * one, o[dt][4 * g + 1] * one, o[dt][4 * g + 2] * one, o[dt][4 * g + 3] * one};
+            if (half == 0) {
+                a.part_ml[at * 2] = l_tot > 0.f ? -(ref[0] * one) : kNegBig;  // (a row that saw no key has no maximum)
+                a.part_ml[at * 2 + 1] = l_tot;
+            }
+            return;
+        }
+    }
     T *orow = reinterpret_cast<T *>(a.out) + (((int64_t)a.q_starts[b] + row) * p.hq + qh) * D;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)

@@ -77,7 +77,8 @@ class Case:
 
 @pytest.mark.parametrize("pieces", [2, 3, 8])
 @pytest.mark.parametrize("d,hq,hkv,dtype", [(128, 8, 2, torch.bfloat16), (64, 4, 1, torch.float16),
-                                           (32, 4, 2, torch.bfloat16)])
+                                           (32, 4, 2, torch.bfloat16), (256, 4, 2, torch.bfloat16),
+                                           (256, 2, 1, torch.float16)])
 def test_one_long_sequence_in_pieces(pieces, d, hq, hkv, dtype):
     announce(f"split prefill: one sequence, {pieces} pieces, d={d} {dtype}")
     c = Case([2900], [150], hq, hkv, d, dtype=dtype, seed=pieces + d)
@@ -136,11 +137,11 @@ def test_context_longer_than_the_kernel_tables_in_pieces():
 def test_workspace_rules():
     c = Case([2900], [150], 8, 2, 128, seed=1)
     q = c.q.reshape(150, 8, 128).to(DEV)
-    # a launch that fills the device needs no workspace; head_dim 256 and fp32 have no split kernel
+    # a launch that fills the device needs no workspace; fp32 and other head sizes have no split kernel
     big = torch.zeros((64, 1024), dtype=torch.int32, device=DEV)
     assert ops.prefill_workspace_bytes(torch.empty((64 * 256, 32, 128), dtype=torch.bfloat16, device=DEV), big, 256, 16, 8) == 0
     assert ops.prefill_workspace_bytes(q.float(), c.dev_tables, 150, 16, 2) == 0
-    assert ops.prefill_workspace_bytes(torch.empty((150, 8, 256), dtype=torch.bfloat16, device=DEV), c.dev_tables, 150, 16, 2) == 0
+    assert ops.prefill_workspace_bytes(torch.empty((150, 8, 96), dtype=torch.bfloat16, device=DEV), c.dev_tables, 150, 16, 2) == 0
     # narrow tables (short contexts at most): no split either
     assert ops.prefill_workspace_bytes(q, c.dev_tables[:, :64].contiguous(), 150, 16, 2) == 0
     # a workspace too small for two pieces: the call is the unsplit one
