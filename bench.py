@@ -8,7 +8,8 @@ JSON line; with the default workload the line also carries short runs of the
 other configurations (c2, c5 decode, c3 append + chunked prefill) under
 ``secondary``.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c5|c1|c3|c3-d256|c3-d64|long-d128|long-d256|engine] [--no-secondary]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary]
+                    [--workload c4|c2|c5|c1|c3|c3-d256|c3-d64|long-d128|long-d256|dense-64x512|dense-4x8192|engine]
     python bench.py --traffic-from-pmc NAME KERNEL FETCH.csv WRITE.csv   # refresh profiles/traffic.json
 """
 
@@ -89,7 +90,8 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c3-d256", "c3-d64", "long-d128", "long-d256", "c4", "c5", "engine"])
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c3-d256", "c3-d64", "long-d128", "long-d256", "dense-64x512",
+                                                         "dense-4x8192", "c4", "c5", "engine"])
     ap.add_argument("--preheat-s", type=float, default=0.5,
                     help="seconds of untimed steps before the warmup steps: an idle GPU sits at its lowest clocks "
                          "and takes a few hundred milliseconds of work to leave them")
@@ -441,6 +443,54 @@ def bench_prefill_long(args, dev, name) -> dict:
     }
 
 
+# dense causal prefill (no cached prefix): workload -> (sequences, tokens each, query heads, kv heads, head_dim, seed)
+PREFILL_DENSE_SHAPES = {"dense-64x512": (64, 512, 32, 8, 128, 1010), "dense-4x8192": (4, 8192, 32, 8, 128, 1011)}
+
+
+def bench_prefill_dense(args, dev, name) -> dict:
+    """Dense causal prefill as ``_prefill_attention`` issues it: the step's own [B, T, Hkv, D] K/V handed to the
+    paged kernel as a pool of B blocks of T tokens with the identity table.  64 prompts of 512 tokens are what an
+    engine step of fresh prompts looks like: eight tiles of keys at most per workgroup, so the kernel's set-up and
+    write-out weigh as much as its loop."""
+    from research_amd import ops
+
+    B, T, hq, hkv, head_dim, seed = PREFILL_DENSE_SHAPES[name]
+    gen = torch.Generator(device=dev).manual_seed(seed)
+    q = torch.randn(B * T, hq, head_dim, device=dev, dtype=torch.bfloat16, generator=gen)
+    k = torch.randn(B * T, hkv, head_dim, device=dev, dtype=torch.bfloat16, generator=gen)
+    v = torch.randn(B * T, hkv, head_dim, device=dev, dtype=torch.bfloat16, generator=gen)
+    tables = torch.arange(B, dtype=torch.int32, device=dev).reshape(B, 1).contiguous()
+    lens = torch.full((B,), T, dtype=torch.int32, device=dev)
+    starts = torch.arange(B, dtype=torch.int32, device=dev) * T
+    out = torch.empty_like(q)
+    scale = head_dim ** -0.5
+
+    def prefill():
+        ops.prefill_paged(q, k, v, tables, lens, lens, starts, T, T, scale, out=out)
+
+    preheat(prefill, args.preheat_s)
+    for _ in range(args.warmup):
+        prefill()
+    ms_step_mean, ms_step = timed_steps(prefill, args.steps)
+    ms_kernel = timed_ms(prefill, max(args.steps, KERNEL_LAUNCHES))
+    flops = 4 * head_dim * hq * B * (T * (T + 1) // 2)  # two products, every visible (row, key) pair
+    achieved = flops / (ms_kernel * 1e-3) / 1e12
+    return {
+        "metric": "prefill-attn TFLOP/s", "value": flops / (ms_step * 1e-3) / 1e12, "unit": "TFLOP/s",
+        "tokens_per_s": B * T / (ms_step * 1e-3), "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "preheat_s": args.preheat_s, "ms_per_step": ms_step, "ms_per_step_mean": ms_step_mean,
+        "step_statistic": "median of the timed steps", "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"dense causal prefill, {B} x {T} tokens, {hq} q / {hkv} kv heads of {head_dim}, bf16",
+                   "num_seqs": B, "prefix_len": 0, "chunk_len": T, "num_q_heads": hq, "num_kv_heads": hkv,
+                   "head_dim": head_dim, "attention_flops": flops, "seed": seed},
+        "roofline": {"bound": "mfma", "kernel": "prefill_asm_kernel", "achieved": achieved,
+                     "peak": MFMA_BF16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": achieved / MFMA_BF16_PEAK_TFLOPS,
+                     "traffic": measured_traffic(name), "kernel_ms": ms_kernel,
+                     "kernel_launches": max(args.steps, KERNEL_LAUNCHES)},
+    }
+
+
 def bench_engine(args, dev) -> int:
     """The engine loop on a Qwen2.5-0.5B-shaped model with random weights (24 layers, 14 query / 2 kv heads of
     64, vocabulary 151 936, bf16): 8 prompts of 512 tokens, 16 rollouts each, 64 new tokens per rollout at
@@ -673,9 +723,10 @@ def secondary(args, dev) -> dict:
     short.copy_calibration = False
     short.secondary_run = True
     out = {}
-    for name in ("c2", "c5", "c3", "c3-d256", "c3-d64"):
+    for name in ("c2", "c5", "c3", "c3-d256", "c3-d64", "dense-64x512", "long-d128"):
         r = (bench_prefill_c3(short, dev) if name == "c3" else bench_prefill_head(short, dev, name) if name in PREFILL_HEAD_SHAPES
-             else bench_decode(name, short, dev))
+             else bench_prefill_dense(short, dev, name) if name in PREFILL_DENSE_SHAPES
+             else bench_prefill_long(short, dev, name) if name in PREFILL_LONG_SHAPES else bench_decode(name, short, dev))
         keep = ("metric", "value", "unit", "ms_per_step", "ms_per_step_mean", "steps", "warmup", "tokens_per_s",
                 "dtype", "roofline", "cpu_baseline", "append", "pct_of_hbm_peak")
         entry = {k: r[k] for k in keep if k in r}
@@ -706,6 +757,8 @@ def main() -> int:
         result = bench_prefill_head(args, dev, args.workload)
     elif args.workload in PREFILL_LONG_SHAPES:
         result = bench_prefill_long(args, dev, args.workload)
+    elif args.workload in PREFILL_DENSE_SHAPES:
+        result = bench_prefill_dense(args, dev, args.workload)
     else:
         result = bench_prefill_c3(args, dev) if args.workload == "c3" else bench_decode(args.workload, args, dev)
     if args.workload == "c4" and not args.no_secondary:

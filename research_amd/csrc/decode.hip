@@ -29,6 +29,7 @@ KernelSet pa_pick_kernels(int q_dtype, int kv_dtype, int d, int nrep_t) {
 int pa_fill_head_mapping(PoolArgs &p, int num_q_heads, int num_kv_heads, int head_dim, int kv_dtype) {
     const HeadPlan h = plan_heads(num_q_heads, num_kv_heads, head_dim, pa_dtype_bytes(kv_dtype));
     if (!h.nrep_t) return 0;
+    p.d = head_dim;
     p.hq = h.hq;
     p.hkv = h.hkv;
     p.n_rep = h.n_rep;
@@ -116,10 +117,12 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
                "one block of %d tokens x %d heads x %d is too large", block_size, num_kv_heads, head_dim);
     DecodeArgs a;
     const int nrep_t = pa_fill_head_mapping(a.p, num_q_heads, num_kv_heads, head_dim, kv_dtype);
-    const KernelSet ks = nrep_t ? pa_pick_kernels(q_dtype, kv_dtype, head_dim, nrep_t) : KernelSet{};
+    const int d_pad = plan_pad_dim(head_dim);  // the head size the kernels are compiled for
+    const KernelSet ks = nrep_t ? pa_pick_kernels(q_dtype, kv_dtype, d_pad, nrep_t) : KernelSet{};
     if (!ks.split)
-        return pa_fail(PA_ERR_UNSUPPORTED, "pa_decode: no kernel for q_dtype=%d kv_dtype=%d head_dim=%d", q_dtype,
-                       kv_dtype, head_dim);
+        return pa_fail(PA_ERR_UNSUPPORTED,
+                       "pa_decode: no kernel for q_dtype=%d kv_dtype=%d head_dim=%d (head_dim must be a multiple of 8, "
+                       "of 16 for an fp8 pool, up to 256)", q_dtype, kv_dtype, head_dim);
     if (batch == 0) return PA_OK;
     PA_REQUIRE(q && out && seq_lens, "NULL q / out / seq_lens");
     PA_REQUIRE(k_cache && v_cache, "NULL cache pointer");
@@ -127,6 +130,7 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
     PA_REQUIRE(kv_dtype != PA_FP8_E4M3 || (k_scale && v_scale), "fp8 KV needs k_scale and v_scale");
     PA_REQUIRE(pa_aligned16(k_cache) && pa_aligned16(v_cache) && pa_aligned16(q),
                "q and cache pointers must be 16-byte aligned");
+    PA_REQUIRE(head_dim * pa_dtype_bytes(q_dtype) % 16 == 0, "head_dim=%d: rows of q must be whole 16-byte vectors", head_dim);
     if (batch > kMaxBatch) {
         // The block prefix sums of a launch live in LDS: a larger batch is taken kMaxBatch sequences at a time, one
         // after the other on the stream, all through the same workspace (sized for kMaxBatch sequences).
@@ -142,13 +146,13 @@ int decode_launch(int phases, const void *q, const void *k_cache, const void *v_
         }
         return PA_OK;
     }
-    PA_REQUIRE(plan_split_lds_bytes(batch, head_dim, pa_dtype_bytes(kv_dtype), nrep_t) <= 65536,
+    PA_REQUIRE(plan_split_lds_bytes(batch, d_pad, pa_dtype_bytes(kv_dtype), nrep_t) <= 65536,
                "batch=%d needs more than 64 KB of LDS per workgroup", batch);
     const int grid = split_grid();
     // A caller's workspace is sized without asking the device (kMaxSplitGrid workgroups); the library's own
     // scratch is laid out for the grid this device really gets, which is what makes its fixed size go far.
     const HeadPlan plan = plan_heads(num_q_heads, num_kv_heads, head_dim, pa_dtype_bytes(kv_dtype));
-    const WsPlan w = plan_workspace(batch, plan, head_dim, use_static ? grid : kMaxSplitGrid);
+    const WsPlan w = plan_workspace(batch, plan, d_pad, use_static ? grid : kMaxSplitGrid);
     if (use_static) {
         if (w.total > kStaticScratchBytes)
             return pa_fail(PA_ERR_WORKSPACE,
@@ -215,7 +219,7 @@ extern "C" size_t pa_decode_workspace_bytes(int batch, int num_q_heads, int num_
         return 0;
     }
     const HeadPlan plan = plan_heads(num_q_heads, num_kv_heads, head_dim, pa_dtype_bytes(kv_dtype));
-    return plan_workspace(batch < kMaxBatch ? batch : kMaxBatch, plan, head_dim, kMaxSplitGrid).total;
+    return plan_workspace(batch < kMaxBatch ? batch : kMaxBatch, plan, plan.d_pad, kMaxSplitGrid).total;
 }
 
 extern "C" int pa_decode_passes(int batch, int num_q_heads, int num_kv_heads, int head_dim, int kv_dtype) {

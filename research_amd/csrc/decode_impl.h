@@ -40,6 +40,7 @@ constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / PA_WAVE;
 constexpr int kMaxBatch = kPlanMaxBatch;  // sequences per call (their block prefix sum lives in LDS)
 constexpr float kNegBig = -1.0e30f;  // finite stand-in for -inf in running maxima
+constexpr int kDeadLaneOffset = 0x40000000;  // byte offset past every buffer descriptor (a block is under 2 GiB / 4)
 
 // What every kernel of this file needs to know about the pool and the heads.
 struct PoolArgs {
@@ -48,6 +49,8 @@ struct PoolArgs {
     int64_t bt_stride;
     const float *k_scale, *v_scale;
     int hq, hkv, n_rep, bs;
+    int d;  // head_dim of the tensors in memory; the kernels' D is d rounded up to 32, 64, 128 or 256 and the lanes
+            // (and d indices) at or past d hold zeros and store nothing
     int64_t num_blocks;
     float scale_log2;  // softmax scale * log2(e)
     int window;        // sliding window: a query at position i sees keys j with i - j < window (0 = all keys)
@@ -158,8 +161,8 @@ __device__ __forceinline__ void load_q(float (&qf)[NREP][EPL], const QT *qrow, c
                                        int rep0, int d0) {
 #pragma unroll
     for (int r = 0; r < NREP; ++r) {
-        const bool live = rep0 + r < p.n_rep;
-        const QT *qp = qrow + ((int64_t)kvh * p.n_rep + rep0 + (live ? r : 0)) * D + d0;
+        const bool live = rep0 + r < p.n_rep && d0 < p.d;
+        const QT *qp = qrow + ((int64_t)kvh * p.n_rep + rep0 + (live ? r : 0)) * p.d + (live ? d0 : 0);
 #pragma unroll
         for (int e = 0; e < EPL; ++e) qf[r][e] = live ? pa_scalar<QT>::load(qp + e) * p.scale_log2 : 0.f;
     }
@@ -175,7 +178,8 @@ __device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EP
     using S = RowShape<KV, D>;
     constexpr int EPL = S::EPL;
     constexpr bool kFp8 = sizeof(KV) == 1;
-    const int64_t tok_stride = (int64_t)p.hkv * D * sizeof(KV);  // bytes between tokens
+    const int64_t tok_stride = (int64_t)p.hkv * p.d * sizeof(KV);  // bytes between tokens
+    const bool lane_live = role.d0 < p.d;                          // (lanes past the row's end read nothing)
 
     for (int blk = blk_begin; blk < blk_end; blk += blk_step) {
         const int ntok = min(p.bs, L - blk * p.bs);
@@ -185,7 +189,7 @@ __device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EP
             if (role.tok_local == 0) st.zero_keys += max(0, ntok - tlo);
             continue;
         }
-        const int64_t base = ((bid * p.bs) * p.hkv + kvh) * (int64_t)(D * sizeof(KV)) + (int64_t)role.lir * 16;
+        const int64_t base = ((bid * p.bs) * p.hkv + kvh) * (int64_t)(p.d * sizeof(KV)) + (int64_t)role.lir * 16;
         const char *kp = reinterpret_cast<const char *>(p.k) + base;
         const char *vp = reinterpret_cast<const char *>(p.v) + base;
         float ks = 1.f, vs = 1.f;
@@ -200,12 +204,12 @@ __device__ __forceinline__ void attend_blocks(RowState<NREP, RowShape<KV, D>::EP
             for (int u = 0; u < U; ++u) {
                 const int t = t0 + u * p.tpw + role.tok_local;
                 ok[u] = t < ntok && t >= tlo;
-                kraw[u] = ok[u] ? ld16_stream(kp + t * tok_stride) : uint4{0, 0, 0, 0};
+                kraw[u] = ok[u] && lane_live ? ld16_stream(kp + t * tok_stride) : uint4{0, 0, 0, 0};
             }
 #pragma unroll
             for (int u = 0; u < U; ++u) {
                 const int t = t0 + u * p.tpw + role.tok_local;
-                vraw[u] = ok[u] ? ld16_stream(vp + t * tok_stride) : uint4{0, 0, 0, 0};
+                vraw[u] = ok[u] && lane_live ? ld16_stream(vp + t * tok_stride) : uint4{0, 0, 0, 0};
             }
             float s[U][NREP];
             float mx[NREP];
@@ -286,8 +290,8 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
                 // local index r of this lane stands for head head_of(r, lane): the order that spares the
                 // reduce-scatter of the logits its selects
                 const int hr = HS::head_of(r, lane);
-                const bool live = rep0 + hr < p.n_rep;
-                const QT *qp = qrow + ((int64_t)kvh * p.n_rep + rep0 + hr) * D + role.d0;
+                const bool live = rep0 + hr < p.n_rep && role.d0 < p.d;
+                const QT *qp = qrow + ((int64_t)kvh * p.n_rep + rep0 + hr) * p.d + role.d0;
 #pragma unroll
                 for (int i = 0; i < NW; i += 4) {
                     const uint4 raw = live ? ld16(qp + 2 * i) : uint4{0, 0, 0, 0};
@@ -296,8 +300,11 @@ template <typename KV, typename QT, int D, int NREP, int U> struct Attender {
             }
             PkState<NREP, HS::VPL, S::EPL> st;
             st.init();
-            const int lane_voff =
-                role.tok_local * (p.hkv * D * (int)sizeof(KV)) + kvh * (D * (int)sizeof(KV)) + role.lir * 16;
+            // (a lane past the end of a head_dim that is not 32, 64, 128 or 256 gets an offset no descriptor covers:
+            // its loads return zeros)
+            const int lane_voff = role.d0 < p.d ? role.tok_local * (p.hkv * p.d * (int)sizeof(KV)) +
+                                                      kvh * (p.d * (int)sizeof(KV)) + role.lir * 16
+                                                : kDeadLaneOffset;
             // uniform choices: few kv heads per wave load and short blocks
             if (U % 4 == 0 && p.bs == 4 * p.tpw && U > 4)  // 4 steps per block: U/4 blocks per iteration
                 attend_blocks_pk_multi<KV, QT, D, NREP, U, (U % 4 == 0 ? 4 : 2)>(
@@ -503,7 +510,7 @@ __device__ __forceinline__ void merge_slots(const DecodeArgs &a, int plane, int 
     const int stride_acc = p.hpw * NREP * D, stride_ml = p.hpw * NREP * 2;
     const int64_t key = (int64_t)plane * a.batch + b;
     const int ez = FINAL && a.extra_zero ? max(0, a.extra_zero[b]) : 0;
-    QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * D;
+    QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * p.d;
     for (int item = tid; item < p.hpw * NREP * (D / 4); item += kThreads) {
         const int idx = item / (D / 4), d = (item - idx * (D / 4)) * 4;
         const int kv_local = idx / NREP, r = idx - kv_local * NREP;
@@ -545,9 +552,10 @@ __device__ __forceinline__ void merge_slots(const DecodeArgs &a, int plane, int 
         }
         if (FINAL) {
             const int qh = (hg * p.hpw + kv_local) * p.n_rep + rep0 + r;
+            if (d >= p.d) continue;
 #pragma unroll
             for (int j = 0; j < 4; ++j)
-                pa_scalar<QT>::store(orow + (int64_t)qh * D + d + j, finish_row(num[j], M, den, ez));
+                pa_scalar<QT>::store(orow + (int64_t)qh * p.d + d + j, finish_row(num[j], M, den, ez));
         } else if ((int64_t)w_first + key < a.slot_cap) {
             const int64_t slot = w_first + key;
             st_coherent(a.part_acc + slot * stride_acc + idx * D + d, num[0], num[1]);
@@ -692,8 +700,8 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
         // no second pass: sequences without a visible key get their zero rows here, dealt out over the grid
         for (int b = blockIdx.x; b < B; b += gridDim.x) {
             if (s_prefix[b + 1] != s_prefix[b]) continue;
-            QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * D;
-            for (int i = tid; i < p.hq * D; i += kThreads) pa_scalar<QT>::store(orow + i, 0.f);
+            QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * p.d;
+            for (int i = tid; i < p.hq * p.d; i += kThreads) pa_scalar<QT>::store(orow + i, 0.f);
         }
     }
     if (total == 0) return;
@@ -724,17 +732,18 @@ __global__ __launch_bounds__(kThreads) void decode_split_kernel(const DecodeArgs
         const int fb = k_lo / p.bs;               // first block with a visible key
 
         RowState<NREP, S::EPL> st = Attender<KV, QT, D, NREP, U>::run(
-            p, reinterpret_cast<const QT *>(a.q) + (int64_t)b * p.hq * D, p.bt + (int64_t)b * p.bt_stride, k_lo, L,
+            p, reinterpret_cast<const QT *>(a.q) + (int64_t)b * p.hq * p.d, p.bt + (int64_t)b * p.bt_stride, k_lo, L,
             fb + blk0, fb + blk1, wave, kWaves, by_chunk, role, lane, kvh, rep0);
         if (blk0 == 0 && blk1 == nblk) {
             // the whole sequence is ours: write the output row
             const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
-            QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * D;
+            QT *orow = reinterpret_cast<QT *>(a.out) + (int64_t)b * p.hq * p.d;
             merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
                                     [&](int qh, int d, const float (&num)[4], float M, float den) {
+                                        if (d >= p.d) return;
 #pragma unroll
                                         for (int j = 0; j < 4; ++j)
-                                            pa_scalar<QT>::store(orow + (int64_t)qh * D + d + j,
+                                            pa_scalar<QT>::store(orow + (int64_t)qh * p.d + d + j,
                                                                  finish_row(num[j], M, den, ez));
                                     });
         } else {
@@ -803,9 +812,9 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_kernel(const DecodeArg
     const int nblk = a.block_prefix[b + 1] - a.block_prefix[b];
     const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
     const int tid = threadIdx.x;
-    QT *orow = reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * D;
+    QT *orow = reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * p.d;
     if (nblk == 0) {
-        for (int d = tid; d < D; d += kThreads) pa_scalar<QT>::store(orow + d, 0.f);
+        for (int d = tid; d < p.d; d += kThreads) pa_scalar<QT>::store(orow + d, 0.f);
         return;
     }
     const int64_t u0 = plane * per_plane + a.block_prefix[b];
@@ -857,7 +866,7 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_kernel(const DecodeArg
         s_l[pl] = den;
     }
     __syncthreads();
-    for (int d = tid; d < D; d += kThreads) {
+    for (int d = tid; d < p.d; d += kThreads) {
         float Mt = kNegBig;
 #pragma unroll
         for (int q = 0; q < PL; ++q) Mt = fmaxf(Mt, s_m[q]);
@@ -896,9 +905,9 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_wave_kernel(const Deco
     const int64_t total = per_plane * p.n_hgroups * p.n_rgroups;
     const int nblk = a.block_prefix[b + 1] - a.block_prefix[b];
     const int ez = a.extra_zero ? max(0, a.extra_zero[b]) : 0;
-    QT *orow = reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * D;
+    QT *orow = reinterpret_cast<QT *>(a.out) + ((int64_t)b * hq + qh) * p.d;
     if (nblk == 0) {
-        for (int d = lane; d < D; d += PA_WAVE) pa_scalar<QT>::store(orow + d, 0.f);
+        for (int d = lane; d < p.d; d += PA_WAVE) pa_scalar<QT>::store(orow + d, 0.f);
         return;
     }
     const int64_t u0 = plane * per_plane + a.block_prefix[b];
@@ -944,7 +953,7 @@ __global__ __launch_bounds__(kThreads) void decode_reduce_wave_kernel(const Deco
 #pragma unroll
     for (int k = 0; k < DPL; ++k) {
         const int d = lane + PA_WAVE * k;
-        if (d < D) pa_scalar<QT>::store(orow + d, finish_row(num[k], M, den, ez));
+        if (d < p.d) pa_scalar<QT>::store(orow + d, finish_row(num[k], M, den, ez));
     }
 }
 
@@ -975,14 +984,15 @@ __global__ __launch_bounds__(kThreads) void prefill_rowwise_kernel(const Rowwise
     if (a.row_lo) k_lo = max(k_lo, min(a.row_lo[qrow], L - 1));
     k_lo = max(k_lo, 0);
     RowState<NREP, S::EPL> st = Attender<KV, QT, D, NREP, U>::run(
-        p, reinterpret_cast<const QT *>(a.q) + qrow * p.hq * D, p.bt + (int64_t)b * p.bt_stride, k_lo, L,
+        p, reinterpret_cast<const QT *>(a.q) + qrow * p.hq * p.d, p.bt + (int64_t)b * p.bt_stride, k_lo, L,
         k_lo / p.bs, nblk, wave, kWaves, false, role, lane, kvh, rep0);
-    QT *orow = reinterpret_cast<QT *>(a.out) + qrow * p.hq * D;
+    QT *orow = reinterpret_cast<QT *>(a.out) + qrow * p.hq * p.d;
     merge_rows<KV, D, NREP>(st, s_part, p, role, wave, tid, hg, rep0,
                             [&](int qh, int d, const float (&num)[4], float M, float den) {
+                                if (d >= p.d) return;
 #pragma unroll
                                 for (int j = 0; j < 4; ++j)
-                                    pa_scalar<QT>::store(orow + (int64_t)qh * D + d + j, den > 0.f ? num[j] / den : 0.f);
+                                    pa_scalar<QT>::store(orow + (int64_t)qh * p.d + d + j, den > 0.f ? num[j] / den : 0.f);
                             });
 }
 

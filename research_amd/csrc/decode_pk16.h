@@ -272,7 +272,7 @@ __device__ __forceinline__ void attend_blocks_pk(
     using PW = PoolWords<KV, AT>;
     constexpr int NW = PW::NW;
     constexpr int VPL = HS::VPL;
-    const int tok_stride = p.hkv * D * (int)sizeof(KV);  // bytes between tokens
+    const int tok_stride = p.hkv * p.d * (int)sizeof(KV);  // bytes between tokens
     const int tok_local = (lane / LPR) / p.hpw;
     const int chunk = p.tpw * U;                          // tokens per chunk
 
@@ -436,7 +436,7 @@ __device__ __forceinline__ void attend_blocks_pk_multi(
     using PW = PoolWords<KV, AT>;
     constexpr int NW = PW::NW;
     constexpr int VPL = HS::VPL;
-    const int tok_stride = p.hkv * D * (int)sizeof(KV);  // bytes between tokens
+    const int tok_stride = p.hkv * p.d * (int)sizeof(KV);  // bytes between tokens
     const int tok_local = (lane / LPR) / p.hpw;
 
     for (int blk0 = blk_begin; blk0 < blk_end; blk0 += G * blk_step) {

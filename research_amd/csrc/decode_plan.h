@@ -33,14 +33,23 @@ struct HeadPlan {
     int hq, hkv, n_rep;
     int hpw, tpw, n_hgroups, n_rgroups;
     int nrep_t;  // padded group size (kernel template parameter); 0 = no kernel for this head_dim / element size
+    int d_pad;   // head_dim rounded up to the next of 32, 64, 128, 256: the head size the kernel is compiled for
     PA_PLAN_FN int planes() const { return n_hgroups * n_rgroups; }
     PA_PLAN_FN int heads_per_slot() const { return hpw * nrep_t; }
 };
 
-PA_PLAN_FN HeadPlan plan_heads(int num_q_heads, int num_kv_heads, int head_dim, int kv_elem_bytes) {
+// The kernels are compiled for head sizes 32, 64, 128 and 256; any other head_dim up to 256 whose rows are whole
+// 16-byte vectors runs the next larger one with the lanes past the row's end idle.
+PA_PLAN_FN int plan_pad_dim(int head_dim) { return head_dim <= 32 ? 32 : head_dim <= 64 ? 64 : head_dim <= 128 ? 128 : 256; }
+
+PA_PLAN_FN HeadPlan plan_heads(int num_q_heads, int num_kv_heads, int head_dim_real, int kv_elem_bytes) {
     HeadPlan h = {};
-    if (kv_elem_bytes <= 0 || (head_dim != 32 && head_dim != 64 && head_dim != 128 && head_dim != 256)) return h;
+    if (kv_elem_bytes <= 0 || head_dim_real <= 0 || head_dim_real > 256 || head_dim_real * kv_elem_bytes % 16 != 0 ||
+        head_dim_real % 8 != 0)
+        return h;
     if (num_q_heads <= 0 || num_kv_heads <= 0 || num_q_heads % num_kv_heads != 0) return h;
+    const int head_dim = plan_pad_dim(head_dim_real);
+    h.d_pad = head_dim;
     const int lpr = head_dim * kv_elem_bytes / 16;  // lanes per K/V row
     const int rpw = 64 / lpr;                        // rows per wave load
     int hpw = 1;                                     // kv heads per wave load: power of two dividing num_kv_heads

@@ -104,9 +104,11 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     PA_REQUIRE(dtype == PA_F32 || dtype == PA_BF16 || dtype == PA_F16, "dtype=%d is not F32, BF16 or F16", dtype);
     RowwiseArgs a;
     const int nrep_t = pa_fill_head_mapping(a.p, num_q_heads, num_kv_heads, head_dim, dtype);
-    const KernelSet ks = nrep_t ? pa_pick_kernels(dtype, dtype, head_dim, nrep_t) : KernelSet{};
+    const KernelSet ks = nrep_t ? pa_pick_kernels(dtype, dtype, plan_pad_dim(head_dim), nrep_t) : KernelSet{};
     if (!ks.rowwise)
-        return pa_fail(PA_ERR_UNSUPPORTED, "pa_prefill_paged: no kernel for dtype=%d head_dim=%d", dtype, head_dim);
+        return pa_fail(PA_ERR_UNSUPPORTED,
+                       "pa_prefill_paged: no kernel for dtype=%d head_dim=%d (head_dim must be a multiple of 8 up to 256)",
+                       dtype, head_dim);
     PA_REQUIRE(batch <= 65535 && max_q_len <= 65535, "batch=%d / max_q_len=%d above 65535", batch, max_q_len);
     if (batch == 0 || max_q_len == 0) return PA_OK;
     PA_REQUIRE(q && out && ctx_lens && q_lens && q_starts, "NULL q / out / ctx_lens / q_lens / q_starts");

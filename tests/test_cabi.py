@@ -89,8 +89,10 @@ def test_decode_argument_errors():
     for entry in ("pa_decode_split", "pa_decode_reduce"):
         rc, msg = _status(entry, *_decode_args(hq=30))
         assert rc == _lib.PA_ERR_INVALID_ARG
-    rc, msg = _status("pa_decode", *_decode_args(d=96))
-    assert rc == _lib.PA_ERR_UNSUPPORTED and "head_dim=96" in msg
+    rc, msg = _status("pa_decode", *_decode_args(d=100))  # (any multiple of 8 up to 256 has a kernel)
+    assert rc == _lib.PA_ERR_UNSUPPORTED and "head_dim=100" in msg
+    rc, msg = _status("pa_decode", *_decode_args(d=264))
+    assert rc == _lib.PA_ERR_UNSUPPORTED
     rc, msg = _status("pa_decode", *_decode_args(qd=_lib.PA_F32))
     assert rc == _lib.PA_ERR_UNSUPPORTED  # q and pool types must match unless the pool is fp8
     rc, msg = _status("pa_decode", *_decode_args(kvd=_lib.PA_FP8_E4M3))
@@ -116,7 +118,7 @@ def test_decode_static_argument_errors():
     static = lambda **kw: _decode_args(**kw)[:-3] + [None]
     rc, msg = _status("pa_decode_static", *static(hq=30))
     assert rc == _lib.PA_ERR_INVALID_ARG and "multiple of num_kv_heads" in msg
-    rc, msg = _status("pa_decode_static", *static(d=96))
+    rc, msg = _status("pa_decode_static", *static(d=100))
     assert rc == _lib.PA_ERR_UNSUPPORTED
     rc, msg = _status("pa_decode_static", *static(batch=8192))
     assert rc == _lib.PA_ERR_WORKSPACE and "scratch" in msg and "pa_decode_workspace_bytes" in msg
@@ -133,7 +135,10 @@ def test_decode_workspace_arithmetic():
     assert lib.pa_decode_workspace_bytes(256, 32, 8, 128, _lib.PA_FP8_E4M3) > 0
     assert lib.pa_decode_workspace_bytes(-1, 32, 8, 128, _lib.PA_BF16) == 0
     assert "pa_decode_workspace_bytes" in _lib.last_error()
-    assert lib.pa_decode_workspace_bytes(4, 32, 8, 96, _lib.PA_BF16) == 0
+    # head sizes between the compiled ones take the next larger kernel (and its workspace); odd ones have none
+    assert (lib.pa_decode_workspace_bytes(4, 32, 8, 96, _lib.PA_BF16)
+            == lib.pa_decode_workspace_bytes(4, 32, 8, 128, _lib.PA_BF16))
+    assert lib.pa_decode_workspace_bytes(4, 32, 8, 100, _lib.PA_BF16) == 0
     assert lib.pa_decode_workspace_bytes(4, 30, 8, 128, _lib.PA_BF16) == 0
 
 

@@ -112,6 +112,14 @@ def test_pool_permutation_and_constant_values():
     (8, 2, 256, torch.float16),    # D=256, group of 4
     (32, 2, 128, torch.float32),   # group of 16: two passes of 8
     (5, 5, 64, torch.float32),     # odd head count: one kv head per wave load
+    (10, 2, 80, torch.bfloat16),   # head sizes between the compiled ones: the next larger kernel, idle lanes masked
+    (6, 3, 96, torch.float16),
+    (4, 1, 112, torch.bfloat16),
+    (8, 2, 160, torch.bfloat16),
+    (6, 2, 192, torch.float16),
+    (4, 2, 40, torch.float32),
+    (4, 2, 24, torch.bfloat16),
+    (2, 2, 8, torch.float32),
 ])
 def test_head_layouts(hq, hkv, d, dtype):
     announce(f"decode heads hq={hq} hkv={hkv} d={d} {dtype}")
@@ -320,6 +328,10 @@ def test_decode_step_in_a_hip_graph():
     (8, 4, 128, "fp8"),    # 2 tokens per load: eight steps are one block
     (4, 2, 64, "fp8"),     # fp8 rows of 4 lanes, 8 tokens per load
     (32, 8, 128, "fp8"),   # the long-context workload's layout: one token per load, 16 steps per block
+    (8, 2, 96, "bf16"),    # head sizes between the compiled ones
+    (6, 2, 80, "fp8"),
+    (4, 1, 192, "fp8"),
+    (4, 4, 160, "f16"),
 ])
 def test_few_kv_heads_with_blocks_of_16(hq, hkv, d, kv):
     """Layouts whose loop takes several blocks per iteration: ragged lengths around block and iteration

@@ -458,3 +458,21 @@ def test_logits_that_grow_along_the_context(d):
                               _i32(np.arange(len(chunk)) * cmax), cmax, bs, d ** -0.5, out=out, window=window)
             assert_close(out.reshape(len(chunk), cmax, hq, d), want, 2e-2,
                          f"logits {'rising' if direction > 0 else 'falling'}, window {window}")
+
+
+@pytest.mark.parametrize("d,dtype,tol", [(80, torch.bfloat16, 2e-2), (96, torch.float16, 2e-2), (192, torch.bfloat16, 2e-2),
+                                         (40, torch.float32, 1e-5), (112, torch.float32, 1e-5)])
+def test_chunked_prefill_other_head_sizes(d, dtype, tol):
+    """Head sizes between the compiled ones (multiples of 8 up to 256) take the vector kernel of the next larger
+    size: chunked prefill over a shared prefix, windows included."""
+    announce(f"chunked prefill head_dim {d} {dtype}")
+    w = make_prefill_c3(num_seqs=3, prefix_len=64, chunk_len=37, num_q_heads=6, num_kv_heads=2, head_dim=d, dtype=dtype)
+    got, kc, vc = _run_chunked(w)
+    want = po.paged_prefill_chunk(w.q, kc.cpu(), vc.cpu(), w.block_tables, [64] * 3, [37] * 3, w.block_size, w.scale)
+    assert_close(got, want, tol, f"head_dim {d}")
+    S, C = w.num_seqs, w.chunk_len
+    win = ops.prefill_paged(w.q.reshape(S * C, 6, d).to(DEV), kc, vc, tables_to_device(w.block_tables),
+                            _i32([64 + C] * S), _i32([C] * S), _i32(np.arange(S) * C), C, w.block_size, w.scale, window=20)
+    want = po.paged_prefill_chunk(w.q, kc.cpu(), vc.cpu(), w.block_tables, [64] * 3, [37] * 3, w.block_size, w.scale,
+                                  window=20)
+    assert_close(win.reshape(S, C, 6, d), want, tol, f"head_dim {d}, window 20")
