@@ -148,7 +148,7 @@ def test_prefill_and_quantize_argument_errors():
     rc, msg = _status("pa_prefill_paged", *args)
     assert rc == _lib.PA_ERR_INVALID_ARG and "dtype" in msg
     args[-2] = _lib.PA_BF16
-    args[14] = 80
+    args[14] = 84  # (not a multiple of 8: no kernel)
     rc, msg = _status("pa_prefill_paged", *args)
     assert rc == _lib.PA_ERR_UNSUPPORTED
     rc, msg = _status("pa_quantize_kv_e4m3", FAKE, FAKE, FAKE, 4, 16, 8, 128, _lib.PA_FP8_E4M3, None)
