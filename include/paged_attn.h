@@ -257,7 +257,8 @@ int pa_prefill_paged_ws(const void *q, const void *k_cache, const void *v_cache,
  * set - nothing else is implied, a causal bound included.  Keys j >= ctx_lens[b] and keys in absent blocks are
  * zero rows (logit 0, zero value), which is what the reference's zero-padded decode gather hands to
  * flex_attention (:253-264); a row with no bit set gives zeros.
- *   q, out  : [total_q][num_q_heads][head_dim], dtype F32 / BF16 / F16 = the pool's dtype
+ *   q, out  : [total_q][num_q_heads][head_dim], dtype F32 / BF16 / F16
+ *   kv_dtype: dtype, or PA_FP8_E4M3 (16-bit q) with k_scale / v_scale float[num_blocks][num_kv_heads] as in pa_decode
  *   mask    : uint32 [total_q][mask_heads][mask_words], bit j of word j/32; mask_heads is 1 (all heads share
  *             the row) or num_q_heads
  * The general path, not a fast one: one workgroup per (head, row), a wave-wide reduction per visible key.  The
@@ -267,7 +268,8 @@ int pa_attend_masked(const void *q, const void *k_cache, const void *v_cache, vo
                      const int32_t *block_tables, int64_t bt_stride, const int32_t *ctx_lens,
                      const int32_t *q_lens, const int32_t *q_starts, const uint32_t *mask, int mask_heads,
                      int mask_words, int n_keys, int batch, int max_q_len, int num_q_heads, int num_kv_heads,
-                     int head_dim, int block_size, int64_t num_blocks, float scale, int dtype, void *stream);
+                     int head_dim, int block_size, int64_t num_blocks, float scale, int dtype, int kv_dtype,
+                     const float *k_scale, const float *v_scale, void *stream);
 
 /*
  * pa_prefill_paged evaluated by the vector kernel (one workgroup per query row, the decode inner loop) whatever

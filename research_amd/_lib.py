@@ -54,7 +54,8 @@ SIGNATURES = {
     "pa_attend_masked": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
-         c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_void_p],
+         c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64, c_float, c_int, c_int, c_void_p,
+         c_void_p, c_void_p],
     ),
     "pa_quantize_kv_e4m3": (
         c_int,

@@ -16,6 +16,7 @@ struct MaskedArgs {
     const int32_t *bt;
     int64_t bt_stride;
     const int32_t *ctx_lens, *q_lens, *q_starts;
+    const float *k_scale, *v_scale;  // fp8 pools: float [num_blocks][hkv]
     const uint32_t *mask;  // [total rows][mask_heads][mask_words]
     int mask_heads, mask_words, n_keys;
     int hq, hkv, d, bs;
@@ -29,8 +30,19 @@ __device__ __forceinline__ float wave_sum(float x) {
     return x;
 }
 
-template <typename T>
+// One element of a pool row as a float: the pool's own 16- or 32-bit type, or an OCP e4m3 byte (the caller
+// multiplies by the tile's scale).
+template <typename KV> struct PoolElem {
+    static __device__ __forceinline__ float load(const KV *p) { return pa_scalar<KV>::load(p); }
+};
+template <> struct PoolElem<pa_fp8> {
+    static __device__ __forceinline__ float load(const pa_fp8 *p) { return __builtin_amdgcn_cvt_f32_fp8((int)p->bits, 0); }
+};
+
+// T: type of q and out; KV: type of the pool (T itself, or fp8-e4m3 with per-(block, kv head) scales).
+template <typename T, typename KV>
 __global__ __launch_bounds__(kMThreads) void attend_masked_kernel(const MaskedArgs a) {
+    constexpr bool kFp8 = sizeof(KV) == 1;
     __shared__ float s_acc[kMWaves][kMaxEpl * PA_WAVE];
     __shared__ float s_ml[kMWaves][2];
     const int h = blockIdx.x, row = blockIdx.y, b = blockIdx.z;
@@ -81,14 +93,19 @@ __global__ __launch_bounds__(kMThreads) void attend_masked_kernel(const MaskedAr
 #pragma unroll
             for (int t = 0; t < kKeysAtOnce; ++t) {
                 const int64_t slot = key[t] >= 0 ? slot_of(key[t]) : -1;
-                const T *kr = reinterpret_cast<const T *>(a.k) + (slot * a.hkv + kvh) * a.d;
-                const T *vr = reinterpret_cast<const T *>(a.v) + (slot * a.hkv + kvh) * a.d;
+                const KV *kr = reinterpret_cast<const KV *>(a.k) + (slot * a.hkv + kvh) * a.d;
+                const KV *vr = reinterpret_cast<const KV *>(a.v) + (slot * a.hkv + kvh) * a.d;
+                float ks = 1.f, vs = 1.f;
+                if (kFp8 && slot >= 0) {
+                    ks = a.k_scale[slot / a.bs * a.hkv + kvh];
+                    vs = a.v_scale[slot / a.bs * a.hkv + kvh];
+                }
 #pragma unroll
                 for (int i = 0; i < kMaxEpl; ++i) {
                     const int e = lane + i * PA_WAVE;
                     const bool live = slot >= 0 && i < epl && e < a.d;
-                    kx[t][i] = live ? pa_scalar<T>::load(kr + e) : 0.f;
-                    vx[t][i] = live ? pa_scalar<T>::load(vr + e) : 0.f;
+                    kx[t][i] = live ? PoolElem<KV>::load(kr + e) * ks : 0.f;
+                    vx[t][i] = live ? PoolElem<KV>::load(vr + e) * vs : 0.f;
                 }
             }
             float s[kKeysAtOnce];
@@ -145,7 +162,7 @@ extern "C" int pa_attend_masked(const void *q, const void *k_cache, const void *
                                 const int32_t *q_lens, const int32_t *q_starts, const uint32_t *mask, int mask_heads,
                                 int mask_words, int n_keys, int batch, int max_q_len, int num_q_heads,
                                 int num_kv_heads, int head_dim, int block_size, int64_t num_blocks, float scale,
-                                int dtype, void *stream) {
+                                int dtype, int kv_dtype, const float *k_scale, const float *v_scale, void *stream) {
     pa_clear_error();
     PA_REQUIRE(batch >= 0 && max_q_len >= 0 && n_keys >= 0, "batch / max_q_len / n_keys must be non-negative");
     PA_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0,
@@ -157,8 +174,12 @@ extern "C" int pa_attend_masked(const void *q, const void *k_cache, const void *
     PA_REQUIRE(batch <= 65535 && max_q_len <= 65535, "batch=%d / max_q_len=%d above 65535", batch, max_q_len);
     if (dtype != PA_F32 && dtype != PA_BF16 && dtype != PA_F16)
         return pa_fail(PA_ERR_UNSUPPORTED, "pa_attend_masked: dtype=%d is not F32, BF16 or F16", dtype);
+    if (kv_dtype != dtype && !(kv_dtype == PA_FP8_E4M3 && dtype != PA_F32))
+        return pa_fail(PA_ERR_UNSUPPORTED,
+                       "pa_attend_masked: kv_dtype=%d must be the dtype of q (%d), or FP8_E4M3 with 16-bit q", kv_dtype, dtype);
     if (batch == 0 || max_q_len == 0) return PA_OK;
     PA_REQUIRE(q && out && ctx_lens && q_lens && q_starts && k_cache && v_cache, "NULL argument");
+    PA_REQUIRE(kv_dtype != PA_FP8_E4M3 || (k_scale && v_scale), "fp8 KV needs k_scale and v_scale");
     PA_REQUIRE(mask || n_keys == 0, "NULL mask");
     PA_REQUIRE(block_tables || bt_stride == 0, "NULL block_tables with bt_stride=%lld", (long long)bt_stride);
     MaskedArgs a;
@@ -169,9 +190,13 @@ extern "C" int pa_attend_masked(const void *q, const void *k_cache, const void *
     a.scale_log2 = scale * 1.4426950408889634f;
     const dim3 grid((unsigned)num_q_heads, (unsigned)max_q_len, (unsigned)batch), block(kMThreads);
     hipStream_t s = (hipStream_t)stream;
-    if (dtype == PA_F32) attend_masked_kernel<float><<<grid, block, 0, s>>>(a);
-    else if (dtype == PA_BF16) attend_masked_kernel<pa_bf16><<<grid, block, 0, s>>>(a);
-    else attend_masked_kernel<pa_f16><<<grid, block, 0, s>>>(a);
+    a.k_scale = k_scale; a.v_scale = v_scale;
+    if (kv_dtype == PA_FP8_E4M3) {
+        if (dtype == PA_BF16) attend_masked_kernel<pa_bf16, pa_fp8><<<grid, block, 0, s>>>(a);
+        else attend_masked_kernel<pa_f16, pa_fp8><<<grid, block, 0, s>>>(a);
+    } else if (dtype == PA_F32) attend_masked_kernel<float, float><<<grid, block, 0, s>>>(a);
+    else if (dtype == PA_BF16) attend_masked_kernel<pa_bf16, pa_bf16><<<grid, block, 0, s>>>(a);
+    else attend_masked_kernel<pa_f16, pa_f16><<<grid, block, 0, s>>>(a);
     PA_CHECK_LAUNCH("pa_attend_masked");
     return PA_OK;
 }

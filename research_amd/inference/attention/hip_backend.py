@@ -519,8 +519,6 @@ class HipPagedAttentionBackend:
         """Decode under an arbitrary predicate, literally as the reference evaluates it (flex_backend.py:203-225):
         the one query row has q_idx 0, kv_idx runs over the batch's longest sequence, and the positions past a
         shorter sequence's end are zero rows that take part wherever the predicate keeps them."""
-        if self._fp8:
-            raise NotImplementedError("arbitrary mask predicates are not evaluated over an fp8 pool")
         cfg = self.config
         batch, _, num_heads, head_dim = q.shape
         self._require_device(q, self.k_cache)
@@ -535,7 +533,9 @@ class HipPagedAttentionBackend:
         words = self._mask_bits(step, mod, batch, num_heads, torch.zeros((batch, 1), dtype=torch.int64), step.max_q_len)
         kc, vc = self._layer(layer_idx)
         out = ops.attend_masked(q.contiguous().view(batch, num_heads, head_dim), kc, vc, step.tables, step.ctx_lens,
-                                step.q_lens, step.q_starts, 1, cfg.block_size, self.scale, words, step.mask_keys)
+                                step.q_lens, step.q_starts, 1, cfg.block_size, self.scale, words, step.mask_keys,
+                                k_scale=self.k_scale[layer_idx] if self._fp8 else None,
+                                v_scale=self.v_scale[layer_idx] if self._fp8 else None)
         return out.view(batch, 1, num_heads, head_dim)
 
     # ------------------------------------------------------------------ prefill
@@ -612,14 +612,14 @@ class HipPagedAttentionBackend:
         tables = step.tables
         if mod is not None:
             # an arbitrary predicate over the cached context: row t of sequence b has q_idx = prefix + t
-            if self._fp8:
-                raise NotImplementedError("arbitrary mask predicates are not evaluated over an fp8 pool")
             totals = self._lens(ctx.seq_lens, batch)
             pos = torch.from_numpy(self._lens(ctx.prefix_lens, batch)[:, None] + np.arange(seq_len, dtype=np.int64)[None, :])
             words = self._mask_bits(step, mod, batch, num_heads, pos, int(totals.max()))
             ops.attend_masked(q.contiguous().view(batch * seq_len, num_heads, head_dim), kc, vc, tables, step.ctx_lens,
                               step.q_lens, step.q_starts, step.max_q_len, cfg.block_size, self.scale, words,
-                              step.mask_keys, out=out.view(batch * seq_len, num_heads, head_dim))
+                              step.mask_keys, out=out.view(batch * seq_len, num_heads, head_dim),
+                              k_scale=self.k_scale[layer_idx] if self._fp8 else None,
+                              v_scale=self.v_scale[layer_idx] if self._fp8 else None)
             return out
         if self._fp8:
             # The matrix-core kernel reads 16-bit pools: dequantise the blocks the tables name into a compact

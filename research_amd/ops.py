@@ -182,10 +182,12 @@ def pack_mask(keep: Tensor) -> Tensor:
 
 def attend_masked(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Tensor, ctx_lens: Tensor, q_lens: Tensor,
                   q_starts: Tensor, max_q_len: int, block_size: int, scale: float, mask_words: Tensor, n_keys: int,
-                  out: Optional[Tensor] = None) -> Tensor:
+                  out: Optional[Tensor] = None, k_scale: Optional[Tensor] = None,
+                  v_scale: Optional[Tensor] = None) -> Tensor:
     """Attention of packed q rows ``[total_q, Hq, D]`` over a paged context under an arbitrary mask
     (``pa_attend_masked``): ``mask_words`` int32 ``[total_q, 1 or Hq, words]`` from ``pack_mask``; row r attends
-    key j < n_keys iff its bit is set; keys at or past ``ctx_lens[b]`` are zero rows."""
+    key j < n_keys iff its bit is set; keys at or past ``ctx_lens[b]`` are zero rows.  An fp8-e4m3 pool comes with
+    its ``k_scale`` / ``v_scale``."""
     total_q, hq, d = q.shape
     total_slots, hkv, _ = k_cache.shape
     if mask_words.dtype != torch.int32 or mask_words.dim() != 3 or mask_words.shape[0] != total_q:
@@ -195,7 +197,8 @@ def attend_masked(q: Tensor, k_cache: Tensor, v_cache: Tensor, block_tables: Ten
     _run("pa_attend_masked", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(out), _ptr(block_tables),
          block_tables.shape[1], _ptr(ctx_lens), _ptr(q_lens), _ptr(q_starts), _ptr(mask_words), mask_words.shape[1],
          mask_words.shape[2], int(n_keys), block_tables.shape[0], max_q_len, hq, hkv, d, block_size,
-         total_slots // block_size, float(scale), PA_DTYPE[q.dtype], _stream(q))
+         total_slots // block_size, float(scale), PA_DTYPE[q.dtype], PA_DTYPE[k_cache.dtype], _ptr(k_scale),
+         _ptr(v_scale), _stream(q))
     return out
 
 

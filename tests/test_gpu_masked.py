@@ -136,3 +136,38 @@ def test_predicates_through_the_backend():
     with pytest.raises(NotImplementedError):
         be.forward(q1.cuda(), None, None, 0, InferenceContext(is_prefill=False, block_tables=tables,
                                                              seq_lens=tuple(ctx_lens), block_mask=object()))
+
+
+def test_predicates_over_an_fp8_pool():
+    """A mask predicate with ``kv_format="fp8_e4m3"``: the masked kernel widens the pool's bytes with the tile's
+    scale; against the checker on the dequantised pool (6e-2), in chunked prefill and in decode."""
+    announce("mask predicates over an fp8 pool")
+    rng = np.random.default_rng(4)
+    bs, nb, hkv, hq, d = 16, 12, 2, 4, 64
+    be = HipPagedAttentionBackend(CacheConfig(num_layers=1, num_kv_heads=hkv, head_dim=d, num_blocks=nb, block_size=bs,
+                                              dtype=torch.bfloat16, device="cuda", kv_format="fp8_e4m3"))
+    be.set_num_heads(hq)
+    kp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+    vp = torch.from_numpy(rng.standard_normal((nb * bs, hkv, d)).astype(np.float32)).to(torch.bfloat16)
+    be.quantize_from(kp.cuda(), vp.cuda(), 0)
+    kd = po.dequantize_kv_e4m3(be.k_cache[0].cpu().view(torch.uint8), be.k_scale[0].cpu(), bs)
+    vd = po.dequantize_kv_e4m3(be.v_cache[0].cpu().view(torch.uint8), be.v_scale[0].cpu(), bs)
+    tables, ctx_lens, pre = ((3, 1, 6, 9), (7, 2, 5)), [60, 41], [52, 33]
+    q = torch.from_numpy(rng.standard_normal((2, 8, hq, d)).astype(np.float32)).to(torch.bfloat16)
+    window = lambda b, h, q_idx, kv_idx: (q_idx >= kv_idx) & (q_idx - kv_idx < 11 + h)
+    ctx = InferenceContext(is_prefill=True, block_tables=tables, seq_lens=tuple(ctx_lens), prefix_lens=tuple(pre),
+                           block_mask=window)
+    out = be.forward(q.cuda(), None, None, 0, ctx)
+    qi = (np.asarray(pre)[:, None] + np.arange(8)[None, :])[:, :, None, None]
+    ki = np.arange(60)[None, None, None, :]
+    hi = np.arange(hq)[None, None, :, None]
+    keep = (qi >= ki) & (qi - ki < 11 + hi)
+    want = po.paged_attend_masked(q, kd, vd, tables, ctx_lens, [8, 8], keep, bs, be.scale)
+    assert_close(out, want, 6e-2, "per-head windows over an fp8 pool, chunked prefill")
+    q1 = q[:, :1]
+    first = lambda b, h, q_idx, kv_idx: kv_idx < 37
+    out = be.forward(q1.cuda(), None, None, 0, InferenceContext(is_prefill=False, block_tables=tables,
+                                                               seq_lens=tuple(ctx_lens), block_mask=first))
+    keep = np.broadcast_to((np.arange(60) < 37)[None, None, None, :], (2, 1, 1, 60))
+    want = po.paged_attend_masked(q1, kd, vd, tables, ctx_lens, [1, 1], keep, bs, be.scale)
+    assert_close(out, want, 6e-2, "decode under a predicate over an fp8 pool")
