@@ -46,7 +46,6 @@ import os
 import sys
 
 NC, NSTAGE = 2, 4
-X = set(os.environ.get("PF_GEN_X", "").split(","))  # experiment switches
 
 
 def configure(head_dim):
@@ -206,7 +205,7 @@ def subtile_ops(ty, j, kt):
         # rows it loaded itself; unsigned compare of the distance covers both ends)
         lds.append(Op(Ins(f"s_waitcnt vmcnt({2 * NG})\n\ts_sub_u32 s56, %[sP], %[splo]\n\ts_cmp_lt_u32 s56, %[spspan]\n"
                           f"\ts_cbranch_scc1 .Lpf_fix_{j}_%=\n.Lpf_fixed_{j}_%=:\n"
-                          "\ts_add_u32 %[sP], %[sP], 1\n\t" + ("s_nop 0" if "nobarrier" in X else "s_barrier"),
+                          "\ts_add_u32 %[sP], %[sP], 1\n\ts_barrier",
                           kind="sync", units=6, n=6), SYNC_GAP, SYNC_GAP))
         STUBS.append([f".Lpf_fix_{j}_%=:", "s_call_b64 s[50:51], .Lpf_fixup_%=", f"s_branch .Lpf_fixed_{j}_%="])
     # K operands of subtile g+2 = subtile kt of the next tile (stage j+1)
@@ -224,8 +223,8 @@ def subtile_ops(ty, j, kt):
         c, jj = n & 1, n >> 1
         s0 = S(cb, c) + 2 * jj
         ta, tb = 80 + 2 * (n % 4), 81 + 2 * (n % 4)
-        return [Ins(f"{'v_mov_b32_e32' if 'noexp' in X else 'v_exp_f32_e32'} v{ta}, v{s0}", units=2, kind="trans", reads=(f"v{s0}",), writes=(f"v{ta}",)),
-                Ins(f"{'v_mov_b32_e32' if 'noexp' in X else 'v_exp_f32_e32'} v{tb}, v{s0 + 1}", units=2, kind="trans", reads=(f"v{s0 + 1}",), writes=(f"v{tb}",))]
+        return [Ins(f"v_exp_f32_e32 v{ta}, v{s0}", units=2, kind="trans", reads=(f"v{s0}",), writes=(f"v{ta}",)),
+                Ins(f"v_exp_f32_e32 v{tb}, v{s0 + 1}", units=2, kind="trans", reads=(f"v{s0 + 1}",), writes=(f"v{tb}",))]
 
     # The row sums are plain fp32 additions: v_dot2 on the packed words would be one instruction instead of
     # two, but it does not run beside the matrix unit (measured: a product followed by two of them takes 58
@@ -330,24 +329,18 @@ def subtile_ops(ty, j, kt):
         ldr.append(Op([Ins(f"s_mul_i32 s44, s{40 + n}, %[stride]", kind="salu"),
                        Ins(f"s_mul_hi_u32 s45, s{40 + n}, %[stride]", kind="salu")], e))
         dst = dst_stage * STAGE + n * 4096
-        ld = "s_nop 0" if "noloads" in X else "global_load_lds_dwordx4"
+        ld = "global_load_lds_dwordx4"
         ldr.append(Op(Ins(f"s_add_u32 m0, %[m0w], {dst}\n\ts_add_u32 s46, %[pklo], s44\n\ts_addc_u32 s47, %[pkhi], s45\n"
-                          f"\t{ld} %[lanek], s[46:47]".replace("s_nop 0 %[lanek], s[46:47]", "s_nop 0"),
+                          f"\t{ld} %[lanek], s[46:47]",
                           kind="vmem", units=5, n=4), e))
         ldr.append(Op(Ins(f"s_add_u32 m0, %[m0w], {dst + TENSOR}\n\ts_add_u32 s48, %[pvlo], s44\n\ts_addc_u32 s49, %[pvhi], s45\n"
-                          f"\t{ld} %[lanev], s[48:49]".replace("s_nop 0 %[lanev], s[48:49]", "s_nop 0"),
+                          f"\t{ld} %[lanev], s[48:49]",
                           kind="vmem", units=5, n=4), e))
     streams["ldr"] = ldr
-    for k in list(streams):
-        if f"drop_{k}" in X:  # (timing experiments only: results are garbage)
-            streams[k] = [op for op in streams[k] if any(i.kind == "sync" for i in op.ins)]
-    if "drop_lds" in X:
-        for ins in mf:
-            ins.need = ()
     return mf, streams
 
 
-def schedule(mf, streams, spare=float(os.environ.get("PF_GEN_SPARE", "0.6"))):
+def schedule(mf, streams, spare=0.6):
     """Places the other instructions into the 33 gaps around the products: earliest deadline first within the
     capacity of a gap, a stream's instructions in their order, everything due in a gap placed there."""
     total = sum(op.units for ops in streams.values() for op in ops)
@@ -562,8 +555,7 @@ def loop_text(ty):
     del STUBS[:]
     bodies = [tile_body(ty, j) for j in range(NSTAGE)]
     bodies = add_waits(bodies)
-    if not (X - {""}):
-        check_hazards(bodies)
+    check_hazards(bodies)
     lines = []
     # prologue: addresses of stages 2 and 3 and the constants
     for ks in range(KS):
