@@ -87,6 +87,9 @@ struct RowwiseArgs {
     // the merge kernel: part_o float [row][head][split][D], part_ml float [row][head][split][2].  1 = no split.
     int splits;
     float *part_o, *part_ml;
+    // prefill_asm_kernel without lower bounds: groups of 8 tasks one workgroup runs in turn (grid.y = chunks of that
+    // many groups); 1 everywhere else.
+    int groups_per_wg;
 };
 
 __device__ __forceinline__ uint4 ld16(const void *p) { return *reinterpret_cast<const uint4 *>(p); }

@@ -124,7 +124,7 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     a.q = q; a.out = out; a.ctx_lens = ctx_lens; a.q_lens = q_lens; a.q_starts = q_starts;
     a.row_lo = row_first_key;
     a.batch = batch; a.max_q_len = max_q_len;
-    a.splits = 1; a.part_o = nullptr; a.part_ml = nullptr;
+    a.splits = 1; a.part_o = nullptr; a.part_ml = nullptr; a.groups_per_wg = 1;
     hipStream_t s = (hipStream_t)stream;
     // bf16 / fp16 with head_dim 32, 64, 128 (and 256, below) run on the matrix cores unless the caller asked for the
     // vector kernel
@@ -154,7 +154,19 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
             while (want > 1 && prefill_ws_bytes(total_q, num_q_heads, head_dim, want) > workspace_bytes) --want;
             split = want;
         }
-        mfma = pa_prefill_asm_kernel(dtype, head_dim, split > 1 || window > 0 || row_first_key != nullptr, !fits);
+        const bool lower_bounds = split > 1 || window > 0 || row_first_key != nullptr;
+        mfma = pa_prefill_asm_kernel(dtype, head_dim, lower_bounds, !fits);
+        if (!lower_bounds && fits) {
+            // The plain instance runs several groups of one (sequence, kv head) per workgroup, which share the
+            // set-up of lengths and slot tables: as many (up to 8) as leave a workgroup for every compute unit.
+            const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
+            const int64_t groups = (row_blocks * (int64_t)a.p.n_rep + kPfTasks - 1) / kPfTasks;
+            const int cus = prefill_cus();
+            int gpw = 1;
+            for (int g = 2; g <= 8; ++g)
+                if ((int64_t)num_kv_heads * ((groups + g - 1) / g) * batch >= cus) gpw = g;
+            a.groups_per_wg = gpw;
+        }
     }
     // head_dim 256: one 32-row task per wave, loads driven by a table of 16-key groups - which must lie inside one
     // pool block (block sizes that are multiples of 16, or a single block per sequence); the kernel fills its table
@@ -182,7 +194,8 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     if (mfma) {
         PA_REQUIRE(pa_aligned16(q) && pa_aligned16(out), "q and out must be 16-byte aligned");
         const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
-        const int groups = (row_blocks * a.p.n_rep + tasks_per_wg - 1) / tasks_per_wg;
+        int groups = (row_blocks * a.p.n_rep + tasks_per_wg - 1) / tasks_per_wg;
+        groups = (groups + a.groups_per_wg - 1) / a.groups_per_wg;  // workgroups along y: chunks of groups
         PA_REQUIRE((int64_t)groups * split <= 65535, "max_q_len=%d is too long for one launch", max_q_len);
         if (split > 1) {
             PA_REQUIRE(((uintptr_t)workspace & 255u) == 0, "workspace must be 256-byte aligned");

@@ -64,24 +64,64 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5, col = lane & 31;
 
-    // workgroup -> (kv head, group of 8 tasks, sequence), heaviest groups first when the prefix is short
-    // (the launch order of prefill_mfma_kernel)
+    // workgroup -> (kv head, chunk of groups of 8 tasks, sequence), heaviest first when the prefix is short (the launch
+    // order of prefill_mfma_kernel).  The plain instance runs the a.groups_per_wg groups of its chunk in turn:
+    // lengths and slot tables are set up once (the groups of one sequence and kv head share them), which is a
+    // third of what a group costs beside its loop and counts where the loop is short (prompts of a few hundred
+    // tokens).
     const int kvh = blockIdx.x;
     const int n_splits = a.splits;  // pieces a workgroup's tiles are cut into (1: none; more only in the LO instance)
-    const int piece = (int)blockIdx.y % n_splits, group_y = (int)blockIdx.y / n_splits;
-    const int n_groups = gridDim.y / n_splits, n_seqs = gridDim.z;
-    const int lin = group_y + n_groups * blockIdx.z;
+    const int gpw = (LO || LONG) ? 1 : a.groups_per_wg;  // groups per workgroup
+    const int piece = (int)blockIdx.y % n_splits, chunk_y = (int)blockIdx.y / n_splits;
+    const int n_chunks = gridDim.y / n_splits, n_seqs = gridDim.z;
+    const int lin = chunk_y + n_chunks * blockIdx.z;
     const bool group_major = a.ctx_lens[0] - a.q_lens[0] < a.q_lens[0];
-    const int group = group_major ? n_groups - 1 - lin / n_seqs : group_y;
+    const int wg_chunk = group_major ? n_chunks - 1 - lin / n_seqs : chunk_y;
     const int b = group_major ? lin % n_seqs : (int)blockIdx.z;
     const int q_len = a.q_lens[b];
     const int ctx_len = a.ctx_lens[b];
     const int prefix = ctx_len - q_len;
     const int n_rowblocks = (q_len + kPfRows - 1) / kPfRows;
     const int n_tasks = n_rowblocks * p.n_rep;
-    const int task0 = group * kPfTasks;
-    if (task0 >= n_tasks || q_len <= 0) return;  // uniform over the workgroup
+    // Groups of this workgroup: one of every n_chunks consecutive groups, the wg_chunk-th from the front in even
+    // rounds and from the back in odd ones, so that under the causal mask (later groups see more keys) the
+    // workgroups' totals come out equal.
+    const int group_end = (n_tasks + kPfTasks - 1) / kPfTasks;
+    if (wg_chunk >= group_end || q_len <= 0) return;  // uniform over the workgroup
+    auto group_of = [&](int i) PF_INLINE { return i * n_chunks + ((i & 1) ? n_chunks - 1 - wg_chunk : wg_chunk); };
+    int first_special_tab = 0;  // (of the tables, which the workgroup's groups share)
+    // Q rows of a group, staged as whole rows through the upper half of the ring (empty between two groups' loops;
+    // the write-out stages its rows through the lower half): 32 rows of each of the wave's two tasks.  The first
+    // group's are requested here, a later group's before the write-out of the group before it, so that they
+    // travel while that group's rows are normalised and stored.
+    constexpr int QRB = D * 2, QCPR = QRB / 16, QRPI = 64 / QCPR;
+    constexpr int kStoresPerTask = 32 / QRPI;  // store instructions of the write-out per task
+    const uint32_t q_stage = (uint32_t)(kRingBytes / 2) + (uint32_t)wave * (NC * 32 * QRB);
+    static_assert(kPfWaves * NC * 32 * QRB == kRingBytes / 2, "the staged rows of the four waves fill half the ring");
+    auto issue_q = [&](int grp) PF_INLINE {
+        const int lrow = lane / QCPR, lslot = lane % QCPR;
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+            const int task = grp * kPfTasks + wave * NC + c;
+            const bool lv = task < n_tasks;
+            const int rb = lv ? task / p.n_rep : 0;
+            const int qhead = kvh * p.n_rep + (lv ? task - rb * p.n_rep : 0);
+            const char *qb = reinterpret_cast<const char *>(a.q) + ((int64_t)a.q_starts[b] * p.hq + qhead) * (D * 2);
+#pragma unroll
+            for (int i = 0; i < 32 / QRPI; ++i) {
+                const int r = i * QRPI + lrow;
+                const int64_t grow = min(rb * kPfRows + r, q_len - 1);
+                pf_dma16(lds_base + q_stage + (uint32_t)((c * 32 + i * QRPI) * QRB),
+                         qb + grow * p.hq * (D * 2) + ((lslot ^ (r & (QCPR - 1))) * 16));
+            }
+        }
+    };
+    issue_q(wg_chunk);
+    int prev_stores = 0;  // store instructions this wave issued behind the current group's Q loads
 
+    for (int gi = 0;;) {  // uniform control flow, stated to the compiler
+    const int group = __builtin_amdgcn_readfirstlane(group_of(gi));
+    const int task0 = group * kPfTasks;
     bool live[NC];
     int row0[NC], qh[NC];
 #pragma unroll
@@ -152,23 +192,6 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     constexpr int kSegTiles = (kPaCapTiles - kPfStages) / kPfStages * kPfStages;  // (the loop starts in ring slot 0)
     const int cap_rel = kPaCapTiles;
 
-    // ---- Q^T operands, staged through the (still empty) ring as whole rows: see prefill_mfma_kernel ----
-    constexpr int QRB = D * 2, QCPR = QRB / 16, QRPI = 64 / QCPR;
-    const uint32_t q_stage = (uint32_t)wave * (NC * 32 * QRB);
-    {
-        const int lrow = lane / QCPR, lslot = lane % QCPR;
-#pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            const char *qb = reinterpret_cast<const char *>(a.q) + ((int64_t)a.q_starts[b] * p.hq + qh[c]) * (D * 2);
-#pragma unroll
-            for (int i = 0; i < 32 / QRPI; ++i) {
-                const int r = i * QRPI + lrow;
-                const int64_t grow = min(row0[c] + r, q_len - 1);
-                pf_dma16(lds_base + q_stage + (uint32_t)((c * 32 + i * QRPI) * QRB),
-                         qb + grow * p.hq * (D * 2) + ((lslot ^ (r & (QCPR - 1))) * 16));
-            }
-        }
-    }
     // ---- slot tables (in flight together with the Q rows) ----
     const int64_t pool_rows = p.num_blocks * p.bs;  // >= 16, < 2^31 (the host checks)
     // Blocks that are not multiples of 16 keys long (one block per sequence, as dense prefill passes its rows):
@@ -189,9 +212,12 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             edge_slot = bid * p.bs + key_last;
         }
     }
+    // the tables hold the tiles of this group, or of the whole sequence when the workgroup runs several groups
+    const int tab_tiles =
+        gpw == 1 ? n_tiles : (ctx_len + kPfKeys - 1) / kPfKeys - t0;  // (several groups: every key of the sequence)
     auto fill_tables = [&](int base) PF_INLINE {
         const int32_t *bt_seq = p.bt + (int64_t)b * p.bt_stride;
-        const int n_rest = n_tiles - base;             // tiles still to run (>= 1)
+        const int n_rest = tab_tiles - base;           // tiles still to run (>= 1)
         const int n_real = min(n_rest, kPaCapTiles);   // those of them with table entries
         const int n_entries = n_real * GPT;  // (the loads of tiles past the last fetch tile 0 again: it has entries)
         int first_special = n_rest;
@@ -220,8 +246,18 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     auto read_special = [&]() PF_INLINE {
         return __builtin_amdgcn_readfirstlane(min(min(s_special[0], s_special[1]), min(s_special[2], s_special[3])));
     };
-    fill_tables(0);
-    pf_wait_loads<0>();
+    const bool first_group = gi == 0;  // uniform
+    if (first_group) {
+        fill_tables(0);
+        pf_wait_loads<0>();
+    } else if (prev_stores == 2 * kStoresPerTask) {
+        // this group's Q rows were requested before the last group's stores: wait for them, not for the stores
+        pf_wait_loads<2 * kStoresPerTask>();
+    } else if (prev_stores == kStoresPerTask) {
+        pf_wait_loads<kStoresPerTask>();
+    } else {
+        pf_wait_loads<0>();
+    }
     const float sc = p.scale_log2;
     X8 qreg[NC][KS];
 #pragma unroll
@@ -243,7 +279,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qreg[c][ks]));
     __syncthreads();  // the tables are complete and the staged rows have been read: the ring may overwrite them
-    int first_special = read_special();
+    if (first_group) first_special_tab = read_special();
+    int first_special = min(first_special_tab, n_tiles);  // (a group before the last runs fewer tiles than the tables hold)
 
     // ---- loads of a tile: wave w fetches rows w*RPL .. w*RPL + RPL-1 of the tile and, NG-1 times, the rows 4*RPL on ----
     const int64_t tok_stride = (int64_t)p.hkv * D * 2;
@@ -551,6 +588,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     }
     // ---- normalise; rows go through LDS so that every store instruction writes whole 256-byte rows ----
     __syncthreads();  // every wave is done with the ring
+    const int group_next = __builtin_amdgcn_readfirstlane(group_of(gi + 1));
+    if (group_next < group_end) issue_q(group_next);  // (uniform) the next group's Q rows travel during the write-out
     const uint32_t out_stage = (uint32_t)wave * (NC * 32 * QRB);  // this wave's 64 rows of 256 bytes
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
@@ -571,20 +610,30 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     }
     // (a wave reads only what it wrote itself: no barrier, the compiler waits for the LDS writes)
     {
-        const int r_in = lane / QCPR, chunk = lane % QCPR;  // 4 rows per instruction, 16 bytes per lane
+        // Stores through a descriptor of the sequence's rows: a row past the chunk's length falls outside it and is
+        // dropped, so every task costs exactly kStoresPerTask store instructions - the count the next group's wait
+        // for its Q rows (requested before these stores) relies on.
+        const int r_in = lane / QCPR, chunk = lane % QCPR;  // QRPI rows per instruction, 16 bytes per lane
+        const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(reinterpret_cast<T *>(a.out) + (int64_t)a.q_starts[b] * p.hq * D), 0, q_len * p.hq * (D * 2), 0x00020000);
+        prev_stores = 0;
 #pragma unroll
         for (int c = 0; c < NC; ++c) {
-            if (!live[c]) continue;
-            T *obase = reinterpret_cast<T *>(a.out) + (((int64_t)a.q_starts[b] + row0[c]) * p.hq + qh[c]) * D;
+            if (!live[c]) continue;  // uniform
+            prev_stores += kStoresPerTask;
 #pragma unroll
             for (int i = 0; i < 32 / QRPI; ++i) {
                 const int r = i * QRPI + r_in;
                 const uint4 v = *reinterpret_cast<const uint4 *>(s_mem + out_stage + (c * 32 + r) * QRB + ((chunk ^ (r & (QCPR - 1))) * 16));
-                if (row0[c] + r < q_len)
-                    *reinterpret_cast<uint4 *>(reinterpret_cast<char *>(obase + (int64_t)r * p.hq * D) + chunk * 16) = v;
+                __builtin_amdgcn_raw_buffer_store_b128(pa_u4{v.x, v.y, v.z, v.w}, rout,
+                                                       ((row0[c] + r) * p.hq + qh[c]) * (D * 2) + chunk * 16, 0, 0);
             }
         }
     }
+    gi = __builtin_amdgcn_readfirstlane(gi + 1);
+    if (group_next >= group_end) break;
+    __syncthreads();  // every wave has read its staged rows: the next group's query rows may land there
+    }  // groups of the workgroup
 }
 
 // nullptr unless the element type has this kernel; `lower_bounds`: the instance for sliding windows and per-row
