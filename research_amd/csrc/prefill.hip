@@ -138,9 +138,11 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // on, which bounds the table's length - or, under a sliding window, the stretch of keys that the rows of a
     // workgroup (at most kPfTasks blocks of kPfRows) see; longer tables take the instance that fills its copy again on
     // the way.
+    // (a chunk's rows of q and out are addressed by 32-bit byte offsets from the sequence's first row)
     if (mfma && (head_dim == 128 || head_dim == 64 || head_dim == 32) && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
-        bt_stride * (int64_t)block_size < (1ll << 31)) {
+        bt_stride * (int64_t)block_size < (1ll << 31) &&
+        (int64_t)max_q_len * num_q_heads * head_dim * 2 < (1ll << 31)) {
         const int64_t cap_keys = (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys;
         const bool fits = bt_stride * (int64_t)block_size <= cap_keys ||
                           (window > 0 && (int64_t)window + kPfTasks * kPfRows + 3 * kPfKeys <= cap_keys);

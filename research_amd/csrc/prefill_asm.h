@@ -78,8 +78,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     const bool group_major = a.ctx_lens[0] - a.q_lens[0] < a.q_lens[0];
     const int wg_chunk = group_major ? n_chunks - 1 - lin / n_seqs : chunk_y;
     const int b = group_major ? lin % n_seqs : (int)blockIdx.z;
-    const int q_len = a.q_lens[b];
-    const int ctx_len = a.ctx_lens[b];
+    // (read once and held in scalar registers: a load behind the direct-to-LDS requests would wait for all of them)
+    const int q_len = __builtin_amdgcn_readfirstlane(a.q_lens[b]);
+    const int ctx_len = __builtin_amdgcn_readfirstlane(a.ctx_lens[b]);
+    const int q_start = __builtin_amdgcn_readfirstlane(a.q_starts[b]);
     const int prefix = ctx_len - q_len;
     const int n_rowblocks = (q_len + kPfRows - 1) / kPfRows;
     const int n_tasks = n_rowblocks * p.n_rep;
@@ -90,14 +92,22 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     if (wg_chunk >= group_end || q_len <= 0) return;  // uniform over the workgroup
     auto group_of = [&](int i) PF_INLINE { return i * n_chunks + ((i & 1) ? n_chunks - 1 - wg_chunk : wg_chunk); };
     int first_special_tab = 0;  // (of the tables, which the workgroup's groups share)
-    // Q rows of a group, staged as whole rows through the upper half of the ring (empty between two groups' loops;
-    // the write-out stages its rows through the lower half): 32 rows of each of the wave's two tasks.  The first
-    // group's are requested here, a later group's before the write-out of the group before it, so that they
-    // travel while that group's rows are normalised and stored.
+    // Between two groups' loops the ring is empty and its four stages hold: stage 0 - tile 0 of the next group
+    // (every group of the workgroup starts at key 0 of the same sequence and kv head); stages 1 and 2 - the next
+    // group's Q rows, staged as whole rows (32 rows of each of a wave's two tasks); stage 3 - the rows being written
+    // out, one task of each wave at a time.  The first group's Q rows are requested here; a later group's, and
+    // its tile 0, before the write-out of the group before it, so that they travel while that group's rows are
+    // normalised and stored.
     constexpr int QRB = D * 2, QCPR = QRB / 16, QRPI = 64 / QCPR;
     constexpr int kStoresPerTask = 32 / QRPI;  // store instructions of the write-out per task
-    const uint32_t q_stage = (uint32_t)(kRingBytes / 2) + (uint32_t)wave * (NC * 32 * QRB);
-    static_assert(kPfWaves * NC * 32 * QRB == kRingBytes / 2, "the staged rows of the four waves fill half the ring");
+    constexpr int kStageBytes = kRingBytes / kPfStages;
+    const uint32_t q_stage = (uint32_t)kStageBytes + (uint32_t)wave * (NC * 32 * QRB);
+    static_assert(kPfWaves * NC * 32 * QRB == 2 * kStageBytes, "the staged rows of the four waves fill two stages");
+    static_assert(kPfWaves * 32 * QRB == kStageBytes, "one task's rows of the four waves fill one stage");
+    // (32-bit byte offsets from the sequence's first row: the host checks that a chunk's rows span less than 2 GiB)
+    const uint32_t q_row_bytes = (uint32_t)p.hq * QRB;
+    const uint32_t q_last_row = (uint32_t)(q_len - 1) * q_row_bytes;
+    const char *q_seq = reinterpret_cast<const char *>(a.q) + (int64_t)q_start * p.hq * QRB;
     auto issue_q = [&](int grp) PF_INLINE {
         const int lrow = lane / QCPR, lslot = lane % QCPR;
 #pragma unroll
@@ -106,18 +116,21 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             const bool lv = task < n_tasks;
             const int rb = lv ? task / p.n_rep : 0;
             const int qhead = kvh * p.n_rep + (lv ? task - rb * p.n_rep : 0);
-            const char *qb = reinterpret_cast<const char *>(a.q) + ((int64_t)a.q_starts[b] * p.hq + qhead) * (D * 2);
+            const char *qb = pf_scalar_ptr(q_seq + qhead * QRB);
+            const uint32_t row_ofs = (uint32_t)(rb * kPfRows + lrow) * q_row_bytes;
 #pragma unroll
             for (int i = 0; i < 32 / QRPI; ++i) {
                 const int r = i * QRPI + lrow;
-                const int64_t grow = min(rb * kPfRows + r, q_len - 1);
-                pf_dma16(lds_base + q_stage + (uint32_t)((c * 32 + i * QRPI) * QRB),
-                         qb + grow * p.hq * (D * 2) + ((lslot ^ (r & (QCPR - 1))) * 16));
+                // (rows past the chunk's end read its last row: they are computed and never stored)
+                const uint32_t ofs = min(row_ofs + (uint32_t)(i * QRPI) * q_row_bytes, q_last_row);
+                pf_dma16(lds_base + q_stage + (uint32_t)((c * 32 + i * QRPI) * QRB), qb,
+                         ofs + (uint32_t)((lslot ^ (r & (QCPR - 1))) * 16));
             }
         }
     };
     issue_q(wg_chunk);
     int prev_stores = 0;  // store instructions this wave issued behind the current group's Q loads
+    bool tile0_ahead = false;  // (uniform) tile 0 of the current group was requested with its Q rows
 
     for (int gi = 0;;) {  // uniform control flow, stated to the compiler
     const int group = __builtin_amdgcn_readfirstlane(group_of(gi));
@@ -148,7 +161,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     int lo[NC] = {0, 0};    // a lane's first visible key per column tile, less 4 * half like lim
     if constexpr (LO) {
         const int win = p.window;
-        const int32_t *rlo = a.row_lo ? a.row_lo + a.q_starts[b] : nullptr;
+        const int32_t *rlo = a.row_lo ? a.row_lo + q_start : nullptr;
         auto row_first = [&](int row) PF_INLINE {
             const int pos = prefix + row;
             int first = win > 0 ? pos - win + 1 : 0;
@@ -172,7 +185,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
                 for (int c = 0; c < NC; ++c) {
                     const int row = row0[c] + col;
                     if (live[c] && row < q_len && half == 0) {
-                        const int64_t at = ((((int64_t)a.q_starts[b] + row) * p.hq + qh[c]) * n_splits + piece) * 2;
+                        const int64_t at = ((((int64_t)q_start + row) * p.hq + qh[c]) * n_splits + piece) * 2;
                         a.part_ml[at] = kNegBig;
                         a.part_ml[at + 1] = 0.f;
                     }
@@ -260,12 +273,19 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     }
     const float sc = p.scale_log2;
     X8 qreg[NC][KS];
+    uint4 q_raw[NC][KS];  // (all reads first: one LDS round trip)
 #pragma unroll
     for (int c = 0; c < NC; ++c)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             const int slot = (2 * ks + half) ^ (col & (QCPR - 1));
-            const uint4 raw = *reinterpret_cast<const uint4 *>(s_mem + q_stage + (c * 32 + col) * QRB + slot * 16);
+            q_raw[c][ks] = *reinterpret_cast<const uint4 *>(s_mem + q_stage + (c * 32 + col) * QRB + slot * 16);
+        }
+#pragma unroll
+    for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const uint4 raw = q_raw[c][ks];
             // scaled by softmax scale * log2(e) here, once per workgroup: S^T then comes out of the products in
             // the units of the exponential's argument (one more rounding of q to its 16-bit type)
             const X8 q8 = __builtin_bit_cast(X8, raw);
@@ -298,37 +318,53 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     auto issue = [&](int tile) PF_INLINE {
         const int src = tile < min(n_tiles, kPaCapTiles) ? tile : 0;
         const uint32_t dst0 = m0w + (uint32_t)(tile % kPfStages) * 2 * G::BYTES;
+        int32_t slots[NG];  // (read together: one wait for the table instead of one per load)
+#pragma unroll
+        for (int n = 0; n < NG; ++n) slots[n] = tab_a[src * GPT + g0 + n * GSTEP];
 #pragma unroll
         for (int n = 0; n < NG; ++n) {
-            const uint32_t slot = (uint32_t)__builtin_amdgcn_readfirstlane(tab_a[src * GPT + g0 + n * GSTEP]);
+            const uint32_t slot = (uint32_t)__builtin_amdgcn_readfirstlane(slots[n]);
             const uint64_t ofs = (uint64_t)slot * (uint32_t)tok_stride;
             pf_dma16(dst0 + n * kLoadStep, pf_scalar_ptr(pool_k + ofs), lane_k);
             pf_dma16(dst0 + G::BYTES + n * kLoadStep, pf_scalar_ptr(pool_v + ofs), lane_v);
         }
     };
-    issue(0);
-    issue(1);
-    issue(2);
-    pf_wait_loads<4 * NG>();  // tile 0 has landed
-    if (first_special == 0) {  // clear the rows of tile 0 that do not exist (the loop does it for later tiles)
-#pragma unroll
-        for (int n = 0; n < NG; ++n)
-            if (arow >= tab_b[g0 + n * GSTEP]) {
-                const uint32_t at = (m0w - lds_base) + n * kLoadStep + lane * 16;
-                *reinterpret_cast<uint4 *>(s_mem + at) = uint4{0, 0, 0, 0};
-                *reinterpret_cast<uint4 *>(s_mem + at + G::BYTES) = uint4{0, 0, 0, 0};
-            }
-    }
     // this wave's load of the group at the end of the pool, as an LDS offset behind the wave's first load (-1: none)
     const int edge_n = edge_group - g0;
     const int edge_ofs = edge_tile >= 0 && edge_n >= 0 && edge_n % GSTEP == 0 ? edge_n / GSTEP * kLoadStep : -1;
-    if (edge_tile == 0 && edge_ofs >= 0 && arow < edge_rows) {  // (in tile 0; the loop does it for later tiles)
-        const uint32_t at = (m0w - lds_base) + edge_ofs + lane * 16;
-        *reinterpret_cast<uint4 *>(s_mem + at) = *reinterpret_cast<const uint4 *>(pool_k + edge_slot * tok_stride + lane_k);
-        *reinterpret_cast<uint4 *>(s_mem + at + G::BYTES) =
-            *reinterpret_cast<const uint4 *>(pool_v + edge_slot * tok_stride + lane_v);
+    auto mend_tile0 = [&]() PF_INLINE {  // (the loop does this for later tiles)
+        if (first_special == 0) {  // clear the rows of tile 0 that do not exist
+#pragma unroll
+            for (int n = 0; n < NG; ++n)
+                if (arow >= tab_b[g0 + n * GSTEP]) {
+                    const uint32_t at = (m0w - lds_base) + n * kLoadStep + lane * 16;
+                    *reinterpret_cast<uint4 *>(s_mem + at) = uint4{0, 0, 0, 0};
+                    *reinterpret_cast<uint4 *>(s_mem + at + G::BYTES) = uint4{0, 0, 0, 0};
+                }
+        }
+        if (edge_tile == 0 && edge_ofs >= 0 && arow < edge_rows) {
+            const uint32_t at = (m0w - lds_base) + edge_ofs + lane * 16;
+            *reinterpret_cast<uint4 *>(s_mem + at) = *reinterpret_cast<const uint4 *>(pool_k + edge_slot * tok_stride + lane_k);
+            *reinterpret_cast<uint4 *>(s_mem + at + G::BYTES) =
+                *reinterpret_cast<const uint4 *>(pool_v + edge_slot * tok_stride + lane_v);
+        }
+    };
+    if (tile0_ahead) {
+        // tile 0 landed with the Q rows and the barrier above published it
+        issue(1);
+        issue(2);
+        if (first_special == 0 || edge_tile == 0) {  // uniform, rare: a context of less than a tile, an absent first block
+            mend_tile0();
+            __syncthreads();
+        }
+    } else {
+        issue(0);
+        issue(1);
+        issue(2);
+        pf_wait_loads<4 * NG>();  // tile 0 has landed
+        mend_tile0();
+        __syncthreads();  // tile 0 is visible
     }
-    __syncthreads();  // tile 0 is visible
 
     // ---- operand read addresses (stage 0), as in prefill_mfma_kernel ----
     uint32_t kad[KS], vad[DT];
@@ -569,7 +605,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
                 const float l_tot = l_run[c] + __shfl_xor(l_run[c], 32, 64);
                 const int row = row0[c] + col;
                 if (!live[c] || row >= q_len) continue;
-                const int64_t at = (((int64_t)a.q_starts[b] + row) * p.hq + qh[c]) * n_splits + piece;
+                const int64_t at = (((int64_t)q_start + row) * p.hq + qh[c]) * n_splits + piece;
                 float *po = a.part_o + at * D + 4 * half;  // lane owns d = 32*dt + 8*g + 4*half + j
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt)
@@ -589,15 +625,29 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     // ---- normalise; rows go through LDS so that every store instruction writes whole 256-byte rows ----
     __syncthreads();  // every wave is done with the ring
     const int group_next = __builtin_amdgcn_readfirstlane(group_of(gi + 1));
-    if (group_next < group_end) issue_q(group_next);  // (uniform) the next group's Q rows travel during the write-out
-    const uint32_t out_stage = (uint32_t)wave * (NC * 32 * QRB);  // this wave's 64 rows of 256 bytes
+    tile0_ahead = false;
+    if (group_next < group_end) {  // (uniform) the next group's Q rows and its tile 0 travel during the write-out
+        issue_q(group_next);
+        if constexpr (!LO && !LONG) {
+            issue(0);
+            tile0_ahead = true;
+        }
+    }
+    const uint32_t out_stage = 3u * kStageBytes + (uint32_t)wave * (32 * QRB);  // this wave's 32 rows of a task
+    // Stores through a descriptor of the sequence's rows: a row past the chunk's length falls outside it and is
+    // dropped, so every task costs exactly kStoresPerTask store instructions - the count the next group's wait
+    // for its Q rows (requested before these stores) relies on.
+    const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(
+        (void *)(reinterpret_cast<T *>(a.out) + (int64_t)q_start * p.hq * D), 0, q_len * p.hq * (D * 2), 0x00020000);
+    prev_stores = 0;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
+        if (!live[c]) continue;  // uniform
         const float l_tot = l_run[c] + __shfl_xor(l_run[c], 32, 64);
         const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
         // lane owns row col, d = 32*dt + 8*g + 4*half + j: the 8 bytes are half `half` of 16-byte chunk 4*dt + g,
         // chunks swizzled by row so that the 32 rows of a store spread over the banks
-        char *rowp = s_mem + out_stage + (c * 32 + col) * QRB;
+        char *rowp = s_mem + out_stage + col * QRB;
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -607,32 +657,24 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
                 w.y = M::pack(o[c][dt][4 * g + 2] * inv, o[c][dt][4 * g + 3] * inv);
                 *reinterpret_cast<uint2 *>(rowp + (((4 * dt + g) ^ (col & (QCPR - 1))) * 16) + 8 * half) = w;
             }
-    }
-    // (a wave reads only what it wrote itself: no barrier, the compiler waits for the LDS writes)
-    {
-        // Stores through a descriptor of the sequence's rows: a row past the chunk's length falls outside it and is
-        // dropped, so every task costs exactly kStoresPerTask store instructions - the count the next group's wait
-        // for its Q rows (requested before these stores) relies on.
+        // (a wave reads only what it wrote itself, and LDS serves a wave in order: no barrier)
         const int r_in = lane / QCPR, chunk = lane % QCPR;  // QRPI rows per instruction, 16 bytes per lane
-        const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(
-            (void *)(reinterpret_cast<T *>(a.out) + (int64_t)a.q_starts[b] * p.hq * D), 0, q_len * p.hq * (D * 2), 0x00020000);
-        prev_stores = 0;
+        prev_stores += kStoresPerTask;
+        uint4 rows[32 / QRPI];  // (all reads before the first store: one LDS round trip, not one per store)
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-            if (!live[c]) continue;  // uniform
-            prev_stores += kStoresPerTask;
-#pragma unroll
-            for (int i = 0; i < 32 / QRPI; ++i) {
-                const int r = i * QRPI + r_in;
-                const uint4 v = *reinterpret_cast<const uint4 *>(s_mem + out_stage + (c * 32 + r) * QRB + ((chunk ^ (r & (QCPR - 1))) * 16));
-                __builtin_amdgcn_raw_buffer_store_b128(pa_u4{v.x, v.y, v.z, v.w}, rout,
-                                                       ((row0[c] + r) * p.hq + qh[c]) * (D * 2) + chunk * 16, 0, 0);
-            }
+        for (int i = 0; i < 32 / QRPI; ++i) {
+            const int r = i * QRPI + r_in;
+            rows[i] = *reinterpret_cast<const uint4 *>(s_mem + out_stage + r * QRB + ((chunk ^ (r & (QCPR - 1))) * 16));
         }
+        const int out_ofs = ((row0[c] + r_in) * p.hq + qh[c]) * (D * 2) + chunk * 16;
+#pragma unroll
+        for (int i = 0; i < 32 / QRPI; ++i)
+            __builtin_amdgcn_raw_buffer_store_b128(pa_u4{rows[i].x, rows[i].y, rows[i].z, rows[i].w}, rout,
+                                                   out_ofs + i * QRPI * (int)q_row_bytes, 0, 0);
     }
     gi = __builtin_amdgcn_readfirstlane(gi + 1);
     if (group_next >= group_end) break;
-    __syncthreads();  // every wave has read its staged rows: the next group's query rows may land there
+    // (no barrier: until the next group's barrier behind its Q^T read, a wave touches only its own staged rows)
     }  // groups of the workgroup
 }
 
