@@ -118,11 +118,12 @@ __device__ __forceinline__ void pf_dma16(uint32_t lds_dst, const char *lane_ptr)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_dst), "v"(lane_ptr) : "memory", "m0");
 }
 // One table entry per lane, loaded behind the compiler's back like the tile loads (a load the compiler knows
-// about would make it wait for ALL loads in flight wherever it cannot prove the value has arrived); the
-// caller waits with pf_wait_loads<0>() before the value is used.
-__device__ __forceinline__ int pf_load_i32(const int32_t *lane_ptr) {
+// about would make it wait for ALL loads in flight wherever it cannot prove the value has arrived).  The load
+// and the wait for it (which is a wait for every load of the wave in flight) are one statement: the
+// compiler never sees the register while the value is still on its way.
+__device__ __forceinline__ int pf_load_i32_wait(const int32_t *lane_ptr) {
     int v;
-    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(lane_ptr) : "memory");
+    asm volatile("global_load_dword %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=&v"(v) : "v"(lane_ptr) : "memory");
     return v;
 }
 // Wait until at most N of this wave's vector memory loads are outstanding (they complete in order).
@@ -341,9 +342,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
             if (tile % WIN == 0 || tile == t0) {  // next window of block ids (once per 16 tiles: latency not hidden)
                 const int idx = (tile - tile % WIN) * BPT + lane;
                 int v = -1;
-                if (idx < p.bt_stride) v = pf_load_i32(bt_row + idx);
-                pf_wait_loads<0>();
-                asm volatile("" : "+v"(v));
+                if (idx < p.bt_stride) v = pf_load_i32_wait(bt_row + idx);
                 bid_win = v;
             }
             const int first = (tile % WIN) * BPT;  // lane of the window that holds the tile's first block
@@ -370,9 +369,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_mfma_kernel(const RowwiseA
                 win_base = g_blk[0];
                 const int idx = win_base + lane;
                 int v = -1;
-                if (idx < p.bt_stride) v = pf_load_i32(bt_row + idx);
-                pf_wait_loads<0>();
-                asm volatile("" : "+v"(v));
+                if (idx < p.bt_stride) v = pf_load_i32_wait(bt_row + idx);
                 bid_win = v;
             }
             uint32_t g_row[NLW];  // pool row (slot) of the first row of each load
