@@ -37,6 +37,15 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 matrix peak, vendor figure
 TRAFFIC_FILE = os.path.join(ROOT, "profiles", "traffic.json")
 
 
+def calibration_copy(dev) -> None:
+    """One device copy of 1 GiB (reads 1 GiB, writes 1 GiB): what `--traffic-from-pmc` scales the counters by."""
+    src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def measured_traffic(name):
     try:
         with open(TRAFFIC_FILE) as f:
@@ -240,11 +249,7 @@ def bench_prefill_c3(args, dev) -> dict:
         prefill()
 
     if args.copy_calibration:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(dev)
     preheat(step, args.preheat_s)
     for _ in range(args.warmup):
         step()
@@ -351,11 +356,7 @@ def bench_prefill_head(args, dev, name) -> dict:
         ops.prefill_paged(q, kc, vc, tables, ctx, ql, qs, C, w.block_size, w.scale, out=out)
 
     if args.copy_calibration:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(dev)
     preheat(prefill, args.preheat_s)
     for _ in range(args.warmup):
         prefill()
@@ -415,11 +416,7 @@ def bench_prefill_long(args, dev, name) -> dict:
         ops.prefill_paged(q, kc, vc, tables, ctx, ql, qs, C, bs, scale, out=out, workspace=ws)
 
     if args.copy_calibration:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(dev)
     preheat(prefill, args.preheat_s)
     for _ in range(args.warmup):
         prefill()
@@ -468,6 +465,8 @@ def bench_prefill_dense(args, dev, name) -> dict:
     def prefill():
         ops.prefill_paged(q, k, v, tables, lens, lens, starts, T, T, scale, out=out)
 
+    if args.copy_calibration:
+        calibration_copy(dev)
     preheat(prefill, args.preheat_s)
     for _ in range(args.warmup):
         prefill()
@@ -589,11 +588,7 @@ def bench_decode(name, args, dev) -> dict:
                    out=out, entry=entry)
 
     if args.copy_calibration:
-        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
-        dst = torch.empty_like(src)
-        dst.copy_(src)  # reads 1 GiB, writes 1 GiB
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(dev)
     preheat(step, args.preheat_s)
     for _ in range(args.warmup):
         step()
