@@ -91,6 +91,37 @@ def test_end_to_end_like_the_reference_script_with_values():
     assert not backend.k_cache.any() and not backend.v_cache.any()
 
 
+@pytest.mark.parametrize("head_dim,dtype", [(96, torch.bfloat16), (80, torch.float16), (192, torch.bfloat16), (40, torch.float32)])
+def test_head_sizes_between_the_compiled_ones_through_the_backend(head_dim, dtype):
+    """The reference takes any head_dim (attention/config.py:22-24): prefill, append and decode of a head size
+    that has no kernel instance of its own, through the backend."""
+    announce(f"backend head_dim {head_dim} {dtype}")
+    cache = PagedKVCache(num_blocks=16, block_size=4)
+    config = CacheConfig(num_layers=1, num_kv_heads=2, head_dim=head_dim, num_blocks=16, block_size=4, device="cuda",
+                         dtype=dtype)
+    backend = HipPagedAttentionBackend(config)
+    backend.set_num_heads(4)
+    layer = Attention(layer_idx=0, backend=backend)
+    torch.manual_seed(head_dim)
+    ctx, _ = allocate_and_build_context(cache, seq_id=0, token_ids=list(range(1, 8)))
+    q = torch.randn(1, 7, 4, head_dim, device="cuda", dtype=dtype)
+    k = torch.randn(1, 7, 2, head_dim, device="cuda", dtype=dtype)
+    v = torch.randn(1, 7, 2, head_dim, device="cuda", dtype=dtype)
+    out = layer(q, k, v, ctx)
+    tol = 2e-2 if dtype != torch.float32 else 1e-4
+    assert_close(out, po.dense_prefill(q.cpu(), k.cpu(), v.cpu(), backend.scale), tol, "prefill")
+    ctx = extend_and_build_context(cache, seq_id=0, new_token=9, current_len=7)
+    q1 = torch.randn(1, 1, 4, head_dim, device="cuda", dtype=dtype)
+    k1 = torch.randn(1, 1, 2, head_dim, device="cuda", dtype=dtype)
+    v1 = torch.randn(1, 1, 2, head_dim, device="cuda", dtype=dtype)
+    out = layer(q1, k1, v1, ctx)
+    k_all, v_all = torch.cat([k, k1], 1).cpu(), torch.cat([v, v1], 1).cpu()
+    want = po.dense_prefill(torch.cat([torch.zeros_like(q), q1], 1).cpu(), k_all, v_all, backend.scale)[:, 7:]
+    assert_close(out, want, tol, "decode sees prompt + its own token")
+    kg, vg = backend._gather_kv_from_cache(0, ctx.block_tables, ctx.seq_lens)
+    assert torch.equal(kg.cpu(), k_all) and torch.equal(vg.cpu(), v_all)
+
+
 def test_dropped_token_when_the_table_cannot_grow():
     """allocate() of exactly one partial block, then decode until the block is full:
     the reference's allocator never adds a block (no hash on a partial block), the
