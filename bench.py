@@ -5,8 +5,9 @@ One step = one ``pa_decode`` call over one batch of the synthetic workload,
 inputs resident in HBM.  The headline workload is workload c4 (Llama-3-8B
 shape, B=256, bf16 pool, lognormal context lengths, seed 1004).  Prints one
 JSON line; with the default workload the line also carries short runs of the
-other configurations (c2, c5 decode, c3 append + chunked prefill) under
-``secondary``.
+other configurations (c2, c5 decode; c3 append + chunked prefill; the c3 shape at
+head_dim 256 and 64; dense prefill of 64 x 512 and 4 x 8192 tokens; one chunk
+behind 200 000 cached keys at head_dim 128 and 256) under ``secondary``.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary]
                     [--workload c4|c2|c5|c1|c3|c3-d256|c3-d64|long-d128|long-d256|dense-64x512|dense-4x8192|engine]
@@ -718,7 +719,7 @@ def secondary(args, dev) -> dict:
     short.copy_calibration = False
     short.secondary_run = True
     out = {}
-    for name in ("c2", "c5", "c3", "c3-d256", "c3-d64", "dense-64x512", "long-d128"):
+    for name in ("c2", "c5", "c3", "c3-d256", "c3-d64", "dense-64x512", "dense-4x8192", "long-d128", "long-d256"):
         r = (bench_prefill_c3(short, dev) if name == "c3" else bench_prefill_head(short, dev, name) if name in PREFILL_HEAD_SHAPES
              else bench_prefill_dense(short, dev, name) if name in PREFILL_DENSE_SHAPES
              else bench_prefill_long(short, dev, name) if name in PREFILL_LONG_SHAPES else bench_decode(name, short, dev))
