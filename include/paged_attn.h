@@ -124,6 +124,8 @@ int pa_decode_passes(int batch, int num_q_heads, int num_kv_heads, int head_dim,
  * value (logit 0), as it does in the reference.  Accumulation is fp32.  All
  * integer inputs stay on the device: the host never reads seq_lens.
  *   q, out        : [batch][num_q_heads][head_dim], dtype q_dtype, 16-byte aligned
+ *   head_dim      : a multiple of 8 up to 256 (of 16 for an fp8 pool; rows of whole 16-byte vectors); the
+ *                   reference takes any head_dim (attention/config.py:22-24)
  *   kv_dtype      : q_dtype, or PA_FP8_E4M3 with k_scale/v_scale =
  *                   float[num_blocks][num_kv_heads] (value = fp8 * scale)
  *   extra_zero_keys: NULL, or int32[batch]: that many additional all-zero
@@ -205,6 +207,8 @@ int pa_decode_static(const void *q, const void *k_cache, const void *v_cache, vo
  *   q, out   : [total_q][num_q_heads][head_dim] packed rows, sequence b's rows
  *              start at q_starts[b]; dtype PA_BF16 or PA_F16 (MFMA path) or
  *              PA_F32 (vector path)
+ *   head_dim : 32, 64, 128 or 256 run on the matrix cores (bf16 / fp16); any other multiple of 8 up to 256,
+ *              and PA_F32, on the vector kernel
  *   ctx_lens, q_lens, q_starts : int32[batch]
  *   max_q_len: upper bound of q_lens (grid sizing)
  *   window   : 0, or the sliding window of CacheConfig.sliding_window (attention/config.py:31): row i at
