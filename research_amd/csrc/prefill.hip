@@ -1,5 +1,6 @@
 // Host entry point of causal prefill attention over a paged context.
 #include "prefill_mfma.h"
+#include "prefill_plan.h"
 
 namespace pa_decode_detail {
 prefill_mfma_fn pa_prefill_asm_kernel(int dtype, int head_dim, bool lower_bounds, bool long_table);
@@ -24,33 +25,12 @@ int prefill_cus() {
     return n;
 }
 
-constexpr int kMaxPrefillSplits = 8;
-constexpr int kMinTilesPerSplit = 24;  // a piece's set-up and write-out cost about six tiles of its loop
-
-// Pieces to cut every workgroup's tiles into, from shapes alone.  The matrix-core kernels run one workgroup per
-// compute unit, each owning 256 (head_dim 256: 128) row-head pairs and all their keys, so a launch of few rows
-// leaves compute units idle however long the context is.  The launch takes rounds of `cus` workgroups, each lasting
-// a piece's tiles plus its fixed cost; the split with the shortest estimate wins (the smaller on ties), as long as a
-// piece keeps kMinTilesPerSplit tiles of the longest context the block tables can describe.
+// (the split rule, the workspace size and the groups a workgroup runs are host-testable arithmetic: prefill_plan.h)
 int prefill_splits(int64_t workgroups, int cus, int64_t max_keys) {
-    const int64_t tiles = max_keys / kPfKeys;
-    constexpr int64_t kFixedTiles = 6;  // set-up and write-out of a workgroup, in tiles of its loop
-    int best = 1;
-    int64_t best_cost = 0;
-    for (int s = 1; s <= kMaxPrefillSplits; ++s) {
-        if (s > 1 && tiles / s < kMinTilesPerSplit) break;
-        const int64_t rounds = (workgroups * s + cus - 1) / cus;
-        const int64_t cost = rounds * (tiles / s + kFixedTiles);
-        if (s == 1 || cost < best_cost) {
-            best_cost = cost;
-            best = s;
-        }
-    }
-    return best;
+    return plan_prefill_splits(workgroups, cus, max_keys, kPfKeys);
 }
-
 size_t prefill_ws_bytes(int64_t total_q, int num_q_heads, int head_dim, int splits) {
-    return splits <= 1 ? 0 : (size_t)total_q * num_q_heads * splits * ((size_t)head_dim + 2) * sizeof(float);
+    return plan_prefill_ws_bytes(total_q, num_q_heads, head_dim, splits);
 }
 
 // Merge of the pieces of a split prefill launch: one thread per (row, head, four consecutive d).
@@ -163,10 +143,7 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
             // set-up of lengths and slot tables: as many (up to 8) as leave a workgroup for every compute unit.
             const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
             const int64_t groups = (row_blocks * (int64_t)a.p.n_rep + kPfTasks - 1) / kPfTasks;
-            const int cus = prefill_cus();
-            int gpw = 1;
-            for (int g = 2; g <= 8; ++g)
-                if ((int64_t)num_kv_heads * ((groups + g - 1) / g) * batch >= cus) gpw = g;
+            const int gpw = plan_groups_per_workgroup(num_kv_heads, groups, batch, prefill_cus());
             a.groups_per_wg = gpw;
         }
     }

@@ -26,6 +26,7 @@
 // one asm statement with pinned operands and little else.
 #pragma once
 #include "prefill_mfma.h"
+#include "prefill_plan.h"
 #include "prefill_mfma_loop.inc"
 
 namespace pa_decode_detail {
@@ -90,7 +91,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     // workgroups' totals come out equal.
     const int group_end = (n_tasks + kPfTasks - 1) / kPfTasks;
     if (wg_chunk >= group_end || q_len <= 0) return;  // uniform over the workgroup
-    auto group_of = [&](int i) PF_INLINE { return i * n_chunks + ((i & 1) ? n_chunks - 1 - wg_chunk : wg_chunk); };
+    auto group_of = [&](int i) PF_INLINE { return plan_group_of(i, n_chunks, wg_chunk); };
     int first_special_tab = 0;  // (of the tables, which the workgroup's groups share)
     // Between two groups' loops the ring is empty and its four stages hold: stage 0 - tile 0 of the next group
     // (every group of the workgroup starts at key 0 of the same sequence and kv head); stages 1 and 2 - the next
@@ -178,8 +179,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             // This workgroup runs piece `piece` of the tiles [t0, t0 + n_all): a later first tile and an earlier
             // last key, nothing else changes (rows that see none of the piece's keys end with an empty sum).
             const int n_all = (wg_keys + kPfKeys - 1) / kPfKeys - t0;
-            const int tb = t0 + (int)((int64_t)piece * n_all / n_splits);
-            const int te = t0 + (int)((int64_t)(piece + 1) * n_all / n_splits);
+            int tb, te;
+            plan_piece_tiles(t0, n_all, piece, n_splits, tb, te);
             if (tb >= te) {  // uniform: fewer tiles than pieces - an empty partial for every row
 #pragma unroll
                 for (int c = 0; c < NC; ++c) {

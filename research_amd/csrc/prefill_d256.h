@@ -29,6 +29,7 @@
 // visible key multiplies exact zeros.
 #pragma once
 #include "prefill_mfma.h"
+#include "prefill_plan.h"
 #include "prefill_d256_loop.inc"
 
 namespace pa_decode_detail {
@@ -109,8 +110,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             // This workgroup runs piece `piece` of the tiles [t0, n_tiles): a later first tile and an earlier last
             // one, nothing else changes (rows that see none of the piece's keys end with an empty sum).
             const int n_all = n_tiles - t0;
-            const int tb = t0 + (int)((int64_t)piece * n_all / n_splits);
-            const int te = t0 + (int)((int64_t)(piece + 1) * n_all / n_splits);
+            int tb, te;
+            plan_piece_tiles(t0, n_all, piece, n_splits, tb, te);
             if (tb >= te) {  // uniform: fewer tiles than pieces - an empty partial for every row
                 const int row = row0 + col;
                 if (live && row < q_len && half == 0) {
