@@ -10,7 +10,7 @@ head_dim 256 and 64; dense prefill of 64 x 512 and 4 x 8192 tokens; one chunk
 behind 200 000 cached keys at head_dim 128 and 256) under ``secondary``.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-secondary]
-                    [--workload c4|c2|c5|c1|c3|c3-d256|c3-d64|long-d128|long-d256|dense-64x512|dense-4x8192|engine]
+                    [--workload c4|c2|c5|c1|c3|c3-d256|c3-d64|c3-d96|long-d128|long-d256|dense-64x512|dense-4x8192|engine]
     python bench.py --traffic-from-pmc NAME KERNEL FETCH.csv WRITE.csv   # refresh profiles/traffic.json
 """
 
@@ -100,7 +100,7 @@ def parse_args():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c3-d256", "c3-d64", "long-d128", "long-d256", "dense-64x512",
+    ap.add_argument("--workload", default="c4", choices=["c1", "c2", "c3", "c3-d256", "c3-d64", "c3-d96", "long-d128", "long-d256", "dense-64x512",
                                                          "dense-4x8192", "c4", "c5", "engine"])
     ap.add_argument("--preheat-s", type=float, default=0.5,
                     help="seconds of untimed steps before the warmup steps: an idle GPU sits at its lowest clocks "
@@ -327,13 +327,15 @@ def bench_prefill_c3(args, dev) -> dict:
 
 # the c3 shape at other head sizes: workload -> (query heads, kv heads, head_dim, seed, kernel)
 PREFILL_HEAD_SHAPES = {"c3-d256": (16, 8, 256, 1006, "prefill_d256_kernel"),
-                       "c3-d64": (32, 8, 64, 1007, "prefill_asm_kernel")}
+                       "c3-d64": (32, 8, 64, 1007, "prefill_asm_kernel"),
+                       # a head size between the compiled ones: the head_dim-128 kernel, rows of 96 in memory
+                       "c3-d96": (32, 8, 96, 1011, "prefill_asm_kernel")}
 
 
 def bench_prefill_head(args, dev, name) -> dict:
-    """The c3 shape (32 x (2048 shared + 256 own) tokens, 16-token blocks, bf16) with 16 query / 8 kv heads of 256
-    or 32 query / 8 kv heads of 64: the chunked-prefill kernel for that head size alone, against the bf16
-    matrix-core peak."""
+    """The c3 shape (32 x (2048 shared + 256 own) tokens, 16-token blocks, bf16) with 16 query / 8 kv heads of 256,
+    or 32 query / 8 kv heads of 64 or 96: the chunked-prefill kernel for that head size alone, against the bf16
+    matrix-core peak (head_dim 96 runs the head_dim-128 kernel; its FLOP count is that of 96)."""
     from research_amd import ops
     from research_amd.workloads import make_prefill_c3
 
@@ -719,7 +721,7 @@ def secondary(args, dev) -> dict:
     short.copy_calibration = False
     short.secondary_run = True
     out = {}
-    for name in ("c2", "c5", "c3", "c3-d256", "c3-d64", "dense-64x512", "dense-4x8192", "long-d128", "long-d256"):
+    for name in ("c2", "c5", "c3", "c3-d256", "c3-d64", "c3-d96", "dense-64x512", "dense-4x8192", "long-d128", "long-d256"):
         r = (bench_prefill_c3(short, dev) if name == "c3" else bench_prefill_head(short, dev, name) if name in PREFILL_HEAD_SHAPES
              else bench_prefill_dense(short, dev, name) if name in PREFILL_DENSE_SHAPES
              else bench_prefill_long(short, dev, name) if name in PREFILL_LONG_SHAPES else bench_decode(name, short, dev))

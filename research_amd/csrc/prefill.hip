@@ -119,16 +119,21 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // workgroup (at most kPfTasks blocks of kPfRows) see; longer tables take the instance that fills its copy again on
     // the way.
     // (a chunk's rows of q and out are addressed by 32-bit byte offsets from the sequence's first row)
-    if (mfma && (head_dim == 128 || head_dim == 64 || head_dim == 32) && (block_size % 16 == 0 || bt_stride == 1) &&
+    // Head sizes between the compiled ones (multiples of 8) run the next larger instance: rows in memory keep their
+    // size, the chunks past a row's end are zero in Q^T and never stored (no pieces over a workspace for these).
+    const int d_pad = plan_pad_dim(head_dim);
+    const bool matrix_types = !force_rowwise && scale > 0.f && (dtype == PA_BF16 || dtype == PA_F16);
+    if (matrix_types && head_dim % 8 == 0 && (d_pad == 128 || d_pad == 64 || d_pad == 32) &&
+        (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
         bt_stride * (int64_t)block_size < (1ll << 31) &&
         (int64_t)max_q_len * num_q_heads * head_dim * 2 < (1ll << 31)) {
-        const int64_t cap_keys = (int64_t)pa_asm_cap_tiles(head_dim) * kPfKeys;
+        const int64_t cap_keys = (int64_t)pa_asm_cap_tiles(d_pad) * kPfKeys;
         const bool fits = bt_stride * (int64_t)block_size <= cap_keys ||
                           (window > 0 && (int64_t)window + kPfTasks * kPfRows + 3 * kPfKeys <= cap_keys);
         // With a workspace, a launch that cannot fill the chip has every workgroup's tiles cut into pieces (the
         // instance with lower bounds runs them: a piece is a later first tile and an earlier last key).
-        if (workspace) {
+        if (workspace && d_pad == head_dim) {
             const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
             const int64_t groups = (row_blocks * (int64_t)a.p.n_rep + kPfTasks - 1) / kPfTasks;
             int want = prefill_splits((int64_t)num_kv_heads * groups * batch, prefill_cus(),
@@ -137,7 +142,7 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
             split = want;
         }
         const bool lower_bounds = split > 1 || window > 0 || row_first_key != nullptr;
-        mfma = pa_prefill_asm_kernel(dtype, head_dim, lower_bounds, !fits);
+        mfma = pa_prefill_asm_kernel(dtype, d_pad, lower_bounds, !fits);
         if (!lower_bounds && fits) {
             // The plain instance runs several groups of one (sequence, kv head) per workgroup, which share the
             // set-up of lengths and slot tables: as many (up to 8) as leave a workgroup for every compute unit.

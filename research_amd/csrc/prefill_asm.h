@@ -106,9 +106,16 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     static_assert(kPfWaves * NC * 32 * QRB == 2 * kStageBytes, "the staged rows of the four waves fill two stages");
     static_assert(kPfWaves * 32 * QRB == kStageBytes, "one task's rows of the four waves fill one stage");
     // (32-bit byte offsets from the sequence's first row: the host checks that a chunk's rows span less than 2 GiB)
-    const uint32_t q_row_bytes = (uint32_t)p.hq * QRB;
+    // Head sizes between the compiled ones (p.d < D, a multiple of 8): rows in memory are p.d elements long, the
+    // kernel's rows D.  The 16-byte chunks past a row's end are requested from chunk 0 instead (any finite data
+    // does) and Q^T holds zeros there, so they add nothing to S^T; what they add to O^T is never stored.
+    const uint32_t row_bytes = (uint32_t)p.d * 2;       // a (token, head) row in memory
+    const uint32_t real_chunks = row_bytes / 16;        // its 16-byte chunks (<= QCPR)
+    const bool padded = real_chunks != (uint32_t)QCPR;  // uniform
+    auto real_chunk = [&](uint32_t chunk) PF_INLINE { return chunk < real_chunks ? chunk : 0u; };
+    const uint32_t q_row_bytes = (uint32_t)p.hq * row_bytes;
     const uint32_t q_last_row = (uint32_t)(q_len - 1) * q_row_bytes;
-    const char *q_seq = reinterpret_cast<const char *>(a.q) + (int64_t)q_start * p.hq * QRB;
+    const char *q_seq = reinterpret_cast<const char *>(a.q) + (int64_t)q_start * p.hq * row_bytes;
     auto issue_q = [&](int grp) PF_INLINE {
         const int lrow = lane / QCPR, lslot = lane % QCPR;
 #pragma unroll
@@ -117,7 +124,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             const bool lv = task < n_tasks;
             const int rb = lv ? task / p.n_rep : 0;
             const int qhead = kvh * p.n_rep + (lv ? task - rb * p.n_rep : 0);
-            const char *qb = pf_scalar_ptr(q_seq + qhead * QRB);
+            const char *qb = pf_scalar_ptr(q_seq + qhead * row_bytes);
             const uint32_t row_ofs = (uint32_t)(rb * kPfRows + lrow) * q_row_bytes;
 #pragma unroll
             for (int i = 0; i < 32 / QRPI; ++i) {
@@ -125,7 +132,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
                 // (rows past the chunk's end read its last row: they are computed and never stored)
                 const uint32_t ofs = min(row_ofs + (uint32_t)(i * QRPI) * q_row_bytes, q_last_row);
                 pf_dma16(lds_base + q_stage + (uint32_t)((c * 32 + i * QRPI) * QRB), qb,
-                         ofs + (uint32_t)((lslot ^ (r & (QCPR - 1))) * 16));
+                         ofs + real_chunk((uint32_t)(lslot ^ (r & (QCPR - 1)))) * 16);
             }
         }
     };
@@ -293,6 +300,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             uint32_t w[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) w[e] = M::pack((float)q8[2 * e] * sc, (float)q8[2 * e + 1] * sc);
+            if (padded && (uint32_t)(2 * ks + half) >= real_chunks) w[0] = w[1] = w[2] = w[3] = 0;  // past the row's end
             qreg[c][ks] = __builtin_bit_cast(X8, uint4{w[0], w[1], w[2], w[3]});
         }
 #pragma unroll
@@ -304,15 +312,15 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     int first_special = min(first_special_tab, n_tiles);  // (a group before the last runs fewer tiles than the tables hold)
 
     // ---- loads of a tile: wave w fetches rows w*RPL .. w*RPL + RPL-1 of the tile and, NG-1 times, the rows 4*RPL on ----
-    const int64_t tok_stride = (int64_t)p.hkv * D * 2;
-    const char *pool_k = reinterpret_cast<const char *>(p.k) + (int64_t)kvh * D * 2;
-    const char *pool_v = reinterpret_cast<const char *>(p.v) + (int64_t)kvh * D * 2;
+    const int64_t tok_stride = (int64_t)p.hkv * row_bytes;
+    const char *pool_k = reinterpret_cast<const char *>(p.k) + (int64_t)kvh * row_bytes;
+    const char *pool_v = reinterpret_cast<const char *>(p.v) + (int64_t)kvh * row_bytes;
     const int ld_row = lane / G::CPR, ld_slot = lane % G::CPR;
     const int tile_row = wave * G::RPL + ld_row;  // this lane's row of the tile in the wave's first load
     const int g0 = (wave * G::RPL) / 16;          // the 16-key group of that load; load n: group g0 + n * GSTEP
     const int arow = tile_row % 16;               // this lane's row inside its 16-key group
-    const uint32_t lane_k = (uint32_t)(arow * tok_stride) + (uint32_t)((ld_slot ^ G::swz_k(tile_row)) * 16);
-    const uint32_t lane_v = (uint32_t)(arow * tok_stride) + (uint32_t)((ld_slot ^ G::swz_v(tile_row)) * 16);
+    const uint32_t lane_k = (uint32_t)(arow * tok_stride) + real_chunk((uint32_t)(ld_slot ^ G::swz_k(tile_row))) * 16;
+    const uint32_t lane_v = (uint32_t)(arow * tok_stride) + real_chunk((uint32_t)(ld_slot ^ G::swz_v(tile_row))) * 16;
     const uint32_t m0w = lds_base + (uint32_t)wave * (G::RPL * G::RB);
     constexpr int kLoadStep = kPfWaves * G::RPL * G::RB;  // LDS bytes between a wave's consecutive loads
     static_assert(kLoadStep == 4096, "the assembly loops place a wave's loads 4 KiB apart");
@@ -639,7 +647,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
     // dropped, so every task costs exactly kStoresPerTask store instructions - the count the next group's wait
     // for its Q rows (requested before these stores) relies on.
     const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc(
-        (void *)(reinterpret_cast<T *>(a.out) + (int64_t)q_start * p.hq * D), 0, q_len * p.hq * (D * 2), 0x00020000);
+        (void *)(reinterpret_cast<char *>(a.out) + (int64_t)q_start * q_row_bytes), 0, q_len * (int)q_row_bytes, 0x00020000);
     prev_stores = 0;
 #pragma unroll
     for (int c = 0; c < NC; ++c) {
@@ -667,7 +675,10 @@ __global__ __launch_bounds__(kPfThreads) void prefill_asm_kernel(const RowwiseAr
             const int r = i * QRPI + r_in;
             rows[i] = *reinterpret_cast<const uint4 *>(s_mem + out_stage + r * QRB + ((chunk ^ (r & (QCPR - 1))) * 16));
         }
-        const int out_ofs = ((row0[c] + r_in) * p.hq + qh[c]) * (D * 2) + chunk * 16;
+        // (a chunk past the end of the row in memory gets an offset outside the descriptor: dropped)
+        const int out_ofs = (uint32_t)chunk < real_chunks
+                                ? (int)(((uint32_t)(row0[c] + r_in) * p.hq + qh[c]) * row_bytes) + chunk * 16
+                                : (int)0x80000000u;
 #pragma unroll
         for (int i = 0; i < 32 / QRPI; ++i)
             __builtin_amdgcn_raw_buffer_store_b128(pa_u4{rows[i].x, rows[i].y, rows[i].z, rows[i].w}, rout,

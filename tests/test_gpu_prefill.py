@@ -463,8 +463,8 @@ def test_logits_that_grow_along_the_context(d):
 @pytest.mark.parametrize("d,dtype,tol", [(80, torch.bfloat16, 2e-2), (96, torch.float16, 2e-2), (192, torch.bfloat16, 2e-2),
                                          (40, torch.float32, 1e-5), (112, torch.float32, 1e-5)])
 def test_chunked_prefill_other_head_sizes(d, dtype, tol):
-    """Head sizes between the compiled ones (multiples of 8 up to 256) take the vector kernel of the next larger
-    size: chunked prefill over a shared prefix, windows included."""
+    """Head sizes between the compiled ones (multiples of 8 up to 256) take the next larger size's kernel (the
+    vector kernel above 128 and for fp32): chunked prefill over a shared prefix, windows included."""
     announce(f"chunked prefill head_dim {d} {dtype}")
     w = make_prefill_c3(num_seqs=3, prefix_len=64, chunk_len=37, num_q_heads=6, num_kv_heads=2, head_dim=d, dtype=dtype)
     got, kc, vc = _run_chunked(w)
@@ -476,3 +476,48 @@ def test_chunked_prefill_other_head_sizes(d, dtype, tol):
     want = po.paged_prefill_chunk(w.q, kc.cpu(), vc.cpu(), w.block_tables, [64] * 3, [37] * 3, w.block_size, w.scale,
                                   window=20)
     assert_close(win.reshape(S, C, 6, d), want, tol, f"head_dim {d}, window 20")
+
+
+@pytest.mark.parametrize("d,dtype", [(96, torch.bfloat16), (72, torch.float16), (120, torch.bfloat16), (104, torch.float16),
+                                     (48, torch.bfloat16), (40, torch.float16), (56, torch.bfloat16),
+                                     (24, torch.bfloat16), (8, torch.float16), (16, torch.bfloat16)])
+def test_head_sizes_between_the_compiled_ones_on_the_matrix_cores(d, dtype):
+    """The reference takes any head_dim (attention/config.py:22-24).  Multiples of 8 below 128 run the assembly-loop
+    kernel of the next larger head size (rows in memory keep their size; the 16-byte chunks past a row's end are
+    zeros in Q^T and are never stored): dense rows of any length as one block per sequence (several groups per
+    workgroup, the group at the end of the pool), with packed documents and a window, and chunked prefill over a
+    shared prefix with ragged chunks - against the checker and against the vector kernel on the same inputs."""
+    announce(f"prefill on the matrix cores, head_dim {d} {dtype}")
+    rng = np.random.default_rng(d)
+    hq, hkv = 8, 2
+    for b, t, doc_lens in ((2, 333, (40, 200, 93)), (3, 6, (2, 4)), (1, 130, (130,))):
+        q, k, v = (torch.from_numpy(rng.standard_normal((b, t, h, d)).astype(np.float32)).to(dtype) for h in (hq, hkv, hkv))
+        ident = torch.arange(b, dtype=torch.int32, device=DEV).reshape(b, 1).contiguous()
+        lens = _i32([t] * b)
+        bounds = np.asarray(po.document_boundaries(doc_lens))
+        first = bounds[np.searchsorted(bounds[1:], np.arange(t), side="right")].astype(np.int32)
+        first = torch.from_numpy(np.tile(first, b)).to(DEV)
+        for docs, window in ((None, 0), (doc_lens, 0), (None, 40), (doc_lens, 40)):
+            args = (q.reshape(b * t, hq, d).to(DEV), k.reshape(b * t, hkv, d).to(DEV), v.reshape(b * t, hkv, d).to(DEV),
+                    ident, lens, lens, _i32(np.arange(b) * t), t, t, d ** -0.5)
+            # the output starts as a pattern: chunks past a row's end must not be stored anywhere
+            out = torch.full((b * t + 1, hq, d), 7.0, dtype=dtype, device=DEV)
+            got = ops.prefill_paged(*args, out=out[: b * t], window=window, row_first_key=first if docs else None)
+            assert (out[b * t] == 7.0).all(), "a store past the last row"
+            vec = ops.prefill_paged(*args, window=window, row_first_key=first if docs else None, rowwise=True)
+            want = po.dense_prefill(q, k, v, d ** -0.5, window=window, doc_lens=docs)
+            assert_close(got.reshape(b, t, hq, d), want, 2e-2, f"{b} x {t}, documents {docs}, window {window}")
+            assert_close(got.reshape(b, t, hq, d), vec.reshape(b, t, hq, d).cpu(), 2e-2, f"{b} x {t} against the vector kernel")
+    # chunked prefill over a shared prefix, ragged chunks and prefixes, 16-token blocks in random order
+    w = make_prefill_c3(num_seqs=3, prefix_len=208, chunk_len=77, num_q_heads=6, num_kv_heads=2, head_dim=d, dtype=dtype)
+    got, kc, vc = _run_chunked(w)
+    want = po.paged_prefill_chunk(w.q, kc.cpu(), vc.cpu(), w.block_tables, [208] * 3, [77] * 3, w.block_size, w.scale)
+    assert_close(got, want, 2e-2, f"chunked, head_dim {d}")
+    S, C = w.num_seqs, w.chunk_len
+    ctx, ql = [208 + 77, 208 + 30, 100 + 5], [77, 30, 5]
+    out = ops.prefill_paged(w.q.reshape(S * C, 6, d).to(DEV), kc, vc, tables_to_device(w.block_tables), _i32(ctx), _i32(ql),
+                            _i32(np.arange(S) * C), C, w.block_size, w.scale).reshape(S, C, 6, d)
+    want = po.paged_prefill_chunk(w.q, kc.cpu(), vc.cpu(), w.block_tables, [c - n for c, n in zip(ctx, ql)], ql,
+                                  w.block_size, w.scale)
+    for s_, n in enumerate(ql):
+        assert_close(out[s_, :n], want[s_, :n], 2e-2, f"ragged chunk {s_}, head_dim {d}")
