@@ -207,9 +207,9 @@ int pa_decode_static(const void *q, const void *k_cache, const void *v_cache, vo
  *   q, out   : [total_q][num_q_heads][head_dim] packed rows, sequence b's rows
  *              start at q_starts[b]; dtype PA_BF16 or PA_F16 (MFMA path) or
  *              PA_F32 (vector path)
- *   head_dim : a multiple of 8 up to 256.  bf16 / fp16 run on the matrix cores for 32, 64, 128, 256 and for
- *              every multiple of 8 below 128 (the kernel of the next larger size, rows in memory keep theirs);
- *              136 .. 248, and PA_F32, run on the vector kernel
+ *   head_dim : a multiple of 8 up to 256.  bf16 / fp16 run on the matrix cores: 32, 64, 128 and 256 have
+ *              kernels of their own, every other multiple of 8 runs the kernel of the next larger size (rows in
+ *              memory keep their length); PA_F32 runs on the vector kernel
  *   ctx_lens, q_lens, q_starts : int32[batch]
  *   max_q_len: upper bound of q_lens (grid sizing)
  *   window   : 0, or the sliding window of CacheConfig.sliding_window (attention/config.py:31): row i at

@@ -157,14 +157,14 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // again whenever the context is longer than what LDS can hold of it
     int tasks_per_wg = kPfTasks;
     // (a pool of fewer than 16 rows has no slot a whole group could be loaded from: the vector kernel)
-    if (!force_rowwise && scale > 0.f && head_dim == 256 && (block_size % 16 == 0 || bt_stride == 1) &&
+    if (matrix_types && head_dim % 8 == 0 && d_pad == 256 && (block_size % 16 == 0 || bt_stride == 1) &&
         num_blocks * (int64_t)block_size >= 16 && num_blocks * (int64_t)block_size < (1ll << 31) &&
         bt_stride * (int64_t)block_size < (1ll << 31)) {
         // (the tables hold kWdCapGroups groups of 16 keys from the workgroup's first tile on; under a sliding window
         // a workgroup's kWdTasks blocks of kPfRows rows, and the tiles its loads run ahead, bound what it needs)
         const bool fits = bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16 ||
                           (window > 0 && (int64_t)window + kWdTasks * kPfRows + 10 * 32 <= (int64_t)kWdCapGroups * 16);
-        if (workspace) {  // (as above; a workgroup of this kernel holds kWdTasks tasks)
+        if (workspace && head_dim == 256) {  // (as above; a workgroup of this kernel holds kWdTasks tasks)
             const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
             const int64_t groups = (row_blocks * (int64_t)a.p.n_rep + kWdTasks - 1) / kWdTasks;
             int want = prefill_splits((int64_t)num_kv_heads * groups * batch, prefill_cus(),

@@ -134,14 +134,22 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     // ---- Q^T operands, staged through the (still empty) ring as whole rows: see prefill_mfma_kernel ----
     constexpr int QRPI = 64 / CPR;  // rows per wave-wide load
     const uint32_t q_stage = (uint32_t)wave * (32 * RB);
+    // Head sizes between 128 and 256 (p.d < D, a multiple of 8): rows in memory are p.d elements long, the kernel's
+    // rows D.  The 16-byte chunks past a row's end are requested from chunk 0 instead (any finite data does) and
+    // Q^T holds zeros there, so they add nothing to S^T; what they add to O^T is never stored.
+    const int64_t row_bytes = (int64_t)p.d * 2;          // a (token, head) row in memory
+    const uint32_t real_chunks = (uint32_t)row_bytes / 16;  // its 16-byte chunks (<= CPR)
+    const bool padded = real_chunks != (uint32_t)CPR;       // uniform
+    auto real_chunk = [&](uint32_t chunk) PF_INLINE { return chunk < real_chunks ? chunk : 0u; };
     {
         const int lrow = lane / CPR, lslot = lane % CPR;
-        const char *qb = reinterpret_cast<const char *>(a.q) + ((int64_t)a.q_starts[b] * p.hq + qh) * RB;
+        const char *qb = reinterpret_cast<const char *>(a.q) + ((int64_t)a.q_starts[b] * p.hq + qh) * row_bytes;
 #pragma unroll
         for (int i = 0; i < 32 / QRPI; ++i) {
             const int r = i * QRPI + lrow;
             const int64_t grow = min(row0 + r, q_len - 1);
-            pf_dma16(lds_base + q_stage + (uint32_t)(i * QRPI * RB), qb + grow * p.hq * RB + ((lslot ^ (r & (CPR - 1))) * 16));
+            pf_dma16(lds_base + q_stage + (uint32_t)(i * QRPI * RB),
+                     qb + grow * p.hq * row_bytes + real_chunk((uint32_t)(lslot ^ (r & (CPR - 1)))) * 16);
         }
     }
     // ---- slot tables (in flight together with the Q rows) ----
@@ -215,6 +223,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
         uint32_t w[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) w[e] = M::pack((float)q8[2 * e] * p.scale_log2, (float)q8[2 * e + 1] * p.scale_log2);
+        if (padded && (uint32_t)(2 * ks + half) >= real_chunks) w[0] = w[1] = w[2] = w[3] = 0;  // past the row's end
         qreg[ks] = __builtin_bit_cast(X8, uint4{w[0], w[1], w[2], w[3]});
     }
 #pragma unroll
@@ -224,9 +233,9 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
     const int first_special = t0 + first_special_rel;
 
     // ---- loads: wave w fetches rows 8w .. 8w+7 of a stage's K and V, two rows (1 KiB) per direct load ----
-    const int64_t tok_stride = (int64_t)p.hkv * RB;
-    const char *pool_k = reinterpret_cast<const char *>(p.k) + (int64_t)kvh * RB;
-    const char *pool_v = reinterpret_cast<const char *>(p.v) + (int64_t)kvh * RB;
+    const int64_t tok_stride = (int64_t)p.hkv * row_bytes;
+    const char *pool_k = reinterpret_cast<const char *>(p.k) + (int64_t)kvh * row_bytes;
+    const char *pool_v = reinterpret_cast<const char *>(p.v) + (int64_t)kvh * row_bytes;
     const int ld_row = lane / CPR, ld_slot = lane % CPR;
     const int arow0 = (wave & 1) * 8 + ld_row;  // this lane's row inside its 16-key group for load 0; +2 per load
     // K: 16 consecutive rows read the same chunk -> chunk index swizzled by row % 16;
@@ -235,8 +244,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
 #pragma unroll
     for (int n = 0; n < NL; ++n) {
         const int r = arow0 + 2 * n;
-        lane_k[n] = (uint32_t)(r * tok_stride) + (uint32_t)((ld_slot ^ (r & 15)) * 16);
-        lane_v[n] = (uint32_t)(r * tok_stride) + (uint32_t)((ld_slot ^ ((r & 3) * 4)) * 16);
+        lane_k[n] = (uint32_t)(r * tok_stride) + real_chunk((uint32_t)(ld_slot ^ (r & 15))) * 16;
+        lane_v[n] = (uint32_t)(r * tok_stride) + real_chunk((uint32_t)(ld_slot ^ ((r & 3) * 4))) * 16;
     }
     const uint32_t wave_rows = (uint32_t)wave * (8 * RB);  // the wave's rows inside a tensor of a stage
     // table entry of the wave's group of tile `tile` (>= 0, at most kLookahead - 1 past the last tile)
@@ -496,7 +505,7 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             return;
         }
     }
-    T *orow = reinterpret_cast<T *>(a.out) + (((int64_t)a.q_starts[b] + row) * p.hq + qh) * D;
+    T *orow = reinterpret_cast<T *>(a.out) + (((int64_t)a.q_starts[b] + row) * p.hq + qh) * p.d;
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
@@ -504,7 +513,8 @@ __global__ __launch_bounds__(kPfThreads) void prefill_d256_kernel(const RowwiseA
             uint2 w;
             w.x = M::pack(o[dt][4 * g] * inv, o[dt][4 * g + 1] * inv);
             w.y = M::pack(o[dt][4 * g + 2] * inv, o[dt][4 * g + 3] * inv);
-            *reinterpret_cast<uint2 *>(orow + 32 * dt + 4 * half + 8 * g) = w;
+            // (p.d is a multiple of 8: the four elements lie on one side of the row's end)
+            if (32 * dt + 4 * half + 8 * g < p.d) *reinterpret_cast<uint2 *>(orow + 32 * dt + 4 * half + 8 * g) = w;
         }
 }
 

@@ -480,9 +480,10 @@ def test_chunked_prefill_other_head_sizes(d, dtype, tol):
 
 @pytest.mark.parametrize("d,dtype", [(96, torch.bfloat16), (72, torch.float16), (120, torch.bfloat16), (104, torch.float16),
                                      (48, torch.bfloat16), (40, torch.float16), (56, torch.bfloat16),
-                                     (24, torch.bfloat16), (8, torch.float16), (16, torch.bfloat16)])
+                                     (24, torch.bfloat16), (8, torch.float16), (16, torch.bfloat16),
+                                     (160, torch.bfloat16), (192, torch.float16), (248, torch.bfloat16), (136, torch.float16)])
 def test_head_sizes_between_the_compiled_ones_on_the_matrix_cores(d, dtype):
-    """The reference takes any head_dim (attention/config.py:22-24).  Multiples of 8 below 128 run the assembly-loop
+    """The reference takes any head_dim (attention/config.py:22-24).  Multiples of 8 up to 256 run the matrix-core
     kernel of the next larger head size (rows in memory keep their size; the 16-byte chunks past a row's end are
     zeros in Q^T and are never stored): dense rows of any length as one block per sequence (several groups per
     workgroup, the group at the end of the pool), with packed documents and a window, and chunked prefill over a
