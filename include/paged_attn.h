@@ -241,8 +241,9 @@ int pa_prefill_paged(const void *q, const void *k_cache, const void *v_cache, vo
  *                    NULL or too small for any split: the call is pa_prefill_paged.  A smaller workspace is used
  *                    for as many pieces as it holds.
  * pa_prefill_workspace_bytes: what the split the library would choose for these shapes on the current device needs
- * (0 when the launch fills the device anyway, or for shapes only the unsplit kernels take: fp32, head sizes other
- * than 32 / 64 / 128 / 256); host arithmetic plus one device-attribute query.
+ * (0 when the launch fills the device anyway, or for fp32, which only the unsplit vector kernel takes; a head size
+ * between 32 / 64 / 128 / 256 is sized for partial rows of the next larger one); host arithmetic plus one
+ * device-attribute query.
  * bt_stride * block_size bounds the context length the split is sized for.
  */
 size_t pa_prefill_workspace_bytes(int batch, int max_q_len, int64_t total_q, int64_t bt_stride, int block_size,

@@ -33,11 +33,12 @@ size_t prefill_ws_bytes(int64_t total_q, int num_q_heads, int head_dim, int spli
     return plan_prefill_ws_bytes(total_q, num_q_heads, head_dim, splits);
 }
 
-// Merge of the pieces of a split prefill launch: one thread per (row, head, four consecutive d).
+// Merge of the pieces of a split prefill launch: one thread per (row, head, four consecutive d).  The partial rows
+// are d_part floats long (the head size the kernel is compiled for), the output rows d_head elements.
 template <typename T>
 __global__ __launch_bounds__(256) void prefill_merge_kernel(const float *part_o, const float *part_ml, T *out,
                                                             const int32_t *q_lens, const int32_t *q_starts, int hq,
-                                                            int d_head, int splits) {
+                                                            int d_head, int d_part, int splits) {
     const int b = blockIdx.z, i = blockIdx.y;
     if (i >= q_lens[b]) return;
     const int item = blockIdx.x * 256 + threadIdx.x, v4 = d_head / 4;
@@ -53,7 +54,7 @@ __global__ __launch_bounds__(256) void prefill_merge_kernel(const float *part_o,
         const float l = part_ml[(base + s) * 2 + 1];
         if (!(l > 0.f)) continue;  // a piece in which the row saw no key wrote no O row
         const float w = __builtin_amdgcn_exp2f(part_ml[(base + s) * 2] - m_all);
-        const float4 o = *reinterpret_cast<const float4 *>(part_o + (base + s) * d_head + d);
+        const float4 o = *reinterpret_cast<const float4 *>(part_o + (base + s) * d_part + d);
         den = fmaf(w, l, den);
         num[0] = fmaf(w, o.x, num[0]);
         num[1] = fmaf(w, o.y, num[1]);
@@ -120,7 +121,7 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
     // the way.
     // (a chunk's rows of q and out are addressed by 32-bit byte offsets from the sequence's first row)
     // Head sizes between the compiled ones (multiples of 8) run the next larger instance: rows in memory keep their
-    // size, the chunks past a row's end are zero in Q^T and never stored (no pieces over a workspace for these).
+    // size, the chunks past a row's end are zero in Q^T and never stored.
     const int d_pad = plan_pad_dim(head_dim);
     const bool matrix_types = !force_rowwise && scale > 0.f && (dtype == PA_BF16 || dtype == PA_F16);
     if (matrix_types && head_dim % 8 == 0 && (d_pad == 128 || d_pad == 64 || d_pad == 32) &&
@@ -133,12 +134,12 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
                           (window > 0 && (int64_t)window + kPfTasks * kPfRows + 3 * kPfKeys <= cap_keys);
         // With a workspace, a launch that cannot fill the chip has every workgroup's tiles cut into pieces (the
         // instance with lower bounds runs them: a piece is a later first tile and an earlier last key).
-        if (workspace && d_pad == head_dim) {
+        if (workspace) {
             const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
             const int64_t groups = (row_blocks * (int64_t)a.p.n_rep + kPfTasks - 1) / kPfTasks;
             int want = prefill_splits((int64_t)num_kv_heads * groups * batch, prefill_cus(),
                                       window > 0 ? (int64_t)window + kPfTasks * kPfRows : bt_stride * (int64_t)block_size);
-            while (want > 1 && prefill_ws_bytes(total_q, num_q_heads, head_dim, want) > workspace_bytes) --want;
+            while (want > 1 && prefill_ws_bytes(total_q, num_q_heads, d_pad, want) > workspace_bytes) --want;
             split = want;
         }
         const bool lower_bounds = split > 1 || window > 0 || row_first_key != nullptr;
@@ -164,12 +165,12 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
         // a workgroup's kWdTasks blocks of kPfRows rows, and the tiles its loads run ahead, bound what it needs)
         const bool fits = bt_stride * (int64_t)block_size <= (int64_t)kWdCapGroups * 16 ||
                           (window > 0 && (int64_t)window + kWdTasks * kPfRows + 10 * 32 <= (int64_t)kWdCapGroups * 16);
-        if (workspace && head_dim == 256) {  // (as above; a workgroup of this kernel holds kWdTasks tasks)
+        if (workspace) {  // (as above; a workgroup of this kernel holds kWdTasks tasks)
             const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
             const int64_t groups = (row_blocks * (int64_t)a.p.n_rep + kWdTasks - 1) / kWdTasks;
             int want = prefill_splits((int64_t)num_kv_heads * groups * batch, prefill_cus(),
                                       window > 0 ? (int64_t)window + kWdTasks * kPfRows : bt_stride * (int64_t)block_size);
-            while (want > 1 && prefill_ws_bytes(total_q, num_q_heads, head_dim, want) > workspace_bytes) --want;
+            while (want > 1 && prefill_ws_bytes(total_q, num_q_heads, d_pad, want) > workspace_bytes) --want;
             split = want;
         }
         mfma = pa_prefill_d256_kernel(dtype, split > 1 || window > 0 || row_first_key != nullptr, !fits);
@@ -185,7 +186,7 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
             PA_REQUIRE(((uintptr_t)workspace & 255u) == 0, "workspace must be 256-byte aligned");
             a.splits = split;
             a.part_o = (float *)workspace;
-            a.part_ml = a.part_o + (size_t)total_q * num_q_heads * split * head_dim;
+            a.part_ml = a.part_o + (size_t)total_q * num_q_heads * split * d_pad;
         }
         mfma<<<dim3((unsigned)num_kv_heads, (unsigned)(groups * split), (unsigned)batch), dim3(kPfThreads), 0, s>>>(a);
         PA_CHECK_LAUNCH("pa_prefill_paged (matrix-core kernel)");
@@ -194,10 +195,10 @@ int prefill_launch(bool force_rowwise, const void *q, const void *k_cache, const
             const dim3 mg(gx, (unsigned)max_q_len, (unsigned)batch);
             if (dtype == PA_BF16)
                 prefill_merge_kernel<pa_bf16><<<mg, dim3(256), 0, s>>>(a.part_o, a.part_ml, (pa_bf16 *)out, q_lens, q_starts,
-                                                                     num_q_heads, head_dim, split);
+                                                                     num_q_heads, head_dim, d_pad, split);
             else
                 prefill_merge_kernel<pa_f16><<<mg, dim3(256), 0, s>>>(a.part_o, a.part_ml, (pa_f16 *)out, q_lens, q_starts,
-                                                                    num_q_heads, head_dim, split);
+                                                                    num_q_heads, head_dim, d_pad, split);
             PA_CHECK_LAUNCH("pa_prefill_paged_ws (merge of the pieces)");
         }
         return PA_OK;
@@ -230,17 +231,18 @@ extern "C" size_t pa_prefill_workspace_bytes(int batch, int max_q_len, int64_t t
         pa_fail(PA_ERR_INVALID_ARG, "pa_prefill_workspace_bytes: negative size or inconsistent head counts");
         return 0;
     }
-    // only the 16-bit kernels with the assembly loop (head_dim 32 / 64 / 128 / 256) split; everything else needs none
-    if ((dtype != PA_BF16 && dtype != PA_F16) ||
-        (head_dim != 256 && head_dim != 128 && head_dim != 64 && head_dim != 32) || batch == 0 || max_q_len == 0)
+    // only the 16-bit kernels with the assembly loop split (head_dim a multiple of 8 up to 256; the partial rows have
+    // the head size the kernel is compiled for); everything else needs none
+    if ((dtype != PA_BF16 && dtype != PA_F16) || head_dim % 8 != 0 || head_dim > 256 || batch == 0 || max_q_len == 0)
         return 0;
+    const int d_pad = plan_pad_dim(head_dim);
     const int n_rep = num_q_heads / num_kv_heads;
     const int row_blocks = (max_q_len + kPfRows - 1) / kPfRows;
-    const int tasks = head_dim == 256 ? kWdTasks : kPfTasks;
+    const int tasks = d_pad == 256 ? kWdTasks : kPfTasks;
     const int64_t groups = (row_blocks * (int64_t)n_rep + tasks - 1) / tasks;
     const int split = prefill_splits((int64_t)num_kv_heads * groups * batch, prefill_cus(),
                                      window > 0 ? (int64_t)window + tasks * kPfRows : bt_stride * (int64_t)block_size);
-    return prefill_ws_bytes(total_q, num_q_heads, head_dim, split);
+    return prefill_ws_bytes(total_q, num_q_heads, d_pad, split);
 }
 
 extern "C" int pa_prefill_paged_ws(PA_PREFILL_PARAMS, int64_t total_q, void *workspace, size_t workspace_bytes) {

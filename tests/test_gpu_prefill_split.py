@@ -60,7 +60,8 @@ class Case:
         ws = None
         if pieces is not None:
             want = ops.prefill_workspace_bytes(q, self.dev_tables, self.cmax, self.bs, self.hkv, window)
-            per_piece = n * self.cmax * self.hq * (self.d + 2) * 4
+            d_rows = next(x for x in (32, 64, 128, 256) if x >= self.d)  # partial rows have the kernel's head size
+            per_piece = n * self.cmax * self.hq * (d_rows + 2) * 4
             assert want >= pieces * per_piece, f"the library would cut this launch into {want // per_piece} pieces only"
             ws = torch.full((pieces * per_piece,), 0xFF, dtype=torch.uint8, device=DEV)  # NaN patterns: nothing is assumed
         out = torch.zeros_like(q)
@@ -78,7 +79,8 @@ class Case:
 @pytest.mark.parametrize("pieces", [2, 3, 8])
 @pytest.mark.parametrize("d,hq,hkv,dtype", [(128, 8, 2, torch.bfloat16), (64, 4, 1, torch.float16),
                                            (32, 4, 2, torch.bfloat16), (256, 4, 2, torch.bfloat16),
-                                           (256, 2, 1, torch.float16)])
+                                           (256, 2, 1, torch.float16), (96, 8, 2, torch.bfloat16),
+                                           (192, 4, 2, torch.float16), (40, 4, 1, torch.bfloat16)])
 def test_one_long_sequence_in_pieces(pieces, d, hq, hkv, dtype):
     announce(f"split prefill: one sequence, {pieces} pieces, d={d} {dtype}")
     c = Case([2900], [150], hq, hkv, d, dtype=dtype, seed=pieces + d)
@@ -137,11 +139,13 @@ def test_context_longer_than_the_kernel_tables_in_pieces():
 def test_workspace_rules():
     c = Case([2900], [150], 8, 2, 128, seed=1)
     q = c.q.reshape(150, 8, 128).to(DEV)
-    # a launch that fills the device needs no workspace; fp32 and other head sizes have no split kernel
+    # a launch that fills the device needs no workspace; fp32 has no split kernel; a head size between the compiled
+    # ones is sized for partial rows of the next larger one
     big = torch.zeros((64, 1024), dtype=torch.int32, device=DEV)
     assert ops.prefill_workspace_bytes(torch.empty((64 * 256, 32, 128), dtype=torch.bfloat16, device=DEV), big, 256, 16, 8) == 0
     assert ops.prefill_workspace_bytes(q.float(), c.dev_tables, 150, 16, 2) == 0
-    assert ops.prefill_workspace_bytes(torch.empty((150, 8, 96), dtype=torch.bfloat16, device=DEV), c.dev_tables, 150, 16, 2) == 0
+    assert (ops.prefill_workspace_bytes(torch.empty((150, 8, 96), dtype=torch.bfloat16, device=DEV), c.dev_tables, 150, 16, 2)
+            == ops.prefill_workspace_bytes(q, c.dev_tables, 150, 16, 2) > 0)
     # narrow tables (short contexts at most): no split either
     assert ops.prefill_workspace_bytes(q, c.dev_tables[:, :64].contiguous(), 150, 16, 2) == 0
     # a workspace too small for two pieces: the call is the unsplit one
