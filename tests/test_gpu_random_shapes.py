@@ -79,6 +79,43 @@ def test_random_decode(seed):
 
 
 @pytest.mark.parametrize("seed", range(16))
+def test_random_decode_head_sizes_between(seed):
+    """Decode with head sizes between the compiled ones (multiples of 8; of 16 for fp8 pools): the next larger
+    instance with the lanes past the row's end idle."""
+    rng = np.random.default_rng(7100 + seed)
+    _, hkv, n_rep, bs, kind, batch = _draw(rng)
+    d = int(rng.choice([16, 48, 80, 96, 112, 144, 160, 192, 208, 240] if kind == "fp8" else
+                       [8, 24, 40, 48, 56, 72, 80, 96, 104, 120, 136, 160, 192, 248]))
+    hq = hkv * n_rep
+    announce(f"random decode seed={seed} hq={hq} hkv={hkv} d={d} bs={bs} {kind} batch={batch}")
+    dtype = {"bf16": torch.bfloat16, "f16": torch.float16, "f32": torch.float32, "fp8": torch.bfloat16}[kind]
+    lens = rng.integers(0, 6 * max(bs, 16) + 1, batch).tolist()
+    if seed % 3 == 0:
+        lens[0] = int(rng.integers(300, 700))
+    tables, nb = _tables(rng, lens, bs)
+    k, v = _pool(rng, nb, bs, hkv, d, dtype)
+    q = torch.from_numpy(rng.standard_normal((batch, hq, d)).astype(np.float32)).to(dtype)
+    scale = d ** -0.5
+    window = int(rng.choice([0, 0, 1, 5, 40]))
+    if kind == "fp8":
+        if bs > 256:
+            pytest.skip("fp8 tile limits")
+        kb, ks = ops.quantize_kv_e4m3(k.to(DEV), bs)
+        vb, vs = ops.quantize_kv_e4m3(v.to(DEV), bs)
+        kref = po.dequantize_kv_e4m3(kb.cpu().view(torch.uint8), ks.cpu(), bs)
+        vref = po.dequantize_kv_e4m3(vb.cpu().view(torch.uint8), vs.cpu(), bs)
+        pools, extra, tol = (kb, vb), (ks, vs), 2e-2
+    else:
+        kref, vref, pools, extra = k, v, (k.to(DEV), v.to(DEV)), (None, None)
+        tol = 1e-5 if kind == "f32" else 2e-2
+    ws = ops.decode_workspace(q.to(DEV), pools[0])
+    got = ops.decode(q.to(DEV), *pools, tables_to_device(tables), torch.tensor(lens, dtype=torch.int32, device=DEV), bs,
+                     scale, ws, None, *extra, window=window)
+    want = po.paged_decode(q, kref, vref, tables, lens, bs, scale, window=window)
+    assert_close(got, want, tol, f"decode window={window}")
+
+
+@pytest.mark.parametrize("seed", range(16))
 def test_random_chunked_prefill(seed):
     rng = np.random.default_rng(9000 + seed)
     d, hkv, n_rep, bs, kind, batch = _draw(rng)
@@ -114,8 +151,18 @@ def test_random_matrix_core_prefill(seed):
     chunks, sliding windows, per-row first keys, absent blocks.  Every case against the vector kernel (which
     states the zero-row rule of absent blocks), cases without absent blocks and first keys also against the
     checker."""
-    rng = np.random.default_rng(9500 + seed)
-    d = int(rng.choice([32, 64, 128, 128, 256]))
+    _matrix_core_case(np.random.default_rng(9500 + seed), seed, [32, 64, 128, 128, 256])
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_matrix_core_prefill_head_sizes_between(seed):
+    """The same with head sizes between the compiled ones (multiples of 8): rows in memory shorter than the
+    kernel's, the reference's "any head_dim" (attention/config.py:22-24)."""
+    _matrix_core_case(np.random.default_rng(9600 + seed), seed, [8, 24, 40, 48, 56, 72, 80, 96, 104, 112, 120, 160, 192, 248])
+
+
+def _matrix_core_case(rng, seed, dims):
+    d = int(rng.choice(dims))
     hkv = int(rng.choice([1, 2, 4]))
     n_rep = int(rng.choice([1, 2, 3, 4, 8]))
     hq = hkv * n_rep
@@ -170,8 +217,17 @@ def test_random_dense_prefill_of_any_length(seed):
     of T rows with the identity table, T of any length (so 16-key groups run into the next sequence's rows and, at
     the end of the pool, past it), head sizes 32 / 64 / 128 / 256, with and without a sliding window; against the
     checker."""
-    rng = np.random.default_rng(9700 + seed)
-    d = int(rng.choice([32, 64, 128, 256]))
+    _dense_case(np.random.default_rng(9700 + seed), seed, [32, 64, 128, 256])
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_dense_prefill_head_sizes_between(seed):
+    """The same with head sizes between the compiled ones."""
+    _dense_case(np.random.default_rng(9800 + seed), seed, [8, 16, 40, 48, 72, 88, 96, 120, 136, 192, 224])
+
+
+def _dense_case(rng, seed, dims):
+    d = int(rng.choice(dims))
     hkv = int(rng.choice([1, 2, 4]))
     hq = hkv * int(rng.choice([1, 2, 4, 7]))
     dtype = torch.bfloat16 if rng.random() < 0.7 else torch.float16
